@@ -1,0 +1,112 @@
+// Shared definitions of the gfx950 kernel library: element types, conversions, wave and
+// block reductions, error reporting.  Wavefronts are 64 lanes wide throughout.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define BH_WAVE 64
+#define BH_PAGE 64  // tokens in one page of the key/value cache
+
+enum BhDtype { BH_F32 = 0, BH_BF16 = 1 };
+
+// bfloat16 kept as its 16 bits; widening is a shift, narrowing rounds to nearest even.
+struct bf16_t {
+  uint16_t bits;
+};
+
+__host__ __device__ inline float bf16_bits_to_f32(uint16_t bits) {
+  union {
+    uint32_t u;
+    float f;
+  } v;
+  v.u = ((uint32_t)bits) << 16;
+  return v.f;
+}
+
+__host__ __device__ inline uint16_t f32_to_bf16_bits(float f) {
+  union {
+    uint32_t u;
+    float f;
+  } v;
+  v.f = f;
+  if ((v.u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((v.u >> 16) | 0x0040u);  // quiet NaN
+  uint32_t rounding = 0x7fffu + ((v.u >> 16) & 1u);
+  return (uint16_t)((v.u + rounding) >> 16);
+}
+
+__device__ inline float to_f32(float x) { return x; }
+__device__ inline float to_f32(bf16_t x) { return bf16_bits_to_f32(x.bits); }
+
+template <typename T>
+__device__ inline T from_f32(float x);
+template <>
+__device__ inline float from_f32<float>(float x) {
+  return x;
+}
+template <>
+__device__ inline bf16_t from_f32<bf16_t>(float x) {
+  bf16_t r;
+  r.bits = f32_to_bf16_bits(x);
+  return r;
+}
+
+// ---- reductions -------------------------------------------------------------------------
+
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+  for (int off = BH_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, BH_WAVE);
+  return v;
+}
+
+__device__ inline float wave_max(float v) {
+#pragma unroll
+  for (int off = BH_WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, BH_WAVE));
+  return v;
+}
+
+// Block-wide sum; `scratch` holds at least blockDim.x / 64 floats.  Every thread gets the result.
+__device__ inline float block_sum(float v, float* scratch) {
+  const int lane = threadIdx.x & (BH_WAVE - 1), wave = threadIdx.x / BH_WAVE;
+  const int n_waves = (blockDim.x + BH_WAVE - 1) / BH_WAVE;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int i = 0; i < n_waves; ++i) total += scratch[i];
+  return total;
+}
+
+__device__ inline float block_max(float v, float* scratch) {
+  const int lane = threadIdx.x & (BH_WAVE - 1), wave = threadIdx.x / BH_WAVE;
+  const int n_waves = (blockDim.x + BH_WAVE - 1) / BH_WAVE;
+  v = wave_max(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = scratch[0];
+  for (int i = 1; i < n_waves; ++i) total = fmaxf(total, scratch[i]);
+  return total;
+}
+
+// ---- errors ------------------------------------------------------------------------------
+
+// Every entry point returns 0 on success; otherwise bh_last_error() gives the reason.
+int bh_fail(const char* format, ...);
+int bh_check_launch(const char* what);
+
+#define BH_REQUIRE(cond, ...)                  \
+  do {                                         \
+    if (!(cond)) return bh_fail(__VA_ARGS__);  \
+  } while (0)
+
+// The cache of one layer as the kernels see it: pages of BH_PAGE tokens,
+// laid [page][kv_head][token in page][head_dim], found through a per-sequence page table.
+struct BhPagedKV {
+  void* k_pages;
+  void* v_pages;
+  const int32_t* page_table;  // [n_seqs, table_stride]
+  int table_stride;
+  int n_pages;                // pages in the pool, for bounds checks on the host
+};

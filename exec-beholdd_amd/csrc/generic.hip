@@ -1,0 +1,408 @@
+// Kernels that take every size and both element types: embedding gather, RMSNorm, a tiled
+// FMA matrix product, per-head q/k norm + rotation + cache write, attention over the paged
+// cache, SwiGLU.  The float32 engine runs on these alone (true 32-bit arithmetic: plain FMA,
+// no matrix-core mode); the bfloat16 engine uses them wherever no faster kernel fits a size.
+// All reductions, norms, softmax and rotation are computed in float32.
+#include "common.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+
+// ---- errors ------------------------------------------------------------------------------
+
+static thread_local char g_error[512] = "";
+
+int bh_fail(const char* format, ...) {
+  va_list args;
+  va_start(args, format);
+  vsnprintf(g_error, sizeof(g_error), format, args);
+  va_end(args);
+  return 1;
+}
+
+int bh_check_launch(const char* what) {
+  hipError_t status = hipGetLastError();
+  if (status != hipSuccess) return bh_fail("%s: launch failed: %s", what, hipGetErrorString(status));
+  return 0;
+}
+
+extern "C" const char* bh_last_error() { return g_error; }
+extern "C" int bh_page_size() { return BH_PAGE; }
+
+// ---- embedding ---------------------------------------------------------------------------
+// hidden[row, :] = table[token[row], :], widened to float32.
+
+template <typename T>
+__global__ void embed_kernel(const int32_t* __restrict__ tokens, const T* __restrict__ table,
+                             float* __restrict__ out, int width) {
+  const int row = blockIdx.x;
+  const T* src = table + (size_t)tokens[row] * width;
+  float* dst = out + (size_t)row * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = to_f32(src[i]);
+}
+
+extern "C" int bh_embed(const int32_t* tokens, const void* table, int table_dtype, float* out,
+                        int n_rows, int width, hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && width > 0, "embed: rows %d and width %d must be positive", n_rows, width);
+  dim3 grid(n_rows), block(256);
+  if (table_dtype == BH_F32)
+    embed_kernel<float><<<grid, block, 0, stream>>>(tokens, (const float*)table, out, width);
+  else if (table_dtype == BH_BF16)
+    embed_kernel<bf16_t><<<grid, block, 0, stream>>>(tokens, (const bf16_t*)table, out, width);
+  else
+    return bh_fail("embed: unknown table dtype %d", table_dtype);
+  return bh_check_launch("embed");
+}
+
+// ---- RMSNorm -----------------------------------------------------------------------------
+// out[r, i] = (x[src, i] * inv) * w[i], inv = 1/sqrt(mean(x^2) + eps), src = rows ? rows[r] : r.
+
+template <typename TW, typename TO>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const int32_t* __restrict__ rows,
+                               const TW* __restrict__ w, TO* __restrict__ out, int width, float eps) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const int src = rows ? rows[r] : r;
+  const float* xr = x + (size_t)src * width;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float v = xr[i];
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+  TO* o = out + (size_t)r * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float y = xr[i] * inv;
+    if (w) y *= to_f32(w[i]);
+    o[i] = from_f32<TO>(y);
+  }
+}
+
+extern "C" int bh_rmsnorm(const float* x, const int32_t* rows, const void* w, int w_dtype, void* out,
+                          int out_dtype, int n_rows, int width, float eps, hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && width > 0, "rmsnorm: rows %d and width %d must be positive", n_rows, width);
+  BH_REQUIRE(eps >= 0.f, "rmsnorm: eps must not be negative");
+  dim3 grid(n_rows), block(width >= 2048 ? 512 : 256);
+#define BH_NORM(TW, TO) \
+  rmsnorm_kernel<TW, TO><<<grid, block, 0, stream>>>(x, rows, (const TW*)w, (TO*)out, width, eps)
+  if (w_dtype == BH_F32 && out_dtype == BH_F32) BH_NORM(float, float);
+  else if (w_dtype == BH_F32 && out_dtype == BH_BF16) BH_NORM(float, bf16_t);
+  else if (w_dtype == BH_BF16 && out_dtype == BH_F32) BH_NORM(bf16_t, float);
+  else if (w_dtype == BH_BF16 && out_dtype == BH_BF16) BH_NORM(bf16_t, bf16_t);
+  else return bh_fail("rmsnorm: unknown dtypes %d/%d", w_dtype, out_dtype);
+#undef BH_NORM
+  return bh_check_launch("rmsnorm");
+}
+
+// ---- matrix product, plain FMA -------------------------------------------------------------
+// C[M, N] (+)= A[M, K] * W[N, K]^T with float32 accumulation; 64x64 tile, 16-wide k slices.
+
+#define GT 64
+#define GK 16
+
+template <typename TA, typename TW, typename TC, bool ACCUMULATE>
+__global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict__ a, const TW* __restrict__ w,
+                                                           TC* __restrict__ c, int M, int N, int K) {
+  __shared__ float as[GK][GT + 1];
+  __shared__ float ws[GK][GT + 1];
+  const int tid = threadIdx.x;
+  const int m0 = blockIdx.y * GT, n0 = blockIdx.x * GT;
+  const int tx = tid % 16, ty = tid / 16;  // thread computes rows ty*4.., columns tx*4..
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < K; k0 += GK) {
+    // 64 rows x 16 k = 1024 elements per operand, 4 per thread
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int e = tid + i * 256;
+      const int r = e / GK, kk = e % GK;
+      const int gm = m0 + r, gn = n0 + r, gk = k0 + kk;
+      as[kk][r] = (gm < M && gk < K) ? to_f32(a[(size_t)gm * K + gk]) : 0.f;
+      ws[kk][r] = (gn < N && gk < K) ? to_f32(w[(size_t)gn * K + gk]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < GK; ++kk) {
+      float av[4], wv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) av[i] = as[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) wv[j] = ws[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int gm = m0 + ty * 4 + i;
+    if (gm >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int gn = n0 + tx * 4 + j;
+      if (gn >= N) continue;
+      const size_t at = (size_t)gm * N + gn;
+      float v = acc[i][j];
+      if (ACCUMULATE) v += to_f32(c[at]);
+      c[at] = from_f32<TC>(v);
+    }
+  }
+}
+
+template <typename TA, typename TW>
+static int gemm_generic_out(const void* a, const void* w, void* c, int c_dtype, int accumulate, int M, int N,
+                            int K, hipStream_t stream) {
+  dim3 grid((N + GT - 1) / GT, (M + GT - 1) / GT), block(256);
+#define BH_GEMM(TC, ACC) \
+  gemm_generic_kernel<TA, TW, TC, ACC><<<grid, block, 0, stream>>>((const TA*)a, (const TW*)w, (TC*)c, M, N, K)
+  if (c_dtype == BH_F32 && accumulate) BH_GEMM(float, true);
+  else if (c_dtype == BH_F32) BH_GEMM(float, false);
+  else if (c_dtype == BH_BF16 && accumulate) BH_GEMM(bf16_t, true);
+  else if (c_dtype == BH_BF16) BH_GEMM(bf16_t, false);
+  else return bh_fail("gemm: unknown output dtype %d", c_dtype);
+#undef BH_GEMM
+  return bh_check_launch("gemm_generic");
+}
+
+extern "C" int bh_gemm_generic(const void* a, int a_dtype, const void* w, int w_dtype, void* c, int c_dtype,
+                               int accumulate, int M, int N, int K, hipStream_t stream) {
+  BH_REQUIRE(M > 0 && N > 0 && K > 0, "gemm: sizes M=%d N=%d K=%d must be positive", M, N, K);
+  BH_REQUIRE((N + GT - 1) / GT <= 2147483647 && (M + GT - 1) / GT <= 65535,
+             "gemm: M=%d needs more than 65535 row tiles", M);
+  if (a_dtype == BH_F32 && w_dtype == BH_F32)
+    return gemm_generic_out<float, float>(a, w, c, c_dtype, accumulate, M, N, K, stream);
+  if (a_dtype == BH_BF16 && w_dtype == BH_BF16)
+    return gemm_generic_out<bf16_t, bf16_t>(a, w, c, c_dtype, accumulate, M, N, K, stream);
+  if (a_dtype == BH_BF16 && w_dtype == BH_F32)
+    return gemm_generic_out<bf16_t, float>(a, w, c, c_dtype, accumulate, M, N, K, stream);
+  if (a_dtype == BH_F32 && w_dtype == BH_BF16)
+    return gemm_generic_out<float, bf16_t>(a, w, c, c_dtype, accumulate, M, N, K, stream);
+  return bh_fail("gemm: unknown operand dtypes %d/%d", a_dtype, w_dtype);
+}
+
+// ---- q/k norm + rotation + cache write -------------------------------------------------------
+// One wave per (row, head) of the fused projection row [q heads | k heads | v heads].
+// q head: optional RMSNorm over the head, rotation at the row's position, written to q_out.
+// k head: the same, written into the cache page of (sequence, position).
+// v head: copied into the cache.  Rotation pairs are (i, i + rot/2) for i < rot/2; elements
+// from rot to head_dim pass through.  With write_kv == 0 only the q heads are processed.
+
+template <typename T, typename TW>
+__global__ __launch_bounds__(64) void qk_norm_rope_cache_kernel(
+    const T* __restrict__ qkv, T* __restrict__ q_out, const TW* __restrict__ q_weight,
+    const TW* __restrict__ k_weight, float eps, const float* __restrict__ cos_table,
+    const float* __restrict__ sin_table, int rot, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ row_seq, T* __restrict__ k_pages, T* __restrict__ v_pages,
+    const int32_t* __restrict__ page_table, int table_stride, int H, int KVH, int hd) {
+  const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const int fused = (H + 2 * KVH) * hd;
+  const T* src = qkv + (size_t)row * fused + (size_t)head * hd;
+  const int pos = positions[row];
+
+  T* dst;
+  const TW* weight;
+  bool is_value = false;
+  if (head < H) {
+    dst = q_out + ((size_t)row * H + head) * hd;
+    weight = q_weight;
+  } else {
+    const int seq = row_seq[row];
+    const int page = page_table[(size_t)seq * table_stride + pos / BH_PAGE];
+    const int kv_head = (head - H) % KVH;
+    is_value = head >= H + KVH;
+    T* pages = is_value ? v_pages : k_pages;
+    dst = pages + (((size_t)page * KVH + kv_head) * BH_PAGE + (pos % BH_PAGE)) * hd;
+    weight = k_weight;
+  }
+  if (is_value) {
+    for (int i = lane; i < hd; i += BH_WAVE) dst[i] = src[i];
+    return;
+  }
+  float inv = 1.f;
+  if (weight) {
+    float ss = 0.f;
+    for (int i = lane; i < hd; i += BH_WAVE) {
+      float v = to_f32(src[i]);
+      ss += v * v;
+    }
+    ss = wave_sum(ss);
+    inv = 1.0f / sqrtf(ss / (float)hd + eps);
+  }
+  const int half = rot / 2;
+  for (int i = lane; i < half; i += BH_WAVE) {
+    float a = to_f32(src[i]), b = to_f32(src[i + half]);
+    if (weight) {
+      a = a * inv * to_f32(weight[i]);
+      b = b * inv * to_f32(weight[i + half]);
+    }
+    float c = 1.f, s = 0.f;
+    if (cos_table) {
+      c = cos_table[(size_t)pos * half + i];
+      s = sin_table[(size_t)pos * half + i];
+    }
+    dst[i] = from_f32<T>(a * c - b * s);
+    dst[i + half] = from_f32<T>(a * s + b * c);
+  }
+  for (int i = rot + lane; i < hd; i += BH_WAVE) {
+    float a = to_f32(src[i]);
+    if (weight) a = a * inv * to_f32(weight[i]);
+    dst[i] = from_f32<T>(a);
+  }
+}
+
+extern "C" int bh_qk_norm_rope_cache(const void* qkv, int dtype, void* q_out, const void* q_weight,
+                                     const void* k_weight, int w_dtype, float eps, const float* cos_table,
+                                     const float* sin_table, int table_positions, int rot,
+                                     const int32_t* positions, const int32_t* row_seq, void* k_pages,
+                                     void* v_pages, const int32_t* page_table, int table_stride, int n_rows,
+                                     int H, int KVH, int hd, int write_kv, int max_position,
+                                     hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && H > 0 && KVH > 0 && hd > 0, "qk_norm_rope: sizes must be positive");
+  BH_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0, "qk_norm_rope: rotary width %d must be even and at most %d", rot, hd);
+  BH_REQUIRE((q_weight == nullptr) == (k_weight == nullptr), "qk_norm_rope: give both norm weights or neither");
+  BH_REQUIRE(cos_table == nullptr || max_position < table_positions,
+             "qk_norm_rope: position %d is outside the rotation table of %d positions", max_position, table_positions);
+  BH_REQUIRE(H + 2 * KVH <= 65535, "qk_norm_rope: too many heads");
+  if (cos_table == nullptr) rot = 0;
+  dim3 grid(n_rows, write_kv ? H + 2 * KVH : H), block(BH_WAVE);
+#define BH_QK(T, TW)                                                                                         \
+  qk_norm_rope_cache_kernel<T, TW><<<grid, block, 0, stream>>>(                                              \
+      (const T*)qkv, (T*)q_out, (const TW*)q_weight, (const TW*)k_weight, eps, cos_table, sin_table, rot,    \
+      positions, row_seq, (T*)k_pages, (T*)v_pages, page_table, table_stride, H, KVH, hd)
+  if (dtype == BH_F32 && w_dtype == BH_F32) BH_QK(float, float);
+  else if (dtype == BH_F32 && w_dtype == BH_BF16) BH_QK(float, bf16_t);
+  else if (dtype == BH_BF16 && w_dtype == BH_F32) BH_QK(bf16_t, float);
+  else if (dtype == BH_BF16 && w_dtype == BH_BF16) BH_QK(bf16_t, bf16_t);
+  else return bh_fail("qk_norm_rope: unknown dtypes %d/%d", dtype, w_dtype);
+#undef BH_QK
+  return bh_check_launch("qk_norm_rope_cache");
+}
+
+// ---- attention over the paged cache, any size -------------------------------------------------
+// One block per (row, query head).  The row at position p of sequence s sees keys
+// max(0, p - window + 1) .. p of that sequence (window 0: all of them).  Keys are taken 256
+// at a time: scores (one thread per key), running maximum and sum in float32 (online softmax),
+// then the value sum with threads spread over (key subset, dimension).
+
+#define AG_THREADS 256
+
+template <typename T>
+__global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
+    const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
+    const int32_t* __restrict__ page_table, int table_stride, const int32_t* __restrict__ row_seq,
+    const int32_t* __restrict__ positions, int H, int KVH, int hd, float scale, int window) {
+  extern __shared__ float smem[];
+  float* qs = smem;                    // [hd]
+  float* probs = qs + hd;              // [AG_THREADS]
+  float* partial = probs + AG_THREADS; // [AG_THREADS]
+  __shared__ float scratch[AG_THREADS / BH_WAVE];
+
+  const int row = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
+  const int kv_head = head / (H / KVH);
+  const int pos = positions[row];
+  const int32_t* table = page_table + (size_t)row_seq[row] * table_stride;
+  const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+
+  const T* qr = q + ((size_t)row * H + head) * hd;
+  for (int i = tid; i < hd; i += AG_THREADS) qs[i] = to_f32(qr[i]);
+  __syncthreads();
+
+  // value phase: groups of hd threads; group g takes keys g, g + n_groups, ... of a chunk
+  const int n_groups = AG_THREADS / hd > 0 ? AG_THREADS / hd : 1;
+  const int group = tid / hd, dim = tid % hd;
+  const bool value_thread = tid < n_groups * hd;  // hd <= AG_THREADS is checked on the host
+
+  float run_max = -INFINITY, run_sum = 0.f, acc = 0.f;
+  for (int c0 = first; c0 <= pos; c0 += AG_THREADS) {
+    const int j = c0 + tid;
+    float s = -INFINITY;
+    if (j <= pos) {
+      const int page = table[j / BH_PAGE];
+      const T* kr = k_pages + (((size_t)page * KVH + kv_head) * BH_PAGE + (j % BH_PAGE)) * hd;
+      float dot = 0.f;
+      for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], to_f32(kr[d]), dot);
+      s = dot * scale;
+    }
+    const float chunk_max = block_max(s, scratch);
+    const float new_max = fmaxf(run_max, chunk_max);
+    const float p = (j <= pos) ? expf(s - new_max) : 0.f;
+    probs[tid] = p;
+    const float chunk_sum = block_sum(p, scratch);  // its barriers also publish probs[]
+    const float alpha = (run_max == -INFINITY) ? 0.f : expf(run_max - new_max);
+    run_sum = run_sum * alpha + chunk_sum;
+    run_max = new_max;
+    if (value_thread) {
+      acc *= alpha;
+      const int n_keys = (pos - c0 + 1 < AG_THREADS) ? pos - c0 + 1 : AG_THREADS;
+      for (int jj = group; jj < n_keys; jj += n_groups) {
+        const int key = c0 + jj;
+        const int page = table[key / BH_PAGE];
+        const T* vr = v_pages + (((size_t)page * KVH + kv_head) * BH_PAGE + (key % BH_PAGE)) * hd;
+        acc = fmaf(probs[jj], to_f32(vr[dim]), acc);
+      }
+    }
+    __syncthreads();  // probs[] is rewritten by the next chunk
+  }
+  partial[tid] = value_thread ? acc : 0.f;
+  __syncthreads();
+  if (tid < hd) {
+    float total = 0.f;
+    for (int g = 0; g < n_groups; ++g) total += partial[g * hd + tid];
+    out[((size_t)row * H + head) * hd + tid] = from_f32<T>(total / run_sum);
+  }
+}
+
+extern "C" int bh_attention_generic(const void* q, void* out, int dtype, const void* k_pages,
+                                    const void* v_pages, const int32_t* page_table, int table_stride,
+                                    const int32_t* row_seq, const int32_t* positions, int n_rows, int H,
+                                    int KVH, int hd, float scale, int window, hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && H > 0 && KVH > 0 && hd > 0, "attention: sizes must be positive");
+  BH_REQUIRE(H % KVH == 0, "attention: %d query heads do not group evenly into %d kv heads", H, KVH);
+  BH_REQUIRE(hd <= AG_THREADS, "attention: head size %d is above the limit of %d", hd, AG_THREADS);
+  BH_REQUIRE(H <= 65535, "attention: too many heads");
+  BH_REQUIRE(window >= 0, "attention: window must not be negative");
+  dim3 grid(n_rows, H), block(AG_THREADS);
+  const size_t smem = (size_t)(hd + 2 * AG_THREADS) * sizeof(float);
+  if (dtype == BH_F32)
+    attention_generic_kernel<float><<<grid, block, smem, stream>>>(
+        (const float*)q, (float*)out, (const float*)k_pages, (const float*)v_pages, page_table, table_stride,
+        row_seq, positions, H, KVH, hd, scale, window);
+  else if (dtype == BH_BF16)
+    attention_generic_kernel<bf16_t><<<grid, block, smem, stream>>>(
+        (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_table,
+        table_stride, row_seq, positions, H, KVH, hd, scale, window);
+  else
+    return bh_fail("attention: unknown dtype %d", dtype);
+  return bh_check_launch("attention_generic");
+}
+
+// ---- SwiGLU ---------------------------------------------------------------------------------
+// out[r, i] = silu(gu[r, i]) * gu[r, F + i], silu(x) = x / (1 + exp(-x)).
+
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int F, size_t total) {
+  const size_t at = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (at >= total) return;
+  const size_t r = at / F;
+  const int i = (int)(at % F);
+  const float g = to_f32(gu[r * 2 * F + i]);
+  const float u = to_f32(gu[r * 2 * F + F + i]);
+  out[at] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+}
+
+extern "C" int bh_swiglu(const void* gu, void* out, int dtype, int n_rows, int F, hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && F > 0, "swiglu: sizes must be positive");
+  const size_t total = (size_t)n_rows * F;
+  const size_t blocks = (total + 255) / 256;
+  BH_REQUIRE(blocks <= 2147483647u, "swiglu: too many elements");
+  dim3 grid((unsigned)blocks), block(256);
+  if (dtype == BH_F32)
+    swiglu_kernel<float><<<grid, block, 0, stream>>>((const float*)gu, (float*)out, F, total);
+  else if (dtype == BH_BF16)
+    swiglu_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, F, total);
+  else
+    return bh_fail("swiglu: unknown dtype %d", dtype);
+  return bh_check_launch("swiglu");
+}

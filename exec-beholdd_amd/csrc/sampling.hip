@@ -1,0 +1,172 @@
+// Token selection from float32 logits, one block per row.
+//   temperature <= 0: argmax, ties to the lowest id.
+//   temperature  > 0: softmax(logits / temperature) in float32 with the maximum subtracted,
+//                     optionally restricted to the top_k largest logits and then to the
+//                     smallest set of most likely tokens whose mass reaches top_p (ties at a
+//                     threshold are kept), then an inverse-CDF draw with the caller's uniform
+//                     number in [0, 1).  Sums run in a fixed order, so a row's result does not
+//                     depend on the other rows.
+// A row with a non-finite logit sets bad[row] = 1 and selects nothing (token -1).
+#include "common.h"
+
+#define SB 1024  // threads per block
+
+__device__ inline uint32_t order_key(float x) {
+  uint32_t u = __float_as_uint(x);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+__global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ logits,
+                                                    const float* __restrict__ temperature,
+                                                    const int32_t* __restrict__ top_k,
+                                                    const float* __restrict__ top_p,
+                                                    const float* __restrict__ uniform,
+                                                    int32_t* __restrict__ tokens, int32_t* __restrict__ bad,
+                                                    int vocab) {
+  __shared__ float scratch[SB / BH_WAVE];
+  __shared__ float best_val[SB];
+  __shared__ int best_idx[SB];
+  __shared__ float prefix[SB + 1];
+  __shared__ int chosen;
+
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const float* x = logits + (size_t)row * vocab;
+
+  // pass 1: maximum with lowest-index ties, and the finiteness check
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  float not_finite = 0.f;
+  for (int i = tid; i < vocab; i += SB) {
+    const float v = x[i];
+    if (!isfinite(v)) not_finite = 1.f;
+    if (v > bv || bi == 0x7fffffff) {
+      bv = v;
+      bi = i;
+    }
+  }
+  not_finite = block_sum(not_finite, scratch);
+  if (not_finite > 0.f) {
+    if (tid == 0) {
+      tokens[row] = -1;
+      bad[row] = 1;
+    }
+    return;
+  }
+  best_val[tid] = bv;
+  best_idx[tid] = bi;
+  __syncthreads();
+  for (int stride = SB / 2; stride > 0; stride >>= 1) {
+    if (tid < stride) {
+      const float ov = best_val[tid + stride];
+      const int oi = best_idx[tid + stride];
+      if (ov > best_val[tid] || (ov == best_val[tid] && oi < best_idx[tid])) {
+        best_val[tid] = ov;
+        best_idx[tid] = oi;
+      }
+    }
+    __syncthreads();
+  }
+  const float max_logit = best_val[0];
+  const int arg_max = best_idx[0];
+  const float temp = temperature ? temperature[row] : 0.f;
+  if (!(temp > 0.f)) {
+    if (tid == 0) {
+      tokens[row] = arg_max;
+      bad[row] = 0;
+    }
+    return;
+  }
+  const float inv_temp = 1.0f / temp;
+
+  // top-k: the k-th largest logit, found bit by bit on the order-preserving integer key
+  uint32_t floor_key = 0;  // tokens with key >= floor_key are kept
+  const int k = top_k ? top_k[row] : 0;
+  if (k > 0 && k < vocab) {
+    uint32_t found = 0;
+    for (int bit = 31; bit >= 0; --bit) {
+      const uint32_t candidate = found | (1u << bit);
+      float count = 0.f;
+      for (int i = tid; i < vocab; i += SB) count += (order_key(x[i]) >= candidate) ? 1.f : 0.f;
+      count = block_sum(count, scratch);
+      if (count >= (float)k) found = candidate;
+    }
+    floor_key = found;
+  }
+
+  // each thread owns a contiguous range of the vocabulary
+  const int per = (vocab + SB - 1) / SB;
+  const int lo = tid * per < vocab ? tid * per : vocab;
+  const int hi = lo + per < vocab ? lo + per : vocab;
+
+  // top-p: the largest key threshold whose kept mass still reaches top_p of the total
+  const float p_keep = top_p ? top_p[row] : 1.f;
+  if (p_keep > 0.f && p_keep < 1.f) {
+    float total = 0.f;
+    for (int i = lo; i < hi; ++i)
+      if (order_key(x[i]) >= floor_key) total += expf((x[i] - max_logit) * inv_temp);
+    total = block_sum(total, scratch);
+    const float need = p_keep * total;
+    uint32_t found = 0;
+    for (int bit = 31; bit >= 0; --bit) {
+      const uint32_t candidate = found | (1u << bit);
+      float mass = 0.f;
+      if (candidate >= floor_key) {
+        for (int i = lo; i < hi; ++i)
+          if (order_key(x[i]) >= candidate) mass += expf((x[i] - max_logit) * inv_temp);
+      } else {
+        mass = 0.f;  // below the top-k floor nothing changes; handled by taking the floor below
+      }
+      mass = block_sum(mass, scratch);
+      if (candidate < floor_key || mass >= need) found = candidate;
+    }
+    if (found > floor_key) floor_key = found;
+  }
+
+  // inverse CDF over the kept tokens in index order
+  float mine = 0.f;
+  for (int i = lo; i < hi; ++i)
+    if (order_key(x[i]) >= floor_key) mine += expf((x[i] - max_logit) * inv_temp);
+  best_val[tid] = mine;
+  if (tid == 0) chosen = arg_max;
+  __syncthreads();
+  if (tid == 0) {
+    float running = 0.f;
+    for (int t = 0; t < SB; ++t) {
+      prefix[t] = running;
+      running += best_val[t];
+    }
+    prefix[SB] = running;
+  }
+  __syncthreads();
+  const float target = uniform[row] * prefix[SB];
+  const bool last_owner = (tid == SB - 1);
+  if (mine > 0.f && target >= prefix[tid] && (target < prefix[tid + 1] || last_owner)) {
+    float running = prefix[tid];
+    int pick = -1, last_kept = -1;
+    for (int i = lo; i < hi; ++i) {
+      if (order_key(x[i]) < floor_key) continue;
+      last_kept = i;
+      running += expf((x[i] - max_logit) * inv_temp);
+      if (running > target) {
+        pick = i;
+        break;
+      }
+    }
+    chosen = pick >= 0 ? pick : last_kept;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    tokens[row] = chosen;
+    bad[row] = 0;
+  }
+}
+
+extern "C" int bh_sample(const float* logits, const float* temperature, const int32_t* top_k,
+                         const float* top_p, const float* uniform, int32_t* tokens, int32_t* bad, int n_rows,
+                         int vocab, hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && vocab > 0, "sample: rows %d and vocabulary %d must be positive", n_rows, vocab);
+  BH_REQUIRE(temperature == nullptr || uniform != nullptr, "sample: temperature sampling needs uniform numbers");
+  sample_kernel<<<dim3(n_rows), dim3(SB), 0, stream>>>(logits, temperature, top_k, top_p, uniform, tokens, bad,
+                                                       vocab);
+  return bh_check_launch("sample");
+}

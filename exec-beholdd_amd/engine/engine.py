@@ -1,0 +1,170 @@
+"""The engine: a loaded model, its cache, the step function and generation above it.
+
+Construction follows the reference's load (crates/beholdd-runtime/src/native.rs:181-337):
+architecture tag -> model class, typed configuration, every tensor bound by name with its
+shape checked, byte accounting before allocation.  The Python entry point mirrors the
+reference's embedded API (crates/beholdd-embed/src/lib.rs:51-105): construct once,
+`generate(...)`, with token ids in place of text.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..cache import SequenceCache
+from ..config.base import read_config_json
+from ..registry import resolve_architecture
+from ..sampling import Sampler, SamplingParams
+from ..weights.binder import bind
+from ..weights.random_init import random_tensor_on_device
+from . import generation
+from .step import StepEntry, build_step
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
+
+
+def parse_dtype(name) -> torch.dtype:
+    if isinstance(name, torch.dtype):
+        if name not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"engine dtype must be bfloat16 or float32, got {name}")
+        return name
+    try:
+        return _DTYPES[str(name).lower()]
+    except KeyError:
+        raise ValueError(f"engine dtype must be bfloat16 or float32, got {name!r}") from None
+
+
+class Engine:
+    """`Engine(model_dir, dtype, max_tokens)`; then `step(...)` or `generate(...)`."""
+
+    def __init__(self, model_dir: str | None = None, dtype="bfloat16", max_tokens: int = 4096,
+                 max_slots: int | None = None, device="cuda:0", kernels=None, model=None,
+                 memory_limit_bytes: int | None = None):
+        self.dtype = parse_dtype(dtype)
+        self.device = torch.device(device)
+        if kernels is None:
+            from ..kernels import HipKernels   # fails loudly without a GPU or the library
+            kernels = HipKernels(self.device)
+        self.kernels = kernels
+        if model is None:
+            if model_dir is None:
+                raise ValueError("give a model folder or a built model")
+            model = load_model(model_dir, self.dtype, self.device)
+        self.model = model
+        self.config = model.config
+        self.cache = SequenceCache(model.entry_needs, max_tokens, self.dtype, self.device, kernels.page_size,
+                                   max_slots=max_slots, max_position=model.max_position)
+        self.cache_plan = self.cache.allocate(limit_bytes=memory_limit_bytes)
+        self.sampler = Sampler(kernels, self.device)
+
+    # ---- what the generation loop needs of a stepper ----
+    @property
+    def page_size(self) -> int:
+        return self.cache.page_size
+
+    @property
+    def capacity_pages(self) -> int:
+        return self.cache.n_pages
+
+    @property
+    def max_slots(self) -> int:
+        return self.cache.max_slots
+
+    @property
+    def max_position(self) -> int:
+        return self.cache.max_position
+
+    def alloc_slot(self) -> int:
+        return self.cache.alloc_slot()
+
+    def free_slot(self, slot: int) -> None:
+        self.cache.free_slot(slot)
+
+    def select(self, logits, params, requests, steps):
+        return self.sampler.select(logits, params, requests, steps)
+
+    # ---- the step function ----
+    def step(self, entries: list):
+        """Run the given tokens of each entry's sequence from the cache; return float32 logits
+        [wanted, vocab] in the order of the entries and of their `want` lists (None if nothing is
+        wanted).  On an error no sequence's length changes."""
+        entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
+        ctx, want_rows, requests = build_step(self.kernels, self.dtype, self.device, self.cache, entries,
+                                              self.model.vocab)
+        self.cache.reserve(requests)
+        try:
+            tables = self.cache.page_tables([slot for slot, _ in requests])
+            runs = self.model.schedule
+            writes = self.model.run_writes
+            entry_needs = self.model.entry_needs
+
+            def cache_for_run(run):
+                entry = runs[run][1]
+                if entry not in entry_needs or self.model.blocks[runs[run][0]].cache_need() is None:
+                    return None
+                return self.cache.layer_cache(entry, writes[run], tables)
+
+            logits = self.model.forward(ctx, cache_for_run, want_rows)
+        except BaseException:
+            self.cache.rollback(requests)
+            raise
+        self.cache.commit(requests)
+        return logits
+
+    # ---- generation ----
+    def generate(self, prompts: list, max_new_tokens=16, temperature: float = 0.0, top_k: int = 0,
+                 top_p: float = 1.0, seed: int = 0, stop_token_ids=(), on_token=None, batch_size=None,
+                 control=None, on_logits=None) -> list:
+        sampling = SamplingParams(temperature=temperature, top_k=top_k, top_p=top_p, seed=seed)
+        return generation.generate(self, prompts, max_new_tokens, sampling, stop_token_ids, on_token,
+                                   batch_size, control, on_logits)
+
+    def memory_plan(self) -> str:
+        weights = sum(t.numel() * t.element_size() for t in _model_tensors(self.model))
+        return f"weights: {weights} bytes\n{self.cache_plan.describe()}"
+
+
+def _model_tensors(model):
+    seen, out = set(), []
+
+    def visit(obj, depth=0):
+        if isinstance(obj, torch.Tensor):
+            if obj.data_ptr() not in seen:
+                seen.add(obj.data_ptr())
+                out.append(obj)
+        elif isinstance(obj, (list, tuple)):
+            for item in obj:
+                visit(item, depth + 1)
+        elif hasattr(obj, "__dict__") and depth < 6 and not isinstance(obj, type):
+            for value in vars(obj).values():
+                visit(value, depth + 1)
+
+    for part in model.parts():
+        visit(part)
+    return out
+
+
+def load_model(model_dir: str, dtype, device):
+    """config.json -> architecture -> model; model.safetensors -> its tensors, bound by name."""
+    dtype = parse_dtype(dtype)
+    data, path = read_config_json(model_dir)
+    entry = resolve_architecture(data, path)
+    config = entry.config_class.from_dict(data, path)
+    model = entry.build(config)
+    weights = bind(model.tensor_specs(), model_dir, dtype, device)
+    try:
+        model.load(weights, device)
+    finally:
+        weights.reader.close()
+    return model
+
+
+def random_model_on_device(config_dict: dict, seed: int, dtype, device):
+    """A model with seeded random weights drawn on the device (nothing is written to disk)."""
+    dtype = parse_dtype(dtype)
+    entry = resolve_architecture(config_dict)
+    config = entry.config_class.from_dict(config_dict)
+    model = entry.build(config)
+    specs = {spec.name: spec for spec in model.tensor_specs()}
+    model.load(lambda name: random_tensor_on_device(specs[name], seed, device, dtype), device)
+    return model

@@ -1,0 +1,146 @@
+"""The generation loop above the step function.
+
+For one sequence this is the reference's loop (crates/beholdd-model/src/qwen3moe/forward.rs:597-686):
+the whole prompt in one step, then one token per step; a selected stop token is reported but
+neither emitted, appended nor evaluated (:655-661); the last emitted token is never evaluated
+(:664), so a request needs prompt + max_new - 1 positions (:612-625); max_new = 0 returns at
+once without touching the model (:628-634).  Here a batch of sequences with unequal prompts
+runs together: all prompts in one step, then one token each; a sequence that ends leaves the
+batch and gives its slot back while the others go on; and requests beyond one batch run as
+one batch after another.
+
+The loop decides on the host and talks to the model only through a *stepper*:
+    stepper.page_size, stepper.capacity_pages, stepper.max_slots, stepper.max_position
+    stepper.alloc_slot() -> slot;  stepper.free_slot(slot)
+    stepper.step(entries: list[StepEntry]) -> logits (one row per entry that wants one)
+    stepper.select(logits, params, request_indices, steps) -> list[int]
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+from ..sampling import SamplingParams
+from .step import StepEntry
+
+FINISH_LENGTH = "length"     # the reference's MaxNewTokens -> Length (crates/beholdd-runtime/src/native.rs:662-665)
+FINISH_STOP = "stop"         # StopToken -> Stop
+
+
+class GenerationError(ValueError):
+    pass
+
+
+@dataclass
+class GenerationResult:
+    token_ids: list = field(default_factory=list)
+    finish_reason: str = FINISH_LENGTH
+    stop_token: int | None = None
+    prompt_tokens: int = 0
+
+    @property
+    def completion_tokens(self) -> int:
+        return len(self.token_ids)
+
+
+def positions_needed(prompt_len: int, max_new: int) -> int:
+    """Positions a request evaluates: the last selected token is never fed back."""
+    return prompt_len + max_new - (1 if max_new > 0 else 0)
+
+
+def plan_batches(prompt_lens: list, max_new: list, page_size: int, capacity_pages: int, max_slots: int,
+                 batch_size: int | None) -> list:
+    """Split requests, in order, into batches that fit the cache: lists of request indices."""
+    limit = min(max_slots, batch_size) if batch_size else max_slots
+    batches, current, pages = [], [], 0
+    for index, (n_prompt, n_new) in enumerate(zip(prompt_lens, max_new)):
+        if n_new == 0:
+            continue
+        need = -(-positions_needed(n_prompt, n_new) // page_size)
+        if need > capacity_pages:
+            raise GenerationError(
+                f"request {index} needs {need} cache pages of {page_size} tokens, the cache has {capacity_pages}")
+        if current and (len(current) >= limit or pages + need > capacity_pages):
+            batches.append(current)
+            current, pages = [], 0
+        current.append(index)
+        pages += need
+    if current:
+        batches.append(current)
+    return batches
+
+
+def generate(stepper, prompts: list, max_new_tokens, sampling=None, stop_token_ids=(), on_token=None,
+             batch_size: int | None = None, control=None, on_logits=None) -> list:
+    """Generate for every prompt (a list of token ids each).
+
+    `max_new_tokens` and `sampling` are one value for all requests or a list with one per
+    request.  `on_token(request_index, token)` is called for every emitted token in order;
+    `control()` is polled before every step and may raise to cancel;
+    `on_logits(request_index, step, logits_row)` sees the device row each token is chosen from.
+    """
+    n = len(prompts)
+    max_new = list(max_new_tokens) if isinstance(max_new_tokens, (list, tuple)) else [max_new_tokens] * n
+    if sampling is None:
+        sampling = SamplingParams()
+    params = list(sampling) if isinstance(sampling, (list, tuple)) else [sampling] * n
+    if len(max_new) != n or len(params) != n:
+        raise GenerationError("one max_new_tokens and one sampling parameter set per prompt")
+    stops = frozenset(int(t) for t in stop_token_ids)
+    for index, (prompt, n_new) in enumerate(zip(prompts, max_new)):
+        if len(prompt) == 0:
+            raise GenerationError(f"request {index}: generation requires at least one prompt token")
+        if n_new < 0:
+            raise GenerationError(f"request {index}: max_new_tokens must not be negative")
+        needed = positions_needed(len(prompt), n_new)
+        if needed > stepper.max_position:
+            raise GenerationError(
+                f"request {index}: prompt plus {n_new} generated tokens needs {needed} evaluated positions, "
+                f"exceeding the context of {stepper.max_position}")
+    results = [GenerationResult(prompt_tokens=len(p)) for p in prompts]
+    batches = plan_batches([len(p) for p in prompts], max_new, stepper.page_size, stepper.capacity_pages,
+                           stepper.max_slots, batch_size)
+    for batch in batches:
+        _run_batch(stepper, batch, prompts, max_new, params, stops, on_token, control, results, on_logits)
+    return results
+
+
+def _run_batch(stepper, batch, prompts, max_new, params, stops, on_token, control, results, on_logits):
+    slots = {}
+    try:
+        for index in batch:
+            slots[index] = stepper.alloc_slot()
+        if control is not None:
+            control()
+        live = list(batch)
+        logits = stepper.step([StepEntry(slots[i], list(prompts[i]), [len(prompts[i]) - 1]) for i in live])
+        step = 0
+        while live:
+            tokens = stepper.select(logits, [params[i] for i in live], live, [step] * len(live))
+            if on_logits is not None:
+                for row, index in enumerate(live):
+                    on_logits(index, step, logits[row])
+            going = []
+            for index, token in zip(live, tokens):
+                result = results[index]
+                if token in stops:
+                    result.finish_reason, result.stop_token = FINISH_STOP, token
+                else:
+                    if on_token is not None:
+                        on_token(index, token)
+                    result.token_ids.append(token)
+                    if len(result.token_ids) < max_new[index]:
+                        going.append((index, token))
+                        continue
+                    result.finish_reason = FINISH_LENGTH
+                stepper.free_slot(slots.pop(index))    # the sequence has ended; its slot is free at once
+            live = [index for index, _ in going]
+            if not live:
+                break
+            if control is not None:
+                control()
+            logits = stepper.step([StepEntry(slots[index], [token], [0]) for index, token in going])
+            step += 1
+    finally:
+        for slot in slots.values():
+            stepper.free_slot(slot)

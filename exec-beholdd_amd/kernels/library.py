@@ -1,0 +1,250 @@
+"""The hand-written gfx950 kernels as Python calls on torch tensors.
+
+`HipKernels` loads `libbeholdd_hip.so` (built from csrc/ on first use) through ctypes and
+checks every argument on the host (device, dtype, contiguity, shapes) before a kernel is
+launched: the kernels themselves trust their arguments.  There is no CPU path: without a GPU
+and the library, construction fails.
+
+Every method launches on torch's current HIP stream and returns nothing; results are written
+into the `out` tensors that the caller passes.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import build as _build
+
+F32, BF16 = 0, 1
+_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+class KernelError(RuntimeError):
+    """A kernel refused its arguments or could not be launched."""
+
+
+def _code(tensor: torch.Tensor, what: str) -> int:
+    code = _CODES.get(tensor.dtype)
+    if code is None:
+        raise KernelError(f"{what}: dtype {tensor.dtype} is not supported (float32 or bfloat16)")
+    return code
+
+
+class HipKernels:
+    """The kernel set of the product path."""
+
+    def __init__(self, device="cuda:0", verbose_build: bool = True):
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible to this process: the HIP kernel library has no CPU fallback")
+        self.device = torch.device(device)
+        if self.device.type != "cuda":
+            raise KernelError(f"the HIP kernel library runs on a GPU, not on {device!r}")
+        path = _build.ensure_built(verbose=verbose_build)
+        try:
+            self.lib = ctypes.CDLL(path)
+        except OSError as error:
+            raise KernelError(f"cannot load the HIP kernel library {path}: {error}") from None
+        self.library_path = path
+        self._declare()
+        self.page_size = int(self.lib.bh_page_size())
+
+    # ---- ctypes declarations ----
+    def _declare(self):
+        lib = self.lib
+        p, i, f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+        lib.bh_last_error.restype = ctypes.c_char_p
+        lib.bh_page_size.restype = i
+        table = {
+            "bh_embed": [p, p, i, p, i, i, p],
+            "bh_rmsnorm": [p, p, p, i, p, i, i, i, f, p],
+            "bh_gemm_generic": [p, i, p, i, p, i, i, i, i, i, p],
+            "bh_qk_norm_rope_cache": [p, i, p, p, p, i, f, p, p, i, i, p, p, p, p, p, i, i, i, i, i, i, i, p],
+            "bh_attention_generic": [p, p, i, p, p, p, i, p, p, i, i, i, i, f, i, p],
+            "bh_swiglu": [p, p, i, i, i, p],
+            "bh_sample": [p, p, p, p, p, p, p, i, i, p],
+        }
+        for name, argtypes in table.items():
+            function = getattr(lib, name)
+            function.argtypes = argtypes
+            function.restype = i
+        self._optional = {}
+        for name, argtypes in {
+            "bh_gemm_bf16": [p, p, p, i, i, i, i, i, p],
+            "bh_attention_prefill_bf16": [p, p, p, p, p, i, p, p, p, i, i, i, i, i, f, i, p],
+            "bh_attention_decode_bf16": [p, p, p, p, p, i, p, p, p, i, i, i, i, i, f, i, p],
+        }.items():
+            function = getattr(lib, name, None)
+            if function is not None:
+                function.argtypes = argtypes
+                function.restype = i
+                self._optional[name] = function
+
+    # ---- helpers ----
+    def _stream(self):
+        return ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+
+    def _check(self, status: int):
+        if status != 0:
+            raise KernelError(self.lib.bh_last_error().decode("utf-8", "replace"))
+
+    def _ptr(self, tensor, what: str, dtypes=None, optional: bool = False):
+        if tensor is None:
+            if optional:
+                return None
+            raise KernelError(f"{what}: tensor is required")
+        if not isinstance(tensor, torch.Tensor) or tensor.device != self.device:
+            raise KernelError(f"{what}: expected a tensor on {self.device}, got "
+                              f"{getattr(tensor, 'device', type(tensor))}")
+        if not tensor.is_contiguous():
+            raise KernelError(f"{what}: tensor must be contiguous")
+        if dtypes is not None and tensor.dtype not in dtypes:
+            raise KernelError(f"{what}: dtype {tensor.dtype} is not one of {dtypes}")
+        return ctypes.c_void_p(tensor.data_ptr())
+
+    # ---- kernels ----
+    def embed(self, tokens, table, out):
+        """out[row] = table[tokens[row]] widened to float32; tokens int32 [T], table [V, D], out f32 [T, D]."""
+        n_rows, width = out.shape
+        if tokens.shape != (n_rows,) or table.dim() != 2 or table.shape[1] != width:
+            raise KernelError(f"embed: shapes tokens {tuple(tokens.shape)}, table {tuple(table.shape)}, "
+                              f"out {tuple(out.shape)} do not fit")
+        self._check(self.lib.bh_embed(
+            self._ptr(tokens, "embed tokens", (torch.int32,)), self._ptr(table, "embed table"),
+            _code(table, "embed table"), self._ptr(out, "embed out", (torch.float32,)), n_rows, width,
+            self._stream()))
+
+    def rmsnorm(self, x, weight, eps, out, rows=None):
+        """out[r] = x[rows[r] if rows is given else r] * inv_rms * weight; x f32 [*, D], out [n, D]."""
+        n_rows, width = out.shape
+        if x.dim() != 2 or x.shape[1] != width or (weight is not None and weight.shape != (width,)):
+            raise KernelError(f"rmsnorm: shapes x {tuple(x.shape)}, out {tuple(out.shape)} do not fit")
+        if rows is None:
+            if x.shape[0] != n_rows:
+                raise KernelError(f"rmsnorm: {x.shape[0]} input rows for {n_rows} output rows")
+        elif rows.shape != (n_rows,):
+            raise KernelError(f"rmsnorm: {tuple(rows.shape)} row indices for {n_rows} output rows")
+        self._check(self.lib.bh_rmsnorm(
+            self._ptr(x, "rmsnorm x", (torch.float32,)), self._ptr(rows, "rmsnorm rows", (torch.int32,), True),
+            self._ptr(weight, "rmsnorm weight", None, True), _code(weight, "rmsnorm weight") if weight is not None else F32,
+            self._ptr(out, "rmsnorm out"), _code(out, "rmsnorm out"), n_rows, width, float(eps), self._stream()))
+
+    def gemm(self, a, w, out, accumulate=False):
+        """out[M, N] (+)= a[M, K] @ w[N, K]^T with float32 accumulation."""
+        if a.dim() != 2 or w.dim() != 2 or out.dim() != 2:
+            raise KernelError("gemm: operands must be matrices")
+        m, k = a.shape
+        n = w.shape[0]
+        if w.shape[1] != k or out.shape != (m, n):
+            raise KernelError(f"gemm: shapes a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
+        fast = self._optional.get("bh_gemm_bf16")
+        if (fast is not None and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and k % 8 == 0):
+            self._check(fast(self._ptr(a, "gemm a"), self._ptr(w, "gemm w"), self._ptr(out, "gemm out"),
+                             _code(out, "gemm out"), int(bool(accumulate)), m, n, k, self._stream()))
+            return
+        self._check(self.lib.bh_gemm_generic(
+            self._ptr(a, "gemm a"), _code(a, "gemm a"), self._ptr(w, "gemm w"), _code(w, "gemm w"),
+            self._ptr(out, "gemm out"), _code(out, "gemm out"), int(bool(accumulate)), m, n, k, self._stream()))
+
+    def qk_norm_rope_cache(self, qkv, q_out, q_weight, k_weight, eps, cos, sin, positions, row_seq,
+                           k_pages, v_pages, page_table, n_heads, n_kv_heads, head_dim, write_kv, max_position):
+        """Per head of the fused [q | k | v] projection rows: RMSNorm (when weights are given),
+        split-half rotation at the row's position (when tables are given), then q to `q_out`
+        and k, v into the cache pages of (sequence, position)."""
+        n_rows = qkv.shape[0]
+        fused = (n_heads + 2 * n_kv_heads) * head_dim
+        if qkv.shape != (n_rows, fused) or q_out.shape != (n_rows, n_heads * head_dim) or q_out.dtype != qkv.dtype:
+            raise KernelError(f"qk_norm_rope: shapes qkv {tuple(qkv.shape)}, q_out {tuple(q_out.shape)} do not fit "
+                              f"{n_heads}+2x{n_kv_heads} heads of {head_dim}")
+        if positions.shape != (n_rows,) or row_seq.shape != (n_rows,):
+            raise KernelError("qk_norm_rope: positions and row_seq must have one entry per row")
+        rot, table_positions = 0, 0
+        if cos is not None:
+            if cos.shape != sin.shape or cos.dim() != 2:
+                raise KernelError("qk_norm_rope: cos and sin tables must be matrices of one shape")
+            table_positions, rot = cos.shape[0], 2 * cos.shape[1]
+        if (q_weight is None) != (k_weight is None):
+            raise KernelError("qk_norm_rope: give both norm weights or neither")
+        w_code = F32
+        if q_weight is not None:
+            if q_weight.shape != (head_dim,) or k_weight.shape != (head_dim,) or q_weight.dtype != k_weight.dtype:
+                raise KernelError("qk_norm_rope: norm weights must be [head_dim] and of one dtype")
+            w_code = _code(q_weight, "qk_norm_rope weight")
+        self._check_pages(k_pages, v_pages, page_table, n_kv_heads, head_dim, qkv.dtype, "qk_norm_rope")
+        self._check(self.lib.bh_qk_norm_rope_cache(
+            self._ptr(qkv, "qkv"), _code(qkv, "qkv"), self._ptr(q_out, "q_out"),
+            self._ptr(q_weight, "q_norm", None, True), self._ptr(k_weight, "k_norm", None, True), w_code,
+            float(eps), self._ptr(cos, "cos", (torch.float32,), True), self._ptr(sin, "sin", (torch.float32,), True),
+            table_positions, rot, self._ptr(positions, "positions", (torch.int32,)),
+            self._ptr(row_seq, "row_seq", (torch.int32,)), self._ptr(k_pages, "k_pages"), self._ptr(v_pages, "v_pages"),
+            self._ptr(page_table, "page_table", (torch.int32,)), page_table.shape[1], n_rows, n_heads, n_kv_heads,
+            head_dim, int(bool(write_kv)), int(max_position), self._stream()))
+
+    def _check_pages(self, k_pages, v_pages, page_table, n_kv_heads, head_dim, dtype, what):
+        expected = (k_pages.shape[0], n_kv_heads, self.page_size, head_dim)
+        if k_pages.shape != expected or v_pages.shape != expected:
+            raise KernelError(f"{what}: cache pages must be [pages, {n_kv_heads}, {self.page_size}, {head_dim}], got "
+                              f"{tuple(k_pages.shape)} and {tuple(v_pages.shape)}")
+        if k_pages.dtype != dtype or v_pages.dtype != dtype:
+            raise KernelError(f"{what}: cache dtype {k_pages.dtype} differs from the activations' {dtype}")
+        if page_table.dim() != 2:
+            raise KernelError(f"{what}: the page table must be [sequences, pages]")
+
+    def attention(self, q, out, k_pages, v_pages, page_table, row_seq, positions, n_heads, n_kv_heads, head_dim,
+                  scale, window=0, layout=None):
+        """out[row, head] = softmax(q . K * scale) V over the keys of the row's sequence that the row
+        may see: positions max(0, p - window + 1) .. p (window 0 = all).  `layout`, when given,
+        describes how rows group into sequences so that a faster kernel can be chosen."""
+        n_rows = q.shape[0]
+        if q.shape != (n_rows, n_heads * head_dim) or out.shape != q.shape or out.dtype != q.dtype:
+            raise KernelError(f"attention: shapes q {tuple(q.shape)}, out {tuple(out.shape)} do not fit")
+        if n_heads % n_kv_heads != 0:
+            raise KernelError(f"attention: {n_heads} query heads do not group evenly into {n_kv_heads} kv heads")
+        if positions.shape != (n_rows,) or row_seq.shape != (n_rows,):
+            raise KernelError("attention: positions and row_seq must have one entry per row")
+        self._check_pages(k_pages, v_pages, page_table, n_kv_heads, head_dim, q.dtype, "attention")
+        common = (self._ptr(q, "q"), self._ptr(out, "attention out"))
+        if q.dtype == torch.bfloat16 and layout is not None and head_dim % 16 == 0:
+            name = "bh_attention_decode_bf16" if layout.is_decode else "bh_attention_prefill_bf16"
+            fast = self._optional.get(name)
+            if fast is not None and head_dim in (64, 128):
+                self._check(fast(*common, self._ptr(k_pages, "k_pages"), self._ptr(v_pages, "v_pages"),
+                                 self._ptr(page_table, "page_table", (torch.int32,)), page_table.shape[1],
+                                 self._ptr(row_seq, "row_seq", (torch.int32,)),
+                                 self._ptr(positions, "positions", (torch.int32,)),
+                                 self._ptr(layout.seq_start, "seq_start", (torch.int32,)), layout.n_seqs,
+                                 n_rows, n_heads, n_kv_heads, head_dim, float(scale), int(window), self._stream()))
+                return
+        self._check(self.lib.bh_attention_generic(
+            *common, _code(q, "q"), self._ptr(k_pages, "k_pages"), self._ptr(v_pages, "v_pages"),
+            self._ptr(page_table, "page_table", (torch.int32,)), page_table.shape[1],
+            self._ptr(row_seq, "row_seq", (torch.int32,)), self._ptr(positions, "positions", (torch.int32,)),
+            n_rows, n_heads, n_kv_heads, head_dim, float(scale), int(window), self._stream()))
+
+    def swiglu(self, gate_up, out):
+        """out[r, i] = silu(gate_up[r, i]) * gate_up[r, F + i]."""
+        n_rows, width = out.shape
+        if gate_up.shape != (n_rows, 2 * width) or gate_up.dtype != out.dtype:
+            raise KernelError(f"swiglu: shapes {tuple(gate_up.shape)} -> {tuple(out.shape)} do not fit")
+        self._check(self.lib.bh_swiglu(self._ptr(gate_up, "gate_up"), self._ptr(out, "swiglu out"),
+                                       _code(out, "swiglu out"), n_rows, width, self._stream()))
+
+    def sample(self, logits, tokens, bad, temperature=None, top_k=None, top_p=None, uniform=None):
+        """tokens[row] = argmax (temperature absent or <= 0) or a draw from the tempered, filtered
+        distribution; bad[row] = 1 where a logit is not finite."""
+        n_rows, vocab = logits.shape
+        for name, tensor, dtype in (("tokens", tokens, torch.int32), ("bad", bad, torch.int32)):
+            if tensor.shape != (n_rows,) or tensor.dtype != dtype:
+                raise KernelError(f"sample: {name} must be {dtype} [{n_rows}]")
+        for name, tensor, dtype in (("temperature", temperature, torch.float32), ("top_k", top_k, torch.int32),
+                                    ("top_p", top_p, torch.float32), ("uniform", uniform, torch.float32)):
+            if tensor is not None and (tensor.shape != (n_rows,) or tensor.dtype != dtype):
+                raise KernelError(f"sample: {name} must be {dtype} [{n_rows}]")
+        if temperature is not None and uniform is None:
+            raise KernelError("sample: temperature sampling needs uniform numbers")
+        self._check(self.lib.bh_sample(
+            self._ptr(logits, "logits", (torch.float32,)), self._ptr(temperature, "temperature", None, True),
+            self._ptr(top_k, "top_k", None, True), self._ptr(top_p, "top_p", None, True),
+            self._ptr(uniform, "uniform", None, True), self._ptr(tokens, "tokens"), self._ptr(bad, "bad"),
+            n_rows, vocab, self._stream()))

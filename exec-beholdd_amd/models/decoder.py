@@ -1,0 +1,93 @@
+"""A decoder as data: embedding, a list of blocks, the order in which they run, final norm, head.
+
+The configuration supplies, layer by layer, the names of the parts (`layer_kinds()`) and the
+order of execution (`schedule()`): a list of (layer index, cache entry index).  A layer may be
+named twice (its weights run twice, each run with a cache entry of its own), and an entry may
+be shared: the first run that names an entry writes it, later runs read it.
+The whole-model order follows the reference: embed, every layer, then final norm and head on
+the rows that are asked for (crates/beholdd-model/src/qwen3moe/forward.rs:811-915, :1416-1455).
+"""
+
+from __future__ import annotations
+
+from ..parts.base import BLOCKS, NORMS, POSITION_ENCODINGS
+from ..parts.embedding import Embedding, LMHead
+
+
+class DecoderModel:
+    def __init__(self, config, embedding, blocks, schedule, final_norm, head, shared_parts=()):
+        self.config = config
+        self.embedding, self.blocks, self.final_norm, self.head = embedding, list(blocks), final_norm, head
+        self.shared_parts = list(shared_parts)
+        self.schedule = [(int(layer), int(entry)) for layer, entry in schedule]
+        for layer, entry in self.schedule:
+            if not 0 <= layer < len(self.blocks):
+                raise ValueError(f"the schedule names layer {layer}, the model has {len(self.blocks)}")
+            if entry < 0:
+                raise ValueError("cache entry indices are not negative")
+        # entry -> need, and which scheduled run owns (writes) each entry
+        self.entry_needs: dict = {}
+        self.run_writes: list = []
+        for layer, entry in self.schedule:
+            need = self.blocks[layer].cache_need()
+            if need is None:
+                self.run_writes.append(False)
+                continue
+            if entry in self.entry_needs:
+                if self.entry_needs[entry] != need:
+                    raise ValueError(f"cache entry {entry} is shared by layers with different needs")
+                self.run_writes.append(False)
+            else:
+                self.entry_needs[entry] = need
+                self.run_writes.append(True)
+
+    @property
+    def vocab(self) -> int:
+        return self.embedding.vocab
+
+    @property
+    def max_position(self) -> int:
+        return self.config.max_position
+
+    def parts(self):
+        return [self.embedding, *self.shared_parts, *self.blocks, self.final_norm, self.head]
+
+    def tensor_specs(self):
+        return [spec for part in self.parts() for spec in part.tensor_specs()]
+
+    def load(self, get, device):
+        for part in self.parts():
+            part.load(get)
+        for part in self.shared_parts:
+            if hasattr(part, "build_tables"):
+                part.build_tables(device)
+
+    def forward(self, ctx, cache_for_run, want_rows):
+        """Run one step.  `cache_for_run(i)` gives the LayerCache of the i-th scheduled run (or
+        None); `want_rows` (int32 device tensor, may be empty) lists the rows whose logits are
+        returned as float32 [len(want_rows), vocab]."""
+        hidden = self.embedding.forward(ctx)
+        for run, (layer, _entry) in enumerate(self.schedule):
+            self.blocks[layer].forward(ctx, hidden, cache_for_run(run))
+        if want_rows is None or want_rows.numel() == 0:
+            return None
+        return self.head.forward(ctx, self.final_norm.forward(ctx, hidden, rows=want_rows))
+
+
+def build_decoder(config, position_encoding: str = "rope", layer_prefix: str = "model.layers.{}.",
+                  embedding_name: str = "model.embed_tokens.weight", final_norm_name: str = "model.norm.weight",
+                  head_name: str = "lm_head.weight", final_norm_kind: str = "rmsnorm") -> DecoderModel:
+    """Put a decoder together from the registered parts that `config` names."""
+    shared = {}
+    shared["position_encoding"] = POSITION_ENCODINGS.get(position_encoding)(config, shared)
+    embedding = Embedding(config.vocab, config.hidden, embedding_name)
+    blocks = []
+    for index, kinds in enumerate(config.layer_kinds()):
+        blocks.append(BLOCKS.get(kinds.block)(config, index, layer_prefix.format(index), kinds, shared))
+    final_norm = NORMS.get(final_norm_kind)(config, config.hidden, final_norm_name, shared)
+    if getattr(config, "tie_word_embeddings", False):
+        head = LMHead(config.vocab, config.hidden, None, tied_to=embedding)
+    else:
+        head = LMHead(config.vocab, config.hidden, head_name)
+    return DecoderModel(config, embedding, blocks, config.schedule(), final_norm, head,
+                        shared_parts=[shared["position_encoding"]])

@@ -1,0 +1,82 @@
+"""Grouped-query attention over the paged cache.
+
+Formulas in the reference's order (crates/beholdd-model/src/qwen3moe/forward.rs:1086-1252):
+q, k, v projections without bias; per-head RMSNorm of q and k with one [head_dim] weight each,
+BEFORE the rotation (:1130-1156); split-half rotation of q and k at the absolute position
+(:1161-1189); keys (normed, rotated) and raw values appended to the cache (:1196); for query
+head h the kv head h // (heads / kv_heads) (crates/beholdd-backend/src/cpu.rs:806); scores
+scaled by `scale`, causal by position, softmax in float32 (cpu.rs:810-833); output projection
+added to the residual (:1236-1252).
+
+Every size and constant is a constructor parameter; the q/k norm, the rotation and a window
+are optional, so the same part serves other stacks.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ..weights.binder import TensorSpec
+from .base import MIXERS, CacheNeed
+from .linear import Linear
+
+
+class GQAAttention:
+    def __init__(self, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int, prefix: str, *,
+                 position_encoding=None, qk_norm_eps: float | None = None, scale: float | None = None,
+                 window: int = 0):
+        if n_heads % n_kv_heads:
+            raise ValueError(f"{n_heads} query heads do not group evenly into {n_kv_heads} kv heads")
+        self.hidden, self.n_heads, self.n_kv_heads, self.head_dim = hidden, n_heads, n_kv_heads, head_dim
+        self.prefix = prefix
+        self.position_encoding = position_encoding
+        self.qk_norm_eps = qk_norm_eps
+        # the reference computes the scale in float32: (head_dim as f32).sqrt().recip() (forward.rs:1192)
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
+        self.window = int(window)
+        q_width, kv_width = n_heads * head_dim, n_kv_heads * head_dim
+        self.qkv = Linear(hidden, [q_width, kv_width, kv_width],
+                          [prefix + "q_proj.weight", prefix + "k_proj.weight", prefix + "v_proj.weight"])
+        self.out = Linear(q_width, hidden, prefix + "o_proj.weight")
+        self.q_norm = self.k_norm = None
+
+    def tensor_specs(self):
+        specs = self.qkv.tensor_specs() + self.out.tensor_specs()
+        if self.qk_norm_eps is not None:
+            specs += [TensorSpec(self.prefix + "q_norm.weight", (self.head_dim,), "norm"),
+                      TensorSpec(self.prefix + "k_norm.weight", (self.head_dim,), "norm")]
+        return specs
+
+    def load(self, get):
+        self.qkv.load(get)
+        self.out.load(get)
+        if self.qk_norm_eps is not None:
+            self.q_norm = get(self.prefix + "q_norm.weight")
+            self.k_norm = get(self.prefix + "k_norm.weight")
+            if self.q_norm.dtype != self.k_norm.dtype:
+                self.q_norm, self.k_norm = self.q_norm.float(), self.k_norm.float()
+
+    def cache_need(self):
+        return CacheNeed(kind="kv", kv_heads=self.n_kv_heads, head_dim=self.head_dim, window=self.window)
+
+    def forward(self, ctx, x, hidden, cache):
+        k = ctx.kernels
+        qkv = self.qkv.forward(ctx, x)
+        q = ctx.new_activations(ctx.n_rows, self.n_heads * self.head_dim)
+        cos, sin = self.position_encoding.tables() if self.position_encoding is not None else (None, None)
+        k.qk_norm_rope_cache(qkv, q, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0, cos, sin,
+                             ctx.positions, ctx.row_seq, cache.k_pages, cache.v_pages, cache.page_table,
+                             self.n_heads, self.n_kv_heads, self.head_dim, cache.writes, ctx.max_position)
+        attended = ctx.new_activations(ctx.n_rows, self.n_heads * self.head_dim)
+        k.attention(q, attended, cache.k_pages, cache.v_pages, cache.page_table, ctx.row_seq, ctx.positions,
+                    self.n_heads, self.n_kv_heads, self.head_dim, self.scale, self.window, layout=ctx)
+        self.out.forward(ctx, attended, out=hidden, accumulate=True)
+
+
+@MIXERS.register("gqa_attention")
+def _build_gqa_attention(config, layer_index, prefix, shared):
+    return GQAAttention(config.hidden, config.n_heads, config.n_kv_heads, config.head_dim,
+                        prefix + "self_attn.", position_encoding=shared["position_encoding"],
+                        qk_norm_eps=config.rms_eps)

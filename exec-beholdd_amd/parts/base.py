@@ -1,0 +1,153 @@
+"""What a part is, what it sees of a step, and the registries that configurations choose from.
+
+A model is put together from parts: a *mixer* (attention here), a *feed-forward*, a *norm*,
+a *position encoding*, arranged by a *block*.  Each part takes its sizes and constants as
+constructor parameters and does not know which model it is in.  A configuration names, layer
+by layer, which registered part to build; the builder functions registered here turn the
+configuration into constructor parameters.
+
+Interfaces
+----------
+Every part:
+    tensor_specs() -> list[TensorSpec]     the checkpoint tensors it needs, by full name
+    load(get)                              take them: get(name) -> device tensor
+Norm:
+    forward(ctx, hidden_f32, rows=None) -> activations [n, width] in ctx.act_dtype
+Position encoding:
+    tables() -> (cos, sin) float32 [positions, rotary/2], or (None, None)
+Mixer:
+    cache_need() -> CacheNeed | None       what it keeps per sequence between steps
+    forward(ctx, x, hidden, cache)         adds its output into `hidden` (float32, the residual)
+Feed-forward:
+    forward(ctx, x, hidden)                adds its output into `hidden`
+Block:
+    mixer, feed_forward attributes; forward(ctx, hidden, cache)
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import torch
+
+
+# ---- what a mixer keeps between steps ------------------------------------------------------
+
+@dataclass(frozen=True)
+class CacheNeed:
+    """Storage one layer needs for each sequence.
+
+    kind "kv":    keys and values of `kv_heads` heads of `head_dim` for every position, or for
+                  the last `window` positions only (window 0 = all); paged.
+    kind "state": one tensor of `state_shape` and `state_dtype` per sequence, of fixed size,
+                  zero when a sequence starts.
+    Layers whose needs are equal share one storage group.
+    """
+    kind: str
+    kv_heads: int = 0
+    head_dim: int = 0
+    window: int = 0
+    state_shape: tuple = ()
+    state_dtype: torch.dtype = torch.float32
+
+    def __post_init__(self):
+        if self.kind not in ("kv", "state"):
+            raise ValueError(f"cache need kind must be 'kv' or 'state', got {self.kind!r}")
+        if self.kind == "kv" and (self.kv_heads <= 0 or self.head_dim <= 0 or self.window < 0):
+            raise ValueError("a kv cache need has positive head count and head size and a window >= 0")
+        if self.kind == "state" and not self.state_shape:
+            raise ValueError("a state cache need has a shape")
+
+
+# ---- what a part sees of one step ------------------------------------------------------------
+
+@dataclass
+class StepContext:
+    """One step: `n_rows` tokens of `n_seqs` sequences, flattened sequence after sequence.
+
+    Device tensors (int32): tokens [T], positions [T] (absolute position of each row),
+    row_seq [T] (index of the row's sequence in this batch), seq_start [B+1] (first row of each
+    sequence), seq_slot [B] (cache slot of each sequence), seq_past [B] (tokens the cache held
+    before this step).  The `host_*` lists carry the same numbers for parts that decide on the
+    host.  `is_decode` says that every sequence brings exactly one token.
+    """
+    kernels: object
+    act_dtype: torch.dtype
+    device: torch.device
+    n_rows: int
+    n_seqs: int
+    tokens: torch.Tensor
+    positions: torch.Tensor
+    row_seq: torch.Tensor
+    seq_start: torch.Tensor
+    seq_slot: torch.Tensor
+    seq_past: torch.Tensor
+    host_seq_start: list
+    host_seq_slot: list
+    host_seq_past: list
+    is_decode: bool
+    max_position: int                      # largest absolute position in this step
+    extras: dict = field(default_factory=dict)
+
+    def new_activations(self, *shape) -> torch.Tensor:
+        return torch.empty(shape, dtype=self.act_dtype, device=self.device)
+
+    def new_f32(self, *shape) -> torch.Tensor:
+        return torch.empty(shape, dtype=torch.float32, device=self.device)
+
+
+@dataclass
+class LayerCache:
+    """The storage of one cache entry as handed to a mixer for one step.
+
+    kv need:    k_pages, v_pages [pages, kv_heads, page_size, head_dim]; page_table int32
+                [n_seqs, width] for the sequences of this step, in batch order.
+    state need: state [max_slots, *state_shape]; index it with ctx.seq_slot.
+    `writes` is False when the schedule lets this layer read another layer's entry.
+    """
+    need: CacheNeed
+    writes: bool = True
+    k_pages: torch.Tensor | None = None
+    v_pages: torch.Tensor | None = None
+    page_table: torch.Tensor | None = None
+    state: torch.Tensor | None = None
+
+
+# ---- registries ---------------------------------------------------------------------------------
+
+class Registry:
+    """Name -> builder.  A builder is `build(config, layer_index, prefix, shared) -> part`."""
+
+    def __init__(self, what: str):
+        self.what = what
+        self._items: dict = {}
+
+    def register(self, name: str, builder=None):
+        if builder is None:                 # decorator form
+            return lambda fn: self.register(name, fn)
+        if name in self._items:
+            raise ValueError(f"{self.what} {name!r} is already registered")
+        self._items[name] = builder
+        return builder
+
+    def unregister(self, name: str):
+        self._items.pop(name, None)
+
+    def get(self, name: str):
+        try:
+            return self._items[name]
+        except KeyError:
+            raise KeyError(f"no {self.what} named {name!r}; registered: {sorted(self._items)}") from None
+
+    def names(self) -> list[str]:
+        return sorted(self._items)
+
+    def __contains__(self, name):
+        return name in self._items
+
+
+MIXERS = Registry("mixer")
+FEED_FORWARDS = Registry("feed-forward")
+NORMS = Registry("norm")
+POSITION_ENCODINGS = Registry("position encoding")
+BLOCKS = Registry("block")

@@ -1,0 +1,43 @@
+"""The arrangement of parts in a layer.
+
+Pre-norm residual block: h = h + Mixer(Norm(h)); h = h + FeedForward(Norm(h))
+(crates/beholdd-model/src/qwen3moe/forward.rs:1022-1414).  The residual `hidden` is float32
+and is updated in place; the mixer and the feed-forward add into it.
+"""
+
+from __future__ import annotations
+
+from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS
+
+
+class PreNormBlock:
+    def __init__(self, mixer_norm, mixer, feed_forward_norm, feed_forward):
+        self.mixer_norm, self.mixer = mixer_norm, mixer
+        self.feed_forward_norm, self.feed_forward = feed_forward_norm, feed_forward
+
+    def parts(self):
+        return [self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward]
+
+    def tensor_specs(self):
+        return [spec for part in self.parts() for spec in part.tensor_specs()]
+
+    def load(self, get):
+        for part in self.parts():
+            part.load(get)
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def forward(self, ctx, hidden, cache):
+        self.mixer.forward(ctx, self.mixer_norm.forward(ctx, hidden), hidden, cache)
+        self.feed_forward.forward(ctx, self.feed_forward_norm.forward(ctx, hidden), hidden)
+
+
+@BLOCKS.register("pre_norm")
+def _build_pre_norm(config, layer_index, prefix, kinds, shared):
+    norm = NORMS.get(kinds.norm)
+    return PreNormBlock(
+        norm(config, config.hidden, prefix + "input_layernorm.weight", shared),
+        MIXERS.get(kinds.mixer)(config, layer_index, prefix, shared),
+        norm(config, config.hidden, prefix + "post_attention_layernorm.weight", shared),
+        FEED_FORWARDS.get(kinds.feed_forward)(config, layer_index, prefix, shared))

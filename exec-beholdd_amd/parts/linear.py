@@ -1,0 +1,52 @@
+"""A bias-free linear map y = W x with W stored [out, in], as checkpoints store it.
+
+The reference applies every weight this way, without transposing or permuting
+(crates/beholdd-backend/src/lib.rs:178, crates/beholdd-backend/src/cpu.rs:206-211).  Several
+checkpoint tensors with the same input may be stacked into one matrix at load time, so that
+one product serves them all; each output row is computed exactly as it would be alone.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..weights.binder import TensorSpec
+
+
+class Linear:
+    def __init__(self, in_features: int, out_features, names):
+        """`names` and `out_features` are one name and size, or equal-length lists to stack."""
+        self.in_features = int(in_features)
+        self.names = [names] if isinstance(names, str) else list(names)
+        self.splits = [int(out_features)] if isinstance(out_features, int) else [int(o) for o in out_features]
+        if len(self.names) != len(self.splits):
+            raise ValueError("one output size per stacked tensor")
+        self.out_features = sum(self.splits)
+        self.weight: torch.Tensor | None = None
+
+    def tensor_specs(self):
+        return [TensorSpec(name, (rows, self.in_features), "linear") for name, rows in zip(self.names, self.splits)]
+
+    def load(self, get):
+        pieces = [get(name) for name in self.names]
+        if len(pieces) == 1:
+            self.weight = pieces[0]
+        else:
+            dtype = pieces[0].dtype
+            if any(p.dtype != dtype for p in pieces):
+                pieces = [p.to(torch.float32) for p in pieces]   # mixed storage: keep the wider one
+            self.weight = torch.cat(pieces, dim=0).contiguous()
+
+    def use(self, weight: torch.Tensor):
+        """Share another part's matrix (a tied head)."""
+        if tuple(weight.shape) != (self.out_features, self.in_features):
+            raise ValueError(f"shared weight has shape {tuple(weight.shape)}, expected "
+                             f"{(self.out_features, self.in_features)}")
+        self.weight = weight
+
+    def forward(self, ctx, x, out=None, accumulate=False, out_dtype=None):
+        """x [n, in] -> out [n, out]; with accumulate the product is added into `out`."""
+        if out is None:
+            out = torch.empty((x.shape[0], self.out_features), dtype=out_dtype or ctx.act_dtype, device=x.device)
+        ctx.kernels.gemm(x, self.weight, out, accumulate=accumulate)
+        return out

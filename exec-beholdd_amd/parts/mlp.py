@@ -1,0 +1,37 @@
+"""Dense SwiGLU feed-forward: out = Wd (silu(Wg x) * (Wu x)), added to the residual.
+
+crates/beholdd-model/src/qwen3moe/forward.rs:1270-1298 with silu(x) = x / (1 + exp(-x)) and no
+clamp (crates/beholdd-kernel/src/vecops.rs:91-110, limit 0 at forward.rs:1288).  The gate and
+up matrices are stacked so that one product computes both.
+"""
+
+from __future__ import annotations
+
+from .base import FEED_FORWARDS
+from .linear import Linear
+
+
+class SwiGLU:
+    def __init__(self, hidden: int, intermediate: int, prefix: str):
+        self.hidden, self.intermediate = hidden, intermediate
+        self.gate_up = Linear(hidden, [intermediate, intermediate],
+                              [prefix + "gate_proj.weight", prefix + "up_proj.weight"])
+        self.down = Linear(intermediate, hidden, prefix + "down_proj.weight")
+
+    def tensor_specs(self):
+        return self.gate_up.tensor_specs() + self.down.tensor_specs()
+
+    def load(self, get):
+        self.gate_up.load(get)
+        self.down.load(get)
+
+    def forward(self, ctx, x, hidden):
+        gate_up = self.gate_up.forward(ctx, x)
+        activated = ctx.new_activations(x.shape[0], self.intermediate)
+        ctx.kernels.swiglu(gate_up, activated)
+        self.down.forward(ctx, activated, out=hidden, accumulate=True)
+
+
+@FEED_FORWARDS.register("swiglu")
+def _build_swiglu(config, layer_index, prefix, shared):
+    return SwiGLU(config.hidden, config.intermediate, prefix + "mlp.")

@@ -1,0 +1,89 @@
+"""Ways of cutting the same requests into steps; shared by the CPU-logic and the GPU tests.
+
+Every function drives `Engine.step` and returns, per request, the float32 logits of every
+position [len(tokens), vocab] as NumPy arrays, so that any two cuts and the plain
+implementation can be compared position by position.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+from beholdd.engine import StepEntry
+
+
+def _rows(logits):
+    return logits.float().cpu().numpy()
+
+
+def whole(engine, requests):
+    """Each request alone, all its tokens in one step."""
+    out = []
+    for tokens in requests:
+        slot = engine.alloc_slot()
+        out.append(_rows(engine.step([StepEntry(slot, list(tokens), list(range(len(tokens))))])))
+        engine.free_slot(slot)
+    return out
+
+
+def tail_one_by_one(engine, requests, tail=32):
+    """Each request alone: the first n - tail tokens in one step, the last `tail` one by one."""
+    out = []
+    for tokens in requests:
+        tokens = list(tokens)
+        cut = max(1, len(tokens) - tail)
+        slot = engine.alloc_slot()
+        rows = [_rows(engine.step([StepEntry(slot, tokens[:cut], list(range(cut)))]))]
+        for token in tokens[cut:]:
+            rows.append(_rows(engine.step([StepEntry(slot, [token], [0])])))
+        engine.free_slot(slot)
+        out.append(np.concatenate(rows, axis=0))
+    return out
+
+
+def batches(engine, requests, batch_size, prompt_fraction=0.6):
+    """Batches of unequal lengths, one after another so that slots and pages are used again:
+    each request's first part (a fraction of its length) goes in with the others' in one
+    step, the rest one token per step; shorter requests end earlier and free their slots."""
+    out = [None] * len(requests)
+    for start in range(0, len(requests), batch_size):
+        group = list(range(start, min(start + batch_size, len(requests))))
+        slots = {i: engine.alloc_slot() for i in group}
+        cuts = {i: max(1, int(len(requests[i]) * prompt_fraction)) for i in group}
+        rows = {i: [] for i in group}
+        logits = _rows(engine.step([StepEntry(slots[i], list(requests[i][:cuts[i]]), list(range(cuts[i])))
+                                    for i in group]))
+        at = 0
+        for i in group:
+            rows[i].append(logits[at:at + cuts[i]])
+            at += cuts[i]
+        done = {i: cuts[i] for i in group}
+        live = [i for i in group if done[i] < len(requests[i])]
+        for i in group:
+            if i not in live:
+                engine.free_slot(slots.pop(i))
+        while live:
+            logits = _rows(engine.step([StepEntry(slots[i], [requests[i][done[i]]], [0]) for i in live]))
+            for row, i in enumerate(live):
+                rows[i].append(logits[row:row + 1])
+                done[i] += 1
+            still = []
+            for i in live:
+                if done[i] < len(requests[i]):
+                    still.append(i)
+                else:
+                    engine.free_slot(slots.pop(i))      # a shorter request ends earlier
+            live = still
+        for i in group:
+            out[i] = np.concatenate(rows[i], axis=0)
+    return out
+
+
+def relative_error(got, want):
+    """max |got - want| / max |want|: the measure the acceptance tolerance is stated in."""
+    return float(np.abs(got.astype(np.float64) - want.astype(np.float64)).max() / np.abs(want).max())
+
+
+def random_requests(vocab, lengths, seed):
+    rng = np.random.default_rng(seed)
+    return [[int(t) for t in rng.integers(0, vocab, size=n)] for n in lengths]
