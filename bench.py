@@ -1,0 +1,173 @@
+"""Decode and prefill throughput of the Qwen3-8B shape with random bfloat16 weights on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C]
+
+A step is one decode step of the batch: every live sequence's next token through the whole
+model, logits of each and a greedy choice.  The sequences' caches are filled with random keys
+and values to just under the context length, so the timed steps read a full-length cache and
+end exactly at the context length.  Prints one JSON line.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBS = 8000.0            # MI355X HBM3E
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+QWEN3_8B = {
+    "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "num_hidden_layers": 36, "hidden_size": 4096,
+    "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128, "intermediate_size": 12288,
+    "vocab_size": 151936, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "max_position_embeddings": 40960,
+    "tie_word_embeddings": False,
+}
+
+
+def parse():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=32)
+    parser.add_argument("--warmup", type=int, default=4)
+    parser.add_argument("--layers", type=int, default=QWEN3_8B["num_hidden_layers"])
+    parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--context", type=int, default=8192)
+    parser.add_argument("--prefill-tokens", type=int, default=2048)
+    parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
+    return parser.parse_args()
+
+
+def fill_cache(engine, slots, length, torch):
+    """Give each slot `length` tokens of random keys and values without running the model."""
+    requests = [(slot, length) for slot in slots]
+    engine.cache.reserve(requests)
+    engine.cache.commit(requests)
+
+
+def randomise_cache(engine, torch):
+    generator = torch.Generator(device=engine.device).manual_seed(1)
+    for group in engine.cache.groups:
+        if group.k is not None:
+            for tensor in (group.k, group.v):
+                for layer in range(tensor.shape[0]):
+                    tensor[layer].normal_(0.0, 1.0, generator=generator)
+
+
+def decode_run(engine, batch, context, steps, warmup, torch):
+    """Time `steps` decode steps of `batch` sequences that end at `context` tokens."""
+    from beholdd.engine import StepEntry
+    from beholdd.sampling import SamplingParams
+
+    start = context - steps - warmup
+    slots = [engine.alloc_slot() for _ in range(batch)]
+    fill_cache(engine, slots, start, torch)
+    greedy = [SamplingParams()] * batch
+    tokens = [(7 * i + 3) % engine.model.vocab for i in range(batch)]
+
+    def one(step):
+        nonlocal tokens
+        logits = engine.step([StepEntry(slot, [token], [0]) for slot, token in zip(slots, tokens)])
+        tokens = engine.select(logits, greedy, list(range(batch)), [step] * batch)
+
+    for step in range(warmup):
+        one(step)
+    torch.cuda.synchronize()
+    begin = time.perf_counter()
+    for step in range(steps):
+        one(warmup + step)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - begin
+    lengths = [engine.cache.length(slot) for slot in slots]
+    for slot in slots:
+        engine.free_slot(slot)
+    mean_length = sum(lengths) / batch - steps / 2.0
+    return elapsed / steps, mean_length
+
+
+def prefill_run(engine, n_tokens, torch, repeats=3):
+    from beholdd.engine import StepEntry
+    tokens = [(31 * i + 5) % engine.model.vocab for i in range(n_tokens)]
+    times = []
+    for _ in range(repeats + 1):          # the first run warms up and is dropped
+        slot = engine.alloc_slot()
+        torch.cuda.synchronize()
+        begin = time.perf_counter()
+        engine.step([StepEntry(slot, tokens, [n_tokens - 1])])
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - begin)
+        engine.free_slot(slot)
+    return min(times[1:])
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU library")
+        return 2
+    import torch
+
+    import beholdd
+    from beholdd.engine import Engine, random_model_on_device
+
+    config = dict(QWEN3_8B, num_hidden_layers=args.layers)
+    device = "cuda:0"
+    dtype_tag = "bf16" if args.dtype == "bfloat16" else "fp32"
+    element = 2 if args.dtype == "bfloat16" else 4
+    model = random_model_on_device(config, seed=0, dtype=args.dtype, device=device)
+    biggest = 1 if args.no_points else 64
+    max_tokens = max(args.batch, biggest) * (-(-args.context // 64) * 64)
+    engine = Engine(model=model, dtype=args.dtype, max_tokens=max_tokens, max_slots=max(args.batch, biggest, 64),
+                    device=device)
+    randomise_cache(engine, torch)
+    cfg = engine.config
+
+    layer_params = (cfg.hidden * (cfg.q_width + 2 * cfg.kv_width) + cfg.q_width * cfg.hidden
+                    + 3 * cfg.hidden * cfg.intermediate)
+    weight_bytes = (cfg.n_layers * layer_params + cfg.vocab * cfg.hidden) * element
+    kv_bytes_per_token = cfg.n_layers * 2 * cfg.kv_width * element
+
+    seconds, mean_length = decode_run(engine, args.batch, args.context, args.steps, args.warmup, torch)
+    step_bytes = weight_bytes + args.batch * mean_length * kv_bytes_per_token
+    achieved = step_bytes / seconds / 1e9
+    value = args.batch / seconds
+
+    prefill_seconds = prefill_run(engine, args.prefill_tokens, torch)
+    t = args.prefill_tokens
+    prefill_flops = (2.0 * cfg.n_layers * layer_params * t + cfg.n_layers * cfg.n_heads * 2.0 * t * t * cfg.head_dim
+                     + 2.0 * cfg.vocab * cfg.hidden)
+    points = {}
+    if not args.no_points:
+        for batch in (1, 64):
+            steps = max(4, args.steps // 2)
+            s, _ = decode_run(engine, batch, args.context, steps, 2, torch)
+            points[f"decode_b{batch}"] = round(batch / s, 2)
+
+    line = {
+        "metric": "decode tok/s @ batch 8 (Qwen3-8B shape, context 8192)", "value": round(value, 2), "unit": "tok/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(seconds * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype_tag,
+        "data": "synthetic: seeded random weights, random token ids, caches filled with random keys and values",
+        "config": {
+            "model": "Qwen3-8B shape", "layers": cfg.n_layers, "layers_of_full_model": QWEN3_8B["num_hidden_layers"],
+            "hidden_size": cfg.hidden, "num_attention_heads": cfg.n_heads, "num_key_value_heads": cfg.n_kv_heads,
+            "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate, "vocab_size": cfg.vocab,
+            "rope_theta": cfg.rope_theta, "rms_norm_eps": cfg.rms_eps, "tie_word_embeddings": cfg.tie_word_embeddings,
+            "global_batch": args.batch, "seq_len": args.context, "prefill_tokens": t, "parallelism": "single GPU",
+        },
+        "prefill": {"value": round(t / prefill_seconds, 1), "tokens": t, "ms": round(prefill_seconds * 1e3, 3),
+                    "frac": round(prefill_flops / prefill_seconds / PEAK_FLOPS[dtype_tag], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+        "points": points,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -37,11 +37,20 @@ TINY_C = {
     "rms_norm_eps": 1e-5, "max_position_embeddings": 1024, "tie_word_embeddings": False,
     "hidden_act": "silu", "attention_bias": False,
 }
+# The head size and group of the large models (128, four query heads per kv head), small otherwise.
+TINY_D = {
+    "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3",
+    "num_hidden_layers": 2, "hidden_size": 320, "num_attention_heads": 8, "num_key_value_heads": 2,
+    "head_dim": 128, "intermediate_size": 896, "vocab_size": 1500, "rope_theta": 1000000.0,
+    "rms_norm_eps": 1e-6, "max_position_embeddings": 2048, "tie_word_embeddings": True,
+    "hidden_act": "silu", "attention_bias": False,
+}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
 
 
 @pytest.fixture(scope="session")
 def tiny_configs():
-    return {"A": dict(TINY_A), "B": dict(TINY_B), "C": dict(TINY_C)}
+    return {name: dict(config) for name, config in CONFIGS.items()}
 
 
 @pytest.fixture(scope="session")
@@ -56,7 +65,7 @@ def model_dirs(tmp_path_factory):
         key = (name, dtype, seed)
         if key not in made:
             folder = tmp_path_factory.mktemp(f"tiny_{name}_{dtype}_{seed}")
-            config = {"A": TINY_A, "B": TINY_B, "C": TINY_C}[name]
+            config = CONFIGS[name]
             beholdd.write_random_model(str(folder), dict(config), seed=seed, dtype=dtype)
             made[key] = str(folder)
         return made[key]

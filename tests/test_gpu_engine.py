@@ -1,0 +1,242 @@
+"""The engine on the GPU against the plain implementation, in float32 and in bfloat16:
+every request alone and whole; with its last 32 tokens one by one; in batches of unequal
+lengths whose shorter requests end earlier, one batch after another so that slots and pages are
+used again; long decoding; the first tokens of a sequence; generation through the entry
+point; trace replay as a program."""
+
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen3 as plain
+import schedules
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+# float32: the acceptance bound.  bfloat16: activations carry 8 bits of mantissa (half an ulp is
+# 2^-9 = 0.002 of a value) through a dozen roundings per layer; the bound is on max|diff| / max|logit|.
+TOLERANCE = {"float32": 1e-4, "bfloat16": 2e-2}
+
+LENGTHS = {"A": [5, 11, 17, 70, 33, 128], "B": [1, 7, 23, 40, 90, 200, 64], "C": [3, 65, 130, 400, 31],
+           "D": [2, 50, 129, 300]}
+
+
+def engine_for(folder, dtype, max_tokens=4096):
+    from beholdd.engine import Engine
+    return Engine(folder, dtype=dtype, max_tokens=max_tokens)
+
+
+@pytest.fixture(scope="module")
+def expected(model_dirs):
+    cache = {}
+
+    def get(name):
+        if name not in cache:
+            folder = model_dirs(name, "bfloat16")
+            cfg, weights = plain.load_plain(folder)
+            requests = schedules.random_requests(cfg.vocab, LENGTHS[name], seed=11)
+            cache[name] = (folder, requests, [plain.forward_logits(cfg, weights, r) for r in requests])
+        return cache[name]
+
+    return get
+
+
+def check(label, got, want, tolerance):
+    for index, (g, e) in enumerate(zip(got, want)):
+        assert g.shape == e.shape, (label, index, g.shape, e.shape)
+        assert np.isfinite(g).all(), (label, index)
+        error = schedules.relative_error(g, e)
+        if error >= tolerance:
+            per_row = np.abs(g.astype(np.float64) - e).max(axis=1) / np.abs(e).max()
+            first = int(np.argmax(per_row >= tolerance))
+            pytest.fail(f"{label}: request {index} (length {len(g)}): error {error:.3e} >= {tolerance}; "
+                        f"first wrong position {first}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+def test_every_cut_matches_the_plain_implementation(expected, name, dtype):
+    folder, requests, want = expected(name)
+    engine = engine_for(folder, dtype)
+    tolerance = TOLERANCE[dtype]
+    whole = schedules.whole(engine, requests)
+    check("whole", whole, want, tolerance)
+    tail = schedules.tail_one_by_one(engine, requests, tail=32)
+    check("last 32 one by one", tail, want, tolerance)
+    for batch_size in (3, len(requests)):
+        batched = schedules.batches(engine, requests, batch_size=batch_size)
+        check(f"batches of {batch_size}", batched, want, tolerance)
+    # the cuts agree with each other more closely than with another implementation
+    check("tail vs whole", tail, whole, tolerance / 2)
+    check("batches vs whole", batched, whole, tolerance / 2)
+    engine.cache.check_invariants()
+    assert engine.cache.live_slots() == [] and engine.cache.free_page_count() == engine.cache.n_pages
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_float32_storage_and_slot_reuse_in_a_small_cache(model_dirs, dtype):
+    """Weights stored in 32-bit; a cache of three pages, so every request runs in pages and slots
+    that earlier requests used."""
+    folder = model_dirs("B", "float32")
+    cfg, weights = plain.load_plain(folder)
+    requests = schedules.random_requests(cfg.vocab, [100, 64, 130, 1, 65], seed=4)
+    want = [plain.forward_logits(cfg, weights, r) for r in requests]
+    engine = engine_for(folder, dtype, max_tokens=192)
+    assert engine.cache.n_pages == 3
+    check("whole", schedules.whole(engine, requests), want, TOLERANCE[dtype])
+    check("tail", schedules.tail_one_by_one(engine, requests, tail=32), want, TOLERANCE[dtype])
+    check("pairs", schedules.batches(engine, [requests[1], requests[3], requests[4], requests[0]], batch_size=2),
+          [want[1], want[3], want[4], want[0]], TOLERANCE[dtype])
+    engine.cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(model_dirs, dtype):
+    """Ten prompt tokens, then 500 tokens one by one (several pages, several key chunks)."""
+    folder = model_dirs("C", "bfloat16")
+    cfg, weights = plain.load_plain(folder)
+    tokens = schedules.random_requests(cfg.vocab, [510], seed=21)[0]
+    want = plain.forward_logits(cfg, weights, tokens)
+    engine = engine_for(folder, dtype)
+    got = schedules.tail_one_by_one(engine, [tokens], tail=500)[0]
+    check("long decoding", [got], [want], TOLERANCE[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_first_tokens_of_a_sequence(model_dirs, name, dtype):
+    folder = model_dirs(name, "bfloat16")
+    cfg, weights = plain.load_plain(folder)
+    engine = engine_for(folder, dtype)
+    for length in (1, 2, 3):
+        tokens = schedules.random_requests(cfg.vocab, [length], seed=length)[0]
+        want = plain.forward_logits(cfg, weights, tokens)
+        check(f"whole {length}", schedules.whole(engine, [tokens]), [want], TOLERANCE[dtype])
+        check(f"one by one {length}", schedules.tail_one_by_one(engine, [tokens], tail=length), [want], TOLERANCE[dtype])
+
+
+def test_greedy_generation_through_the_entry_point(model_dirs):
+    """BASELINE's tiny configuration A: prompts of 5, 11 and 17 tokens, 8 greedy tokens each."""
+    import beholdd
+    folder = model_dirs("A", "bfloat16")
+    cfg, weights = plain.load_plain(folder)
+    prompts = schedules.random_requests(cfg.vocab, [5, 11, 17], seed=2)
+    engine = beholdd.Engine(folder, dtype="float32", max_tokens=512)
+    results = engine.generate(prompts, max_new_tokens=8)
+    for prompt, result in zip(prompts, results):
+        want, _ = plain.greedy_generate(cfg, weights, prompt, 8)
+        assert result.token_ids == want and result.finish_reason == "length"
+        assert result.prompt_tokens == len(prompt) and result.completion_tokens == 8
+    # a stop token ends one sequence early; the others are not disturbed
+    stop = results[1].token_ids[3]
+    again = engine.generate(prompts, max_new_tokens=8, stop_token_ids=[stop])
+    for before, after in zip(results, again):
+        if stop in before.token_ids:
+            cut = before.token_ids.index(stop)
+            assert after.token_ids == before.token_ids[:cut] and after.finish_reason == "stop" and after.stop_token == stop
+        else:
+            assert after.token_ids == before.token_ids
+    # bfloat16: every chosen token is the plain implementation's choice, or as good within rounding
+    engine16 = beholdd.Engine(folder, dtype="bfloat16", max_tokens=512)
+    for prompt, result in zip(prompts, engine16.generate(prompts, max_new_tokens=8)):
+        tokens = list(prompt)
+        for token in result.token_ids:
+            logits = plain.forward_logits(cfg, weights, tokens)[-1]
+            assert logits[token] >= logits.max() - 2e-2 * np.abs(logits).max()
+            tokens.append(token)
+    engine.cache.check_invariants()
+    assert engine.cache.live_slots() == []
+
+
+def test_temperature_sampling_is_seeded_and_independent_of_the_batch(model_dirs):
+    """BASELINE's tiny configuration B: prompts of 1, 7, 23 and 40 tokens, temperature 0.8, 12 tokens."""
+    import beholdd
+    folder = model_dirs("B", "bfloat16")
+    prompts = schedules.random_requests(384, [1, 7, 23, 40], seed=6)
+    engine = beholdd.Engine(folder, dtype="float32", max_tokens=1024)
+    first = engine.generate(prompts, max_new_tokens=12, temperature=0.8, seed=5)
+    again = engine.generate(prompts, max_new_tokens=12, temperature=0.8, seed=5)
+    other = engine.generate(prompts, max_new_tokens=12, temperature=0.8, seed=6)
+    assert [r.token_ids for r in first] == [r.token_ids for r in again]
+    assert [r.token_ids for r in first] != [r.token_ids for r in other]
+    assert all(len(r.token_ids) == 12 for r in first)
+    in_pairs = engine.generate(prompts, max_new_tokens=12, temperature=0.8, seed=5, batch_size=2)
+    assert [r.token_ids for r in in_pairs] == [r.token_ids for r in first]
+    greedy = engine.generate(prompts, max_new_tokens=12)
+    assert [r.token_ids for r in greedy] != [r.token_ids for r in first]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_replay_program(model_dirs, tmp_path, dtype):
+    """bin/trace_run as a user runs it: a batch of three unequal requests, their prompts in one
+    step, then one token each; the shortest ends first; then a second batch in the freed room."""
+    folder = model_dirs("B", "bfloat16")
+    cfg, weights = plain.load_plain(folder)
+    requests = dict(zip("abcde", schedules.random_requests(cfg.vocab, [40, 70, 55, 64, 20], seed=9)))
+    want = {name: plain.forward_logits(cfg, weights, tokens) for name, tokens in requests.items()}
+    steps, expect, number = [], {}, 0
+
+    def run_batch(names, prompt_len):
+        nonlocal number
+        done = {n: prompt_len[n] for n in names}
+        ended = [n for n in names if done[n] == len(requests[n])]
+        steps.append({"step": number, "entries": [{"id": n, "tokens": requests[n][:done[n]],
+                                                   "want": [done[n] - 1, 0] if done[n] > 1 else [0]} for n in names],
+                      "end": ended})
+        expect[number] = np.concatenate([want[n][[done[n] - 1, 0] if done[n] > 1 else [0]] for n in names])
+        number += 1
+        live = [n for n in names if n not in ended]
+        while live:
+            entries = [{"id": n, "tokens": [requests[n][done[n]]], "want": [0] if done[n] % 2 else []} for n in live]
+            rows = [want[n][done[n]:done[n] + 1] for n in live if done[n] % 2]
+            for n in live:
+                done[n] += 1
+            ended = [n for n in live if done[n] == len(requests[n])]
+            steps.append({"step": number, "entries": entries, "end": ended})
+            if rows:
+                expect[number] = np.concatenate(rows)
+            number += 1
+            live = [n for n in live if n not in ended]
+
+    run_batch(["a", "b", "c"], {"a": 30, "b": 50, "c": 55})
+    run_batch(["d", "e"], {"d": 60, "e": 5})
+    out_dir = tmp_path / "out"
+    trace = "\n".join(json.dumps(s) for s in steps) + "\n"
+    # live tokens, each request rounded up to 64: a 64 + b 128 + c 64 = 256 at most
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                          "--out", str(out_dir), "--max-tokens", "256"], input=trace, capture_output=True, text=True,
+                         timeout=600)
+    assert run.returncode == 0, run.stderr[-2000:]
+    assert [line for line in run.stdout.splitlines() if line.startswith("done")] == [f"done {s['step']}" for s in steps]
+    assert sorted(os.listdir(out_dir)) == sorted(f"{n}.f32" for n in expect)
+    for number, rows in expect.items():
+        got = np.fromfile(out_dir / f"{number}.f32", dtype="<f4").reshape(-1, cfg.vocab)
+        assert got.shape == rows.shape
+        assert schedules.relative_error(got, rows) < TOLERANCE[dtype], number
+
+
+def test_command_line_generate(model_dirs, tmp_path):
+    import beholdd
+    from beholdd.engine.artifact import read_logits_artifact
+    folder = model_dirs("A", "bfloat16")
+    cfg, weights = plain.load_plain(folder)
+    capture = tmp_path / "logits.bin"
+    timing = tmp_path / "steps.tsv"
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "beholdd"), "generate", "--model", folder,
+                          "--dtype", "float32", "--prompt-ids", "5,17,3,200", "--max-new-tokens", "6",
+                          "--logits-out", str(capture), "--step-timing-out", str(timing)],
+                         capture_output=True, text=True, timeout=600)
+    assert run.returncode == 0, run.stderr[-2000:]
+    want, _ = plain.greedy_generate(cfg, weights, [5, 17, 3, 200], 6)
+    assert f"generated: {want}" in run.stdout
+    prompt, generated, logits = read_logits_artifact(str(capture))
+    assert prompt == [5, 17, 3, 200] and generated == want and logits.shape == (6, cfg.vocab)
+    full = plain.forward_logits(cfg, weights, [5, 17, 3, 200] + want[:-1])
+    assert schedules.relative_error(logits, full[3:]) < 1e-4
+    assert timing.read_text().splitlines()[0] == "step\tduration_ms"

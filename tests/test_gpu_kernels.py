@@ -1,0 +1,393 @@
+"""Each HIP kernel alone against a plain torch reference of the same operation, at sizes other
+than the engine tests use (head sizes in steps of 16, odd head counts and groups, widths and a
+vocabulary that are no power of two)."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+PAGE = 64
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def K():
+    from beholdd.kernels import HipKernels
+    return HipKernels("cuda:0")
+
+
+def dev(t):
+    return t.to("cuda:0")
+
+
+def tol(dtype, f32=2e-5, bf16=1.6e-2):
+    return f32 if dtype == torch.float32 else bf16
+
+
+def rel(got, want):
+    got, want = got.double().cpu(), want.double().cpu()
+    return float((got - want).abs().max() / want.abs().max().clamp_min(1e-30))
+
+
+def test_library_is_the_in_tree_one(K):
+    assert K.library_path.endswith("libbeholdd_hip.so")
+    assert K.page_size == PAGE
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,width,vocab", [(1, 96, 331), (37, 1000, 77), (5, 4096, 513)])
+def test_embed(K, dtype, rows, width, vocab):
+    g = torch.Generator().manual_seed(rows)
+    table = torch.randn(vocab, width, generator=g).to(dtype)
+    tokens = torch.randint(0, vocab, (rows,), generator=g, dtype=torch.int32)
+    tokens[0], tokens[-1] = vocab - 1, 0
+    out = torch.empty(rows, width, dtype=torch.float32, device="cuda:0")
+    K.embed(dev(tokens), dev(table), out)
+    assert torch.equal(out.cpu(), table[tokens.long()].float())
+
+
+@pytest.mark.parametrize("out_dtype", DTYPES)
+@pytest.mark.parametrize("w_dtype", DTYPES)
+@pytest.mark.parametrize("rows,width,eps", [(1, 48, 1e-6), (33, 1000, 1e-5), (4, 5120, 1e-6), (3, 4097, 1e-2)])
+def test_rmsnorm(K, out_dtype, w_dtype, rows, width, eps):
+    g = torch.Generator().manual_seed(width)
+    x = torch.randn(rows, width, generator=g) * 3 + 0.5
+    w = (1 + 0.1 * torch.randn(width, generator=g)).to(w_dtype)
+    out = torch.empty(rows, width, dtype=out_dtype, device="cuda:0")
+    K.rmsnorm(dev(x), dev(w), eps, out)
+    want = x.double() / torch.sqrt((x.double() ** 2).mean(-1, keepdim=True) + eps) * w.double()
+    assert rel(out, want) < tol(out_dtype, 2e-6, 4e-3)
+    # gathered rows, no weight
+    index = torch.tensor([rows - 1, 0, rows - 1], dtype=torch.int32)
+    out2 = torch.empty(3, width, dtype=out_dtype, device="cuda:0")
+    K.rmsnorm(dev(x), None, eps, out2, rows=dev(index))
+    want2 = (x.double() / torch.sqrt((x.double() ** 2).mean(-1, keepdim=True) + eps))[index.long()]
+    assert rel(out2, want2) < tol(out_dtype, 2e-6, 4e-3)
+
+
+@pytest.mark.parametrize("a_dtype,w_dtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                             (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("m,n,k", [(1, 96, 120), (7, 331, 200), (64, 130, 72), (65, 257, 1000), (200, 64, 48),
+                                   (3, 1000, 4096), (130, 520, 264)])
+def test_gemm(K, a_dtype, w_dtype, m, n, k):
+    g = torch.Generator().manual_seed(m * 1000 + n)
+    a = torch.randn(m, k, generator=g).to(a_dtype)
+    w = (torch.randn(n, k, generator=g) * 0.05).to(w_dtype)
+    want = a.double() @ w.double().t()
+    for out_dtype in (torch.float32, a_dtype):
+        out = torch.empty(m, n, dtype=out_dtype, device="cuda:0")
+        K.gemm(dev(a), dev(w), out)
+        assert rel(out, want) < tol(out_dtype, 2e-6, 4e-3), (out_dtype, rel(out, want))
+    base = torch.randn(m, n, generator=g)
+    acc = dev(base.clone())
+    K.gemm(dev(a), dev(w), acc, accumulate=True)
+    assert rel(acc, want + base.double()) < 2e-6
+
+
+def make_cache(n_seqs, lengths, kv_heads, head_dim, dtype, seed, extra_pages=3):
+    """Random keys/values for sequences of the given lengths, scattered over shuffled pages.
+    Returns (k_pages, v_pages, page_table, dense keys list, dense values list)."""
+    g = torch.Generator().manual_seed(seed)
+    pages_per = [-(-n // PAGE) for n in lengths]
+    n_pages = sum(pages_per) + extra_pages
+    order = torch.randperm(n_pages, generator=g).tolist()
+    k_pages = torch.randn(n_pages, kv_heads, PAGE, head_dim, generator=g).to(dtype)   # garbage everywhere
+    v_pages = torch.randn(n_pages, kv_heads, PAGE, head_dim, generator=g).to(dtype)
+    width = max(pages_per)
+    table = torch.zeros(n_seqs, width, dtype=torch.int32)
+    keys, values = [], []
+    for s, n in enumerate(lengths):
+        mine = [order.pop() for _ in range(pages_per[s])]
+        table[s, :len(mine)] = torch.tensor(mine, dtype=torch.int32)
+        k = torch.randn(n, kv_heads, head_dim, generator=g).to(dtype)
+        v = torch.randn(n, kv_heads, head_dim, generator=g).to(dtype)
+        for p in range(n):
+            k_pages[mine[p // PAGE], :, p % PAGE] = k[p]
+            v_pages[mine[p // PAGE], :, p % PAGE] = v[p]
+        keys.append(k)
+        values.append(v)
+    return k_pages, v_pages, table, keys, values
+
+
+def attention_reference(q, keys, values, pos, n_heads, kv_heads, head_dim, scale, window):
+    group = n_heads // kv_heads
+    first = max(0, pos - window + 1) if window else 0
+    out = torch.empty(n_heads, head_dim, dtype=torch.float64)
+    for h in range(n_heads):
+        k = keys[first:pos + 1, h // group].double()
+        v = values[first:pos + 1, h // group].double()
+        p = torch.softmax(k @ q[h].double() * scale, 0)
+        out[h] = p @ v
+    return out
+
+
+class Layout:
+    def __init__(self, is_decode, seq_start, n_seqs):
+        self.is_decode, self.seq_start, self.n_seqs = is_decode, seq_start, n_seqs
+
+
+ATTN_SHAPES = [  # heads, kv heads, head size
+    (4, 2, 16), (6, 2, 48), (8, 8, 64), (5, 1, 80), (8, 2, 128), (3, 3, 256), (12, 4, 96), (14, 2, 128),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_heads,kv_heads,head_dim", ATTN_SHAPES)
+@pytest.mark.parametrize("window", [0, 70])
+def test_attention_decode_rows(K, dtype, n_heads, kv_heads, head_dim, window):
+    """One query per sequence at the end of caches of unequal lengths (page edges included)."""
+    lengths = [1, 63, 64, 65, 130, 517]
+    kp, vp, table, keys, values = make_cache(len(lengths), lengths, kv_heads, head_dim, dtype, seed=head_dim + n_heads)
+    g = torch.Generator().manual_seed(7)
+    q = torch.randn(len(lengths), n_heads * head_dim, generator=g).to(dtype)
+    positions = torch.tensor([n - 1 for n in lengths], dtype=torch.int32)
+    row_seq = torch.arange(len(lengths), dtype=torch.int32)
+    out = torch.empty(len(lengths), n_heads * head_dim, dtype=dtype, device="cuda:0")
+    scale = 1 / math.sqrt(head_dim)
+    layout = Layout(True, dev(torch.arange(len(lengths) + 1, dtype=torch.int32)), len(lengths))
+    K.attention(dev(q), out, dev(kp), dev(vp), dev(table), dev(row_seq), dev(positions), n_heads, kv_heads,
+                head_dim, scale, window, layout=layout)
+    for s, n in enumerate(lengths):
+        want = attention_reference(q[s].reshape(n_heads, head_dim), keys[s], values[s], n - 1, n_heads, kv_heads,
+                                   head_dim, scale, window)
+        assert rel(out[s].reshape(n_heads, head_dim), want) < tol(dtype, 1e-5, 1.2e-2), (s, n)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_heads,kv_heads,head_dim", ATTN_SHAPES)
+def test_attention_prefill_rows_ragged(K, dtype, n_heads, kv_heads, head_dim):
+    """Several sequences in one step: new tokens after pasts of different lengths (0 included)."""
+    pasts, news = [0, 5, 64, 100, 0], [70, 1, 3, 131, 1]
+    lengths = [p + n for p, n in zip(pasts, news)]
+    kp, vp, table, keys, values = make_cache(len(lengths), lengths, kv_heads, head_dim, dtype, seed=3 * head_dim + n_heads)
+    g = torch.Generator().manual_seed(11)
+    n_rows = sum(news)
+    q = torch.randn(n_rows, n_heads * head_dim, generator=g).to(dtype)
+    positions = torch.tensor([p + t for p, n in zip(pasts, news) for t in range(n)], dtype=torch.int32)
+    row_seq = torch.tensor([s for s, n in enumerate(news) for _ in range(n)], dtype=torch.int32)
+    starts = torch.tensor(np.concatenate([[0], np.cumsum(news)]), dtype=torch.int32)
+    out = torch.empty(n_rows, n_heads * head_dim, dtype=dtype, device="cuda:0")
+    scale = 1 / math.sqrt(head_dim)
+    K.attention(dev(q), out, dev(kp), dev(vp), dev(table), dev(row_seq), dev(positions), n_heads, kv_heads,
+                head_dim, scale, 0, layout=Layout(False, dev(starts), len(lengths)))
+    worst = 0.0
+    for row in range(n_rows):
+        s = int(row_seq[row])
+        want = attention_reference(q[row].reshape(n_heads, head_dim), keys[s], values[s], int(positions[row]),
+                                   n_heads, kv_heads, head_dim, scale, 0)
+        worst = max(worst, rel(out[row].reshape(n_heads, head_dim), want))
+    assert worst < tol(dtype, 1e-5, 1.2e-2), worst
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("far", [0, 63, 64, 127, 128, 300, 511, 640])
+def test_attention_finds_one_far_key_among_hundreds(K, dtype, far):
+    """The query and one key are made to fit each other so that this key takes all the weight:
+    the output must be that key's value, wherever in the pages it lies."""
+    n_heads, kv_heads, head_dim, n = 4, 2, 64, 700
+    kp, vp, table, keys, values = make_cache(1, [n], kv_heads, head_dim, dtype, seed=far)
+    q = torch.zeros(2, n_heads, head_dim)
+    direction = torch.nn.functional.normalize(torch.randn(head_dim, generator=torch.Generator().manual_seed(1)), dim=0)
+    q[:] = direction * 30
+    page = int(table[0, far // PAGE])
+    kp[page, :, far % PAGE] = (direction * 30).to(dtype)
+    keys[0][far] = (direction * 30).to(dtype)
+    q = q.reshape(2, n_heads * head_dim).to(dtype)
+    positions = torch.tensor([n - 1, max(far, 1)], dtype=torch.int32)      # the last row sees the key as its newest
+    row_seq = torch.zeros(2, dtype=torch.int32)
+    out = torch.empty(2, n_heads * head_dim, dtype=dtype, device="cuda:0")
+    K.attention(dev(q), out, dev(kp), dev(vp), dev(table), dev(row_seq), dev(positions), n_heads, kv_heads,
+                head_dim, 1 / math.sqrt(head_dim), 0, layout=None)
+    got = out.float().cpu().reshape(2, n_heads, head_dim)
+    for h in range(n_heads):
+        assert torch.allclose(got[0, h], values[0][far, h // 2].float(), atol=2e-2), (far, h)
+        assert torch.allclose(got[1, h], values[0][far, h // 2].float(), atol=2e-2), (far, h)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_window_edge(K, dtype):
+    """A key just outside the window must be invisible, the one just inside visible."""
+    n_heads, kv_heads, head_dim, n, window = 2, 1, 32, 200, 70
+    kp, vp, table, keys, values = make_cache(1, [n], kv_heads, head_dim, dtype, seed=5)
+    direction = torch.ones(head_dim) / math.sqrt(head_dim)
+    pos = n - 1
+    outside, inside = pos - window, pos - window + 1
+    for where in (outside, inside):
+        page = int(table[0, where // PAGE])
+        kp[page, :, where % PAGE] = (direction * (40 if where == outside else 25)).to(dtype)
+    q = (direction * 30).repeat(n_heads).reshape(1, -1).to(dtype)
+    out = torch.empty(1, n_heads * head_dim, dtype=dtype, device="cuda:0")
+    args = (dev(kp), dev(vp), dev(table), dev(torch.zeros(1, dtype=torch.int32)), dev(torch.tensor([pos], dtype=torch.int32)),
+            n_heads, kv_heads, head_dim, 1 / math.sqrt(head_dim))
+    K.attention(dev(q), out, *args, window)
+    assert torch.allclose(out.float().cpu().reshape(n_heads, head_dim)[0], values[0][inside, 0].float(), atol=2e-2)
+    K.attention(dev(q), out, *args, 0)
+    assert torch.allclose(out.float().cpu().reshape(n_heads, head_dim)[0], values[0][outside, 0].float(), atol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("w_dtype", DTYPES)
+@pytest.mark.parametrize("n_heads,kv_heads,head_dim,rot", [(4, 2, 16, 16), (6, 2, 48, 48), (5, 1, 80, 32),
+                                                           (8, 2, 128, 128), (3, 3, 256, 256)])
+def test_qk_norm_rope_cache(K, dtype, w_dtype, n_heads, kv_heads, head_dim, rot):
+    g = torch.Generator().manual_seed(head_dim)
+    pasts, news = [0, 62, 130], [3, 5, 1]
+    n_rows = sum(news)
+    fused = (n_heads + 2 * kv_heads) * head_dim
+    qkv = torch.randn(n_rows, fused, generator=g).to(dtype)
+    qw = (1 + 0.2 * torch.randn(head_dim, generator=g)).to(w_dtype)
+    kw = (1 + 0.2 * torch.randn(head_dim, generator=g)).to(w_dtype)
+    eps, theta, max_pos = 1e-5, 10000.0, 256
+    freqs = 1.0 / theta ** (torch.arange(0, rot, 2, dtype=torch.float64) / rot)
+    angles = torch.arange(max_pos, dtype=torch.float64)[:, None] * freqs
+    cos, sin = angles.cos().float(), angles.sin().float()
+    positions = torch.tensor([p + t for p, n in zip(pasts, news) for t in range(n)], dtype=torch.int32)
+    row_seq = torch.tensor([s for s, n in enumerate(news) for _ in range(n)], dtype=torch.int32)
+    n_pages = 9
+    table = torch.tensor([[4, 0, 0], [7, 2, 0], [1, 8, 3]], dtype=torch.int32)
+    sentinel = 777.0
+    kp = torch.full((n_pages, kv_heads, PAGE, head_dim), sentinel).to(dtype)
+    vp = torch.full((n_pages, kv_heads, PAGE, head_dim), sentinel).to(dtype)
+    kp_d, vp_d = dev(kp), dev(vp)
+    q_out = torch.empty(n_rows, n_heads * head_dim, dtype=dtype, device="cuda:0")
+    K.qk_norm_rope_cache(dev(qkv), q_out, dev(qw), dev(kw), eps, dev(cos), dev(sin), dev(positions), dev(row_seq),
+                         kp_d, vp_d, dev(table), n_heads, kv_heads, head_dim, True, int(positions.max()))
+
+    def reference(x, w, pos):      # x [heads, head_dim] float64
+        y = x / torch.sqrt((x ** 2).mean(-1, keepdim=True) + eps) * w.double()
+        half = rot // 2
+        c, s = cos[pos].double(), sin[pos].double()
+        a, b = y[:, :half], y[:, half:rot]
+        return torch.cat([a * c - b * s, a * s + b * c, y[:, rot:]], dim=-1)
+
+    written = torch.zeros(n_pages, PAGE, dtype=torch.bool)
+    for row in range(n_rows):
+        pos, seq = int(positions[row]), int(row_seq[row])
+        x = qkv[row].double()
+        q_want = reference(x[:n_heads * head_dim].reshape(n_heads, head_dim), qw, pos)
+        k_want = reference(x[n_heads * head_dim:(n_heads + kv_heads) * head_dim].reshape(kv_heads, head_dim), kw, pos)
+        v_want = x[(n_heads + kv_heads) * head_dim:].reshape(kv_heads, head_dim)
+        page = int(table[seq, pos // PAGE])
+        written[page, pos % PAGE] = True
+        assert rel(q_out[row].reshape(n_heads, head_dim), q_want) < tol(dtype, 2e-6, 4e-3)
+        assert rel(kp_d[page, :, pos % PAGE], k_want) < tol(dtype, 2e-6, 4e-3)
+        assert torch.equal(vp_d[page, :, pos % PAGE].cpu().double(), v_want)
+    # nothing else in the cache was touched
+    untouched = ~written[:, None, :, None].expand(n_pages, kv_heads, PAGE, head_dim)
+    assert bool((kp_d.cpu().float()[untouched] == sentinel).all()) and bool((vp_d.cpu().float()[untouched] == sentinel).all())
+    # without weights and tables the heads pass through; without write_kv the cache stays as it is
+    kp2, vp2 = dev(kp), dev(vp)
+    K.qk_norm_rope_cache(dev(qkv), q_out, None, None, 0.0, None, None, dev(positions), dev(row_seq), kp2, vp2,
+                         dev(table), n_heads, kv_heads, head_dim, False, int(positions.max()))
+    assert torch.equal(q_out.cpu(), qkv[:, :n_heads * head_dim])
+    assert torch.equal(kp2.cpu(), kp) and torch.equal(vp2.cpu(), vp)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,width", [(1, 10), (7, 200), (33, 12288), (2, 25600)])
+def test_swiglu(K, dtype, rows, width):
+    g = torch.Generator().manual_seed(width)
+    gu = (torch.randn(rows, 2 * width, generator=g) * 3).to(dtype)
+    out = torch.empty(rows, width, dtype=dtype, device="cuda:0")
+    K.swiglu(dev(gu), out)
+    gate, up = gu[:, :width].double(), gu[:, width:].double()
+    assert rel(out, gate / (1 + torch.exp(-gate)) * up) < tol(dtype, 2e-6, 4e-3)
+
+
+@pytest.mark.parametrize("vocab", [7, 331, 1024, 1500, 151936])
+def test_argmax_ties_go_to_the_lowest_id(K, vocab):
+    g = torch.Generator().manual_seed(vocab)
+    logits = torch.randn(5, vocab, generator=g)
+    logits[1, vocab - 1] = 50.0
+    logits[2, 0] = 50.0
+    top = min(vocab - 1, 700)
+    logits[3, top] = 60.0
+    logits[3, top // 2] = 60.0               # a tie: the lower id wins
+    logits[4, :] = 1.25                      # all equal: id 0
+    tokens = torch.empty(5, dtype=torch.int32, device="cuda:0")
+    bad = torch.empty(5, dtype=torch.int32, device="cuda:0")
+    K.sample(dev(logits), tokens, bad)
+    assert tokens.cpu().tolist() == [int(torch.argmax(logits[0])), vocab - 1, 0, top // 2, 0]
+    assert bad.cpu().tolist() == [0] * 5
+
+
+def test_sample_flags_rows_that_are_not_finite(K):
+    logits = torch.randn(3, 100)
+    logits[1, 40] = float("nan")
+    logits[2, 99] = float("inf")
+    tokens = torch.empty(3, dtype=torch.int32, device="cuda:0")
+    bad = torch.empty(3, dtype=torch.int32, device="cuda:0")
+    K.sample(dev(logits), tokens, bad)
+    assert bad.cpu().tolist() == [0, 1, 1] and tokens.cpu().tolist()[1:] == [-1, -1]
+
+
+@pytest.mark.parametrize("vocab", [331, 2048, 151936])
+def test_temperature_sampling_is_an_inverse_cdf_draw(K, vocab):
+    g = torch.Generator().manual_seed(vocab)
+    n = 64
+    logits = torch.randn(n, vocab, generator=g) * 2
+    temperature = torch.rand(n, generator=g) * 1.5 + 0.2
+    uniform = torch.rand(n, generator=g)
+    uniform[0], uniform[1] = 0.0, 0.99999994
+    tokens = torch.empty(n, dtype=torch.int32, device="cuda:0")
+    bad = torch.empty(n, dtype=torch.int32, device="cuda:0")
+    K.sample(dev(logits), tokens, bad, temperature=dev(temperature), uniform=dev(uniform))
+    probs = torch.softmax(logits.double() / temperature.double()[:, None], -1)
+    cdf = torch.cumsum(probs, -1)
+    for row, token in enumerate(tokens.cpu().tolist()):
+        lower = float(cdf[row, token - 1]) if token > 0 else 0.0
+        u = float(uniform[row])
+        assert lower - 1e-5 <= u <= float(cdf[row, token]) + 1e-5, (row, token, lower, u, float(cdf[row, token]))
+    # rows do not influence each other
+    alone = torch.empty(1, dtype=torch.int32, device="cuda:0")
+    K.sample(dev(logits[5:6]), alone, bad[:1].clone(), temperature=dev(temperature[5:6]), uniform=dev(uniform[5:6]))
+    assert int(alone.cpu()) == int(tokens[5].cpu())
+
+
+def test_top_k_and_top_p_restrict_the_draw(K):
+    vocab, n = 1000, 200
+    g = torch.Generator().manual_seed(3)
+    logits = (torch.randn(1, vocab, generator=g) * 3).repeat(n, 1)
+    uniform = torch.rand(n, generator=g)
+    temperature = torch.ones(n)
+    tokens = torch.empty(n, dtype=torch.int32, device="cuda:0")
+    bad = torch.empty(n, dtype=torch.int32, device="cuda:0")
+    top_k = torch.full((n,), 5, dtype=torch.int32)
+    K.sample(dev(logits), tokens, bad, temperature=dev(temperature), top_k=dev(top_k), uniform=dev(uniform))
+    allowed = set(torch.topk(logits[0], 5).indices.tolist())
+    drawn = set(tokens.cpu().tolist())
+    assert drawn <= allowed and len(drawn) > 1
+    # top-p: the smallest set of most likely tokens whose mass reaches p
+    p = 0.6
+    probs = torch.softmax(logits[0].double(), 0)
+    order = torch.argsort(probs, descending=True)
+    count = int(torch.searchsorted(torch.cumsum(probs[order], 0), torch.tensor(p, dtype=torch.float64))) + 1
+    nucleus = set(order[:count].tolist())
+    K.sample(dev(logits), tokens, bad, temperature=dev(temperature), top_p=dev(torch.full((n,), p)), uniform=dev(uniform))
+    drawn = set(tokens.cpu().tolist())
+    assert drawn <= nucleus and len(drawn) > 1
+    # k = 1 is greedy whatever the uniform number
+    K.sample(dev(logits), tokens, bad, temperature=dev(temperature), top_k=dev(torch.ones(n, dtype=torch.int32)),
+             uniform=dev(uniform))
+    assert set(tokens.cpu().tolist()) == {int(torch.argmax(logits[0]))}
+
+
+def test_kernels_refuse_what_they_cannot_do(K):
+    from beholdd.kernels import KernelError
+    x = torch.zeros(2, 8, device="cuda:0")
+    with pytest.raises(KernelError):
+        K.gemm(x, torch.zeros(4, 9, device="cuda:0"), torch.zeros(2, 4, device="cuda:0"))
+    with pytest.raises(KernelError):
+        K.gemm(x.cpu(), torch.zeros(4, 8, device="cuda:0"), torch.zeros(2, 4, device="cuda:0"))
+    with pytest.raises(KernelError):
+        K.rmsnorm(x, torch.ones(7, device="cuda:0"), 1e-6, torch.zeros(2, 8, device="cuda:0"))
+    with pytest.raises(KernelError):      # a head size above the attention kernels' limit
+        hd = 512
+        K.attention(torch.zeros(1, hd, device="cuda:0"), torch.zeros(1, hd, device="cuda:0"),
+                    torch.zeros(1, 1, PAGE, hd, device="cuda:0"), torch.zeros(1, 1, PAGE, hd, device="cuda:0"),
+                    torch.zeros(1, 1, dtype=torch.int32, device="cuda:0"), torch.zeros(1, dtype=torch.int32, device="cuda:0"),
+                    torch.zeros(1, dtype=torch.int32, device="cuda:0"), 1, 1, hd, 1.0)
