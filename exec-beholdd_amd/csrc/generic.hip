@@ -121,6 +121,9 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
       ws[kk][r] = (gn < N && gk < K) ? to_f32(w[(size_t)gn * K + gk]) : 0.f;
     }
     __syncthreads();
+    // blocked summation: each 16-wide slice is summed on its own and then added, so the
+    // rounding error grows with K/16 + 16 terms instead of K
+    float part[4][4] = {};
 #pragma unroll
     for (int kk = 0; kk < GK; ++kk) {
       float av[4], wv[4];
@@ -131,8 +134,12 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+        for (int j = 0; j < 4; ++j) part[i][j] = fmaf(av[i], wv[j], part[i][j]);
     }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] += part[i][j];
     __syncthreads();
   }
 #pragma unroll

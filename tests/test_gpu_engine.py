@@ -91,8 +91,8 @@ def test_float32_storage_and_slot_reuse_in_a_small_cache(model_dirs, dtype):
     assert engine.cache.n_pages == 3
     check("whole", schedules.whole(engine, requests), want, TOLERANCE[dtype])
     check("tail", schedules.tail_one_by_one(engine, requests, tail=32), want, TOLERANCE[dtype])
-    check("pairs", schedules.batches(engine, [requests[1], requests[3], requests[4], requests[0]], batch_size=2),
-          [want[1], want[3], want[4], want[0]], TOLERANCE[dtype])
+    check("pairs", schedules.batches(engine, [requests[1], requests[3], requests[4], requests[3]], batch_size=2),
+          [want[1], want[3], want[4], want[3]], TOLERANCE[dtype])      # 64 + 1, then 65 + 1 tokens: 2, then 3 pages
     engine.cache.check_invariants()
 
 

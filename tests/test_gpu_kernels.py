@@ -78,14 +78,15 @@ def test_gemm(K, a_dtype, w_dtype, m, n, k):
     a = torch.randn(m, k, generator=g).to(a_dtype)
     w = (torch.randn(n, k, generator=g) * 0.05).to(w_dtype)
     want = a.double() @ w.double().t()
+    f32_bound = 4 * math.sqrt(k) * 2.0 ** -24      # float32 accumulation of k products, a few standard deviations
     for out_dtype in (torch.float32, a_dtype):
         out = torch.empty(m, n, dtype=out_dtype, device="cuda:0")
         K.gemm(dev(a), dev(w), out)
-        assert rel(out, want) < tol(out_dtype, 2e-6, 4e-3), (out_dtype, rel(out, want))
+        assert rel(out, want) < tol(out_dtype, f32_bound, 4e-3), (out_dtype, rel(out, want))
     base = torch.randn(m, n, generator=g)
     acc = dev(base.clone())
     K.gemm(dev(a), dev(w), acc, accumulate=True)
-    assert rel(acc, want + base.double()) < 2e-6
+    assert rel(acc, want + base.double()) < f32_bound
 
 
 def make_cache(n_seqs, lengths, kv_heads, head_dim, dtype, seed, extra_pages=3):
@@ -249,7 +250,7 @@ def test_qk_norm_rope_cache(K, dtype, w_dtype, n_heads, kv_heads, head_dim, rot)
     row_seq = torch.tensor([s for s, n in enumerate(news) for _ in range(n)], dtype=torch.int32)
     n_pages = 9
     table = torch.tensor([[4, 0, 0], [7, 2, 0], [1, 8, 3]], dtype=torch.int32)
-    sentinel = 777.0
+    sentinel = 768.0        # exact in bfloat16
     kp = torch.full((n_pages, kv_heads, PAGE, head_dim), sentinel).to(dtype)
     vp = torch.full((n_pages, kv_heads, PAGE, head_dim), sentinel).to(dtype)
     kp_d, vp_d = dev(kp), dev(vp)
