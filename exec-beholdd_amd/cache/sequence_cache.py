@@ -3,8 +3,10 @@
 Layout.  A *slot* is one sequence's handle: its length, its pages and its row in every state
 region.  Layers are sorted into *groups* by what they need (`CacheNeed`): every group has
 storage of its own.  A key/value group holds, for each of its cache entries (one per
-scheduled layer run that writes a cache), two tensors [pages, kv_heads, page_size, head_dim];
-a sequence's positions p live in page `table[p // page_size]` at row `p % page_size`, and a
+scheduled layer run that writes a cache), keys [pages, kv_heads, page_size, head_dim] and values
+[pages, kv_heads, head_dim, page_size] (transposed inside a page, the layout the matrix-core
+attention kernels load directly); a sequence's position p lives in page `table[p // page_size]`
+at token `p % page_size`, and a
 group with a window gives pages back once every position in them has left the window.  A
 state group holds [entries, max_slots, *shape] and a slot's rows are zero when it starts.
 
@@ -124,9 +126,10 @@ class SequenceCache:
             raise CacheFull(f"the cache needs {plan.total_bytes} bytes, the limit is {limit_bytes}")
         for g in self.groups:
             if g.need.kind == "kv":
-                shape = (len(g.entries), self.n_pages, g.need.kv_heads, self.page_size, g.need.head_dim)
-                g.k = torch.empty(shape, dtype=self.dtype, device=self.device)
-                g.v = torch.empty(shape, dtype=self.dtype, device=self.device)
+                head = (len(g.entries), self.n_pages, g.need.kv_heads)
+                # zeros, not empty: rows of a page that no token has written yet must hold finite numbers
+                g.k = torch.zeros((*head, self.page_size, g.need.head_dim), dtype=self.dtype, device=self.device)
+                g.v = torch.zeros((*head, g.need.head_dim, self.page_size), dtype=self.dtype, device=self.device)
                 g.free_pages = list(range(self.n_pages - 1, -1, -1))   # pop() hands out page 0 first
             else:
                 g.state = torch.zeros((len(g.entries), self.max_slots, *g.need.state_shape),

@@ -1,0 +1,289 @@
+// bfloat16 attention over the paged cache on the gfx950 matrix cores, for prefill and decode.
+//
+// A *column* is one (row, query head) pair.  A workgroup takes 16 columns that share a sequence
+// and a kv head (consecutive rows x the heads of one group) and a range of that sequence's cache
+// pages; its four waves take the pages of the range in turn.  For each page of 64 keys a wave
+// computes, with v_mfma_f32_16x16x32_bf16,
+//     S^T[key, column] = K[key, :] . Q[column, :]        (keys as rows: K is loaded straight from
+//                                                          the cache in operand layout)
+//     running maximum / sum per column in float32 (online softmax, exponent base 2)
+//     O^T[d, column] += V^T[d, key] . P^T[key, column]   (the cache keeps V transposed inside a
+//                                                          page, so this operand is a straight load too)
+// The rows of an S^T tile are assigned to keys so that every lane ends up with 16 consecutive
+// keys of the page: tile t, row i <-> key 16*(i/4) + 4*t + i%4.  Lane (column j, group g) then
+// holds keys 16g .. 16g+15, which is exactly the k-slice its P^T operand needs.
+// The waves' results are merged through LDS.  When the keys of a sequence are split over several
+// workgroups (decode: few columns, long caches) each writes an unnormalised partial result and
+// its (maximum, sum) to scratch memory and a second kernel combines them.
+//
+// head_dim must be a multiple of 32, at most 256.  Masking is by position: column j sees keys
+// lo_j .. pos_j.  Rows of a page beyond the last written key are never multiplied in: their
+// probabilities are zero and their V values are zeroed before use.
+#include "common.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x8_t __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+__device__ inline bf16x8_t as_bf16x8(u32x4_t v) { return __builtin_bit_cast(bf16x8_t, v); }
+__device__ inline u32x4_t load16(const uint16_t* p) { return *reinterpret_cast<const u32x4_t*>(p); }
+
+__device__ inline int wave_max_int(int v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = max(v, __shfl_xor(v, off, 64));
+  return v;
+}
+__device__ inline int wave_min_int(int v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = min(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+__device__ inline uint32_t pack_bf16(float lo, float hi) {
+  return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+}
+
+// keep the first `n_valid` (0..8) bfloat16 elements of a 16-byte vector, zero the rest
+__device__ inline u32x4_t keep_first(u32x4_t v, int n_valid) {
+#pragma unroll
+  for (int word = 0; word < 4; ++word) {
+    const uint32_t mask = (2 * word + 1 < n_valid) ? 0xffffffffu : (2 * word < n_valid ? 0x0000ffffu : 0u);
+    v[word] &= mask;
+  }
+  return v;
+}
+
+template <int NS>
+__global__ __launch_bounds__(256) void attention_mfma_kernel(
+    const uint16_t* __restrict__ q, uint16_t* __restrict__ out, float* __restrict__ part_o,
+    float* __restrict__ part_ml, const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages,
+    const int32_t* __restrict__ page_table, int table_stride, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ seq_start, int H, int KVH, float scale_log2, int window, int n_splits,
+    int pages_per_split) {
+  constexpr int HD = 32 * NS;
+  constexpr int LANE_D = 8 * NS;  // head_dim elements per lane group
+  __shared__ float sm_m[4][16];
+  __shared__ float sm_l[4][16];
+  __shared__ float sm_o[4][16][HD + 1];
+
+  const int tile = blockIdx.x, kvh = blockIdx.y;
+  const int seq = blockIdx.z / n_splits, split = blockIdx.z % n_splits;
+  const int G = H / KVH;
+  const int row0 = seq_start[seq];
+  const int n_cols = (seq_start[seq + 1] - row0) * G;
+  if (tile * 16 >= n_cols) return;
+
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int j = lane % 16, g = lane / 16;
+  const int c = (tile * 16 + j < n_cols) ? tile * 16 + j : n_cols - 1;
+  const int row = row0 + c / G, head = kvh * G + c % G;
+  const int pos = positions[row];
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int pos_max = wave_max_int(pos), pos_min = wave_min_int(pos);
+  const int lo_min = wave_min_int(lo), lo_max = wave_max_int(lo);
+
+  const int begin = lo_min / BH_PAGE + split * pages_per_split;
+  const int last = pos_max / BH_PAGE;
+  const int end = (begin + pages_per_split < last + 1) ? begin + pages_per_split : last + 1;
+  const int32_t* table = page_table + (size_t)seq * table_stride;
+
+  bf16x8_t q_vec[NS];
+  {
+    const uint16_t* qp = q + ((size_t)row * H + head) * HD + g * LANE_D;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) q_vec[s] = as_bf16x8(load16(qp + 8 * s));
+  }
+  f32x4_t o[2 * NS];
+#pragma unroll
+  for (int dt = 0; dt < 2 * NS; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float run_max = -INFINITY, run_sum = 0.f;  // run_sum: this lane's share of the column's sum
+
+  for (int p = begin + wave; p < end; p += 4) {
+    const int page = table[p];
+    const uint16_t* kb = k_pages + ((size_t)page * KVH + kvh) * BH_PAGE * HD;
+    const uint16_t* vb = v_pages + ((size_t)page * KVH + kvh) * HD * BH_PAGE;
+    u32x4_t k_vec[4][NS], v_vec[2 * NS][2];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const uint16_t* kr = kb + (size_t)(16 * (j / 4) + 4 * t + j % 4) * HD + g * LANE_D;
+#pragma unroll
+      for (int s = 0; s < NS; ++s) k_vec[t][s] = load16(kr + 8 * s);
+    }
+#pragma unroll
+    for (int dt = 0; dt < 2 * NS; ++dt) {
+      const uint16_t* vr = vb + (size_t)(16 * dt + j) * BH_PAGE + 16 * g;
+      v_vec[dt][0] = load16(vr);
+      v_vec[dt][1] = load16(vr + 8);
+    }
+    f32x4_t st[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < NS; ++s)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(k_vec[t][s]), q_vec[s], acc, 0, 0, 0);
+      st[t] = acc;
+    }
+    // lane (j, g) now holds keys key0 + 4t + r of its column, for t, r in 0..3
+    const int key0 = p * BH_PAGE + 16 * g;
+    const bool mask_needed = (p * BH_PAGE + BH_PAGE - 1 > pos_min) || (p * BH_PAGE < lo_max);
+    float local_max = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float v = st[t][r] * scale_log2;
+        if (mask_needed) {
+          const int key = key0 + 4 * t + r;
+          if (key > pos || key < lo) v = -INFINITY;
+        }
+        st[t][r] = v;
+        local_max = fmaxf(local_max, v);
+      }
+    local_max = fmaxf(local_max, __shfl_xor(local_max, 16, 64));
+    local_max = fmaxf(local_max, __shfl_xor(local_max, 32, 64));
+    const float new_max = fmaxf(run_max, local_max);
+    const float safe_max = (new_max == -INFINITY) ? 0.f : new_max;
+    const float alpha = exp2f(run_max - safe_max);  // 0 when nothing was seen before
+    float page_sum = 0.f;
+    u32x4_t p_vec[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const int t = 2 * u + half;
+        const float e0 = exp2f(st[t][0] - safe_max), e1 = exp2f(st[t][1] - safe_max);
+        const float e2 = exp2f(st[t][2] - safe_max), e3 = exp2f(st[t][3] - safe_max);
+        page_sum += (e0 + e1) + (e2 + e3);
+        p_vec[u][2 * half] = pack_bf16(e0, e1);
+        p_vec[u][2 * half + 1] = pack_bf16(e2, e3);
+      }
+    run_sum = run_sum * alpha + page_sum;
+    run_max = new_max;
+    if (p * BH_PAGE + BH_PAGE - 1 > pos_max) {  // the page's tail was never written for this step: zero it
+      const int valid = pos_max + 1 - key0;
+#pragma unroll
+      for (int dt = 0; dt < 2 * NS; ++dt) {
+        v_vec[dt][0] = keep_first(v_vec[dt][0], valid);
+        v_vec[dt][1] = keep_first(v_vec[dt][1], valid - 8);
+      }
+    }
+#pragma unroll
+    for (int dt = 0; dt < 2 * NS; ++dt) {
+      f32x4_t acc = o[dt] * alpha;
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(v_vec[dt][0]), as_bf16x8(p_vec[0]), acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(v_vec[dt][1]), as_bf16x8(p_vec[1]), acc, 0, 0, 0);
+      o[dt] = acc;
+    }
+  }
+
+  // merge the four waves: lane (j, g) holds O^T[16dt + 4g + r, j]
+  run_sum += __shfl_xor(run_sum, 16, 64);
+  run_sum += __shfl_xor(run_sum, 32, 64);
+  if (g == 0) {
+    sm_m[wave][j] = run_max;
+    sm_l[wave][j] = run_sum;
+  }
+#pragma unroll
+  for (int dt = 0; dt < 2 * NS; ++dt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) sm_o[wave][j][16 * dt + 4 * g + r] = o[dt][r];
+  __syncthreads();
+  for (int e = threadIdx.x; e < 16 * HD; e += 256) {
+    const int col = e / HD, d = e % HD;
+    const int cc = tile * 16 + col;
+    if (cc >= n_cols) continue;
+    float top = fmaxf(fmaxf(sm_m[0][col], sm_m[1][col]), fmaxf(sm_m[2][col], sm_m[3][col]));
+    const float safe_top = (top == -INFINITY) ? 0.f : top;
+    float sum = 0.f, value = 0.f;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const float f = exp2f(sm_m[v][col] - safe_top);
+      sum += sm_l[v][col] * f;
+      value += sm_o[v][col][d] * f;
+    }
+    const size_t column = (size_t)(row0 + cc / G) * H + kvh * G + cc % G;
+    if (n_splits == 1) {
+      out[column * HD + d] = f32_to_bf16_bits(value / sum);
+    } else {
+      part_o[(column * n_splits + split) * HD + d] = value;
+      if (d == 0) {
+        part_ml[(column * n_splits + split) * 2] = top;
+        part_ml[(column * n_splits + split) * 2 + 1] = sum;
+      }
+    }
+  }
+}
+
+__global__ void attention_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                         uint16_t* __restrict__ out, int n_splits, int HD) {
+  const size_t column = blockIdx.x;
+  const float* ml = part_ml + column * n_splits * 2;
+  float top = -INFINITY;
+  for (int s = 0; s < n_splits; ++s) top = fmaxf(top, ml[2 * s]);
+  float sum = 0.f;
+  for (int s = 0; s < n_splits; ++s) sum += ml[2 * s + 1] * exp2f(ml[2 * s] - top);
+  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+    float value = 0.f;
+    for (int s = 0; s < n_splits; ++s)
+      value += part_o[(column * n_splits + s) * HD + d] * exp2f(ml[2 * s] - top);
+    out[column * HD + d] = f32_to_bf16_bits(value / sum);
+  }
+}
+
+// How many ways the keys are split for a given launch; the caller sizes the scratch from it.
+extern "C" int bh_attention_bf16_splits(int n_seqs, int max_rows_per_seq, int H, int KVH, int max_position) {
+  if (n_seqs <= 0 || max_rows_per_seq <= 0 || H <= 0 || KVH <= 0 || H % KVH) return 1;
+  const int G = H / KVH;
+  const long tiles = (long)((max_rows_per_seq * G + 15) / 16) * KVH * n_seqs;
+  const int pages = max_position / BH_PAGE + 1;
+  if (tiles >= 512 || pages < 8) return 1;
+  long want = (1024 + tiles - 1) / tiles;
+  if (want > pages / 2) want = pages / 2;  // at least two pages per split
+  if (want < 1) want = 1;
+  const int per = (int)((pages + want - 1) / want);
+  return (pages + per - 1) / per;
+}
+
+extern "C" int bh_attention_bf16(const void* q, void* out, void* part_o, void* part_ml, const void* k_pages,
+                                 const void* v_pages, const int32_t* page_table, int table_stride,
+                                 const int32_t* positions, const int32_t* seq_start, int n_seqs, int n_rows,
+                                 int max_rows_per_seq, int H, int KVH, int hd, float scale, int window,
+                                 int max_position, int n_splits, hipStream_t stream) {
+  BH_REQUIRE(n_seqs > 0 && n_rows > 0 && max_rows_per_seq > 0, "attention_bf16: empty batch");
+  BH_REQUIRE(H > 0 && KVH > 0 && H % KVH == 0, "attention_bf16: %d query heads do not group evenly into %d kv heads", H, KVH);
+  BH_REQUIRE(hd % 32 == 0 && hd >= 32 && hd <= 256, "attention_bf16: head size %d is not a multiple of 32 up to 256", hd);
+  BH_REQUIRE(window >= 0 && max_position >= 0, "attention_bf16: window and positions must not be negative");
+  BH_REQUIRE(n_splits >= 1 && (n_splits == 1 || (part_o && part_ml)), "attention_bf16: split keys need scratch memory");
+  const int G = H / KVH;
+  const int tiles = (max_rows_per_seq * G + 15) / 16;
+  const int pages = max_position / BH_PAGE + 1;
+  const int per = (pages + n_splits - 1) / n_splits;
+  BH_REQUIRE((long)n_seqs * n_splits <= 65535 && KVH <= 65535, "attention_bf16: too many sequences x splits");
+  dim3 grid(tiles, KVH, n_seqs * n_splits), block(256);
+  const float scale_log2 = scale * 1.4426950408889634f;
+#define BH_ATT(NS)                                                                                              \
+  attention_mfma_kernel<NS><<<grid, block, 0, stream>>>(                                                        \
+      (const uint16_t*)q, (uint16_t*)out, (float*)part_o, (float*)part_ml, (const uint16_t*)k_pages,            \
+      (const uint16_t*)v_pages, page_table, table_stride, positions, seq_start, H, KVH, scale_log2, window,     \
+      n_splits, per)
+  switch (hd / 32) {
+    case 1: BH_ATT(1); break;
+    case 2: BH_ATT(2); break;
+    case 3: BH_ATT(3); break;
+    case 4: BH_ATT(4); break;
+    case 5: BH_ATT(5); break;
+    case 6: BH_ATT(6); break;
+    case 7: BH_ATT(7); break;
+    default: BH_ATT(8); break;
+  }
+#undef BH_ATT
+  if (int status = bh_check_launch("attention_mfma")) return status;
+  if (n_splits > 1) {
+    attention_combine_kernel<<<dim3(n_rows * H), dim3(hd >= 128 ? 128 : 64), 0, stream>>>(
+        (const float*)part_o, (const float*)part_ml, (uint16_t*)out, n_splits, hd);
+    return bh_check_launch("attention_combine");
+  }
+  return 0;
+}

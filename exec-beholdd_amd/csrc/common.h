@@ -101,12 +101,7 @@ int bh_check_launch(const char* what);
     if (!(cond)) return bh_fail(__VA_ARGS__);  \
   } while (0)
 
-// The cache of one layer as the kernels see it: pages of BH_PAGE tokens,
-// laid [page][kv_head][token in page][head_dim], found through a per-sequence page table.
-struct BhPagedKV {
-  void* k_pages;
-  void* v_pages;
-  const int32_t* page_table;  // [n_seqs, table_stride]
-  int table_stride;
-  int n_pages;                // pages in the pool, for bounds checks on the host
-};
+// The cache of one layer as the kernels see it: pages of BH_PAGE tokens found through a
+// per-sequence page table.  Keys lie [page][kv_head][token in page][head_dim]; values lie
+// transposed, [page][kv_head][head_dim][token in page], so that a matrix-core operand of
+// "head_dim rows x consecutive tokens" is a contiguous load.

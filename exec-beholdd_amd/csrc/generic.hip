@@ -193,7 +193,7 @@ extern "C" int bh_gemm_generic(const void* a, int a_dtype, const void* w, int w_
 // One wave per (row, head) of the fused projection row [q heads | k heads | v heads].
 // q head: optional RMSNorm over the head, rotation at the row's position, written to q_out.
 // k head: the same, written into the cache page of (sequence, position).
-// v head: copied into the cache.  Rotation pairs are (i, i + rot/2) for i < rot/2; elements
+// v head: copied into the cache (transposed within its page).  Rotation pairs are (i, i + rot/2) for i < rot/2; elements
 // from rot to head_dim pass through.  With write_kv == 0 only the q heads are processed.
 
 template <typename T, typename TW>
@@ -210,7 +210,6 @@ __global__ __launch_bounds__(64) void qk_norm_rope_cache_kernel(
 
   T* dst;
   const TW* weight;
-  bool is_value = false;
   if (head < H) {
     dst = q_out + ((size_t)row * H + head) * hd;
     weight = q_weight;
@@ -218,14 +217,14 @@ __global__ __launch_bounds__(64) void qk_norm_rope_cache_kernel(
     const int seq = row_seq[row];
     const int page = page_table[(size_t)seq * table_stride + pos / BH_PAGE];
     const int kv_head = (head - H) % KVH;
-    is_value = head >= H + KVH;
-    T* pages = is_value ? v_pages : k_pages;
-    dst = pages + (((size_t)page * KVH + kv_head) * BH_PAGE + (pos % BH_PAGE)) * hd;
+    const bool is_value = head >= H + KVH;
     weight = k_weight;
-  }
-  if (is_value) {
-    for (int i = lane; i < hd; i += BH_WAVE) dst[i] = src[i];
-    return;
+    if (is_value) {  // values lie transposed in a page: [head_dim][token]
+      T* column = v_pages + ((size_t)page * KVH + kv_head) * BH_PAGE * hd + (pos % BH_PAGE);
+      for (int i = lane; i < hd; i += BH_WAVE) column[(size_t)i * BH_PAGE] = src[i];
+      return;
+    }
+    dst = k_pages + (((size_t)page * KVH + kv_head) * BH_PAGE + (pos % BH_PAGE)) * hd;
   }
   float inv = 1.f;
   if (weight) {
@@ -346,8 +345,8 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
       for (int jj = group; jj < n_keys; jj += n_groups) {
         const int key = c0 + jj;
         const int page = table[key / BH_PAGE];
-        const T* vr = v_pages + (((size_t)page * KVH + kv_head) * BH_PAGE + (key % BH_PAGE)) * hd;
-        acc = fmaf(probs[jj], to_f32(vr[dim]), acc);
+        const T* vr = v_pages + ((size_t)page * KVH + kv_head) * BH_PAGE * hd + (key % BH_PAGE);
+        acc = fmaf(probs[jj], to_f32(vr[(size_t)dim * BH_PAGE]), acc);
       }
     }
     __syncthreads();  // probs[] is rewritten by the next chunk

@@ -70,5 +70,6 @@ def build_step(kernels, act_dtype, device, cache, entries: list, vocab: int):
         kernels=kernels, act_dtype=act_dtype, device=torch.device(device), n_rows=n_rows, n_seqs=n_seqs,
         tokens=views[0], positions=views[1], row_seq=views[2], seq_start=views[3], seq_slot=views[4],
         seq_past=views[5], host_seq_start=seq_start, host_seq_slot=seq_slot, host_seq_past=seq_past,
-        is_decode=(n_rows == n_seqs), max_position=max(positions))
+        is_decode=(n_rows == n_seqs), max_position=max(positions),
+        max_rows_per_seq=max(n for _, n in requests))
     return ctx, views[6], requests

@@ -72,8 +72,8 @@ class HipKernels:
         self._optional = {}
         for name, argtypes in {
             "bh_gemm_bf16": [p, p, p, i, i, i, i, i, p],
-            "bh_attention_prefill_bf16": [p, p, p, p, p, i, p, p, p, i, i, i, i, i, f, i, p],
-            "bh_attention_decode_bf16": [p, p, p, p, p, i, p, p, p, i, i, i, i, i, f, i, p],
+            "bh_attention_bf16": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, i, i, f, i, i, i, p],
+            "bh_attention_bf16_splits": [i, i, i, i, i],
         }.items():
             function = getattr(lib, name, None)
             if function is not None:
@@ -183,8 +183,10 @@ class HipKernels:
 
     def _check_pages(self, k_pages, v_pages, page_table, n_kv_heads, head_dim, dtype, what):
         expected = (k_pages.shape[0], n_kv_heads, self.page_size, head_dim)
-        if k_pages.shape != expected or v_pages.shape != expected:
-            raise KernelError(f"{what}: cache pages must be [pages, {n_kv_heads}, {self.page_size}, {head_dim}], got "
+        expected_v = (k_pages.shape[0], n_kv_heads, head_dim, self.page_size)
+        if k_pages.shape != expected or v_pages.shape != expected_v:
+            raise KernelError(f"{what}: key pages must be [pages, {n_kv_heads}, {self.page_size}, {head_dim}] and value "
+                              f"pages [pages, {n_kv_heads}, {head_dim}, {self.page_size}], got "
                               f"{tuple(k_pages.shape)} and {tuple(v_pages.shape)}")
         if k_pages.dtype != dtype or v_pages.dtype != dtype:
             raise KernelError(f"{what}: cache dtype {k_pages.dtype} differs from the activations' {dtype}")
@@ -195,7 +197,9 @@ class HipKernels:
                   scale, window=0, layout=None):
         """out[row, head] = softmax(q . K * scale) V over the keys of the row's sequence that the row
         may see: positions max(0, p - window + 1) .. p (window 0 = all).  `layout`, when given,
-        describes how rows group into sequences so that a faster kernel can be chosen."""
+        says how rows group into sequences (seq_start int32 [n_seqs + 1] on the device, n_seqs,
+        max_rows_per_seq, max_position), which the matrix-core kernel needs; rows of one sequence
+        are consecutive and in position order."""
         n_rows = q.shape[0]
         if q.shape != (n_rows, n_heads * head_dim) or out.shape != q.shape or out.dtype != q.dtype:
             raise KernelError(f"attention: shapes q {tuple(q.shape)}, out {tuple(out.shape)} do not fit")
@@ -205,17 +209,27 @@ class HipKernels:
             raise KernelError("attention: positions and row_seq must have one entry per row")
         self._check_pages(k_pages, v_pages, page_table, n_kv_heads, head_dim, q.dtype, "attention")
         common = (self._ptr(q, "q"), self._ptr(out, "attention out"))
-        if q.dtype == torch.bfloat16 and layout is not None and head_dim % 16 == 0:
-            name = "bh_attention_decode_bf16" if layout.is_decode else "bh_attention_prefill_bf16"
-            fast = self._optional.get(name)
-            if fast is not None and head_dim in (64, 128):
-                self._check(fast(*common, self._ptr(k_pages, "k_pages"), self._ptr(v_pages, "v_pages"),
-                                 self._ptr(page_table, "page_table", (torch.int32,)), page_table.shape[1],
-                                 self._ptr(row_seq, "row_seq", (torch.int32,)),
-                                 self._ptr(positions, "positions", (torch.int32,)),
-                                 self._ptr(layout.seq_start, "seq_start", (torch.int32,)), layout.n_seqs,
-                                 n_rows, n_heads, n_kv_heads, head_dim, float(scale), int(window), self._stream()))
-                return
+        fast = self._optional.get("bh_attention_bf16")
+        if (fast is not None and q.dtype == torch.bfloat16 and layout is not None and head_dim % 32 == 0
+                and head_dim <= 256):
+            n_seqs, max_rows = int(layout.n_seqs), int(layout.max_rows_per_seq)
+            if layout.seq_start.shape != (n_seqs + 1,) or page_table.shape[0] < n_seqs:
+                raise KernelError("attention: seq_start must have one entry per sequence and one more, and the page "
+                                  "table a row per sequence")
+            n_splits = int(self._optional["bh_attention_bf16_splits"](n_seqs, max_rows, n_heads, n_kv_heads,
+                                                                      int(layout.max_position)))
+            part_o = part_ml = None
+            if n_splits > 1:   # partial results of the key splits: scratch for this call only
+                part_o = torch.empty(n_rows * n_heads * n_splits * head_dim, dtype=torch.float32, device=self.device)
+                part_ml = torch.empty(n_rows * n_heads * n_splits * 2, dtype=torch.float32, device=self.device)
+            self._check(fast(*common, self._ptr(part_o, "partial o", None, True),
+                             self._ptr(part_ml, "partial sums", None, True), self._ptr(k_pages, "k_pages"),
+                             self._ptr(v_pages, "v_pages"), self._ptr(page_table, "page_table", (torch.int32,)),
+                             page_table.shape[1], self._ptr(positions, "positions", (torch.int32,)),
+                             self._ptr(layout.seq_start, "seq_start", (torch.int32,)), n_seqs, n_rows, max_rows,
+                             n_heads, n_kv_heads, head_dim, float(scale), int(window), int(layout.max_position),
+                             n_splits, self._stream()))
+            return
         self._check(self.lib.bh_attention_generic(
             *common, _code(q, "q"), self._ptr(k_pages, "k_pages"), self._ptr(v_pages, "v_pages"),
             self._ptr(page_table, "page_table", (torch.int32,)), page_table.shape[1],

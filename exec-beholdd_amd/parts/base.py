@@ -87,6 +87,7 @@ class StepContext:
     host_seq_past: list
     is_decode: bool
     max_position: int                      # largest absolute position in this step
+    max_rows_per_seq: int = 1              # most tokens any one sequence brings
     extras: dict = field(default_factory=dict)
 
     def new_activations(self, *shape) -> torch.Tensor:
@@ -100,7 +101,8 @@ class StepContext:
 class LayerCache:
     """The storage of one cache entry as handed to a mixer for one step.
 
-    kv need:    k_pages, v_pages [pages, kv_heads, page_size, head_dim]; page_table int32
+    kv need:    k_pages [pages, kv_heads, page_size, head_dim], v_pages [pages, kv_heads, head_dim,
+                page_size]; page_table int32
                 [n_seqs, width] for the sequences of this step, in batch order.
     state need: state [max_slots, *state_shape]; index it with ctx.seq_slot.
     `writes` is False when the schedule lets this layer read another layer's entry.

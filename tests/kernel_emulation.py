@@ -71,7 +71,7 @@ class TorchKernels:
             pos = int(positions[row])
             page = int(page_table[int(row_seq[row]), pos // PAGE])
             k_pages[page, :, pos % PAGE, :] = k[row].to(k_pages.dtype)
-            v_pages[page, :, pos % PAGE, :] = v[row].to(v_pages.dtype)
+            v_pages[page, :, :, pos % PAGE] = v[row].to(v_pages.dtype)
 
     def attention(self, q, out, k_pages, v_pages, page_table, row_seq, positions, n_heads, n_kv_heads, head_dim,
                   scale, window=0, layout=None):
@@ -86,7 +86,7 @@ class TorchKernels:
             index = torch.arange(first, pos + 1)
             pages = page_table[seq, index // PAGE].long()
             keys = k_pages[pages, :, index % PAGE, :].float()      # [n, kv_heads, head_dim]
-            values = v_pages[pages, :, index % PAGE, :].float()
+            values = v_pages[pages, :, :, index % PAGE].float()
             for head in range(n_heads):
                 kv = head // group
                 scores = (keys[:, kv, :].double() @ qh[row, head].double()).float() * scale

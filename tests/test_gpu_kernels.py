@@ -72,7 +72,8 @@ def test_rmsnorm(K, out_dtype, w_dtype, rows, width, eps):
 @pytest.mark.parametrize("a_dtype,w_dtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
                                              (torch.bfloat16, torch.float32)])
 @pytest.mark.parametrize("m,n,k", [(1, 96, 120), (7, 331, 200), (64, 130, 72), (65, 257, 1000), (200, 64, 48),
-                                   (3, 1000, 4096), (130, 520, 264)])
+                                   (3, 1000, 4096), (130, 520, 264), (17, 40, 100), (33, 100, 2048), (48, 16, 8),
+                                   (8, 4096, 12288), (300, 1000, 1024), (1, 15, 64)])
 def test_gemm(K, a_dtype, w_dtype, m, n, k):
     g = torch.Generator().manual_seed(m * 1000 + n)
     a = torch.randn(m, k, generator=g).to(a_dtype)
@@ -97,7 +98,7 @@ def make_cache(n_seqs, lengths, kv_heads, head_dim, dtype, seed, extra_pages=3):
     n_pages = sum(pages_per) + extra_pages
     order = torch.randperm(n_pages, generator=g).tolist()
     k_pages = torch.randn(n_pages, kv_heads, PAGE, head_dim, generator=g).to(dtype)   # garbage everywhere
-    v_pages = torch.randn(n_pages, kv_heads, PAGE, head_dim, generator=g).to(dtype)
+    v_pages = torch.randn(n_pages, kv_heads, head_dim, PAGE, generator=g).to(dtype)           # transposed in a page
     width = max(pages_per)
     table = torch.zeros(n_seqs, width, dtype=torch.int32)
     keys, values = [], []
@@ -108,7 +109,7 @@ def make_cache(n_seqs, lengths, kv_heads, head_dim, dtype, seed, extra_pages=3):
         v = torch.randn(n, kv_heads, head_dim, generator=g).to(dtype)
         for p in range(n):
             k_pages[mine[p // PAGE], :, p % PAGE] = k[p]
-            v_pages[mine[p // PAGE], :, p % PAGE] = v[p]
+            v_pages[mine[p // PAGE], :, :, p % PAGE] = v[p]
         keys.append(k)
         values.append(v)
     return k_pages, v_pages, table, keys, values
@@ -127,8 +128,9 @@ def attention_reference(q, keys, values, pos, n_heads, kv_heads, head_dim, scale
 
 
 class Layout:
-    def __init__(self, is_decode, seq_start, n_seqs):
+    def __init__(self, is_decode, seq_start, n_seqs, max_rows_per_seq, max_position):
         self.is_decode, self.seq_start, self.n_seqs = is_decode, seq_start, n_seqs
+        self.max_rows_per_seq, self.max_position = max_rows_per_seq, max_position
 
 
 ATTN_SHAPES = [  # heads, kv heads, head size
@@ -149,13 +151,42 @@ def test_attention_decode_rows(K, dtype, n_heads, kv_heads, head_dim, window):
     row_seq = torch.arange(len(lengths), dtype=torch.int32)
     out = torch.empty(len(lengths), n_heads * head_dim, dtype=dtype, device="cuda:0")
     scale = 1 / math.sqrt(head_dim)
-    layout = Layout(True, dev(torch.arange(len(lengths) + 1, dtype=torch.int32)), len(lengths))
+    layout = Layout(True, dev(torch.arange(len(lengths) + 1, dtype=torch.int32)), len(lengths), 1, max(lengths) - 1)
     K.attention(dev(q), out, dev(kp), dev(vp), dev(table), dev(row_seq), dev(positions), n_heads, kv_heads,
                 head_dim, scale, window, layout=layout)
     for s, n in enumerate(lengths):
         want = attention_reference(q[s].reshape(n_heads, head_dim), keys[s], values[s], n - 1, n_heads, kv_heads,
                                    head_dim, scale, window)
         assert rel(out[s].reshape(n_heads, head_dim), want) < tol(dtype, 1e-5, 1.2e-2), (s, n)
+
+
+@pytest.mark.parametrize("n_heads,kv_heads,head_dim", [(8, 2, 128), (4, 4, 64), (6, 1, 96), (32, 8, 128)])
+def test_attention_decode_with_split_keys_and_garbage_beyond_the_end(K, n_heads, kv_heads, head_dim):
+    """Long caches and few sequences: the keys are split over workgroups and combined.  Whatever lies in
+    a page beyond a sequence's last token (here NaN) must not reach the result."""
+    dtype = torch.bfloat16
+    lengths = [3000, 1, 1500, 2049]
+    kp, vp, table, keys, values = make_cache(len(lengths), lengths, kv_heads, head_dim, dtype, seed=head_dim)
+    for s, n in enumerate(lengths):
+        if n % PAGE:
+            page = int(table[s, (n - 1) // PAGE])
+            kp[page, :, n % PAGE:, :] = float("nan")
+            vp[page, :, :, n % PAGE:] = float("nan")
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(len(lengths), n_heads * head_dim, generator=g).to(dtype)
+    positions = torch.tensor([n - 1 for n in lengths], dtype=torch.int32)
+    row_seq = torch.arange(len(lengths), dtype=torch.int32)
+    out = torch.empty(len(lengths), n_heads * head_dim, dtype=dtype, device="cuda:0")
+    scale = 1 / math.sqrt(head_dim)
+    layout = Layout(True, dev(torch.arange(len(lengths) + 1, dtype=torch.int32)), len(lengths), 1, max(lengths) - 1)
+    assert K.lib.bh_attention_bf16_splits(len(lengths), 1, n_heads, kv_heads, max(lengths) - 1) > 1
+    K.attention(dev(q), out, dev(kp), dev(vp), dev(table), dev(row_seq), dev(positions), n_heads, kv_heads,
+                head_dim, scale, 0, layout=layout)
+    assert bool(torch.isfinite(out.float()).all())
+    for s, n in enumerate(lengths):
+        want = attention_reference(q[s].reshape(n_heads, head_dim), keys[s], values[s], n - 1, n_heads, kv_heads,
+                                   head_dim, scale, 0)
+        assert rel(out[s].reshape(n_heads, head_dim), want) < 1.2e-2, (s, n)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -174,7 +205,7 @@ def test_attention_prefill_rows_ragged(K, dtype, n_heads, kv_heads, head_dim):
     out = torch.empty(n_rows, n_heads * head_dim, dtype=dtype, device="cuda:0")
     scale = 1 / math.sqrt(head_dim)
     K.attention(dev(q), out, dev(kp), dev(vp), dev(table), dev(row_seq), dev(positions), n_heads, kv_heads,
-                head_dim, scale, 0, layout=Layout(False, dev(starts), len(lengths)))
+                head_dim, scale, 0, layout=Layout(False, dev(starts), len(lengths), max(news), max(lengths) - 1))
     worst = 0.0
     for row in range(n_rows):
         s = int(row_seq[row])
@@ -200,13 +231,15 @@ def test_attention_finds_one_far_key_among_hundreds(K, dtype, far):
     q = q.reshape(2, n_heads * head_dim).to(dtype)
     positions = torch.tensor([n - 1, max(far, 1)], dtype=torch.int32)      # the last row sees the key as its newest
     row_seq = torch.zeros(2, dtype=torch.int32)
-    out = torch.empty(2, n_heads * head_dim, dtype=dtype, device="cuda:0")
-    K.attention(dev(q), out, dev(kp), dev(vp), dev(table), dev(row_seq), dev(positions), n_heads, kv_heads,
-                head_dim, 1 / math.sqrt(head_dim), 0, layout=None)
-    got = out.float().cpu().reshape(2, n_heads, head_dim)
-    for h in range(n_heads):
-        assert torch.allclose(got[0, h], values[0][far, h // 2].float(), atol=2e-2), (far, h)
-        assert torch.allclose(got[1, h], values[0][far, h // 2].float(), atol=2e-2), (far, h)
+    grouped = Layout(False, dev(torch.tensor([0, 2], dtype=torch.int32)), 1, 2, n - 1)
+    for layout in (None, grouped):          # the kernel for any size, and the matrix-core kernel
+        out = torch.empty(2, n_heads * head_dim, dtype=dtype, device="cuda:0")
+        K.attention(dev(q), out, dev(kp), dev(vp), dev(table), dev(row_seq), dev(positions), n_heads, kv_heads,
+                    head_dim, 1 / math.sqrt(head_dim), 0, layout=layout)
+        got = out.float().cpu().reshape(2, n_heads, head_dim)
+        for h in range(n_heads):
+            assert torch.allclose(got[0, h], values[0][far, h // 2].float(), atol=2e-2), (far, h, layout)
+            assert torch.allclose(got[1, h], values[0][far, h // 2].float(), atol=2e-2), (far, h, layout)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -252,7 +285,7 @@ def test_qk_norm_rope_cache(K, dtype, w_dtype, n_heads, kv_heads, head_dim, rot)
     table = torch.tensor([[4, 0, 0], [7, 2, 0], [1, 8, 3]], dtype=torch.int32)
     sentinel = 768.0        # exact in bfloat16
     kp = torch.full((n_pages, kv_heads, PAGE, head_dim), sentinel).to(dtype)
-    vp = torch.full((n_pages, kv_heads, PAGE, head_dim), sentinel).to(dtype)
+    vp = torch.full((n_pages, kv_heads, head_dim, PAGE), sentinel).to(dtype)
     kp_d, vp_d = dev(kp), dev(vp)
     q_out = torch.empty(n_rows, n_heads * head_dim, dtype=dtype, device="cuda:0")
     K.qk_norm_rope_cache(dev(qkv), q_out, dev(qw), dev(kw), eps, dev(cos), dev(sin), dev(positions), dev(row_seq),
@@ -276,10 +309,11 @@ def test_qk_norm_rope_cache(K, dtype, w_dtype, n_heads, kv_heads, head_dim, rot)
         written[page, pos % PAGE] = True
         assert rel(q_out[row].reshape(n_heads, head_dim), q_want) < tol(dtype, 2e-6, 4e-3)
         assert rel(kp_d[page, :, pos % PAGE], k_want) < tol(dtype, 2e-6, 4e-3)
-        assert torch.equal(vp_d[page, :, pos % PAGE].cpu().double(), v_want)
+        assert torch.equal(vp_d[page, :, :, pos % PAGE].cpu().double(), v_want)
     # nothing else in the cache was touched
     untouched = ~written[:, None, :, None].expand(n_pages, kv_heads, PAGE, head_dim)
-    assert bool((kp_d.cpu().float()[untouched] == sentinel).all()) and bool((vp_d.cpu().float()[untouched] == sentinel).all())
+    assert bool((kp_d.cpu().float()[untouched] == sentinel).all())
+    assert bool((vp_d.cpu().float().transpose(2, 3)[untouched] == sentinel).all())
     # without weights and tables the heads pass through; without write_kv the cache stays as it is
     kp2, vp2 = dev(kp), dev(vp)
     K.qk_norm_rope_cache(dev(qkv), q_out, None, None, 0.0, None, None, dev(positions), dev(row_seq), kp2, vp2,
@@ -389,6 +423,6 @@ def test_kernels_refuse_what_they_cannot_do(K):
     with pytest.raises(KernelError):      # a head size above the attention kernels' limit
         hd = 512
         K.attention(torch.zeros(1, hd, device="cuda:0"), torch.zeros(1, hd, device="cuda:0"),
-                    torch.zeros(1, 1, PAGE, hd, device="cuda:0"), torch.zeros(1, 1, PAGE, hd, device="cuda:0"),
+                    torch.zeros(1, 1, PAGE, hd, device="cuda:0"), torch.zeros(1, 1, hd, PAGE, device="cuda:0"),
                     torch.zeros(1, 1, dtype=torch.int32, device="cuda:0"), torch.zeros(1, dtype=torch.int32, device="cuda:0"),
                     torch.zeros(1, dtype=torch.int32, device="cuda:0"), 1, 1, hd, 1.0)
