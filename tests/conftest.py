@@ -48,9 +48,10 @@ TINY_D = {
 CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
 
 
-@pytest.fixture(scope="session")
+@pytest.fixture()
 def tiny_configs():
-    return {name: dict(config) for name, config in CONFIGS.items()}
+    import copy
+    return copy.deepcopy(CONFIGS)
 
 
 @pytest.fixture(scope="session")

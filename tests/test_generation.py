@@ -1,0 +1,187 @@
+"""The generation loop's decisions, with a stepper that needs no model: which tokens are
+emitted, when a sequence ends, when its slot is freed, how requests are split into batches."""
+
+import pytest
+import torch
+
+from beholdd.engine import (FINISH_LENGTH, FINISH_STOP, GenerationError, generate, plan_batches, positions_needed)
+from beholdd.sampling import SamplingParams, uniform
+
+
+class ScriptedStepper:
+    """A sequence's next token is a function of its length and its first token; logits carry it."""
+
+    page_size = 64
+
+    def __init__(self, capacity_pages=64, max_slots=8, max_position=4096, vocab=50):
+        self.capacity_pages, self.max_slots, self.max_position, self.vocab = capacity_pages, max_slots, max_position, vocab
+        self.free = list(range(max_slots))
+        self.state = {}           # slot -> (first token, length)
+        self.steps = []           # (kind, [slots])
+        self.peak_slots = 0
+        self.log = []
+
+    def alloc_slot(self):
+        slot = self.free.pop(0)
+        self.state[slot] = None
+        self.peak_slots = max(self.peak_slots, len(self.state))
+        self.log.append(("alloc", slot))
+        return slot
+
+    def free_slot(self, slot):
+        assert slot in self.state, "freed twice"
+        del self.state[slot]
+        self.free.insert(0, slot)
+        self.log.append(("free", slot))
+
+    def next_token(self, first, length):
+        return (first * 7 + length * 3) % self.vocab
+
+    def step(self, entries):
+        kinds = {len(e.tokens) == 1 and self.state[e.slot] is not None for e in entries}
+        assert len(kinds) == 1, "a step either starts all its sequences or continues all of them"
+        rows = []
+        for e in entries:
+            if self.state[e.slot] is None:
+                self.state[e.slot] = (e.tokens[0], len(e.tokens))
+            else:
+                first, length = self.state[e.slot]
+                assert e.tokens == [self.next_token(first, length)], "the token fed back is the one that was chosen"
+                self.state[e.slot] = (first, length + 1)
+            first, length = self.state[e.slot]
+            assert e.want == [len(e.tokens) - 1]
+            row = torch.zeros(self.vocab)
+            row[self.next_token(first, length)] = 5.0
+            rows.append(row)
+        self.steps.append(("prefill" if kinds == {False} else "decode", [e.slot for e in entries]))
+        return torch.stack(rows)
+
+    def select(self, logits, params, requests, steps):
+        assert len(params) == len(requests) == len(steps) == logits.shape[0]
+        return [int(torch.argmax(row)) for row in logits]
+
+
+def expected_tokens(stepper, prompt, n):
+    return [stepper.next_token(prompt[0], len(prompt) + i) for i in range(n)]
+
+
+def test_unequal_prompts_one_step_then_one_token_each():
+    s = ScriptedStepper()
+    prompts = [[1, 2, 3, 4, 5], [9] * 11, [4] * 17]
+    results = generate(s, prompts, 8)
+    for prompt, result in zip(prompts, results):
+        assert result.token_ids == expected_tokens(s, prompt, 8)
+        assert result.finish_reason == FINISH_LENGTH and result.stop_token is None
+        assert result.prompt_tokens == len(prompt) and result.completion_tokens == 8
+    assert s.steps[0] == ("prefill", [0, 1, 2]) and all(kind == "decode" for kind, _ in s.steps[1:])
+    assert len(s.steps) == 8                   # prefill + 7 decode steps: the last token is never evaluated
+    assert s.state == {}
+
+
+def test_stop_token_is_not_emitted_and_others_go_on():
+    s = ScriptedStepper()
+    prompts = [[1, 2, 3], [2, 2], [5]]
+    free_run = [expected_tokens(s, p, 6) for p in prompts]
+    stop = free_run[1][2]
+    seen = []
+    results = generate(s, prompts, 6, stop_token_ids=[stop], on_token=lambda i, t: seen.append((i, t)))
+    for i, (result, tokens) in enumerate(zip(results, free_run)):
+        if stop in tokens:
+            cut = tokens.index(stop)
+            assert result.token_ids == tokens[:cut] and result.finish_reason == FINISH_STOP and result.stop_token == stop
+        else:
+            assert result.token_ids == tokens and result.finish_reason == FINISH_LENGTH
+        assert [t for j, t in seen if j == i] == result.token_ids       # the callback sees exactly what is emitted
+    assert results[1].finish_reason == FINISH_STOP
+    later = [slots for kind, slots in s.steps if kind == "decode"][-1]
+    assert 1 not in later                                                # the stopped sequence left the batch
+    assert s.state == {}
+
+
+def test_sequences_that_end_earlier_free_their_slots_at_once():
+    s = ScriptedStepper()
+    generate(s, [[1], [2], [3]], [2, 5, 3])
+    order = [entry for entry in s.log if entry[0] == "free"]
+    assert order == [("free", 0), ("free", 2), ("free", 1)]
+    sizes = [len(slots) for _, slots in s.steps]
+    assert sizes == [3, 3, 2, 1, 1]
+
+
+def test_zero_new_tokens_touches_nothing():
+    s = ScriptedStepper()
+    results = generate(s, [[1, 2], [3]], [0, 2])
+    assert results[0].token_ids == [] and results[0].finish_reason == FINISH_LENGTH
+    assert results[1].completion_tokens == 2
+    assert s.steps[0] == ("prefill", [0])                # only the second request ever ran
+    assert generate(ScriptedStepper(), [[1]], 0)[0].token_ids == []
+
+
+def test_context_boundary():
+    # crates/beholdd-model/src/qwen3moe/forward.rs:3053-3065: a prompt of the whole context may select one token
+    s = ScriptedStepper(max_position=10)
+    assert positions_needed(10, 1) == 10 and positions_needed(10, 0) == 10 and positions_needed(3, 8) == 10
+    assert generate(s, [[1] * 10], 1)[0].completion_tokens == 1
+    assert generate(ScriptedStepper(max_position=10), [[1] * 3], 8)[0].completion_tokens == 8
+    with pytest.raises(GenerationError, match="needs 11 evaluated positions"):
+        generate(ScriptedStepper(max_position=10), [[1] * 3], 9)
+    with pytest.raises(GenerationError, match="at least one prompt token"):
+        generate(ScriptedStepper(), [[]], 1)
+    with pytest.raises(GenerationError, match="negative"):
+        generate(ScriptedStepper(), [[1]], -1)
+
+
+def test_requests_run_as_one_batch_after_another():
+    s = ScriptedStepper(max_slots=3)
+    prompts = [[i + 1] * (i + 1) for i in range(8)]
+    results = generate(s, prompts, 4)
+    assert [r.token_ids for r in results] == [expected_tokens(s, p, 4) for p in prompts]
+    prefills = [slots for kind, slots in s.steps if kind == "prefill"]
+    assert [len(p) for p in prefills] == [3, 3, 2] and s.peak_slots == 3
+    assert sorted(prefills[1]) == sorted(prefills[0])    # the second batch runs in the slots the first gave back
+    assert [len(b) for b in plan_batches([5] * 8, [4] * 8, 64, 64, 8, 2)] == [2, 2, 2, 2]
+    # the cache's pages bound a batch too: each request needs 2 pages of 64, the cache has 5
+    assert [len(b) for b in plan_batches([100] * 5, [20] * 5, 64, 5, 8, None)] == [2, 2, 1]
+    with pytest.raises(GenerationError, match="cache pages"):
+        plan_batches([1000], [10], 64, 5, 8, None)
+
+
+def test_callback_error_aborts_and_frees_everything():
+    s = ScriptedStepper()
+
+    def on_token(index, token):
+        if index == 1:
+            raise RuntimeError("consumer went away")
+
+    with pytest.raises(RuntimeError, match="went away"):
+        generate(s, [[1], [2], [3]], 4, on_token=on_token)
+    assert s.state == {}
+    calls = {"n": 0}
+
+    def control():
+        calls["n"] += 1
+        if calls["n"] == 3:
+            raise KeyboardInterrupt
+
+    s = ScriptedStepper()
+    with pytest.raises(KeyboardInterrupt):
+        generate(s, [[1], [2]], 10, control=control)
+    assert s.state == {} and len(s.steps) == 2           # the prefill and one decode step ran before the third poll
+
+
+def test_per_request_limits_and_parameters():
+    s = ScriptedStepper()
+    results = generate(s, [[1], [2]], [1, 3], [SamplingParams(), SamplingParams(temperature=0.5, seed=3)])
+    assert [r.completion_tokens for r in results] == [1, 3]
+    with pytest.raises(GenerationError, match="one max_new_tokens"):
+        generate(s, [[1], [2]], [1])
+
+
+def test_uniform_numbers_are_a_pure_function_of_seed_request_step():
+    values = {uniform(s, r, t) for s in range(3) for r in range(5) for t in range(20)}
+    assert len(values) == 300 and all(0.0 <= v < 1.0 for v in values)
+    assert uniform(1, 2, 3) == uniform(1, 2, 3)
+    mean = sum(uniform(0, 0, t) for t in range(4000)) / 4000
+    assert abs(mean - 0.5) < 0.03
+    for bad in (dict(temperature=-1.0), dict(top_k=-1), dict(top_p=0.0), dict(top_p=1.5)):
+        with pytest.raises(ValueError):
+            SamplingParams(**bad)
