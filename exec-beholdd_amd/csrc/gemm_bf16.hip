@@ -1,15 +1,24 @@
 // bfloat16 matrix products on the gfx950 matrix cores: C[M, N] (+)= A[M, K] * W[N, K]^T,
-// float32 accumulation, C in float32 or bfloat16.
+// float32 accumulation, C in float32 or bfloat16; optionally C[M, F] = silu(A Wg^T) * (A Wu^T)
+// for W = [Wg; Wu] stacked (the SwiGLU feed-forward's first half in one pass).
+//
+// Weight layouts.  `rows`: W as checkpoints store it, [N, K] row-major.  `tiles`: the same
+// numbers regrouped at load time into blocks of 16 rows x 64 k, block (nb, kb) at
+// (nb * K/64 + kb) * 1024 elements, and inside a block [half u][lane l][8] with
+// row = l % 16, k = 16 * (l / 16) + 8 * u + e.  A wave then reads a block as two fully
+// contiguous 1 KB loads that are already in matrix-core operand order; streaming a weight once
+// from HBM (decode) runs about a third faster from this layout than from strided rows.
+// Tiles need K % 64 == 0; rows beyond N in the last block are zero.
 //
 // Two kernels.
-//   skinny (M <= 64, the decode shapes): the product is bound by reading W once from HBM.  A
-//     workgroup owns 16 rows of W; its waves split K between them in 64-wide chunks, each lane
-//     reading 32 contiguous bytes of a row so that four lanes cover a 128-byte line, and feed
+//   skinny (M <= 64, the decode shapes): bound by reading W once.  A workgroup owns 16 rows of W
+//     (a gate block and its up block for SwiGLU); its 8 waves split K in 64-wide chunks and feed
 //     v_mfma_f32_16x16x32_bf16 with W as the row operand and the activations as the column
 //     operand; the waves' partial tiles are summed through LDS in a fixed order.
 //   tiled (M > 64, the prefill shapes): 128x128 output tile per workgroup of four waves, 64-wide
 //     k slices staged through padded LDS with the next slice's global loads in flight during
-//     the multiplies; v_mfma_f32_32x32x16_bf16, each wave a 64x64 quarter.
+//     the multiplies; v_mfma_f32_32x32x16_bf16, each wave a 64x64 quarter.  For SwiGLU a wave's
+//     two 32-column halves are the gate and the up columns of the same 32 outputs.
 // K must be a multiple of 8 (16-byte loads); other sizes are free.
 //
 // Operand layouts relied on (wave of 64 lanes, l = lane):
@@ -43,98 +52,130 @@ __device__ inline void store_out<bf16_t>(bf16_t* c, size_t at, float v, bool acc
   c[at] = from_f32<bf16_t>(v);
 }
 
-// ---- skinny --------------------------------------------------------------------------------
+__device__ inline float silu_mul(float gate, float up) { return gate / (1.0f + expf(-gate)) * up; }
 
-template <int MB, int WAVES, typename TC>
+#define MFMA16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(b), c, 0, 0, 0)
+
+// ---- skinny --------------------------------------------------------------------------------
+// RT = 1: plain product.  RT = 2: SwiGLU; the second row block lies `pair_blocks` blocks after the first.
+
+template <int MB, int WAVES, bool TILES, int RT, typename TC>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t* __restrict__ a,
                                                                  const uint16_t* __restrict__ w,
                                                                  TC* __restrict__ c, int M, int N, int K,
-                                                                 int accumulate) {
-  __shared__ float partial[WAVES][MB][256];
+                                                                 int accumulate, int pair_blocks) {
+  __shared__ float partial[WAVES][RT][MB][256];
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int i = lane % 16, g = lane / 16;
   const int n0 = blockIdx.x * 16;
-  const int w_row = (n0 + i < N) ? n0 + i : N - 1;
-  const uint16_t* wp = w + (size_t)w_row * K + g * 16;
+  const int full = K / 64;
+  // per row block: base pointer, distance between consecutive 64-wide chunks, distance to the second half
+  const uint16_t* wp[RT];
+  const size_t chunk_stride = TILES ? 1024 : 64;
+  const int half_offset = TILES ? 512 : 8;
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    const int block = blockIdx.x + t * pair_blocks;
+    if (TILES) {
+      wp[t] = w + (size_t)block * full * 1024 + lane * 8;
+    } else {
+      const int rows = RT == 2 ? 2 * N : N;  // SwiGLU: N counts outputs, W has twice as many rows
+      const int row = (block * 16 + i < rows) ? block * 16 + i : rows - 1;
+      wp[t] = w + (size_t)row * K + g * 16;
+    }
+  }
   const uint16_t* xp[MB];
 #pragma unroll
   for (int b = 0; b < MB; ++b) {
     const int row = (b * 16 + i < M) ? b * 16 + i : M - 1;
     xp[b] = a + (size_t)row * K + g * 16;
   }
-  f32x4_t acc[MB];
+  f32x4_t acc[RT][MB];
 #pragma unroll
-  for (int b = 0; b < MB; ++b) acc[b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < RT; ++t)
+#pragma unroll
+    for (int b = 0; b < MB; ++b) acc[t][b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  const int full = K / 64;
   int chunk = wave;
   // U chunks per trip, all their loads issued before the first multiply, to keep bytes in flight
-  constexpr int U = MB <= 2 ? 4 : 2;
+  constexpr int U = (MB * RT <= 2) ? 4 : (MB * RT <= 4 ? 2 : 1);
   for (; chunk + (U - 1) * WAVES < full; chunk += U * WAVES) {
-    u32x4_t wv[U][2], xv[U][MB][2];
+    u32x4_t wv[U][RT][2], xv[U][MB][2];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int k = (chunk + u * WAVES) * 64;
-      wv[u][0] = load16_stream(wp + k);
-      wv[u][1] = load16_stream(wp + k + 8);
+      const int at = chunk + u * WAVES;
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
+        const uint16_t* p = wp[t] + (size_t)at * chunk_stride;
+        wv[u][t][0] = TILES ? load16_stream(p) : load16(p);
+        wv[u][t][1] = TILES ? load16_stream(p + half_offset) : load16(p + half_offset);
+      }
 #pragma unroll
       for (int b = 0; b < MB; ++b) {
-        xv[u][b][0] = load16(xp[b] + k);
-        xv[u][b][1] = load16(xp[b] + k + 8);
+        xv[u][b][0] = load16(xp[b] + at * 64);
+        xv[u][b][1] = load16(xp[b] + at * 64 + 8);
       }
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int b = 0; b < MB; ++b) {
-        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wv[u][0]), as_bf16x8(xv[u][b][0]), acc[b], 0, 0, 0);
-        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wv[u][1]), as_bf16x8(xv[u][b][1]), acc[b], 0, 0, 0);
-      }
+      for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+          acc[t][b] = MFMA16(wv[u][t][0], xv[u][b][0], acc[t][b]);
+          acc[t][b] = MFMA16(wv[u][t][1], xv[u][b][1], acc[t][b]);
+        }
   }
   for (; chunk < full; chunk += WAVES) {
-    const int k = chunk * 64;
-    const u32x4_t w0 = load16_stream(wp + k), w1 = load16_stream(wp + k + 8);
 #pragma unroll
-    for (int b = 0; b < MB; ++b) {
-      const u32x4_t x0 = load16(xp[b] + k), x1 = load16(xp[b] + k + 8);
-      acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(w0), as_bf16x8(x0), acc[b], 0, 0, 0);
-      acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(w1), as_bf16x8(x1), acc[b], 0, 0, 0);
+    for (int t = 0; t < RT; ++t) {
+      const uint16_t* p = wp[t] + (size_t)chunk * chunk_stride;
+      const u32x4_t w0 = load16(p), w1 = load16(p + half_offset);
+#pragma unroll
+      for (int b = 0; b < MB; ++b) {
+        const u32x4_t x0 = load16(xp[b] + chunk * 64), x1 = load16(xp[b] + chunk * 64 + 8);
+        acc[t][b] = MFMA16(w0, x0, acc[t][b]);
+        acc[t][b] = MFMA16(w1, x1, acc[t][b]);
+      }
     }
   }
-  if (chunk == full && full * 64 < K) {  // the last, partial chunk: 8-element pieces beyond K are zero
+  if (!TILES && chunk == full && full * 64 < K) {  // rows layout: the last, partial chunk; pieces beyond K are zero
     const int k = full * 64, at = k + g * 16;
     const u32x4_t zero = {0u, 0u, 0u, 0u};
-    const u32x4_t w0 = at < K ? load16_stream(wp + k) : zero, w1 = at + 8 < K ? load16_stream(wp + k + 8) : zero;
 #pragma unroll
-    for (int b = 0; b < MB; ++b) {
-      const u32x4_t x0 = at < K ? load16(xp[b] + k) : zero, x1 = at + 8 < K ? load16(xp[b] + k + 8) : zero;
-      acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(w0), as_bf16x8(x0), acc[b], 0, 0, 0);
-      acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(w1), as_bf16x8(x1), acc[b], 0, 0, 0);
+    for (int t = 0; t < RT; ++t) {
+      const u32x4_t w0 = at < K ? load16(wp[t] + k) : zero, w1 = at + 8 < K ? load16(wp[t] + k + 8) : zero;
+#pragma unroll
+      for (int b = 0; b < MB; ++b) {
+        const u32x4_t x0 = at < K ? load16(xp[b] + k) : zero, x1 = at + 8 < K ? load16(xp[b] + k + 8) : zero;
+        acc[t][b] = MFMA16(w0, x0, acc[t][b]);
+        acc[t][b] = MFMA16(w1, x1, acc[t][b]);
+      }
     }
   }
   // D: lane holds column (activation row) i and rows (W rows) 4g..4g+3; lay it out as [m][n]
 #pragma unroll
-  for (int b = 0; b < MB; ++b)
+  for (int t = 0; t < RT; ++t)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) partial[wave][b][i * 16 + 4 * g + r] = acc[b][r];
+    for (int b = 0; b < MB; ++b)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) partial[wave][t][b][i * 16 + 4 * g + r] = acc[t][b][r];
   __syncthreads();
   for (int e = threadIdx.x; e < MB * 256; e += WAVES * 64) {
     const int b = e / 256, m = b * 16 + (e % 256) / 16, n = n0 + e % 16;
     if (m >= M || n >= N) continue;
-    float sum = 0.f;
+    float sum[RT];
 #pragma unroll
-    for (int v = 0; v < WAVES; ++v) sum += partial[v][b][e % 256];
-    store_out<TC>(c, (size_t)m * N + n, sum, accumulate != 0);
+    for (int t = 0; t < RT; ++t) {
+      sum[t] = 0.f;
+#pragma unroll
+      for (int v = 0; v < WAVES; ++v) sum[t] += partial[v][t][b][e % 256];
+    }
+    if (RT == 2)
+      store_out<TC>(c, (size_t)m * N + n, silu_mul(sum[0], sum[RT - 1]), false);
+    else
+      store_out<TC>(c, (size_t)m * N + n, sum[0], accumulate != 0);
   }
-}
-
-template <int MB, typename TC>
-static void launch_skinny(const void* a, const void* w, void* c, int M, int N, int K, int accumulate,
-                          hipStream_t stream) {
-  constexpr int WAVES = 8;
-  dim3 grid((N + 15) / 16), block(WAVES * 64);
-  gemm_skinny_kernel<MB, WAVES, TC><<<grid, block, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, (TC*)c, M,
-                                                                N, K, accumulate);
 }
 
 // ---- tiled -----------------------------------------------------------------------------------
@@ -143,46 +184,72 @@ static void launch_skinny(const void* a, const void* w, void* c, int M, int N, i
 #define TK 64           // k slice
 #define TPITCH (TK + 8) // LDS row pitch in elements: 144 bytes, so 16-byte reads of 16 rows hit 64 distinct banks
 
-template <typename TC>
+// SWIGLU: the tile's 128 W rows are, per wave column half (32 outputs), 32 gate rows then the 32 up
+// rows of the same outputs; N counts outputs and the up rows start `N` rows (N/16 blocks) further on.
+template <bool TILES, bool SWIGLU, typename TC>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restrict__ a,
                                                          const uint16_t* __restrict__ w, TC* __restrict__ c,
                                                          int M, int N, int K, int accumulate) {
   __shared__ __attribute__((aligned(16))) uint16_t as[2][TB * TPITCH];
   __shared__ __attribute__((aligned(16))) uint16_t ws[2][TB * TPITCH];
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
-  const int m0 = blockIdx.y * TB, n0 = blockIdx.x * TB;
-  const int wm = (wave / 2) * 64, wn = (wave % 2) * 64;  // this wave's quarter of the tile
+  const int m0 = blockIdx.y * TB;
+  const int n0 = blockIdx.x * (SWIGLU ? TB / 2 : TB);   // first output column of the tile
+  const int wm = (wave / 2) * 64, wn = (wave % 2) * 64;  // this wave's quarter of the tile (in LDS rows)
+  const int w_rows = SWIGLU ? 2 * N : N;
+  const int w_blocks = (w_rows + 15) / 16;
+
+  // LDS row r of the W tile -> row of W
+  auto w_row_of = [&](int r) {
+    if (!SWIGLU) return n0 + r;
+    const int half = r / 64, inner = r % 64;              // wave column half, then 32 gate rows + 32 up rows
+    return (inner < 32 ? 0 : N) + n0 + half * 32 + inner % 32;
+  };
 
   // global -> LDS staging: a slice is 128 rows x 8 pieces of 16 bytes; a thread moves 4 pieces per operand
-  int st_row[4], st_piece[4];
+  int a_at[4], w_at[4], a_piece[4];
   const uint16_t* a_src[4];
   const uint16_t* w_src[4];
+  size_t w_step;
 #pragma unroll
   for (int s = 0; s < 4; ++s) {
     const int e = tid + s * 256;
-    st_row[s] = e / 8;
-    st_piece[s] = e % 8;
-    const int am = (m0 + st_row[s] < M) ? m0 + st_row[s] : M - 1;
-    const int wr = (n0 + st_row[s] < N) ? n0 + st_row[s] : N - 1;
-    a_src[s] = a + (size_t)am * K + st_piece[s] * 8;
-    w_src[s] = w + (size_t)wr * K + st_piece[s] * 8;
+    const int row = e / 8, piece = e % 8;
+    const int am = (m0 + row < M) ? m0 + row : M - 1;
+    a_src[s] = a + (size_t)am * K + piece * 8;
+    a_at[s] = row * TPITCH + piece * 8;
+    a_piece[s] = piece;
+    if (TILES) {
+      // 8 blocks of 16 rows; inside a block piece p = u * 64 + l holds row l % 16, k 16 * (l / 16) + 8 * u
+      const int block = e / 128, p = e % 128, u = p / 64, l = p % 64;
+      int global_block = w_row_of(block * 16) / 16;
+      if (global_block >= w_blocks) global_block = w_blocks - 1;
+      w_src[s] = w + (size_t)global_block * (K / 64) * 1024 + p * 8;
+      w_at[s] = (block * 16 + l % 16) * TPITCH + 16 * (l / 16) + 8 * u;
+    } else {
+      int wr = w_row_of(row);
+      if (wr >= w_rows) wr = w_rows - 1;
+      w_src[s] = w + (size_t)wr * K + piece * 8;
+      w_at[s] = a_at[s];
+    }
   }
+  w_step = TILES ? 1024 : TK;
   u32x4_t a_reg[4], w_reg[4];
   const u32x4_t zero = {0u, 0u, 0u, 0u};
-  auto fetch = [&](int k0) {
+  auto fetch = [&](int slice) {
+    const int k0 = slice * TK;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      const bool inside = k0 + st_piece[s] * 8 < K;
+      const bool inside = k0 + a_piece[s] * 8 < K;
       a_reg[s] = inside ? load16(a_src[s] + k0) : zero;
-      w_reg[s] = inside ? load16(w_src[s] + k0) : zero;
+      w_reg[s] = (TILES || inside) ? load16(w_src[s] + (size_t)slice * w_step) : zero;
     }
   };
   auto stash = [&](int buffer) {
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      const int at = st_row[s] * TPITCH + st_piece[s] * 8;
-      *reinterpret_cast<u32x4_t*>(&as[buffer][at]) = a_reg[s];
-      *reinterpret_cast<u32x4_t*>(&ws[buffer][at]) = w_reg[s];
+      *reinterpret_cast<u32x4_t*>(&as[buffer][a_at[s]]) = a_reg[s];
+      *reinterpret_cast<u32x4_t*>(&ws[buffer][w_at[s]]) = w_reg[s];
     }
   };
 
@@ -201,7 +268,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
   const int frag_row = lane % 32, frag_k = (lane / 32) * 8;
   for (int s = 0; s < slices; ++s) {
     const int buffer = s & 1;
-    if (s + 1 < slices) fetch((s + 1) * TK);
+    if (s + 1 < slices) fetch(s + 1);
 #pragma unroll
     for (int kk = 0; kk < TK; kk += 16) {
       bf16x8_t af[2], wf[2];
@@ -222,47 +289,94 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
   }
   // D of one 32x32 block: column (n) lane%32, rows (m) 8*(e/4) + 4*(lane/32) + e%4
 #pragma unroll
-  for (int x = 0; x < 2; ++x)
-#pragma unroll
-    for (int y = 0; y < 2; ++y) {
-      const int n = n0 + wn + y * 32 + lane % 32;
+  for (int x = 0; x < 2; ++x) {
+    if (SWIGLU) {
+      const int n = n0 + (wave % 2) * 32 + lane % 32;
       if (n >= N) continue;
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const int m = m0 + wm + x * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
-        if (m < M) store_out<TC>(c, (size_t)m * N + n, acc[x][y][e], accumulate != 0);
+        if (m < M) store_out<TC>(c, (size_t)m * N + n, silu_mul(acc[x][0][e], acc[x][1][e]), false);
+      }
+    } else {
+#pragma unroll
+      for (int y = 0; y < 2; ++y) {
+        const int n = n0 + wn + y * 32 + lane % 32;
+        if (n >= N) continue;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int m = m0 + wm + x * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
+          if (m < M) store_out<TC>(c, (size_t)m * N + n, acc[x][y][e], accumulate != 0);
+        }
       }
     }
+  }
 }
 
 // ---- entry -------------------------------------------------------------------------------------
 
+template <bool TILES, int RT, typename TC>
+static void launch_skinny(const void* a, const void* w, void* c, int M, int N, int K, int accumulate,
+                          int pair_blocks, hipStream_t stream) {
+  constexpr int WAVES = 8;
+  dim3 grid((N + 15) / 16), block(WAVES * 64);
+#define BH_SKINNY(MB)                                                                                     \
+  gemm_skinny_kernel<MB, WAVES, TILES, RT, TC><<<grid, block, 0, stream>>>(                               \
+      (const uint16_t*)a, (const uint16_t*)w, (TC*)c, M, N, K, accumulate, pair_blocks)
+  switch ((M + 15) / 16) {
+    case 1: BH_SKINNY(1); break;
+    case 2: BH_SKINNY(2); break;
+    case 3: BH_SKINNY(3); break;
+    default: BH_SKINNY(4); break;
+  }
+#undef BH_SKINNY
+}
+
+template <bool TILES, bool SWIGLU, typename TC>
+static void launch_tiled(const void* a, const void* w, void* c, int M, int N, int K, int accumulate,
+                         hipStream_t stream) {
+  const int columns = SWIGLU ? TB / 2 : TB;
+  dim3 grid((N + columns - 1) / columns, (M + TB - 1) / TB), block(256);
+  gemm_tiled_kernel<TILES, SWIGLU, TC><<<grid, block, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, (TC*)c, M,
+                                                                   N, K, accumulate);
+}
+
+// layout: 0 = rows, 1 = tiles.  activation: 0 = none; 1 = SwiGLU (W has 2 * N rows: gate rows then up rows).
 extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, int accumulate, int M, int N, int K,
-                            hipStream_t stream) {
+                            int layout, int activation, hipStream_t stream) {
   BH_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_bf16: sizes M=%d N=%d K=%d must be positive", M, N, K);
   BH_REQUIRE(K % 8 == 0, "gemm_bf16: K=%d must be a multiple of 8", K);
   BH_REQUIRE(c_dtype == BH_F32 || c_dtype == BH_BF16, "gemm_bf16: unknown output dtype %d", c_dtype);
   BH_REQUIRE(((uintptr_t)a | (uintptr_t)w) % 16 == 0, "gemm_bf16: operands must be 16-byte aligned");
+  BH_REQUIRE(layout == 0 || (layout == 1 && K % 64 == 0), "gemm_bf16: the tiles layout needs K=%d to be a multiple of 64", K);
+  BH_REQUIRE(activation == 0 || activation == 1, "gemm_bf16: unknown activation %d", activation);
+  BH_REQUIRE(activation == 0 || (N % 16 == 0 && !accumulate),
+             "gemm_bf16: SwiGLU needs a multiple of 16 outputs (got %d) and no accumulation", N);
+  BH_REQUIRE((M + TB - 1) / TB <= 65535, "gemm_bf16: M=%d needs more than 65535 row tiles", M);
+  const bool f32 = c_dtype == BH_F32;
+#define BH_PICK(FN, TILES, EXTRA, ...)                                             \
+  do {                                                                              \
+    if (f32) FN<TILES, EXTRA, float>(__VA_ARGS__);                                  \
+    else FN<TILES, EXTRA, bf16_t>(__VA_ARGS__);                                     \
+  } while (0)
   if (M <= 64) {
-    const int blocks = (M + 15) / 16;
-#define BH_SKINNY(MB)                                                                               \
-  if (c_dtype == BH_F32) launch_skinny<MB, float>(a, w, c, M, N, K, accumulate, stream);             \
-  else launch_skinny<MB, bf16_t>(a, w, c, M, N, K, accumulate, stream)
-    if (blocks == 1) { BH_SKINNY(1); }
-    else if (blocks == 2) { BH_SKINNY(2); }
-    else if (blocks == 3) { BH_SKINNY(3); }
-    else { BH_SKINNY(4); }
-#undef BH_SKINNY
+    const int pair_blocks = N / 16;
+    if (activation) {
+      if (layout) BH_PICK(launch_skinny, true, 2, a, w, c, M, N, K, 0, pair_blocks, stream);
+      else BH_PICK(launch_skinny, false, 2, a, w, c, M, N, K, 0, pair_blocks, stream);
+    } else {
+      if (layout) BH_PICK(launch_skinny, true, 1, a, w, c, M, N, K, accumulate, 0, stream);
+      else BH_PICK(launch_skinny, false, 1, a, w, c, M, N, K, accumulate, 0, stream);
+    }
     return bh_check_launch("gemm_skinny");
   }
-  const int row_tiles = (M + TB - 1) / TB;
-  BH_REQUIRE(row_tiles <= 65535, "gemm_bf16: M=%d needs more than 65535 row tiles", M);
-  dim3 grid((N + TB - 1) / TB, row_tiles), block(256);
-  if (c_dtype == BH_F32)
-    gemm_tiled_kernel<float><<<grid, block, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, (float*)c, M, N, K,
-                                                         accumulate);
-  else
-    gemm_tiled_kernel<bf16_t><<<grid, block, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, (bf16_t*)c, M, N,
-                                                          K, accumulate);
+  if (activation) {
+    if (layout) BH_PICK(launch_tiled, true, true, a, w, c, M, N, K, 0, stream);
+    else BH_PICK(launch_tiled, false, true, a, w, c, M, N, K, 0, stream);
+  } else {
+    if (layout) BH_PICK(launch_tiled, true, false, a, w, c, M, N, K, accumulate, stream);
+    else BH_PICK(launch_tiled, false, false, a, w, c, M, N, K, accumulate, stream);
+  }
+#undef BH_PICK
   return bh_check_launch("gemm_tiled");
 }

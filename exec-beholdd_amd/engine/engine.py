@@ -52,6 +52,8 @@ class Engine:
             model = load_model(model_dir, self.dtype, self.device)
         self.model = model
         self.config = model.config
+        if hasattr(model, "prepare"):
+            model.prepare(kernels)
         self.cache = SequenceCache(model.entry_needs, max_tokens, self.dtype, self.device, kernels.page_size,
                                    max_slots=max_slots, max_position=model.max_position)
         self.cache_plan = self.cache.allocate(limit_bytes=memory_limit_bytes)

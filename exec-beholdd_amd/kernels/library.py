@@ -25,6 +25,18 @@ class KernelError(RuntimeError):
     """A kernel refused its arguments or could not be launched."""
 
 
+class PackedWeight:
+    """A bfloat16 weight matrix regrouped into 16-row x 64-column blocks in matrix-core operand
+    order (the `tiles` layout of csrc/gemm_bf16.hip).  `shape` and `dtype` are those of the
+    matrix it stands for; `data` is the regrouped buffer (rows padded to a multiple of 16)."""
+
+    def __init__(self, data: torch.Tensor, rows: int, cols: int):
+        self.data, self.shape, self.dtype = data, (rows, cols), data.dtype
+
+    def dim(self):
+        return 2
+
+
 def _code(tensor: torch.Tensor, what: str) -> int:
     code = _CODES.get(tensor.dtype)
     if code is None:
@@ -71,7 +83,7 @@ class HipKernels:
             function.restype = i
         self._optional = {}
         for name, argtypes in {
-            "bh_gemm_bf16": [p, p, p, i, i, i, i, i, p],
+            "bh_gemm_bf16": [p, p, p, i, i, i, i, i, i, i, p],
             "bh_attention_bf16": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, i, i, f, i, i, i, p],
             "bh_attention_bf16_splits": [i, i, i, i, i],
         }.items():
@@ -130,22 +142,64 @@ class HipKernels:
             self._ptr(weight, "rmsnorm weight", None, True), _code(weight, "rmsnorm weight") if weight is not None else F32,
             self._ptr(out, "rmsnorm out"), _code(out, "rmsnorm out"), n_rows, width, float(eps), self._stream()))
 
+    def pack_weight(self, w):
+        """The form of a weight matrix that the matrix products read fastest: a `PackedWeight` for a
+        bfloat16 matrix whose width is a multiple of 64, else the matrix itself."""
+        if (isinstance(w, torch.Tensor) and w.dim() == 2 and w.dtype == torch.bfloat16 and w.shape[1] % 64 == 0
+                and "bh_gemm_bf16" in self._optional):
+            rows, cols = w.shape
+            padded = -(-rows // 16) * 16
+            if padded != rows:
+                w = torch.cat([w, torch.zeros(padded - rows, cols, dtype=w.dtype, device=w.device)])
+            # [block of 16 rows][block of 64 k][half u][lane group g][row i][8]
+            data = w.view(padded // 16, 16, cols // 64, 4, 2, 8).permute(0, 2, 4, 3, 1, 5).contiguous()
+            return PackedWeight(data, rows, cols)
+        return w
+
+    def _gemm_fast(self, a, w, out, accumulate, activation):
+        """Launch the matrix-core product if it takes these operands; say whether it did."""
+        fast = self._optional.get("bh_gemm_bf16")
+        packed = isinstance(w, PackedWeight)
+        if fast is None or a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or a.shape[1] % 8:
+            if packed:
+                raise KernelError("gemm: a packed weight needs bfloat16 activations")
+            return False
+        if activation and (out.shape[1] % 16 or accumulate):
+            return False
+        m, k = a.shape
+        self._check(fast(self._ptr(a, "gemm a"), self._ptr(w.data if packed else w, "gemm w"),
+                         self._ptr(out, "gemm out"), _code(out, "gemm out"), int(bool(accumulate)), m, out.shape[1], k,
+                         int(packed), int(activation), self._stream()))
+        return True
+
     def gemm(self, a, w, out, accumulate=False):
-        """out[M, N] (+)= a[M, K] @ w[N, K]^T with float32 accumulation."""
+        """out[M, N] (+)= a[M, K] @ w[N, K]^T with float32 accumulation; `w` may be a PackedWeight."""
         if a.dim() != 2 or w.dim() != 2 or out.dim() != 2:
             raise KernelError("gemm: operands must be matrices")
         m, k = a.shape
         n = w.shape[0]
         if w.shape[1] != k or out.shape != (m, n):
             raise KernelError(f"gemm: shapes a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
-        fast = self._optional.get("bh_gemm_bf16")
-        if (fast is not None and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and k % 8 == 0):
-            self._check(fast(self._ptr(a, "gemm a"), self._ptr(w, "gemm w"), self._ptr(out, "gemm out"),
-                             _code(out, "gemm out"), int(bool(accumulate)), m, n, k, self._stream()))
+        if self._gemm_fast(a, w, out, accumulate, 0):
             return
         self._check(self.lib.bh_gemm_generic(
             self._ptr(a, "gemm a"), _code(a, "gemm a"), self._ptr(w, "gemm w"), _code(w, "gemm w"),
             self._ptr(out, "gemm out"), _code(out, "gemm out"), int(bool(accumulate)), m, n, k, self._stream()))
+
+    def gemm_swiglu(self, a, w, out):
+        """out[M, F] = silu(a @ w[:F]^T) * (a @ w[F:]^T) for w [2F, K] = gate rows, then up rows."""
+        if a.dim() != 2 or w.dim() != 2 or out.dim() != 2:
+            raise KernelError("gemm_swiglu: operands must be matrices")
+        m, k = a.shape
+        width = out.shape[1]
+        if w.shape != (2 * width, k) or out.shape[0] != m or out.dtype != a.dtype:
+            raise KernelError(f"gemm_swiglu: shapes a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} "
+                              "do not fit")
+        if self._gemm_fast(a, w, out, False, 1):
+            return
+        both = torch.empty((m, 2 * width), dtype=a.dtype, device=self.device)
+        self.gemm(a, w, both)
+        self.swiglu(both, out)
 
     def qk_norm_rope_cache(self, qkv, q_out, q_weight, k_weight, eps, cos, sin, positions, row_seq,
                            k_pages, v_pages, page_table, n_heads, n_kv_heads, head_dim, write_kv, max_position):

@@ -62,6 +62,12 @@ class DecoderModel:
             if hasattr(part, "build_tables"):
                 part.build_tables(device)
 
+    def prepare(self, kernels):
+        """After loading: parts may have the kernel library regroup their weights."""
+        for part in self.parts():
+            if hasattr(part, "prepare"):
+                part.prepare(kernels)
+
     def forward(self, ctx, cache_for_run, want_rows):
         """Run one step.  `cache_for_run(i)` gives the LayerCache of the i-th scheduled run (or
         None); `want_rows` (int32 device tensor, may be empty) lists the rows whose logits are

@@ -58,6 +58,10 @@ class GQAAttention:
             if self.q_norm.dtype != self.k_norm.dtype:
                 self.q_norm, self.k_norm = self.q_norm.float(), self.k_norm.float()
 
+    def prepare(self, kernels):
+        self.qkv.prepare(kernels)
+        self.out.prepare(kernels)
+
     def cache_need(self):
         return CacheNeed(kind="kv", kv_heads=self.n_kv_heads, head_dim=self.head_dim, window=self.window)
 

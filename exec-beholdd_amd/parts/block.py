@@ -25,6 +25,11 @@ class PreNormBlock:
         for part in self.parts():
             part.load(get)
 
+    def prepare(self, kernels):
+        for part in self.parts():
+            if hasattr(part, "prepare"):
+                part.prepare(kernels)
+
     def cache_need(self):
         return self.mixer.cache_need()
 

@@ -47,6 +47,9 @@ class LMHead:
         else:
             self.linear.load(get)
 
+    def prepare(self, kernels):
+        self.linear.prepare(kernels)        # a tied head keeps the embedding's own matrix
+
     def forward(self, ctx, x):
         """x [n, width] -> float32 logits [n, vocab]."""
         return self.linear.forward(ctx, x, out_dtype=torch.float32)

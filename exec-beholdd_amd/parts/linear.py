@@ -22,7 +22,8 @@ class Linear:
         if len(self.names) != len(self.splits):
             raise ValueError("one output size per stacked tensor")
         self.out_features = sum(self.splits)
-        self.weight: torch.Tensor | None = None
+        self.weight = None          # a tensor, or the kernel library's packed form of it
+        self.shared = False
 
     def tensor_specs(self):
         return [TensorSpec(name, (rows, self.in_features), "linear") for name, rows in zip(self.names, self.splits)]
@@ -43,6 +44,12 @@ class Linear:
             raise ValueError(f"shared weight has shape {tuple(weight.shape)}, expected "
                              f"{(self.out_features, self.in_features)}")
         self.weight = weight
+        self.shared = True
+
+    def prepare(self, kernels):
+        """Let the kernel library regroup the matrix into the layout it reads fastest."""
+        if not self.shared and hasattr(kernels, "pack_weight"):
+            self.weight = kernels.pack_weight(self.weight)
 
     def forward(self, ctx, x, out=None, accumulate=False, out_dtype=None):
         """x [n, in] -> out [n, out]; with accumulate the product is added into `out`."""

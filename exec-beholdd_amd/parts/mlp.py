@@ -25,10 +25,13 @@ class SwiGLU:
         self.gate_up.load(get)
         self.down.load(get)
 
+    def prepare(self, kernels):
+        self.gate_up.prepare(kernels)
+        self.down.prepare(kernels)
+
     def forward(self, ctx, x, hidden):
-        gate_up = self.gate_up.forward(ctx, x)
         activated = ctx.new_activations(x.shape[0], self.intermediate)
-        ctx.kernels.swiglu(gate_up, activated)
+        ctx.kernels.gemm_swiglu(x, self.gate_up.weight, activated)     # both products and the gate in one pass
         self.down.forward(ctx, activated, out=hidden, accumulate=True)
 
 

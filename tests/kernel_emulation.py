@@ -94,6 +94,15 @@ class TorchKernels:
                 result[row, head] = (probs.double() @ values[:, kv, :].double()).float()
         out.copy_(result.reshape(n_rows, n_heads * head_dim).to(out.dtype))
 
+    def pack_weight(self, w):
+        return w
+
+    def gemm_swiglu(self, a, w, out):
+        self.calls.append("gemm_swiglu")
+        both = torch.empty(a.shape[0], w.shape[0], dtype=a.dtype)
+        self.gemm(a, w, both)
+        self.swiglu(both, out)
+
     def swiglu(self, gate_up, out):
         self.calls.append("swiglu")
         width = out.shape[1]

@@ -90,6 +90,49 @@ def test_gemm(K, a_dtype, w_dtype, m, n, k):
     assert rel(acc, want + base.double()) < f32_bound
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 96, 128), (8, 331, 192), (64, 130, 64), (65, 257, 1024), (200, 64, 448),
+                                   (3, 1000, 4096), (130, 520, 256), (16, 24, 64), (33, 16, 2048),
+                                   (8, 4096, 12288), (300, 1000, 1024), (129, 129, 128)])
+def test_gemm_with_packed_weights(K, m, n, k):
+    """The same product from the regrouped (16 x 64 blocks) weight layout."""
+    from beholdd.kernels import PackedWeight
+    g = torch.Generator().manual_seed(m * 7 + n)
+    a = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(n, k, generator=g) * 0.05).to(torch.bfloat16)
+    packed = K.pack_weight(dev(w))
+    assert isinstance(packed, PackedWeight) and packed.shape == (n, k) and packed.data.numel() == -(-n // 16) * 16 * k
+    assert not isinstance(K.pack_weight(dev(w[:, :k - 8].contiguous())), PackedWeight)      # width not a multiple of 64
+    assert not isinstance(K.pack_weight(dev(w.float())), PackedWeight)
+    want = a.double() @ w.double().t()
+    f32_bound = 4 * math.sqrt(k) * 2.0 ** -24
+    for out_dtype in (torch.float32, torch.bfloat16):
+        out = torch.empty(m, n, dtype=out_dtype, device="cuda:0")
+        K.gemm(dev(a), packed, out)
+        assert rel(out, want) < tol(out_dtype, f32_bound, 4e-3), (out_dtype, rel(out, want))
+    base = torch.randn(m, n, generator=g)
+    acc = dev(base.clone())
+    K.gemm(dev(a), packed, acc, accumulate=True)
+    assert rel(acc, want + base.double()) < f32_bound
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("m,width,k", [(1, 16, 64), (8, 160, 128), (40, 896, 320), (64, 48, 192), (65, 64, 64),
+                                       (130, 208, 256), (300, 1000, 128), (7, 100, 64), (8, 12288, 4096), (5, 32, 72)])
+def test_gemm_swiglu(K, dtype, packed, m, width, k):
+    """silu(a Wg^T) * (a Wu^T) in one pass (or in two where the sizes do not allow one), from both layouts."""
+    g = torch.Generator().manual_seed(m + width)
+    a = torch.randn(m, k, generator=g).to(dtype)
+    w = (torch.randn(2 * width, k, generator=g) * 0.08).to(dtype)
+    gate = a.double() @ w[:width].double().t()
+    up = a.double() @ w[width:].double().t()
+    want = gate / (1 + torch.exp(-gate)) * up
+    weight = K.pack_weight(dev(w)) if packed else dev(w)
+    out = torch.empty(m, width, dtype=dtype, device="cuda:0")
+    K.gemm_swiglu(dev(a), weight, out)
+    assert rel(out, want) < tol(dtype, 1e-5, 6e-3), rel(out, want)
+
+
 def make_cache(n_seqs, lengths, kv_heads, head_dim, dtype, seed, extra_pages=3):
     """Random keys/values for sequences of the given lengths, scattered over shuffled pages.
     Returns (k_pages, v_pages, page_table, dense keys list, dense values list)."""
