@@ -21,6 +21,11 @@
 //     two 32-column halves are the gate and the up columns of the same 32 outputs.
 // K must be a multiple of 8 (16-byte loads); other sizes are free.
 //
+// Fused input norm.  With NORM the activations are the float32 residual rows (optionally gathered
+// through a row index) and an RMSNorm weight: the operand is bf16(x[k] * w[k]) and the row's
+// 1/sqrt(mean(x^2) + eps), a scalar that factors out of the sum over k, multiplies the
+// accumulator in the epilogue.  The sum of squares is gathered in float32 on the way.
+//
 // Operand layouts relied on (wave of 64 lanes, l = lane):
 //   16x16x32: A row l%16, k 8*(l/16)..+7;  B column l%16, the same k;  D column l%16, rows 4*(l/16)..+3
 //   32x32x16: A row l%32, k 8*(l/32)..+7;  B column l%32, the same k;  D column l%32,
@@ -56,15 +61,36 @@ __device__ inline float silu_mul(float gate, float up) { return gate / (1.0f + e
 
 #define MFMA16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(b), c, 0, 0, 0)
 
+typedef float f32x4v_t __attribute__((ext_vector_type(4)));
+
+// eight float32 values at `x` times eight norm weights at `nw`, rounded to bfloat16; adds their squares to `ssq`
+__device__ inline u32x4_t normed_piece(const float* x, const float* nw, float& ssq) {
+  const f32x4v_t x0 = *reinterpret_cast<const f32x4v_t*>(x), x1 = *reinterpret_cast<const f32x4v_t*>(x + 4);
+  const f32x4v_t w0 = *reinterpret_cast<const f32x4v_t*>(nw), w1 = *reinterpret_cast<const f32x4v_t*>(nw + 4);
+  ssq += (x0[0] * x0[0] + x0[1] * x0[1]) + (x0[2] * x0[2] + x0[3] * x0[3]) +
+         (x1[0] * x1[0] + x1[1] * x1[1]) + (x1[2] * x1[2] + x1[3] * x1[3]);
+  u32x4_t r;
+  r[0] = (uint32_t)f32_to_bf16_bits(x0[0] * w0[0]) | ((uint32_t)f32_to_bf16_bits(x0[1] * w0[1]) << 16);
+  r[1] = (uint32_t)f32_to_bf16_bits(x0[2] * w0[2]) | ((uint32_t)f32_to_bf16_bits(x0[3] * w0[3]) << 16);
+  r[2] = (uint32_t)f32_to_bf16_bits(x1[0] * w1[0]) | ((uint32_t)f32_to_bf16_bits(x1[1] * w1[1]) << 16);
+  r[3] = (uint32_t)f32_to_bf16_bits(x1[2] * w1[2]) | ((uint32_t)f32_to_bf16_bits(x1[3] * w1[3]) << 16);
+  return r;
+}
+
 // ---- skinny --------------------------------------------------------------------------------
 // RT = 1: plain product.  RT = 2: SwiGLU; the second row block lies `pair_blocks` blocks after the first.
 
-template <int MB, int WAVES, bool TILES, int RT, typename TC>
-__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t* __restrict__ a,
+template <int MB, int WAVES, bool TILES, int RT, bool NORM, typename TC>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __restrict__ a_any,
                                                                  const uint16_t* __restrict__ w,
                                                                  TC* __restrict__ c, int M, int N, int K,
-                                                                 int accumulate, int pair_blocks) {
+                                                                 int accumulate, int pair_blocks,
+                                                                 const float* __restrict__ norm_w,
+                                                                 const int32_t* __restrict__ rows, float eps) {
   __shared__ float partial[WAVES][RT][MB][256];
+  __shared__ float ssq_part[WAVES][MB][16];
+  const uint16_t* a = (const uint16_t*)a_any;     // bfloat16 activations, or
+  const float* hidden = (const float*)a_any;      // with NORM: float32 rows to be normalised
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int i = lane % 16, g = lane / 16;
   const int n0 = blockIdx.x * 16;
@@ -85,11 +111,27 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
     }
   }
   const uint16_t* xp[MB];
+  const float* hp[MB];
+  float ssq[MB];
 #pragma unroll
   for (int b = 0; b < MB; ++b) {
-    const int row = (b * 16 + i < M) ? b * 16 + i : M - 1;
+    int row = (b * 16 + i < M) ? b * 16 + i : M - 1;
+    if (NORM && rows) row = rows[row];
     xp[b] = a + (size_t)row * K + g * 16;
+    hp[b] = hidden + (size_t)row * K + g * 16;
+    ssq[b] = 0.f;
   }
+  const float* nwp = NORM ? norm_w + g * 16 : nullptr;
+  // the 16 operand elements of chunk `at` for activation block b, as two 8-element pieces
+  auto x_pieces = [&](int b, int at, u32x4_t& p0, u32x4_t& p1) {
+    if (NORM) {
+      p0 = normed_piece(hp[b] + at * 64, nwp + at * 64, ssq[b]);
+      p1 = normed_piece(hp[b] + at * 64 + 8, nwp + at * 64 + 8, ssq[b]);
+    } else {
+      p0 = load16(xp[b] + at * 64);
+      p1 = load16(xp[b] + at * 64 + 8);
+    }
+  };
   f32x4_t acc[RT][MB];
 #pragma unroll
   for (int t = 0; t < RT; ++t)
@@ -111,10 +153,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
         wv[u][t][1] = TILES ? load16_stream(p + half_offset) : load16(p + half_offset);
       }
 #pragma unroll
-      for (int b = 0; b < MB; ++b) {
-        xv[u][b][0] = load16(xp[b] + at * 64);
-        xv[u][b][1] = load16(xp[b] + at * 64 + 8);
-      }
+      for (int b = 0; b < MB; ++b) x_pieces(b, at, xv[u][b][0], xv[u][b][1]);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -133,7 +172,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
       const u32x4_t w0 = load16(p), w1 = load16(p + half_offset);
 #pragma unroll
       for (int b = 0; b < MB; ++b) {
-        const u32x4_t x0 = load16(xp[b] + chunk * 64), x1 = load16(xp[b] + chunk * 64 + 8);
+        u32x4_t x0, x1;
+        float unused = 0.f;
+        if (NORM && t > 0) {   // the squares of this chunk were counted with the first row block
+          x0 = normed_piece(hp[b] + chunk * 64, nwp + chunk * 64, unused);
+          x1 = normed_piece(hp[b] + chunk * 64 + 8, nwp + chunk * 64 + 8, unused);
+        } else {
+          x_pieces(b, chunk, x0, x1);
+        }
         acc[t][b] = MFMA16(w0, x0, acc[t][b]);
         acc[t][b] = MFMA16(w1, x1, acc[t][b]);
       }
@@ -147,7 +193,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
       const u32x4_t w0 = at < K ? load16(wp[t] + k) : zero, w1 = at + 8 < K ? load16(wp[t] + k + 8) : zero;
 #pragma unroll
       for (int b = 0; b < MB; ++b) {
-        const u32x4_t x0 = at < K ? load16(xp[b] + k) : zero, x1 = at + 8 < K ? load16(xp[b] + k + 8) : zero;
+        u32x4_t x0 = zero, x1 = zero;
+        float unused = 0.f;
+        if (NORM) {
+          if (at < K) x0 = normed_piece(hp[b] + k, nwp + k, t == 0 ? ssq[b] : unused);
+          if (at + 8 < K) x1 = normed_piece(hp[b] + k + 8, nwp + k + 8, t == 0 ? ssq[b] : unused);
+        } else {
+          if (at < K) x0 = load16(xp[b] + k);
+          if (at + 8 < K) x1 = load16(xp[b] + k + 8);
+        }
         acc[t][b] = MFMA16(w0, x0, acc[t][b]);
         acc[t][b] = MFMA16(w1, x1, acc[t][b]);
       }
@@ -160,16 +214,33 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
     for (int b = 0; b < MB; ++b)
 #pragma unroll
       for (int r = 0; r < 4; ++r) partial[wave][t][b][i * 16 + 4 * g + r] = acc[t][b][r];
+  if (NORM) {
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {  // lanes i, i+16, i+32, i+48 hold the four k quarters of row i
+      float v = ssq[b];
+      v += __shfl_xor(v, 16, 64);
+      v += __shfl_xor(v, 32, 64);
+      if (g == 0) ssq_part[wave][b][i] = v;
+    }
+  }
   __syncthreads();
   for (int e = threadIdx.x; e < MB * 256; e += WAVES * 64) {
     const int b = e / 256, m = b * 16 + (e % 256) / 16, n = n0 + e % 16;
     if (m >= M || n >= N) continue;
+    float inv = 1.f;
+    if (NORM) {
+      float total = 0.f;
+#pragma unroll
+      for (int v = 0; v < WAVES; ++v) total += ssq_part[v][b][(e % 256) / 16];
+      inv = 1.0f / sqrtf(total / (float)K + eps);
+    }
     float sum[RT];
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
       sum[t] = 0.f;
 #pragma unroll
       for (int v = 0; v < WAVES; ++v) sum[t] += partial[v][t][b][e % 256];
+      sum[t] *= inv;
     }
     if (RT == 2)
       store_out<TC>(c, (size_t)m * N + n, silu_mul(sum[0], sum[RT - 1]), false);
@@ -186,12 +257,17 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
 
 // SWIGLU: the tile's 128 W rows are, per wave column half (32 outputs), 32 gate rows then the 32 up
 // rows of the same outputs; N counts outputs and the up rows start `N` rows (N/16 blocks) further on.
-template <bool TILES, bool SWIGLU, typename TC>
-__global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restrict__ a,
+template <bool TILES, bool SWIGLU, bool NORM, typename TC>
+__global__ __launch_bounds__(256) void gemm_tiled_kernel(const void* __restrict__ a_any,
                                                          const uint16_t* __restrict__ w, TC* __restrict__ c,
-                                                         int M, int N, int K, int accumulate) {
+                                                         int M, int N, int K, int accumulate,
+                                                         const float* __restrict__ norm_w,
+                                                         const int32_t* __restrict__ rows, float eps) {
   __shared__ __attribute__((aligned(16))) uint16_t as[2][TB * TPITCH];
   __shared__ __attribute__((aligned(16))) uint16_t ws[2][TB * TPITCH];
+  __shared__ float inv_rms[TB];
+  const uint16_t* a = (const uint16_t*)a_any;     // bfloat16 activations, or
+  const float* hidden = (const float*)a_any;      // with NORM: float32 rows to be normalised
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int m0 = blockIdx.y * TB;
   const int n0 = blockIdx.x * (SWIGLU ? TB / 2 : TB);   // first output column of the tile
@@ -209,14 +285,18 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
   // global -> LDS staging: a slice is 128 rows x 8 pieces of 16 bytes; a thread moves 4 pieces per operand
   int a_at[4], w_at[4], a_piece[4];
   const uint16_t* a_src[4];
+  const float* h_src[4];
   const uint16_t* w_src[4];
+  float ssq[4] = {0.f, 0.f, 0.f, 0.f};   // NORM: squares of the pieces this thread stages, one row each
   size_t w_step;
 #pragma unroll
   for (int s = 0; s < 4; ++s) {
     const int e = tid + s * 256;
     const int row = e / 8, piece = e % 8;
-    const int am = (m0 + row < M) ? m0 + row : M - 1;
+    int am = (m0 + row < M) ? m0 + row : M - 1;
+    if (NORM && rows) am = rows[am];
     a_src[s] = a + (size_t)am * K + piece * 8;
+    h_src[s] = hidden + (size_t)am * K + piece * 8;
     a_at[s] = row * TPITCH + piece * 8;
     a_piece[s] = piece;
     if (TILES) {
@@ -241,7 +321,10 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       const bool inside = k0 + a_piece[s] * 8 < K;
-      a_reg[s] = inside ? load16(a_src[s] + k0) : zero;
+      if (NORM)
+        a_reg[s] = inside ? normed_piece(h_src[s] + k0, norm_w + k0 + a_piece[s] * 8, ssq[s]) : zero;
+      else
+        a_reg[s] = inside ? load16(a_src[s] + k0) : zero;
       w_reg[s] = (TILES || inside) ? load16(w_src[s] + (size_t)slice * w_step) : zero;
     }
   };
@@ -287,6 +370,25 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
     if (s + 1 < slices) stash(buffer ^ 1);
     __syncthreads();
   }
+  if (NORM) {  // the 8 threads tid%8 = 0..7 staged the 8 pieces of each slice of rows tid/8 + 32 s
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      float v = ssq[s];
+      v += __shfl_xor(v, 1, 64);
+      v += __shfl_xor(v, 2, 64);
+      v += __shfl_xor(v, 4, 64);
+      if (tid % 8 == 0) inv_rms[tid / 8 + 32 * s] = 1.0f / sqrtf(v / (float)K + eps);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int x = 0; x < 2; ++x)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const float inv = inv_rms[wm + x * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4];
+        acc[x][0][e] *= inv;
+        acc[x][1][e] *= inv;
+      }
+  }
   // D of one 32x32 block: column (n) lane%32, rows (m) 8*(e/4) + 4*(lane/32) + e%4
 #pragma unroll
   for (int x = 0; x < 2; ++x) {
@@ -315,15 +417,26 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
 
 // ---- entry -------------------------------------------------------------------------------------
 
-template <bool TILES, int RT, typename TC>
-static void launch_skinny(const void* a, const void* w, void* c, int M, int N, int K, int accumulate,
-                          int pair_blocks, hipStream_t stream) {
+struct GemmArgs {
+  const void* a;
+  const void* w;
+  void* c;
+  int M, N, K, accumulate;
+  const float* norm_w;
+  const int32_t* rows;
+  float eps;
+  hipStream_t stream;
+};
+
+template <bool TILES, int RT, bool NORM, typename TC>
+static void launch_skinny(const GemmArgs& g) {
   constexpr int WAVES = 8;
-  dim3 grid((N + 15) / 16), block(WAVES * 64);
-#define BH_SKINNY(MB)                                                                                     \
-  gemm_skinny_kernel<MB, WAVES, TILES, RT, TC><<<grid, block, 0, stream>>>(                               \
-      (const uint16_t*)a, (const uint16_t*)w, (TC*)c, M, N, K, accumulate, pair_blocks)
-  switch ((M + 15) / 16) {
+  dim3 grid((g.N + 15) / 16), block(WAVES * 64);
+  const int pair_blocks = RT == 2 ? g.N / 16 : 0;
+#define BH_SKINNY(MB)                                                                                        \
+  gemm_skinny_kernel<MB, WAVES, TILES, RT, NORM, TC><<<grid, block, 0, g.stream>>>(                          \
+      g.a, (const uint16_t*)g.w, (TC*)g.c, g.M, g.N, g.K, g.accumulate, pair_blocks, g.norm_w, g.rows, g.eps)
+  switch ((g.M + 15) / 16) {
     case 1: BH_SKINNY(1); break;
     case 2: BH_SKINNY(2); break;
     case 3: BH_SKINNY(3); break;
@@ -332,51 +445,54 @@ static void launch_skinny(const void* a, const void* w, void* c, int M, int N, i
 #undef BH_SKINNY
 }
 
-template <bool TILES, bool SWIGLU, typename TC>
-static void launch_tiled(const void* a, const void* w, void* c, int M, int N, int K, int accumulate,
-                         hipStream_t stream) {
+template <bool TILES, bool SWIGLU, bool NORM, typename TC>
+static void launch_tiled(const GemmArgs& g) {
   const int columns = SWIGLU ? TB / 2 : TB;
-  dim3 grid((N + columns - 1) / columns, (M + TB - 1) / TB), block(256);
-  gemm_tiled_kernel<TILES, SWIGLU, TC><<<grid, block, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, (TC*)c, M,
-                                                                   N, K, accumulate);
+  dim3 grid((g.N + columns - 1) / columns, (g.M + TB - 1) / TB), block(256);
+  gemm_tiled_kernel<TILES, SWIGLU, NORM, TC><<<grid, block, 0, g.stream>>>(
+      g.a, (const uint16_t*)g.w, (TC*)g.c, g.M, g.N, g.K, g.accumulate, g.norm_w, g.rows, g.eps);
+}
+
+template <bool TILES, bool SWIGLU, bool NORM>
+static void launch_shape(const GemmArgs& g, bool f32) {
+  if (g.M <= 64) {
+    if (f32) launch_skinny<TILES, SWIGLU ? 2 : 1, NORM, float>(g);
+    else launch_skinny<TILES, SWIGLU ? 2 : 1, NORM, bf16_t>(g);
+  } else {
+    if (f32) launch_tiled<TILES, SWIGLU, NORM, float>(g);
+    else launch_tiled<TILES, SWIGLU, NORM, bf16_t>(g);
+  }
 }
 
 // layout: 0 = rows, 1 = tiles.  activation: 0 = none; 1 = SwiGLU (W has 2 * N rows: gate rows then up rows).
+// norm_w != null: `a` is float32 [*, K]; its rows (gathered through `rows` when given) are RMS-normalised
+// with weight norm_w (float32 [K]) and eps on the way in.  Otherwise `a` is bfloat16 [M, K].
 extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, int accumulate, int M, int N, int K,
-                            int layout, int activation, hipStream_t stream) {
+                            int layout, int activation, const float* norm_w, const int32_t* rows, float eps,
+                            hipStream_t stream) {
   BH_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_bf16: sizes M=%d N=%d K=%d must be positive", M, N, K);
   BH_REQUIRE(K % 8 == 0, "gemm_bf16: K=%d must be a multiple of 8", K);
   BH_REQUIRE(c_dtype == BH_F32 || c_dtype == BH_BF16, "gemm_bf16: unknown output dtype %d", c_dtype);
-  BH_REQUIRE(((uintptr_t)a | (uintptr_t)w) % 16 == 0, "gemm_bf16: operands must be 16-byte aligned");
+  BH_REQUIRE(((uintptr_t)a | (uintptr_t)w | (uintptr_t)norm_w) % 16 == 0, "gemm_bf16: operands must be 16-byte aligned");
   BH_REQUIRE(layout == 0 || (layout == 1 && K % 64 == 0), "gemm_bf16: the tiles layout needs K=%d to be a multiple of 64", K);
   BH_REQUIRE(activation == 0 || activation == 1, "gemm_bf16: unknown activation %d", activation);
   BH_REQUIRE(activation == 0 || (N % 16 == 0 && !accumulate),
              "gemm_bf16: SwiGLU needs a multiple of 16 outputs (got %d) and no accumulation", N);
+  BH_REQUIRE(norm_w != nullptr || rows == nullptr, "gemm_bf16: a row index comes with a norm only");
+  BH_REQUIRE(norm_w == nullptr || eps >= 0.f, "gemm_bf16: eps must not be negative");
   BH_REQUIRE((M + TB - 1) / TB <= 65535, "gemm_bf16: M=%d needs more than 65535 row tiles", M);
+  const GemmArgs g{a, w, c, M, N, K, accumulate, norm_w, rows, eps, stream};
   const bool f32 = c_dtype == BH_F32;
-#define BH_PICK(FN, TILES, EXTRA, ...)                                             \
-  do {                                                                              \
-    if (f32) FN<TILES, EXTRA, float>(__VA_ARGS__);                                  \
-    else FN<TILES, EXTRA, bf16_t>(__VA_ARGS__);                                     \
-  } while (0)
-  if (M <= 64) {
-    const int pair_blocks = N / 16;
-    if (activation) {
-      if (layout) BH_PICK(launch_skinny, true, 2, a, w, c, M, N, K, 0, pair_blocks, stream);
-      else BH_PICK(launch_skinny, false, 2, a, w, c, M, N, K, 0, pair_blocks, stream);
-    } else {
-      if (layout) BH_PICK(launch_skinny, true, 1, a, w, c, M, N, K, accumulate, 0, stream);
-      else BH_PICK(launch_skinny, false, 1, a, w, c, M, N, K, accumulate, 0, stream);
-    }
-    return bh_check_launch("gemm_skinny");
+  const int which = (layout ? 4 : 0) | (activation ? 2 : 0) | (norm_w ? 1 : 0);
+  switch (which) {
+    case 0: launch_shape<false, false, false>(g, f32); break;
+    case 1: launch_shape<false, false, true>(g, f32); break;
+    case 2: launch_shape<false, true, false>(g, f32); break;
+    case 3: launch_shape<false, true, true>(g, f32); break;
+    case 4: launch_shape<true, false, false>(g, f32); break;
+    case 5: launch_shape<true, false, true>(g, f32); break;
+    case 6: launch_shape<true, true, false>(g, f32); break;
+    default: launch_shape<true, true, true>(g, f32); break;
   }
-  if (activation) {
-    if (layout) BH_PICK(launch_tiled, true, true, a, w, c, M, N, K, 0, stream);
-    else BH_PICK(launch_tiled, false, true, a, w, c, M, N, K, 0, stream);
-  } else {
-    if (layout) BH_PICK(launch_tiled, true, false, a, w, c, M, N, K, accumulate, stream);
-    else BH_PICK(launch_tiled, false, false, a, w, c, M, N, K, accumulate, stream);
-  }
-#undef BH_PICK
-  return bh_check_launch("gemm_tiled");
+  return bh_check_launch(M <= 64 ? "gemm_skinny" : "gemm_tiled");
 }

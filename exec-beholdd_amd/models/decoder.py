@@ -12,6 +12,7 @@ from __future__ import annotations
 
 from ..parts.base import BLOCKS, NORMS, POSITION_ENCODINGS
 from ..parts.embedding import Embedding, LMHead
+from ..parts.norm import NormedInput, RMSNorm
 
 
 class DecoderModel:
@@ -77,6 +78,8 @@ class DecoderModel:
             self.blocks[layer].forward(ctx, hidden, cache_for_run(run))
         if want_rows is None or want_rows.numel() == 0:
             return None
+        if isinstance(self.final_norm, RMSNorm):
+            return self.head.forward(ctx, NormedInput(ctx, self.final_norm, hidden, rows=want_rows))
         return self.head.forward(ctx, self.final_norm.forward(ctx, hidden, rows=want_rows))
 
 

@@ -65,6 +65,8 @@ class GQAAttention:
     def cache_need(self):
         return CacheNeed(kind="kv", kv_heads=self.n_kv_heads, head_dim=self.head_dim, window=self.window)
 
+    takes_normed_input = True     # x goes straight into the q/k/v product
+
     def forward(self, ctx, x, hidden, cache):
         k = ctx.kernels
         qkv = self.qkv.forward(ctx, x)

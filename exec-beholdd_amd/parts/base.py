@@ -20,6 +20,9 @@ Mixer:
     forward(ctx, x, hidden, cache)         adds its output into `hidden` (float32, the residual)
 Feed-forward:
     forward(ctx, x, hidden)                adds its output into `hidden`
+A mixer or feed-forward whose first operation is a `Linear` may set `takes_normed_input = True`;
+`x` is then a `NormedInput` (the not yet computed rmsnorm of the residual) that `Linear.forward`
+fuses into its product, and `x.tensor()` is the plain tensor.
 Block:
     mixer, feed_forward attributes; forward(ctx, hidden, cache)
 """

@@ -29,9 +29,17 @@ class SwiGLU:
         self.gate_up.prepare(kernels)
         self.down.prepare(kernels)
 
+    takes_normed_input = True
+
     def forward(self, ctx, x, hidden):
-        activated = ctx.new_activations(x.shape[0], self.intermediate)
-        ctx.kernels.gemm_swiglu(x, self.gate_up.weight, activated)     # both products and the gate in one pass
+        from .norm import NormedInput
+        n_rows = x.n_rows if isinstance(x, NormedInput) else x.shape[0]
+        activated = ctx.new_activations(n_rows, self.intermediate)
+        if isinstance(x, NormedInput):     # norm, both products and the gate in one pass
+            ctx.kernels.gemm_swiglu_normed(x.hidden, x.norm.weight, x.norm.eps, self.gate_up.weight, activated,
+                                           ctx.act_dtype, rows=x.rows)
+        else:
+            ctx.kernels.gemm_swiglu(x, self.gate_up.weight, activated)
         self.down.forward(ctx, activated, out=hidden, accumulate=True)
 
 

@@ -33,6 +33,23 @@ class RMSNorm:
         return out
 
 
+class NormedInput:
+    """rmsnorm(hidden[rows]) that has not been computed yet.
+
+    A part that starts with a linear map can hand this to `Linear.forward`, which fuses the norm
+    into the product; `tensor()` computes it the plain way for any other use."""
+
+    def __init__(self, ctx, norm: RMSNorm, hidden, rows=None):
+        self.ctx, self.norm, self.hidden, self.rows = ctx, norm, hidden, rows
+        self.n_rows = hidden.shape[0] if rows is None else rows.shape[0]
+        self._tensor = None
+
+    def tensor(self):
+        if self._tensor is None:
+            self._tensor = self.norm.forward(self.ctx, self.hidden, rows=self.rows)
+        return self._tensor
+
+
 @NORMS.register("rmsnorm")
 def _build_rmsnorm(config, width, name, shared):
     return RMSNorm(width, config.rms_eps, name)
