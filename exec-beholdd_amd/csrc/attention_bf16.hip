@@ -40,8 +40,13 @@ __device__ inline int wave_min_int(int v) {
   return v;
 }
 
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+// two float32 values rounded to nearest-even bfloat16 and packed (one v_cvt_pk_bf16_f32)
 __device__ inline uint32_t pack_bf16(float lo, float hi) {
-  return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
 // keep the first `n_valid` (0..8) bfloat16 elements of a 16-byte vector, zero the rest

@@ -21,7 +21,7 @@
 //     two 32-column halves are the gate and the up columns of the same 32 outputs.
 // K must be a multiple of 8 (16-byte loads); other sizes are free.
 //
-// Fused input norm.  With NORM the activations are the float32 residual rows (optionally gathered
+// Fused input norm (skinny kernel, at most 16 rows).  With NORM the activations are the float32 residual rows (optionally gathered
 // through a row index) and an RMSNorm weight: the operand is bf16(x[k] * w[k]) and the row's
 // 1/sqrt(mean(x^2) + eps), a scalar that factors out of the sum over k, multiplies the
 // accumulator in the epilogue.  The sum of squares is gathered in float32 on the way.
@@ -62,6 +62,14 @@ __device__ inline float silu_mul(float gate, float up) { return gate / (1.0f + e
 #define MFMA16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(b), c, 0, 0, 0)
 
 typedef float f32x4v_t __attribute__((ext_vector_type(4)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+// two float32 values rounded to nearest-even bfloat16 and packed (one v_cvt_pk_bf16_f32)
+__device__ inline uint32_t pack_bf16x2(float lo, float hi) {
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
 
 // eight float32 values at `x` times eight norm weights at `nw`, rounded to bfloat16; adds their squares to `ssq`
 __device__ inline u32x4_t normed_piece(const float* x, const float* nw, float& ssq) {
@@ -70,10 +78,10 @@ __device__ inline u32x4_t normed_piece(const float* x, const float* nw, float& s
   ssq += (x0[0] * x0[0] + x0[1] * x0[1]) + (x0[2] * x0[2] + x0[3] * x0[3]) +
          (x1[0] * x1[0] + x1[1] * x1[1]) + (x1[2] * x1[2] + x1[3] * x1[3]);
   u32x4_t r;
-  r[0] = (uint32_t)f32_to_bf16_bits(x0[0] * w0[0]) | ((uint32_t)f32_to_bf16_bits(x0[1] * w0[1]) << 16);
-  r[1] = (uint32_t)f32_to_bf16_bits(x0[2] * w0[2]) | ((uint32_t)f32_to_bf16_bits(x0[3] * w0[3]) << 16);
-  r[2] = (uint32_t)f32_to_bf16_bits(x1[0] * w1[0]) | ((uint32_t)f32_to_bf16_bits(x1[1] * w1[1]) << 16);
-  r[3] = (uint32_t)f32_to_bf16_bits(x1[2] * w1[2]) | ((uint32_t)f32_to_bf16_bits(x1[3] * w1[3]) << 16);
+  r[0] = pack_bf16x2(x0[0] * w0[0], x0[1] * w0[1]);
+  r[1] = pack_bf16x2(x0[2] * w0[2], x0[3] * w0[3]);
+  r[2] = pack_bf16x2(x1[0] * w1[0], x1[1] * w1[1]);
+  r[3] = pack_bf16x2(x1[2] * w1[2], x1[3] * w1[3]);
   return r;
 }
 
@@ -257,17 +265,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
 
 // SWIGLU: the tile's 128 W rows are, per wave column half (32 outputs), 32 gate rows then the 32 up
 // rows of the same outputs; N counts outputs and the up rows start `N` rows (N/16 blocks) further on.
-template <bool TILES, bool SWIGLU, bool NORM, typename TC>
-__global__ __launch_bounds__(256) void gemm_tiled_kernel(const void* __restrict__ a_any,
+template <bool TILES, bool SWIGLU, typename TC>
+__global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restrict__ a,
                                                          const uint16_t* __restrict__ w, TC* __restrict__ c,
-                                                         int M, int N, int K, int accumulate,
-                                                         const float* __restrict__ norm_w,
-                                                         const int32_t* __restrict__ rows, float eps) {
+                                                         int M, int N, int K, int accumulate) {
   __shared__ __attribute__((aligned(16))) uint16_t as[2][TB * TPITCH];
   __shared__ __attribute__((aligned(16))) uint16_t ws[2][TB * TPITCH];
-  __shared__ float inv_rms[TB];
-  const uint16_t* a = (const uint16_t*)a_any;     // bfloat16 activations, or
-  const float* hidden = (const float*)a_any;      // with NORM: float32 rows to be normalised
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int m0 = blockIdx.y * TB;
   const int n0 = blockIdx.x * (SWIGLU ? TB / 2 : TB);   // first output column of the tile
@@ -285,18 +288,14 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const void* __restrict_
   // global -> LDS staging: a slice is 128 rows x 8 pieces of 16 bytes; a thread moves 4 pieces per operand
   int a_at[4], w_at[4], a_piece[4];
   const uint16_t* a_src[4];
-  const float* h_src[4];
   const uint16_t* w_src[4];
-  float ssq[4] = {0.f, 0.f, 0.f, 0.f};   // NORM: squares of the pieces this thread stages, one row each
   size_t w_step;
 #pragma unroll
   for (int s = 0; s < 4; ++s) {
     const int e = tid + s * 256;
     const int row = e / 8, piece = e % 8;
-    int am = (m0 + row < M) ? m0 + row : M - 1;
-    if (NORM && rows) am = rows[am];
+    const int am = (m0 + row < M) ? m0 + row : M - 1;
     a_src[s] = a + (size_t)am * K + piece * 8;
-    h_src[s] = hidden + (size_t)am * K + piece * 8;
     a_at[s] = row * TPITCH + piece * 8;
     a_piece[s] = piece;
     if (TILES) {
@@ -321,10 +320,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const void* __restrict_
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       const bool inside = k0 + a_piece[s] * 8 < K;
-      if (NORM)
-        a_reg[s] = inside ? normed_piece(h_src[s] + k0, norm_w + k0 + a_piece[s] * 8, ssq[s]) : zero;
-      else
-        a_reg[s] = inside ? load16(a_src[s] + k0) : zero;
+      a_reg[s] = inside ? load16(a_src[s] + k0) : zero;
       w_reg[s] = (TILES || inside) ? load16(w_src[s] + (size_t)slice * w_step) : zero;
     }
   };
@@ -370,25 +366,6 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const void* __restrict_
     if (s + 1 < slices) stash(buffer ^ 1);
     __syncthreads();
   }
-  if (NORM) {  // the 8 threads tid%8 = 0..7 staged the 8 pieces of each slice of rows tid/8 + 32 s
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      float v = ssq[s];
-      v += __shfl_xor(v, 1, 64);
-      v += __shfl_xor(v, 2, 64);
-      v += __shfl_xor(v, 4, 64);
-      if (tid % 8 == 0) inv_rms[tid / 8 + 32 * s] = 1.0f / sqrtf(v / (float)K + eps);
-    }
-    __syncthreads();
-#pragma unroll
-    for (int x = 0; x < 2; ++x)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const float inv = inv_rms[wm + x * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4];
-        acc[x][0][e] *= inv;
-        acc[x][1][e] *= inv;
-      }
-  }
   // D of one 32x32 block: column (n) lane%32, rows (m) 8*(e/4) + 4*(lane/32) + e%4
 #pragma unroll
   for (int x = 0; x < 2; ++x) {
@@ -433,24 +410,28 @@ static void launch_skinny(const GemmArgs& g) {
   constexpr int WAVES = 8;
   dim3 grid((g.N + 15) / 16), block(WAVES * 64);
   const int pair_blocks = RT == 2 ? g.N / 16 : 0;
-#define BH_SKINNY(MB)                                                                                        \
-  gemm_skinny_kernel<MB, WAVES, TILES, RT, NORM, TC><<<grid, block, 0, g.stream>>>(                          \
+#define BH_SKINNY(MB, WITH_NORM)                                                                             \
+  gemm_skinny_kernel<MB, WAVES, TILES, RT, WITH_NORM, TC><<<grid, block, 0, g.stream>>>(                     \
       g.a, (const uint16_t*)g.w, (TC*)g.c, g.M, g.N, g.K, g.accumulate, pair_blocks, g.norm_w, g.rows, g.eps)
+  if (NORM) {  // the entry point admits a fused norm for at most 16 rows only
+    BH_SKINNY(1, NORM);
+    return;
+  }
   switch ((g.M + 15) / 16) {
-    case 1: BH_SKINNY(1); break;
-    case 2: BH_SKINNY(2); break;
-    case 3: BH_SKINNY(3); break;
-    default: BH_SKINNY(4); break;
+    case 1: BH_SKINNY(1, false); break;
+    case 2: BH_SKINNY(2, false); break;
+    case 3: BH_SKINNY(3, false); break;
+    default: BH_SKINNY(4, false); break;
   }
 #undef BH_SKINNY
 }
 
-template <bool TILES, bool SWIGLU, bool NORM, typename TC>
+template <bool TILES, bool SWIGLU, typename TC>
 static void launch_tiled(const GemmArgs& g) {
   const int columns = SWIGLU ? TB / 2 : TB;
   dim3 grid((g.N + columns - 1) / columns, (g.M + TB - 1) / TB), block(256);
-  gemm_tiled_kernel<TILES, SWIGLU, NORM, TC><<<grid, block, 0, g.stream>>>(
-      g.a, (const uint16_t*)g.w, (TC*)g.c, g.M, g.N, g.K, g.accumulate, g.norm_w, g.rows, g.eps);
+  gemm_tiled_kernel<TILES, SWIGLU, TC><<<grid, block, 0, g.stream>>>(
+      (const uint16_t*)g.a, (const uint16_t*)g.w, (TC*)g.c, g.M, g.N, g.K, g.accumulate);
 }
 
 template <bool TILES, bool SWIGLU, bool NORM>
@@ -459,14 +440,15 @@ static void launch_shape(const GemmArgs& g, bool f32) {
     if (f32) launch_skinny<TILES, SWIGLU ? 2 : 1, NORM, float>(g);
     else launch_skinny<TILES, SWIGLU ? 2 : 1, NORM, bf16_t>(g);
   } else {
-    if (f32) launch_tiled<TILES, SWIGLU, NORM, float>(g);
-    else launch_tiled<TILES, SWIGLU, NORM, bf16_t>(g);
+    if (f32) launch_tiled<TILES, SWIGLU, float>(g);
+    else launch_tiled<TILES, SWIGLU, bf16_t>(g);
   }
 }
 
 // layout: 0 = rows, 1 = tiles.  activation: 0 = none; 1 = SwiGLU (W has 2 * N rows: gate rows then up rows).
-// norm_w != null: `a` is float32 [*, K]; its rows (gathered through `rows` when given) are RMS-normalised
-// with weight norm_w (float32 [K]) and eps on the way in.  Otherwise `a` is bfloat16 [M, K].
+// norm_w != null (M <= 16 only): `a` is float32 [*, K]; its rows (gathered through `rows` when given) are
+// RMS-normalised with weight norm_w (float32 [K]) and eps on the way in.  Otherwise `a` is bfloat16 [M, K].
+// (For more rows the conversion work, repeated by every workgroup, costs more than a norm kernel of its own.)
 extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, int accumulate, int M, int N, int K,
                             int layout, int activation, const float* norm_w, const int32_t* rows, float eps,
                             hipStream_t stream) {
@@ -480,6 +462,7 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
              "gemm_bf16: SwiGLU needs a multiple of 16 outputs (got %d) and no accumulation", N);
   BH_REQUIRE(norm_w != nullptr || rows == nullptr, "gemm_bf16: a row index comes with a norm only");
   BH_REQUIRE(norm_w == nullptr || eps >= 0.f, "gemm_bf16: eps must not be negative");
+  BH_REQUIRE(norm_w == nullptr || M <= 16, "gemm_bf16: the fused norm takes at most 16 rows, got %d", M);
   BH_REQUIRE((M + TB - 1) / TB <= 65535, "gemm_bf16: M=%d needs more than 65535 row tiles", M);
   const GemmArgs g{a, w, c, M, N, K, accumulate, norm_w, rows, eps, stream};
   const bool f32 = c_dtype == BH_F32;

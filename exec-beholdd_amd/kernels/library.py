@@ -169,6 +169,8 @@ class HipKernels:
             return False
         if activation and (out.shape[1] % 16 or accumulate):
             return False
+        if norm is not None and out.shape[0] > 16:
+            return False      # every workgroup would redo the conversion of all rows: a norm kernel is cheaper
         norm_w = rows = None
         eps = 0.0
         if norm is not None:
