@@ -21,11 +21,6 @@
 //     two 32-column halves are the gate and the up columns of the same 32 outputs.
 // K must be a multiple of 8 (16-byte loads); other sizes are free.
 //
-// Fused input norm (skinny kernel, at most 16 rows).  With NORM the activations are the float32 residual rows (optionally gathered
-// through a row index) and an RMSNorm weight: the operand is bf16(x[k] * w[k]) and the row's
-// 1/sqrt(mean(x^2) + eps), a scalar that factors out of the sum over k, multiplies the
-// accumulator in the epilogue.  The sum of squares is gathered in float32 on the way.
-//
 // Operand layouts relied on (wave of 64 lanes, l = lane):
 //   16x16x32: A row l%16, k 8*(l/16)..+7;  B column l%16, the same k;  D column l%16, rows 4*(l/16)..+3
 //   32x32x16: A row l%32, k 8*(l/32)..+7;  B column l%32, the same k;  D column l%32,
@@ -61,44 +56,15 @@ __device__ inline float silu_mul(float gate, float up) { return gate / (1.0f + e
 
 #define MFMA16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(b), c, 0, 0, 0)
 
-typedef float f32x4v_t __attribute__((ext_vector_type(4)));
-typedef float f32x2_t __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-
-// two float32 values rounded to nearest-even bfloat16 and packed (one v_cvt_pk_bf16_f32)
-__device__ inline uint32_t pack_bf16x2(float lo, float hi) {
-  const f32x2_t v = {lo, hi};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
-}
-
-// eight float32 values at `x` times eight norm weights at `nw`, rounded to bfloat16; adds their squares to `ssq`
-__device__ inline u32x4_t normed_piece(const float* x, const float* nw, float& ssq) {
-  const f32x4v_t x0 = *reinterpret_cast<const f32x4v_t*>(x), x1 = *reinterpret_cast<const f32x4v_t*>(x + 4);
-  const f32x4v_t w0 = *reinterpret_cast<const f32x4v_t*>(nw), w1 = *reinterpret_cast<const f32x4v_t*>(nw + 4);
-  ssq += (x0[0] * x0[0] + x0[1] * x0[1]) + (x0[2] * x0[2] + x0[3] * x0[3]) +
-         (x1[0] * x1[0] + x1[1] * x1[1]) + (x1[2] * x1[2] + x1[3] * x1[3]);
-  u32x4_t r;
-  r[0] = pack_bf16x2(x0[0] * w0[0], x0[1] * w0[1]);
-  r[1] = pack_bf16x2(x0[2] * w0[2], x0[3] * w0[3]);
-  r[2] = pack_bf16x2(x1[0] * w1[0], x1[1] * w1[1]);
-  r[3] = pack_bf16x2(x1[2] * w1[2], x1[3] * w1[3]);
-  return r;
-}
-
 // ---- skinny --------------------------------------------------------------------------------
 // RT = 1: plain product.  RT = 2: SwiGLU; the second row block lies `pair_blocks` blocks after the first.
 
-template <int MB, int WAVES, bool TILES, int RT, bool NORM, typename TC>
-__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __restrict__ a_any,
+template <int MB, int WAVES, bool TILES, int RT, typename TC>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t* __restrict__ a,
                                                                  const uint16_t* __restrict__ w,
                                                                  TC* __restrict__ c, int M, int N, int K,
-                                                                 int accumulate, int pair_blocks,
-                                                                 const float* __restrict__ norm_w,
-                                                                 const int32_t* __restrict__ rows, float eps) {
+                                                                 int accumulate, int pair_blocks) {
   __shared__ float partial[WAVES][RT][MB][256];
-  __shared__ float ssq_part[WAVES][MB][16];
-  const uint16_t* a = (const uint16_t*)a_any;     // bfloat16 activations, or
-  const float* hidden = (const float*)a_any;      // with NORM: float32 rows to be normalised
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int i = lane % 16, g = lane / 16;
   const int n0 = blockIdx.x * 16;
@@ -119,27 +85,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
     }
   }
   const uint16_t* xp[MB];
-  const float* hp[MB];
-  float ssq[MB];
 #pragma unroll
   for (int b = 0; b < MB; ++b) {
-    int row = (b * 16 + i < M) ? b * 16 + i : M - 1;
-    if (NORM && rows) row = rows[row];
+    const int row = (b * 16 + i < M) ? b * 16 + i : M - 1;
     xp[b] = a + (size_t)row * K + g * 16;
-    hp[b] = hidden + (size_t)row * K + g * 16;
-    ssq[b] = 0.f;
   }
-  const float* nwp = NORM ? norm_w + g * 16 : nullptr;
-  // the 16 operand elements of chunk `at` for activation block b, as two 8-element pieces
-  auto x_pieces = [&](int b, int at, u32x4_t& p0, u32x4_t& p1) {
-    if (NORM) {
-      p0 = normed_piece(hp[b] + at * 64, nwp + at * 64, ssq[b]);
-      p1 = normed_piece(hp[b] + at * 64 + 8, nwp + at * 64 + 8, ssq[b]);
-    } else {
-      p0 = load16(xp[b] + at * 64);
-      p1 = load16(xp[b] + at * 64 + 8);
-    }
-  };
   f32x4_t acc[RT][MB];
 #pragma unroll
   for (int t = 0; t < RT; ++t)
@@ -161,7 +111,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
         wv[u][t][1] = TILES ? load16_stream(p + half_offset) : load16(p + half_offset);
       }
 #pragma unroll
-      for (int b = 0; b < MB; ++b) x_pieces(b, at, xv[u][b][0], xv[u][b][1]);
+      for (int b = 0; b < MB; ++b) {
+        xv[u][b][0] = load16(xp[b] + at * 64);
+        xv[u][b][1] = load16(xp[b] + at * 64 + 8);
+      }
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -180,14 +133,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
       const u32x4_t w0 = load16(p), w1 = load16(p + half_offset);
 #pragma unroll
       for (int b = 0; b < MB; ++b) {
-        u32x4_t x0, x1;
-        float unused = 0.f;
-        if (NORM && t > 0) {   // the squares of this chunk were counted with the first row block
-          x0 = normed_piece(hp[b] + chunk * 64, nwp + chunk * 64, unused);
-          x1 = normed_piece(hp[b] + chunk * 64 + 8, nwp + chunk * 64 + 8, unused);
-        } else {
-          x_pieces(b, chunk, x0, x1);
-        }
+        const u32x4_t x0 = load16(xp[b] + chunk * 64), x1 = load16(xp[b] + chunk * 64 + 8);
         acc[t][b] = MFMA16(w0, x0, acc[t][b]);
         acc[t][b] = MFMA16(w1, x1, acc[t][b]);
       }
@@ -201,15 +147,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
       const u32x4_t w0 = at < K ? load16(wp[t] + k) : zero, w1 = at + 8 < K ? load16(wp[t] + k + 8) : zero;
 #pragma unroll
       for (int b = 0; b < MB; ++b) {
-        u32x4_t x0 = zero, x1 = zero;
-        float unused = 0.f;
-        if (NORM) {
-          if (at < K) x0 = normed_piece(hp[b] + k, nwp + k, t == 0 ? ssq[b] : unused);
-          if (at + 8 < K) x1 = normed_piece(hp[b] + k + 8, nwp + k + 8, t == 0 ? ssq[b] : unused);
-        } else {
-          if (at < K) x0 = load16(xp[b] + k);
-          if (at + 8 < K) x1 = load16(xp[b] + k + 8);
-        }
+        const u32x4_t x0 = at < K ? load16(xp[b] + k) : zero, x1 = at + 8 < K ? load16(xp[b] + k + 8) : zero;
         acc[t][b] = MFMA16(w0, x0, acc[t][b]);
         acc[t][b] = MFMA16(w1, x1, acc[t][b]);
       }
@@ -222,33 +160,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const void* __r
     for (int b = 0; b < MB; ++b)
 #pragma unroll
       for (int r = 0; r < 4; ++r) partial[wave][t][b][i * 16 + 4 * g + r] = acc[t][b][r];
-  if (NORM) {
-#pragma unroll
-    for (int b = 0; b < MB; ++b) {  // lanes i, i+16, i+32, i+48 hold the four k quarters of row i
-      float v = ssq[b];
-      v += __shfl_xor(v, 16, 64);
-      v += __shfl_xor(v, 32, 64);
-      if (g == 0) ssq_part[wave][b][i] = v;
-    }
-  }
   __syncthreads();
   for (int e = threadIdx.x; e < MB * 256; e += WAVES * 64) {
     const int b = e / 256, m = b * 16 + (e % 256) / 16, n = n0 + e % 16;
     if (m >= M || n >= N) continue;
-    float inv = 1.f;
-    if (NORM) {
-      float total = 0.f;
-#pragma unroll
-      for (int v = 0; v < WAVES; ++v) total += ssq_part[v][b][(e % 256) / 16];
-      inv = 1.0f / sqrtf(total / (float)K + eps);
-    }
     float sum[RT];
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
       sum[t] = 0.f;
 #pragma unroll
       for (int v = 0; v < WAVES; ++v) sum[t] += partial[v][t][b][e % 256];
-      sum[t] *= inv;
     }
     if (RT == 2)
       store_out<TC>(c, (size_t)m * N + n, silu_mul(sum[0], sum[RT - 1]), false);
@@ -394,88 +315,68 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
 
 // ---- entry -------------------------------------------------------------------------------------
 
-struct GemmArgs {
-  const void* a;
-  const void* w;
-  void* c;
-  int M, N, K, accumulate;
-  const float* norm_w;
-  const int32_t* rows;
-  float eps;
-  hipStream_t stream;
-};
-
-template <bool TILES, int RT, bool NORM, typename TC>
-static void launch_skinny(const GemmArgs& g) {
+template <bool TILES, int RT, typename TC>
+static void launch_skinny(const void* a, const void* w, void* c, int M, int N, int K, int accumulate,
+                          int pair_blocks, hipStream_t stream) {
   constexpr int WAVES = 8;
-  dim3 grid((g.N + 15) / 16), block(WAVES * 64);
-  const int pair_blocks = RT == 2 ? g.N / 16 : 0;
-#define BH_SKINNY(MB, WITH_NORM)                                                                             \
-  gemm_skinny_kernel<MB, WAVES, TILES, RT, WITH_NORM, TC><<<grid, block, 0, g.stream>>>(                     \
-      g.a, (const uint16_t*)g.w, (TC*)g.c, g.M, g.N, g.K, g.accumulate, pair_blocks, g.norm_w, g.rows, g.eps)
-  if (NORM) {  // the entry point admits a fused norm for at most 16 rows only
-    BH_SKINNY(1, NORM);
-    return;
-  }
-  switch ((g.M + 15) / 16) {
-    case 1: BH_SKINNY(1, false); break;
-    case 2: BH_SKINNY(2, false); break;
-    case 3: BH_SKINNY(3, false); break;
-    default: BH_SKINNY(4, false); break;
+  dim3 grid((N + 15) / 16), block(WAVES * 64);
+#define BH_SKINNY(MB)                                                                                     \
+  gemm_skinny_kernel<MB, WAVES, TILES, RT, TC><<<grid, block, 0, stream>>>(                               \
+      (const uint16_t*)a, (const uint16_t*)w, (TC*)c, M, N, K, accumulate, pair_blocks)
+  switch ((M + 15) / 16) {
+    case 1: BH_SKINNY(1); break;
+    case 2: BH_SKINNY(2); break;
+    case 3: BH_SKINNY(3); break;
+    default: BH_SKINNY(4); break;
   }
 #undef BH_SKINNY
 }
 
 template <bool TILES, bool SWIGLU, typename TC>
-static void launch_tiled(const GemmArgs& g) {
+static void launch_tiled(const void* a, const void* w, void* c, int M, int N, int K, int accumulate,
+                         hipStream_t stream) {
   const int columns = SWIGLU ? TB / 2 : TB;
-  dim3 grid((g.N + columns - 1) / columns, (g.M + TB - 1) / TB), block(256);
-  gemm_tiled_kernel<TILES, SWIGLU, TC><<<grid, block, 0, g.stream>>>(
-      (const uint16_t*)g.a, (const uint16_t*)g.w, (TC*)g.c, g.M, g.N, g.K, g.accumulate);
-}
-
-template <bool TILES, bool SWIGLU, bool NORM>
-static void launch_shape(const GemmArgs& g, bool f32) {
-  if (g.M <= 64) {
-    if (f32) launch_skinny<TILES, SWIGLU ? 2 : 1, NORM, float>(g);
-    else launch_skinny<TILES, SWIGLU ? 2 : 1, NORM, bf16_t>(g);
-  } else {
-    if (f32) launch_tiled<TILES, SWIGLU, float>(g);
-    else launch_tiled<TILES, SWIGLU, bf16_t>(g);
-  }
+  dim3 grid((N + columns - 1) / columns, (M + TB - 1) / TB), block(256);
+  gemm_tiled_kernel<TILES, SWIGLU, TC><<<grid, block, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, (TC*)c, M,
+                                                                   N, K, accumulate);
 }
 
 // layout: 0 = rows, 1 = tiles.  activation: 0 = none; 1 = SwiGLU (W has 2 * N rows: gate rows then up rows).
-// norm_w != null (M <= 16 only): `a` is float32 [*, K]; its rows (gathered through `rows` when given) are
-// RMS-normalised with weight norm_w (float32 [K]) and eps on the way in.  Otherwise `a` is bfloat16 [M, K].
-// (For more rows the conversion work, repeated by every workgroup, costs more than a norm kernel of its own.)
 extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, int accumulate, int M, int N, int K,
-                            int layout, int activation, const float* norm_w, const int32_t* rows, float eps,
-                            hipStream_t stream) {
+                            int layout, int activation, hipStream_t stream) {
   BH_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_bf16: sizes M=%d N=%d K=%d must be positive", M, N, K);
   BH_REQUIRE(K % 8 == 0, "gemm_bf16: K=%d must be a multiple of 8", K);
   BH_REQUIRE(c_dtype == BH_F32 || c_dtype == BH_BF16, "gemm_bf16: unknown output dtype %d", c_dtype);
-  BH_REQUIRE(((uintptr_t)a | (uintptr_t)w | (uintptr_t)norm_w) % 16 == 0, "gemm_bf16: operands must be 16-byte aligned");
+  BH_REQUIRE(((uintptr_t)a | (uintptr_t)w) % 16 == 0, "gemm_bf16: operands must be 16-byte aligned");
   BH_REQUIRE(layout == 0 || (layout == 1 && K % 64 == 0), "gemm_bf16: the tiles layout needs K=%d to be a multiple of 64", K);
   BH_REQUIRE(activation == 0 || activation == 1, "gemm_bf16: unknown activation %d", activation);
   BH_REQUIRE(activation == 0 || (N % 16 == 0 && !accumulate),
              "gemm_bf16: SwiGLU needs a multiple of 16 outputs (got %d) and no accumulation", N);
-  BH_REQUIRE(norm_w != nullptr || rows == nullptr, "gemm_bf16: a row index comes with a norm only");
-  BH_REQUIRE(norm_w == nullptr || eps >= 0.f, "gemm_bf16: eps must not be negative");
-  BH_REQUIRE(norm_w == nullptr || M <= 16, "gemm_bf16: the fused norm takes at most 16 rows, got %d", M);
   BH_REQUIRE((M + TB - 1) / TB <= 65535, "gemm_bf16: M=%d needs more than 65535 row tiles", M);
-  const GemmArgs g{a, w, c, M, N, K, accumulate, norm_w, rows, eps, stream};
   const bool f32 = c_dtype == BH_F32;
-  const int which = (layout ? 4 : 0) | (activation ? 2 : 0) | (norm_w ? 1 : 0);
-  switch (which) {
-    case 0: launch_shape<false, false, false>(g, f32); break;
-    case 1: launch_shape<false, false, true>(g, f32); break;
-    case 2: launch_shape<false, true, false>(g, f32); break;
-    case 3: launch_shape<false, true, true>(g, f32); break;
-    case 4: launch_shape<true, false, false>(g, f32); break;
-    case 5: launch_shape<true, false, true>(g, f32); break;
-    case 6: launch_shape<true, true, false>(g, f32); break;
-    default: launch_shape<true, true, true>(g, f32); break;
+#define BH_PICK(FN, TILES, EXTRA, ...)                                             \
+  do {                                                                              \
+    if (f32) FN<TILES, EXTRA, float>(__VA_ARGS__);                                  \
+    else FN<TILES, EXTRA, bf16_t>(__VA_ARGS__);                                     \
+  } while (0)
+  if (M <= 64) {
+    const int pair_blocks = N / 16;
+    if (activation) {
+      if (layout) BH_PICK(launch_skinny, true, 2, a, w, c, M, N, K, 0, pair_blocks, stream);
+      else BH_PICK(launch_skinny, false, 2, a, w, c, M, N, K, 0, pair_blocks, stream);
+    } else {
+      if (layout) BH_PICK(launch_skinny, true, 1, a, w, c, M, N, K, accumulate, 0, stream);
+      else BH_PICK(launch_skinny, false, 1, a, w, c, M, N, K, accumulate, 0, stream);
+    }
+    return bh_check_launch("gemm_skinny");
   }
-  return bh_check_launch(M <= 64 ? "gemm_skinny" : "gemm_tiled");
+  if (activation) {
+    if (layout) BH_PICK(launch_tiled, true, true, a, w, c, M, N, K, 0, stream);
+    else BH_PICK(launch_tiled, false, true, a, w, c, M, N, K, 0, stream);
+  } else {
+    if (layout) BH_PICK(launch_tiled, true, false, a, w, c, M, N, K, accumulate, stream);
+    else BH_PICK(launch_tiled, false, false, a, w, c, M, N, K, accumulate, stream);
+  }
+#undef BH_PICK
+  return bh_check_launch("gemm_tiled");
 }

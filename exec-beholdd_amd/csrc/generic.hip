@@ -57,13 +57,37 @@ extern "C" int bh_embed(const int32_t* tokens, const void* table, int table_dtyp
 // ---- RMSNorm -----------------------------------------------------------------------------
 // out[r, i] = (x[src, i] * inv) * w[i], inv = 1/sqrt(mean(x^2) + eps), src = rows ? rows[r] : r.
 
-template <typename TW, typename TO>
+// PER > 0: the row fits PER elements per thread; x and w are loaded into registers before the
+// reduction so that both memory round trips overlap (a decode step runs this on a handful of rows,
+// where latency is all there is).  PER == 0: any width, in loops.
+template <typename TW, typename TO, int PER>
 __global__ void rmsnorm_kernel(const float* __restrict__ x, const int32_t* __restrict__ rows,
                                const TW* __restrict__ w, TO* __restrict__ out, int width, float eps) {
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const int src = rows ? rows[r] : r;
   const float* xr = x + (size_t)src * width;
+  TO* o = out + (size_t)r * width;
+  if (PER > 0) {
+    float xv[PER > 0 ? PER : 1], wv[PER > 0 ? PER : 1];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int i = threadIdx.x + j * blockDim.x;
+      xv[j] = i < width ? xr[i] : 0.f;
+      wv[j] = (w && i < width) ? to_f32(w[i]) : 1.f;
+    }
+#pragma unroll
+    for (int j = 0; j < PER; ++j) ss += xv[j] * xv[j];
+    ss = block_sum(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int i = threadIdx.x + j * blockDim.x;
+      if (i < width) o[i] = from_f32<TO>(xv[j] * inv * wv[j]);
+    }
+    return;
+  }
   float ss = 0.f;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     float v = xr[i];
@@ -71,7 +95,6 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const int32_t* __res
   }
   ss = block_sum(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / (float)width + eps);
-  TO* o = out + (size_t)r * width;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     float y = xr[i] * inv;
     if (w) y *= to_f32(w[i]);
@@ -79,19 +102,29 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const int32_t* __res
   }
 }
 
+template <typename TW, typename TO>
+static void launch_rmsnorm(const float* x, const int32_t* rows, const void* w, void* out, int n_rows, int width,
+                           float eps, hipStream_t stream) {
+  const int threads = width >= 4096 ? 1024 : (width >= 1024 ? 512 : 256);
+  const int per = (width + threads - 1) / threads;
+  dim3 grid(n_rows), block(threads);
+#define BH_NORM(PER) \
+  rmsnorm_kernel<TW, TO, PER><<<grid, block, 0, stream>>>(x, rows, (const TW*)w, (TO*)out, width, eps)
+  if (per <= 4) BH_NORM(4);
+  else if (per <= 8) BH_NORM(8);
+  else BH_NORM(0);
+#undef BH_NORM
+}
+
 extern "C" int bh_rmsnorm(const float* x, const int32_t* rows, const void* w, int w_dtype, void* out,
                           int out_dtype, int n_rows, int width, float eps, hipStream_t stream) {
   BH_REQUIRE(n_rows > 0 && width > 0, "rmsnorm: rows %d and width %d must be positive", n_rows, width);
   BH_REQUIRE(eps >= 0.f, "rmsnorm: eps must not be negative");
-  dim3 grid(n_rows), block(width >= 2048 ? 512 : 256);
-#define BH_NORM(TW, TO) \
-  rmsnorm_kernel<TW, TO><<<grid, block, 0, stream>>>(x, rows, (const TW*)w, (TO*)out, width, eps)
-  if (w_dtype == BH_F32 && out_dtype == BH_F32) BH_NORM(float, float);
-  else if (w_dtype == BH_F32 && out_dtype == BH_BF16) BH_NORM(float, bf16_t);
-  else if (w_dtype == BH_BF16 && out_dtype == BH_F32) BH_NORM(bf16_t, float);
-  else if (w_dtype == BH_BF16 && out_dtype == BH_BF16) BH_NORM(bf16_t, bf16_t);
+  if (w_dtype == BH_F32 && out_dtype == BH_F32) launch_rmsnorm<float, float>(x, rows, w, out, n_rows, width, eps, stream);
+  else if (w_dtype == BH_F32 && out_dtype == BH_BF16) launch_rmsnorm<float, bf16_t>(x, rows, w, out, n_rows, width, eps, stream);
+  else if (w_dtype == BH_BF16 && out_dtype == BH_F32) launch_rmsnorm<bf16_t, float>(x, rows, w, out, n_rows, width, eps, stream);
+  else if (w_dtype == BH_BF16 && out_dtype == BH_BF16) launch_rmsnorm<bf16_t, bf16_t>(x, rows, w, out, n_rows, width, eps, stream);
   else return bh_fail("rmsnorm: unknown dtypes %d/%d", w_dtype, out_dtype);
-#undef BH_NORM
   return bh_check_launch("rmsnorm");
 }
 

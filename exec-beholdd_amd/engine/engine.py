@@ -18,7 +18,8 @@ from ..sampling import Sampler, SamplingParams
 from ..weights.binder import bind
 from ..weights.random_init import random_tensor_on_device
 from . import generation
-from .step import StepEntry, build_step
+from .graphs import DecodeGraphs
+from .step import StepEntry, build_step, check_entries
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
 
@@ -39,7 +40,7 @@ class Engine:
 
     def __init__(self, model_dir: str | None = None, dtype="bfloat16", max_tokens: int = 4096,
                  max_slots: int | None = None, device="cuda:0", kernels=None, model=None,
-                 memory_limit_bytes: int | None = None):
+                 memory_limit_bytes: int | None = None, use_graphs: bool = True):
         self.dtype = parse_dtype(dtype)
         self.device = torch.device(device)
         if kernels is None:
@@ -58,6 +59,7 @@ class Engine:
                                    max_slots=max_slots, max_position=model.max_position)
         self.cache_plan = self.cache.allocate(limit_bytes=memory_limit_bytes)
         self.sampler = Sampler(kernels, self.device)
+        self.graphs = DecodeGraphs(self) if use_graphs and self.device.type == "cuda" else None
 
     # ---- what the generation loop needs of a stepper ----
     @property
@@ -91,6 +93,8 @@ class Engine:
         [wanted, vocab] in the order of the entries and of their `want` lists (None if nothing is
         wanted).  On an error no sequence's length changes."""
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
+        if self.graphs is not None and entries and self.graphs.usable(entries):
+            return self._graph_step(entries)
         ctx, want_rows, requests = build_step(self.kernels, self.dtype, self.device, self.cache, entries,
                                               self.model.vocab)
         self.cache.reserve(requests)
@@ -112,6 +116,25 @@ class Engine:
             raise
         self.cache.commit(requests)
         return logits
+
+    def _graph_step(self, entries: list):
+        """A decode step (one token per sequence) replayed from a captured HIP graph."""
+        check_entries(entries, self.cache, self.model.vocab)
+        requests = [(e.slot, 1) for e in entries]
+        self.cache.reserve(requests)
+        try:
+            pasts = [self.cache.length(e.slot) for e in entries]
+            logits = self.graphs.step(entries, pasts)
+        except BaseException:
+            self.cache.rollback(requests)
+            raise
+        self.cache.commit(requests)
+        wanted = [row for row, e in enumerate(entries) if e.want]
+        if not wanted:
+            return None
+        if len(wanted) == len(entries):
+            return logits
+        return logits[torch.tensor(wanted, device=self.device)]
 
     # ---- generation ----
     def generate(self, prompts: list, max_new_tokens=16, temperature: float = 0.0, top_k: int = 0,

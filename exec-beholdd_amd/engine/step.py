@@ -30,25 +30,34 @@ class StepEntry:
     want: list = field(default_factory=list)   # indices into `tokens` whose logits are returned
 
 
-def build_step(kernels, act_dtype, device, cache, entries: list, vocab: int):
-    """Check the entries and lay the step out.  Returns (context, want_rows tensor, requests)."""
+def check_entries(entries: list, cache, vocab: int) -> None:
+    """Refuse malformed entries before anything is changed or computed."""
     if not entries:
         raise StepError("a step needs at least one entry")
-    tokens, positions, row_seq, seq_start, seq_slot, seq_past, want_rows = [], [], [], [0], [], [], []
-    requests = []
     for index, entry in enumerate(entries):
         n_new = len(entry.tokens)
         if n_new == 0:
             raise StepError(f"entry {index} (slot {entry.slot}) brings no tokens")
-        past = cache.length(entry.slot)
+        cache.length(entry.slot)       # raises for a slot that is not in use
         for token in entry.tokens:
             if not isinstance(token, (int, np.integer)) or isinstance(token, bool) or not 0 <= token < vocab:
                 raise StepError(f"entry {index} (slot {entry.slot}): token {token!r} is outside the vocabulary "
                                 f"of {vocab}")
         for place in entry.want:
-            if not isinstance(place, (int, np.integer)) or not 0 <= place < n_new:
+            if not isinstance(place, (int, np.integer)) or isinstance(place, bool) or not 0 <= place < n_new:
                 raise StepError(f"entry {index} (slot {entry.slot}): wanted place {place!r} is outside its "
                                 f"{n_new} tokens")
+
+
+def build_step(kernels, act_dtype, device, cache, entries: list, vocab: int):
+    """Check the entries and lay the step out.  Returns (context, want_rows tensor, requests)."""
+    check_entries(entries, cache, vocab)
+    tokens, positions, row_seq, seq_start, seq_slot, seq_past, want_rows = [], [], [], [0], [], [], []
+    requests = []
+    for index, entry in enumerate(entries):
+        n_new = len(entry.tokens)
+        past = cache.length(entry.slot)
+        for place in entry.want:
             want_rows.append(len(tokens) + int(place))
         tokens.extend(int(t) for t in entry.tokens)
         positions.extend(range(past, past + n_new))

@@ -60,7 +60,6 @@ class HipKernels:
             raise KernelError(f"cannot load the HIP kernel library {path}: {error}") from None
         self.library_path = path
         self._declare()
-        self._norm_weights = {}
         self.page_size = int(self.lib.bh_page_size())
 
     # ---- ctypes declarations ----
@@ -84,7 +83,7 @@ class HipKernels:
             function.restype = i
         self._optional = {}
         for name, argtypes in {
-            "bh_gemm_bf16": [p, p, p, i, i, i, i, i, i, i, p, p, f, p],
+            "bh_gemm_bf16": [p, p, p, i, i, i, i, i, i, i, p],
             "bh_attention_bf16": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, i, i, f, i, i, i, p],
             "bh_attention_bf16_splits": [i, i, i, i, i],
         }.items():
@@ -157,71 +156,21 @@ class HipKernels:
             return PackedWeight(data, rows, cols)
         return w
 
-    def _gemm_fast(self, a, w, out, accumulate, activation, norm=None):
-        """Launch the matrix-core product if it takes these operands; say whether it did.
-        `norm` = (weight, eps, rows): `a` is then the float32 residual, normalised on the way in."""
+    def _gemm_fast(self, a, w, out, accumulate, activation):
+        """Launch the matrix-core product if it takes these operands; say whether it did."""
         fast = self._optional.get("bh_gemm_bf16")
         packed = isinstance(w, PackedWeight)
-        wanted = torch.float32 if norm is not None else torch.bfloat16
-        if fast is None or a.dtype != wanted or w.dtype != torch.bfloat16 or a.shape[1] % 8:
+        if fast is None or a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or a.shape[1] % 8:
             if packed:
-                raise KernelError("gemm: a packed weight needs bfloat16 activations or a fused norm")
+                raise KernelError("gemm: a packed weight needs bfloat16 activations")
             return False
         if activation and (out.shape[1] % 16 or accumulate):
             return False
-        if norm is not None and out.shape[0] > 16:
-            return False      # every workgroup would redo the conversion of all rows: a norm kernel is cheaper
-        norm_w = rows = None
-        eps = 0.0
-        if norm is not None:
-            weight, eps, rows = norm
-            norm_w = self._float_copy(weight)
+        m, k = a.shape
         self._check(fast(self._ptr(a, "gemm a"), self._ptr(w.data if packed else w, "gemm w"),
-                         self._ptr(out, "gemm out"), _code(out, "gemm out"), int(bool(accumulate)), out.shape[0],
-                         out.shape[1], a.shape[1], int(packed), int(activation),
-                         self._ptr(norm_w, "norm weight", (torch.float32,), True),
-                         self._ptr(rows, "rows", (torch.int32,), True), float(eps), self._stream()))
+                         self._ptr(out, "gemm out"), _code(out, "gemm out"), int(bool(accumulate)), m, out.shape[1], k,
+                         int(packed), int(activation), self._stream()))
         return True
-
-    def _float_copy(self, weight):
-        """A float32 copy of a (small, long-lived) norm weight, made once."""
-        if weight.dtype == torch.float32:
-            return weight
-        key = (weight.data_ptr(), tuple(weight.shape))
-        cached = self._norm_weights.get(key)
-        if cached is None or cached[0] is not weight:
-            cached = (weight, weight.float().contiguous())
-            self._norm_weights[key] = cached
-        return cached[1]
-
-    def _check_normed(self, hidden, norm_weight, w, out, rows, columns):
-        if hidden.dim() != 2 or w.dim() != 2 or out.dim() != 2 or hidden.dtype != torch.float32:
-            raise KernelError("gemm_normed: hidden must be a float32 matrix, w and out matrices")
-        k = hidden.shape[1]
-        n_rows = hidden.shape[0] if rows is None else rows.shape[0]
-        if norm_weight.shape != (k,) or w.shape[1] != k or out.shape != (n_rows, columns):
-            raise KernelError(f"gemm_normed: shapes hidden {tuple(hidden.shape)}, w {tuple(w.shape)}, "
-                              f"out {tuple(out.shape)} do not fit")
-        return n_rows, k
-
-    def gemm_normed(self, hidden, norm_weight, eps, w, out, act_dtype, rows=None, accumulate=False):
-        """out (+)= rmsnorm(hidden[rows]; norm_weight, eps) @ w^T, the norm fused into the product where
-        the sizes allow, else as two kernels with activations of `act_dtype` between them."""
-        n_rows, k = self._check_normed(hidden, norm_weight, w, out, rows, w.shape[0])
-        if self._gemm_fast(hidden, w, out, accumulate, 0, norm=(norm_weight, eps, rows)):
-            return
-        x = torch.empty((n_rows, k), dtype=act_dtype, device=self.device)
-        self.rmsnorm(hidden, norm_weight, eps, x, rows=rows)
-        self.gemm(x, w, out, accumulate=accumulate)
-
-    def gemm_swiglu_normed(self, hidden, norm_weight, eps, w, out, act_dtype, rows=None):
-        """out = silu(x @ w[:F]^T) * (x @ w[F:]^T) with x = rmsnorm(hidden[rows])."""
-        n_rows, k = self._check_normed(hidden, norm_weight, w, out, rows, w.shape[0] // 2)
-        if out.dtype == act_dtype and self._gemm_fast(hidden, w, out, False, 1, norm=(norm_weight, eps, rows)):
-            return
-        x = torch.empty((n_rows, k), dtype=act_dtype, device=self.device)
-        self.rmsnorm(hidden, norm_weight, eps, x, rows=rows)
-        self.gemm_swiglu(x, w, out)
 
     def gemm(self, a, w, out, accumulate=False):
         """out[M, N] (+)= a[M, K] @ w[N, K]^T with float32 accumulation; `w` may be a PackedWeight."""

@@ -12,7 +12,6 @@ from __future__ import annotations
 
 from ..parts.base import BLOCKS, NORMS, POSITION_ENCODINGS
 from ..parts.embedding import Embedding, LMHead
-from ..parts.norm import NormedInput, RMSNorm
 
 
 class DecoderModel:
@@ -53,6 +52,13 @@ class DecoderModel:
     def parts(self):
         return [self.embedding, *self.shared_parts, *self.blocks, self.final_norm, self.head]
 
+    @property
+    def graph_safe(self):
+        """True when a decode step of this model may be captured as a HIP graph: every part's
+        forward depends on the step's device tensors only."""
+        return all(getattr(part, "graph_safe", False)
+                   for part in (self.embedding, *self.blocks, self.final_norm, self.head))
+
     def tensor_specs(self):
         return [spec for part in self.parts() for spec in part.tensor_specs()]
 
@@ -78,8 +84,6 @@ class DecoderModel:
             self.blocks[layer].forward(ctx, hidden, cache_for_run(run))
         if want_rows is None or want_rows.numel() == 0:
             return None
-        if isinstance(self.final_norm, RMSNorm):
-            return self.head.forward(ctx, NormedInput(ctx, self.final_norm, hidden, rows=want_rows))
         return self.head.forward(ctx, self.final_norm.forward(ctx, hidden, rows=want_rows))
 
 

@@ -3,7 +3,7 @@
 from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, CacheNeed, LayerCache,
                    Registry, StepContext)
 from .linear import Linear
-from .norm import NormedInput, RMSNorm
+from .norm import RMSNorm
 from .rope import NoPositionEncoding, RotaryEncoding
 from .attention import GQAAttention
 from .mlp import SwiGLU
@@ -11,5 +11,5 @@ from .block import PreNormBlock
 from .embedding import Embedding, LMHead
 
 __all__ = ["BLOCKS", "FEED_FORWARDS", "MIXERS", "NORMS", "POSITION_ENCODINGS", "CacheNeed", "LayerCache",
-           "Registry", "StepContext", "Linear", "NormedInput", "RMSNorm", "NoPositionEncoding", "RotaryEncoding",
+           "Registry", "StepContext", "Linear", "RMSNorm", "NoPositionEncoding", "RotaryEncoding",
            "GQAAttention", "SwiGLU", "PreNormBlock", "Embedding", "LMHead"]

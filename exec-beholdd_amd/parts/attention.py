@@ -24,6 +24,7 @@ from .linear import Linear
 
 
 class GQAAttention:
+    graph_safe = True      # forward reads only the step's device tensors
     def __init__(self, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int, prefix: str, *,
                  position_encoding=None, qk_norm_eps: float | None = None, scale: float | None = None,
                  window: int = 0):
@@ -64,8 +65,6 @@ class GQAAttention:
 
     def cache_need(self):
         return CacheNeed(kind="kv", kv_heads=self.n_kv_heads, head_dim=self.head_dim, window=self.window)
-
-    takes_normed_input = True     # x goes straight into the q/k/v product
 
     def forward(self, ctx, x, hidden, cache):
         k = ctx.kernels

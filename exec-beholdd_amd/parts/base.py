@@ -20,11 +20,11 @@ Mixer:
     forward(ctx, x, hidden, cache)         adds its output into `hidden` (float32, the residual)
 Feed-forward:
     forward(ctx, x, hidden)                adds its output into `hidden`
-A mixer or feed-forward whose first operation is a `Linear` may set `takes_normed_input = True`;
-`x` is then a `NormedInput` (the not yet computed rmsnorm of the residual) that `Linear.forward`
-fuses into its product, and `x.tensor()` is the plain tensor.
 Block:
     mixer, feed_forward attributes; forward(ctx, hidden, cache)
+A part may declare `graph_safe = True`: its forward uses only the device tensors of the step
+context (never the host_* lists, never a host-side decision that changes from step to step).
+Decode steps of a model whose parts all say so are captured and replayed as HIP graphs.
 """
 
 from __future__ import annotations

@@ -8,7 +8,6 @@ and is updated in place; the mixer and the feed-forward add into it.
 from __future__ import annotations
 
 from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS
-from .norm import NormedInput, RMSNorm
 
 
 class PreNormBlock:
@@ -18,6 +17,10 @@ class PreNormBlock:
 
     def parts(self):
         return [self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward]
+
+    @property
+    def graph_safe(self):
+        return all(getattr(part, "graph_safe", False) for part in self.parts())
 
     def tensor_specs(self):
         return [spec for part in self.parts() for spec in part.tensor_specs()]
@@ -34,16 +37,9 @@ class PreNormBlock:
     def cache_need(self):
         return self.mixer.cache_need()
 
-    @staticmethod
-    def _normed(ctx, norm, consumer, hidden):
-        """The consumer's input: left for it to fuse when it says it can, else computed here."""
-        if isinstance(norm, RMSNorm) and getattr(consumer, "takes_normed_input", False):
-            return NormedInput(ctx, norm, hidden)
-        return norm.forward(ctx, hidden)
-
     def forward(self, ctx, hidden, cache):
-        self.mixer.forward(ctx, self._normed(ctx, self.mixer_norm, self.mixer, hidden), hidden, cache)
-        self.feed_forward.forward(ctx, self._normed(ctx, self.feed_forward_norm, self.feed_forward, hidden), hidden)
+        self.mixer.forward(ctx, self.mixer_norm.forward(ctx, hidden), hidden, cache)
+        self.feed_forward.forward(ctx, self.feed_forward_norm.forward(ctx, hidden), hidden)
 
 
 @BLOCKS.register("pre_norm")

@@ -15,6 +15,7 @@ from .linear import Linear
 
 
 class Embedding:
+    graph_safe = True      # forward reads only the step's device tensors
     def __init__(self, vocab: int, width: int, name: str):
         self.vocab, self.width, self.name = vocab, width, name
         self.weight: torch.Tensor | None = None
@@ -32,6 +33,7 @@ class Embedding:
 
 
 class LMHead:
+    graph_safe = True      # forward reads only the step's device tensors
     def __init__(self, vocab: int, width: int, name: str | None, tied_to: Embedding | None = None):
         if (name is None) == (tied_to is None):
             raise ValueError("a head has either its own tensor or an embedding it is tied to")

@@ -14,6 +14,7 @@ from ..weights.binder import TensorSpec
 
 
 class Linear:
+    graph_safe = True      # forward reads only the step's device tensors
     def __init__(self, in_features: int, out_features, names):
         """`names` and `out_features` are one name and size, or equal-length lists to stack."""
         self.in_features = int(in_features)
@@ -52,15 +53,8 @@ class Linear:
             self.weight = kernels.pack_weight(self.weight)
 
     def forward(self, ctx, x, out=None, accumulate=False, out_dtype=None):
-        """x [n, in] -> out [n, out]; with accumulate the product is added into `out`.
-        `x` may be a `NormedInput`: the norm is then fused into the product."""
-        from .norm import NormedInput
-        n_rows = x.n_rows if isinstance(x, NormedInput) else x.shape[0]
+        """x [n, in] -> out [n, out]; with accumulate the product is added into `out`."""
         if out is None:
-            out = torch.empty((n_rows, self.out_features), dtype=out_dtype or ctx.act_dtype, device=ctx.device)
-        if isinstance(x, NormedInput):
-            ctx.kernels.gemm_normed(x.hidden, x.norm.weight, x.norm.eps, self.weight, out, ctx.act_dtype,
-                                    rows=x.rows, accumulate=accumulate)
-        else:
-            ctx.kernels.gemm(x, self.weight, out, accumulate=accumulate)
+            out = torch.empty((x.shape[0], self.out_features), dtype=out_dtype or ctx.act_dtype, device=x.device)
+        ctx.kernels.gemm(x, self.weight, out, accumulate=accumulate)
         return out

@@ -12,6 +12,7 @@ from .linear import Linear
 
 
 class SwiGLU:
+    graph_safe = True      # forward reads only the step's device tensors
     def __init__(self, hidden: int, intermediate: int, prefix: str):
         self.hidden, self.intermediate = hidden, intermediate
         self.gate_up = Linear(hidden, [intermediate, intermediate],
@@ -29,17 +30,9 @@ class SwiGLU:
         self.gate_up.prepare(kernels)
         self.down.prepare(kernels)
 
-    takes_normed_input = True
-
     def forward(self, ctx, x, hidden):
-        from .norm import NormedInput
-        n_rows = x.n_rows if isinstance(x, NormedInput) else x.shape[0]
-        activated = ctx.new_activations(n_rows, self.intermediate)
-        if isinstance(x, NormedInput):     # norm, both products and the gate in one pass
-            ctx.kernels.gemm_swiglu_normed(x.hidden, x.norm.weight, x.norm.eps, self.gate_up.weight, activated,
-                                           ctx.act_dtype, rows=x.rows)
-        else:
-            ctx.kernels.gemm_swiglu(x, self.gate_up.weight, activated)
+        activated = ctx.new_activations(x.shape[0], self.intermediate)
+        ctx.kernels.gemm_swiglu(x, self.gate_up.weight, activated)     # both products and the gate in one pass
         self.down.forward(ctx, activated, out=hidden, accumulate=True)
 
 

@@ -14,6 +14,7 @@ from .base import NORMS
 
 
 class RMSNorm:
+    graph_safe = True      # forward reads only the step's device tensors
     def __init__(self, width: int, eps: float, name: str):
         if not (eps > 0.0):
             raise ValueError(f"RMSNorm epsilon must be positive, got {eps}")
@@ -31,23 +32,6 @@ class RMSNorm:
         out = ctx.new_activations(n, self.width)
         ctx.kernels.rmsnorm(hidden, self.weight, self.eps, out, rows=rows)
         return out
-
-
-class NormedInput:
-    """rmsnorm(hidden[rows]) that has not been computed yet.
-
-    A part that starts with a linear map can hand this to `Linear.forward`, which fuses the norm
-    into the product; `tensor()` computes it the plain way for any other use."""
-
-    def __init__(self, ctx, norm: RMSNorm, hidden, rows=None):
-        self.ctx, self.norm, self.hidden, self.rows = ctx, norm, hidden, rows
-        self.n_rows = hidden.shape[0] if rows is None else rows.shape[0]
-        self._tensor = None
-
-    def tensor(self):
-        if self._tensor is None:
-            self._tensor = self.norm.forward(self.ctx, self.hidden, rows=self.rows)
-        return self._tensor
 
 
 @NORMS.register("rmsnorm")

@@ -103,18 +103,6 @@ class TorchKernels:
         self.gemm(a, w, both)
         self.swiglu(both, out)
 
-    def gemm_normed(self, hidden, norm_weight, eps, w, out, act_dtype, rows=None, accumulate=False):
-        n = hidden.shape[0] if rows is None else rows.shape[0]
-        x = torch.empty(n, hidden.shape[1], dtype=act_dtype)
-        self.rmsnorm(hidden, norm_weight, eps, x, rows=rows)
-        self.gemm(x, w, out, accumulate=accumulate)
-
-    def gemm_swiglu_normed(self, hidden, norm_weight, eps, w, out, act_dtype, rows=None):
-        n = hidden.shape[0] if rows is None else rows.shape[0]
-        x = torch.empty(n, hidden.shape[1], dtype=act_dtype)
-        self.rmsnorm(hidden, norm_weight, eps, x, rows=rows)
-        self.gemm_swiglu(x, w, out)
-
     def swiglu(self, gate_up, out):
         self.calls.append("swiglu")
         width = out.shape[1]

@@ -121,6 +121,51 @@ def test_first_tokens_of_a_sequence(model_dirs, name, dtype):
         check(f"one by one {length}", schedules.tail_one_by_one(engine, [tokens], tail=length), [want], TOLERANCE[dtype])
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replays_equal_eager_steps(model_dirs, dtype):
+    """Decode steps replayed from captured HIP graphs against the same steps launched one kernel at
+    a time: every replay is checked, with other work (a prefill of another request, a sampling
+    kernel, synchronisations) between the replays, across a page boundary, across a change of the
+    batch and across the page-table bucket (1,024 tokens) that makes a new graph."""
+    from beholdd.engine import Engine, StepEntry
+    folder = model_dirs("D", "bfloat16")
+    graphed = Engine(folder, dtype=dtype, max_tokens=4096)
+    eager = Engine(folder, dtype=dtype, max_tokens=4096, use_graphs=False)
+    assert graphed.graphs is not None and eager.graphs is None and graphed.model.graph_safe
+    requests = schedules.random_requests(1500, [1000, 40, 1075], seed=17)
+    prompts = [990, 30, 1]
+    worst = 0.0
+    for engine in (graphed, eager):
+        engine.slots = [engine.alloc_slot() for _ in requests]
+        engine.step([StepEntry(s, r[:p], []) for s, r, p in zip(engine.slots, requests, prompts)])
+    done = list(prompts)
+    live = [0, 1, 2]
+    for step in range(40):
+        if step == 12:
+            live = [0, 2]             # the batch shrinks: another graph
+        outs = []
+        for engine in (graphed, eager):
+            logits = engine.step([StepEntry(engine.slots[i], [requests[i][done[i]]], [0]) for i in live])
+            outs.append(logits.float().cpu().numpy())
+            if step % 5 == 0:         # other work between replays
+                extra = engine.alloc_slot()
+                engine.step([StepEntry(extra, requests[1][:33], [32])])
+                engine.select(logits, [__import__("beholdd").SamplingParams()] * len(live), live, [step] * len(live))
+                engine.free_slot(extra)
+                torch.cuda.synchronize()
+        for i in live:
+            done[i] += 1
+        if dtype == "float32":
+            assert np.array_equal(outs[0], outs[1]), step
+        else:
+            worst = max(worst, schedules.relative_error(outs[0], outs[1]))
+    assert worst < 5e-3, worst
+    assert len(graphed.graphs.graphs) >= 3        # (3, 16 pages), (2, 16 pages), (2, 32 pages)
+    cfg, weights = plain.load_plain(folder)
+    final = plain.forward_logits(cfg, weights, requests[0][:done[0]])[-1]
+    assert schedules.relative_error(outs[0][0], final) < TOLERANCE[dtype]
+
+
 def test_greedy_generation_through_the_entry_point(model_dirs):
     """BASELINE's tiny configuration A: prompts of 5, 11 and 17 tokens, 8 greedy tokens each."""
     import beholdd

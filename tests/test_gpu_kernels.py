@@ -133,42 +133,6 @@ def test_gemm_swiglu(K, dtype, packed, m, width, k):
     assert rel(out, want) < tol(dtype, 1e-5, 6e-3), rel(out, want)
 
 
-@pytest.mark.parametrize("w_dtype", DTYPES)
-@pytest.mark.parametrize("packed", [False, True])
-@pytest.mark.parametrize("m,n,k,gather", [(1, 96, 128, False), (8, 331, 192, True), (64, 130, 64, False),
-                                          (65, 256, 1024, True), (200, 64, 448, False), (16, 1000, 4096, True),
-                                          (300, 100, 128, True), (5, 40, 72, False), (8, 6144, 4096, False)])
-def test_gemm_with_fused_rmsnorm(K, w_dtype, packed, m, n, k, gather):
-    """rmsnorm(hidden[rows]) @ W^T with the norm inside the product (bfloat16 weights) or before it."""
-    g = torch.Generator().manual_seed(m + n + k)
-    total_rows = m + 7 if gather else m
-    hidden = torch.randn(total_rows, k, generator=g) * 2 + 0.3
-    rows = torch.randperm(total_rows, generator=g)[:m].to(torch.int32) if gather else None
-    norm_w = (1 + 0.2 * torch.randn(k, generator=g)).to(w_dtype)
-    w = (torch.randn(n, k, generator=g) * 0.05).to(w_dtype)
-    eps = 1e-5
-    src = hidden[rows.long()] if gather else hidden
-    x = src.double() / torch.sqrt((src.double() ** 2).mean(-1, keepdim=True) + eps) * norm_w.double()
-    want = x @ w.double().t()
-    weight = K.pack_weight(dev(w)) if packed else dev(w)
-    act = torch.bfloat16 if w_dtype == torch.bfloat16 else torch.float32
-    bound = tol(act, 4 * math.sqrt(k) * 2.0 ** -24, 6e-3)
-    for out_dtype in (torch.float32, act):
-        out = torch.empty(m, n, dtype=out_dtype, device="cuda:0")
-        K.gemm_normed(dev(hidden), dev(norm_w), eps, weight, out, act, rows=None if rows is None else dev(rows))
-        assert rel(out, want) < bound, (out_dtype, rel(out, want))
-    base = torch.randn(m, n, generator=g)
-    acc = dev(base.clone())
-    K.gemm_normed(dev(hidden), dev(norm_w), eps, weight, acc, act, rows=None if rows is None else dev(rows), accumulate=True)
-    assert rel(acc, want + base.double()) < bound
-    if n % 2 == 0:
-        half = n // 2
-        gate, up = want[:, :half], want[:, half:]
-        out = torch.empty(m, half, dtype=act, device="cuda:0")
-        K.gemm_swiglu_normed(dev(hidden), dev(norm_w), eps, weight, out, act, rows=None if rows is None else dev(rows))
-        assert rel(out, gate / (1 + torch.exp(-gate)) * up) < tol(act, 1e-5, 8e-3)
-
-
 def make_cache(n_seqs, lengths, kv_heads, head_dim, dtype, seed, extra_pages=3):
     """Random keys/values for sequences of the given lengths, scattered over shuffled pages.
     Returns (k_pages, v_pages, page_table, dense keys list, dense values list)."""
