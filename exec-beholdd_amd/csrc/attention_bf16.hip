@@ -14,7 +14,9 @@
 // holds keys 16g .. 16g+15, which is exactly the k-slice its P^T operand needs.
 // The waves' results are merged through LDS.  When the keys of a sequence are split over several
 // workgroups (decode: few columns, long caches) each writes an unnormalised partial result and
-// its (maximum, sum) to scratch memory, and the workgroup that finishes last combines them.
+// its (maximum, sum) to scratch memory and a second kernel combines them.  (Letting the last
+// workgroup combine, behind a device-wide fence and an arrival counter, was measured: the fences
+// write back the L2 of every workgroup's XCD and cost several times what the second launch costs.)
 //
 // head_dim must be a multiple of 32, at most 256.  Masking is by position: column j sees keys
 // lo_j .. pos_j.  Rows of a page beyond the last written key are never multiplied in: their
@@ -62,8 +64,7 @@ __device__ inline u32x4_t keep_first(u32x4_t v, int n_valid) {
 template <int NS>
 __global__ __launch_bounds__(256) void attention_mfma_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ out, float* __restrict__ part_o,
-    float* __restrict__ part_ml, int32_t* __restrict__ counters, const uint16_t* __restrict__ k_pages,
-    const uint16_t* __restrict__ v_pages,
+    float* __restrict__ part_ml, const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages,
     const int32_t* __restrict__ page_table, int table_stride, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ seq_start, int H, int KVH, float scale_log2, int window, int n_splits,
     int pages_per_split) {
@@ -72,7 +73,6 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
   __shared__ float sm_m[4][16];
   __shared__ float sm_l[4][16];
   __shared__ float sm_o[4][16][HD + 1];
-  __shared__ int is_last;
 
   const int tile = blockIdx.x, kvh = blockIdx.y;
   const int seq = blockIdx.z / n_splits, split = blockIdx.z % n_splits;
@@ -221,36 +221,20 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
       }
     }
   }
-  if (n_splits == 1) return;
+}
 
-  // The workgroup that finishes last among the splits of these 16 columns combines them.  Each
-  // workgroup publishes its partial results (fence), then counts itself; the one that counts
-  // n_splits - 1 others before it knows that all partial results are published.
-  __threadfence();
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int32_t* counter = counters + ((size_t)seq * KVH + kvh) * gridDim.x + tile;
-    const int before = atomicAdd(counter, 1);
-    is_last = (before == n_splits - 1);
-    if (is_last) *counter = 0;  // every split has counted: leave the counter ready for the next launch
-  }
-  __syncthreads();
-  if (!is_last) return;
-  __threadfence();
-  for (int e = threadIdx.x; e < 16 * HD; e += 256) {
-    const int col = e / HD, d = e % HD;
-    const int cc = tile * 16 + col;
-    if (cc >= n_cols) continue;
-    const size_t column = (size_t)(row0 + cc / G) * H + kvh * G + cc % G;
-    const float* ml = part_ml + column * n_splits * 2;
-    float top = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) top = fmaxf(top, ml[2 * s]);
-    float sum = 0.f, value = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-      const float f = exp2f(ml[2 * s] - top);
-      sum += ml[2 * s + 1] * f;
-      value += part_o[(column * n_splits + s) * HD + d] * f;
-    }
+__global__ void attention_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                         uint16_t* __restrict__ out, int n_splits, int HD) {
+  const size_t column = blockIdx.x;
+  const float* ml = part_ml + column * n_splits * 2;
+  float top = -INFINITY;
+  for (int s = 0; s < n_splits; ++s) top = fmaxf(top, ml[2 * s]);
+  float sum = 0.f;
+  for (int s = 0; s < n_splits; ++s) sum += ml[2 * s + 1] * exp2f(ml[2 * s] - top);
+  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+    float value = 0.f;
+    for (int s = 0; s < n_splits; ++s)
+      value += part_o[(column * n_splits + s) * HD + d] * exp2f(ml[2 * s] - top);
     out[column * HD + d] = f32_to_bf16_bits(value / sum);
   }
 }
@@ -270,12 +254,8 @@ extern "C" int bh_attention_bf16_splits(int n_seqs, int max_rows_per_seq, int H,
   return (pages + per - 1) / per;
 }
 
-// With n_splits > 1: part_o (float32 [rows * H * n_splits * hd]) and part_ml ([rows * H * n_splits * 2])
-// take the partial results, and `counters` (int32, at least n_seqs * KVH * tiles entries, all zero
-// before the first launch; every launch leaves them zero) tells the last workgroup of each tile that it
-// is the last.  Launches that share `counters` must not overlap.
-extern "C" int bh_attention_bf16(const void* q, void* out, void* part_o, void* part_ml, int32_t* counters,
-                                 int n_counters, const void* k_pages, const void* v_pages, const int32_t* page_table, int table_stride,
+extern "C" int bh_attention_bf16(const void* q, void* out, void* part_o, void* part_ml, const void* k_pages,
+                                 const void* v_pages, const int32_t* page_table, int table_stride,
                                  const int32_t* positions, const int32_t* seq_start, int n_seqs, int n_rows,
                                  int max_rows_per_seq, int H, int KVH, int hd, float scale, int window,
                                  int max_position, int n_splits, hipStream_t stream) {
@@ -283,12 +263,9 @@ extern "C" int bh_attention_bf16(const void* q, void* out, void* part_o, void* p
   BH_REQUIRE(H > 0 && KVH > 0 && H % KVH == 0, "attention_bf16: %d query heads do not group evenly into %d kv heads", H, KVH);
   BH_REQUIRE(hd % 32 == 0 && hd >= 32 && hd <= 256, "attention_bf16: head size %d is not a multiple of 32 up to 256", hd);
   BH_REQUIRE(window >= 0 && max_position >= 0, "attention_bf16: window and positions must not be negative");
-  BH_REQUIRE(n_splits >= 1 && (n_splits == 1 || (part_o && part_ml && counters)),
-             "attention_bf16: split keys need scratch memory and counters");
+  BH_REQUIRE(n_splits >= 1 && (n_splits == 1 || (part_o && part_ml)), "attention_bf16: split keys need scratch memory");
   const int G = H / KVH;
   const int tiles = (max_rows_per_seq * G + 15) / 16;
-  BH_REQUIRE(n_splits == 1 || (long)n_seqs * KVH * tiles <= n_counters,
-             "attention_bf16: %ld counters are needed, %d are given", (long)n_seqs * KVH * tiles, n_counters);
   const int pages = max_position / BH_PAGE + 1;
   const int per = (pages + n_splits - 1) / n_splits;
   BH_REQUIRE((long)n_seqs * n_splits <= 65535 && KVH <= 65535, "attention_bf16: too many sequences x splits");
@@ -296,7 +273,7 @@ extern "C" int bh_attention_bf16(const void* q, void* out, void* part_o, void* p
   const float scale_log2 = scale * 1.4426950408889634f;
 #define BH_ATT(NS)                                                                                              \
   attention_mfma_kernel<NS><<<grid, block, 0, stream>>>(                                                        \
-      (const uint16_t*)q, (uint16_t*)out, (float*)part_o, (float*)part_ml, counters, (const uint16_t*)k_pages,  \
+      (const uint16_t*)q, (uint16_t*)out, (float*)part_o, (float*)part_ml, (const uint16_t*)k_pages,            \
       (const uint16_t*)v_pages, page_table, table_stride, positions, seq_start, H, KVH, scale_log2, window,     \
       n_splits, per)
   switch (hd / 32) {
@@ -310,5 +287,11 @@ extern "C" int bh_attention_bf16(const void* q, void* out, void* part_o, void* p
     default: BH_ATT(8); break;
   }
 #undef BH_ATT
-  return bh_check_launch("attention_mfma");
+  if (int status = bh_check_launch("attention_mfma")) return status;
+  if (n_splits > 1) {
+    attention_combine_kernel<<<dim3(n_rows * H), dim3(hd >= 128 ? 128 : 64), 0, stream>>>(
+        (const float*)part_o, (const float*)part_ml, (uint16_t*)out, n_splits, hd);
+    return bh_check_launch("attention_combine");
+  }
+  return 0;
 }

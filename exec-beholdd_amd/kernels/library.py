@@ -60,8 +60,6 @@ class HipKernels:
             raise KernelError(f"cannot load the HIP kernel library {path}: {error}") from None
         self.library_path = path
         self._declare()
-        # per-tile arrival counters of the key-split attention: zero between launches
-        self._attention_counters = torch.zeros(1 << 16, dtype=torch.int32, device=self.device)
         self.page_size = int(self.lib.bh_page_size())
 
     # ---- ctypes declarations ----
@@ -86,7 +84,7 @@ class HipKernels:
         self._optional = {}
         for name, argtypes in {
             "bh_gemm_bf16": [p, p, p, i, i, i, i, i, i, i, p],
-            "bh_attention_bf16": [p, p, p, p, p, i, p, p, p, i, p, p, i, i, i, i, i, i, f, i, i, i, p],
+            "bh_attention_bf16": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, i, i, f, i, i, i, p],
             "bh_attention_bf16_splits": [i, i, i, i, i],
         }.items():
             function = getattr(lib, name, None)
@@ -279,9 +277,7 @@ class HipKernels:
                 part_o = torch.empty(n_rows * n_heads * n_splits * head_dim, dtype=torch.float32, device=self.device)
                 part_ml = torch.empty(n_rows * n_heads * n_splits * 2, dtype=torch.float32, device=self.device)
             self._check(fast(*common, self._ptr(part_o, "partial o", None, True),
-                             self._ptr(part_ml, "partial sums", None, True),
-                             self._ptr(self._attention_counters, "counters"), self._attention_counters.numel(),
-                             self._ptr(k_pages, "k_pages"),
+                             self._ptr(part_ml, "partial sums", None, True), self._ptr(k_pages, "k_pages"),
                              self._ptr(v_pages, "v_pages"), self._ptr(page_table, "page_table", (torch.int32,)),
                              page_table.shape[1], self._ptr(positions, "positions", (torch.int32,)),
                              self._ptr(layout.seq_start, "seq_start", (torch.int32,)), n_seqs, n_rows, max_rows,
