@@ -9,9 +9,11 @@
 //     running maximum / sum per column in float32 (online softmax, exponent base 2)
 //     O^T[d, column] += V^T[d, key] . P^T[key, column]   (the cache keeps V transposed inside a
 //                                                          page, so this operand is a straight load too)
-// The rows of an S^T tile are assigned to keys so that every lane ends up with 16 consecutive
-// keys of the page: tile t, row i <-> key 16*(i/4) + 4*t + i%4.  Lane (column j, group g) then
-// holds keys 16g .. 16g+15, which is exactly the k-slice its P^T operand needs.
+// The rows of an S^T tile are assigned to keys so that every lane ends up with the keys its P^T
+// operand needs: tile t, row i <-> key 32*(t/2) + 4*(t%2) + 8*(i/4) + i%4.  Lane (column j, group g)
+// then holds keys 8g..8g+7 (tiles 0, 1) and 32+8g..32+8g+7 (tiles 2, 3): the k-slices of the two
+// P.V products of a page, whose V^T operands are 16 contiguous bytes per lane and 64 contiguous
+// bytes per row and instruction.  The same holds for K along head_dim.
 // The waves' results are merged through LDS.  When the keys of a sequence are split over several
 // workgroups (decode: few columns, long caches) each writes an unnormalised partial result and
 // its (maximum, sum) to scratch memory and a second kernel combines them.  (Letting the last
@@ -61,7 +63,9 @@ __device__ inline u32x4_t keep_first(u32x4_t v, int n_valid) {
   return v;
 }
 
-template <int NS>
+// NS = head_dim / 32.  CT = column tiles (of 16 columns) per workgroup: every page a wave loads is
+// used for all CT tiles, which divides the cache traffic of a prefill by CT.
+template <int NS, int CT>
 __global__ __launch_bounds__(256) void attention_mfma_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages,
@@ -69,155 +73,180 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
     const int32_t* __restrict__ seq_start, int H, int KVH, float scale_log2, int window, int n_splits,
     int pages_per_split) {
   constexpr int HD = 32 * NS;
-  constexpr int LANE_D = 8 * NS;  // head_dim elements per lane group
   __shared__ float sm_m[4][16];
   __shared__ float sm_l[4][16];
   __shared__ float sm_o[4][16][HD + 1];
 
-  const int tile = blockIdx.x, kvh = blockIdx.y;
+  const int tile0 = blockIdx.x * CT, kvh = blockIdx.y;
   const int seq = blockIdx.z / n_splits, split = blockIdx.z % n_splits;
   const int G = H / KVH;
   const int row0 = seq_start[seq];
   const int n_cols = (seq_start[seq + 1] - row0) * G;
-  if (tile * 16 >= n_cols) return;
+  if (tile0 * 16 >= n_cols) return;
 
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int j = lane % 16, g = lane / 16;
-  const int c = (tile * 16 + j < n_cols) ? tile * 16 + j : n_cols - 1;
-  const int row = row0 + c / G, head = kvh * G + c % G;
-  const int pos = positions[row];
-  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int pos_max = wave_max_int(pos), pos_min = wave_min_int(pos);
-  const int lo_min = wave_min_int(lo), lo_max = wave_max_int(lo);
+  int pos[CT], lo[CT];
+  bf16x8_t q_vec[CT][NS];
+  int pos_max = 0, pos_min = 0x7fffffff, lo_min = 0x7fffffff, lo_max = 0;
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int wanted = (tile0 + ct) * 16 + j;
+    const int c = wanted < n_cols ? wanted : n_cols - 1;
+    const int row = row0 + c / G, head = kvh * G + c % G;
+    pos[ct] = positions[row];
+    lo[ct] = (window > 0 && pos[ct] - window + 1 > 0) ? pos[ct] - window + 1 : 0;
+    pos_max = max(pos_max, pos[ct]);
+    pos_min = min(pos_min, pos[ct]);
+    lo_min = min(lo_min, lo[ct]);
+    lo_max = max(lo_max, lo[ct]);
+    const uint16_t* qp = q + ((size_t)row * H + head) * HD + 8 * g;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) q_vec[ct][s] = as_bf16x8(load16(qp + 32 * s));
+  }
+  pos_max = wave_max_int(pos_max);
+  pos_min = wave_min_int(pos_min);
+  lo_min = wave_min_int(lo_min);
+  lo_max = wave_max_int(lo_max);
 
   const int begin = lo_min / BH_PAGE + split * pages_per_split;
   const int last = pos_max / BH_PAGE;
   const int end = (begin + pages_per_split < last + 1) ? begin + pages_per_split : last + 1;
   const int32_t* table = page_table + (size_t)seq * table_stride;
 
-  bf16x8_t q_vec[NS];
-  {
-    const uint16_t* qp = q + ((size_t)row * H + head) * HD + g * LANE_D;
+  f32x4_t o[CT][2 * NS];
+  float run_max[CT], run_sum[CT];  // run_sum: this lane's share of the column's sum
 #pragma unroll
-    for (int s = 0; s < NS; ++s) q_vec[s] = as_bf16x8(load16(qp + 8 * s));
+  for (int ct = 0; ct < CT; ++ct) {
+    run_max[ct] = -INFINITY;
+    run_sum[ct] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < 2 * NS; ++dt) o[ct][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
-  f32x4_t o[2 * NS];
-#pragma unroll
-  for (int dt = 0; dt < 2 * NS; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  float run_max = -INFINITY, run_sum = 0.f;  // run_sum: this lane's share of the column's sum
 
   for (int p = begin + wave; p < end; p += 4) {
     const int page = table[p];
     const uint16_t* kb = k_pages + ((size_t)page * KVH + kvh) * BH_PAGE * HD;
     const uint16_t* vb = v_pages + ((size_t)page * KVH + kvh) * HD * BH_PAGE;
     u32x4_t k_vec[4][NS], v_vec[2 * NS][2];
+    // every load instruction covers 64 contiguous bytes of each of its 16 rows (lane group g the g-th 16)
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      const uint16_t* kr = kb + (size_t)(16 * (j / 4) + 4 * t + j % 4) * HD + g * LANE_D;
+      const uint16_t* kr = kb + (size_t)(32 * (t / 2) + 4 * (t % 2) + 8 * (j / 4) + j % 4) * HD + 8 * g;
 #pragma unroll
-      for (int s = 0; s < NS; ++s) k_vec[t][s] = load16(kr + 8 * s);
+      for (int s = 0; s < NS; ++s) k_vec[t][s] = load16(kr + 32 * s);
     }
 #pragma unroll
     for (int dt = 0; dt < 2 * NS; ++dt) {
-      const uint16_t* vr = vb + (size_t)(16 * dt + j) * BH_PAGE + 16 * g;
+      const uint16_t* vr = vb + (size_t)(16 * dt + j) * BH_PAGE + 8 * g;
       v_vec[dt][0] = load16(vr);
-      v_vec[dt][1] = load16(vr + 8);
+      v_vec[dt][1] = load16(vr + 32);
     }
-    f32x4_t st[4];
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int s = 0; s < NS; ++s)
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(k_vec[t][s]), q_vec[s], acc, 0, 0, 0);
-      st[t] = acc;
-    }
-    // lane (j, g) now holds keys key0 + 4t + r of its column, for t, r in 0..3
-    const int key0 = p * BH_PAGE + 16 * g;
+    const int key0 = p * BH_PAGE + 8 * g;  // lane (j, g) holds keys key0 + 32 * (t / 2) + 4 * (t % 2) + r
     const bool mask_needed = (p * BH_PAGE + BH_PAGE - 1 > pos_min) || (p * BH_PAGE < lo_max);
-    float local_max = -INFINITY;
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+    for (int ct = 0; ct < CT; ++ct) {
+      if (CT > 1 && (tile0 + ct) * 16 >= n_cols) continue;  // a tile beyond the sequence's columns
+      f32x4_t st[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float v = st[t][r] * scale_log2;
-        if (mask_needed) {
-          const int key = key0 + 4 * t + r;
-          if (key > pos || key < lo) v = -INFINITY;
+      for (int t = 0; t < 4; ++t) {
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(k_vec[t][s]), q_vec[ct][s], acc, 0, 0, 0);
+        st[t] = acc;
+      }
+      float local_max = -INFINITY;
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float v = st[t][r] * scale_log2;
+          if (mask_needed) {
+            const int key = key0 + 32 * (t / 2) + 4 * (t % 2) + r;
+            if (key > pos[ct] || key < lo[ct]) v = -INFINITY;
+          }
+          st[t][r] = v;
+          local_max = fmaxf(local_max, v);
         }
-        st[t][r] = v;
-        local_max = fmaxf(local_max, v);
-      }
-    local_max = fmaxf(local_max, __shfl_xor(local_max, 16, 64));
-    local_max = fmaxf(local_max, __shfl_xor(local_max, 32, 64));
-    const float new_max = fmaxf(run_max, local_max);
-    const float safe_max = (new_max == -INFINITY) ? 0.f : new_max;
-    const float alpha = exp2f(run_max - safe_max);  // 0 when nothing was seen before
-    float page_sum = 0.f;
-    u32x4_t p_vec[2];
+      local_max = fmaxf(local_max, __shfl_xor(local_max, 16, 64));
+      local_max = fmaxf(local_max, __shfl_xor(local_max, 32, 64));
+      const float new_max = fmaxf(run_max[ct], local_max);
+      const float safe_max = (new_max == -INFINITY) ? 0.f : new_max;
+      const float alpha = exp2f(run_max[ct] - safe_max);  // 0 when nothing was seen before
+      float page_sum = 0.f;
+      u32x4_t p_vec[2];
 #pragma unroll
-    for (int u = 0; u < 2; ++u)
+      for (int u = 0; u < 2; ++u)
 #pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        const int t = 2 * u + half;
-        const float e0 = exp2f(st[t][0] - safe_max), e1 = exp2f(st[t][1] - safe_max);
-        const float e2 = exp2f(st[t][2] - safe_max), e3 = exp2f(st[t][3] - safe_max);
-        page_sum += (e0 + e1) + (e2 + e3);
-        p_vec[u][2 * half] = pack_bf16(e0, e1);
-        p_vec[u][2 * half + 1] = pack_bf16(e2, e3);
+        for (int half = 0; half < 2; ++half) {
+          const int t = 2 * u + half;
+          const float e0 = exp2f(st[t][0] - safe_max), e1 = exp2f(st[t][1] - safe_max);
+          const float e2 = exp2f(st[t][2] - safe_max), e3 = exp2f(st[t][3] - safe_max);
+          page_sum += (e0 + e1) + (e2 + e3);
+          p_vec[u][2 * half] = pack_bf16(e0, e1);
+          p_vec[u][2 * half + 1] = pack_bf16(e2, e3);
+        }
+      run_sum[ct] = run_sum[ct] * alpha + page_sum;
+      run_max[ct] = new_max;
+      if (ct == 0 && p * BH_PAGE + BH_PAGE - 1 > pos_max) {  // the page's tail was never written: zero it
+        const int valid = pos_max + 1 - key0;
+#pragma unroll
+        for (int dt = 0; dt < 2 * NS; ++dt) {
+          v_vec[dt][0] = keep_first(v_vec[dt][0], valid);
+          v_vec[dt][1] = keep_first(v_vec[dt][1], valid - 32);
+        }
       }
-    run_sum = run_sum * alpha + page_sum;
-    run_max = new_max;
-    if (p * BH_PAGE + BH_PAGE - 1 > pos_max) {  // the page's tail was never written for this step: zero it
-      const int valid = pos_max + 1 - key0;
 #pragma unroll
       for (int dt = 0; dt < 2 * NS; ++dt) {
-        v_vec[dt][0] = keep_first(v_vec[dt][0], valid);
-        v_vec[dt][1] = keep_first(v_vec[dt][1], valid - 8);
+        f32x4_t acc = o[ct][dt] * alpha;
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(v_vec[dt][0]), as_bf16x8(p_vec[0]), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(v_vec[dt][1]), as_bf16x8(p_vec[1]), acc, 0, 0, 0);
+        o[ct][dt] = acc;
       }
-    }
-#pragma unroll
-    for (int dt = 0; dt < 2 * NS; ++dt) {
-      f32x4_t acc = o[dt] * alpha;
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(v_vec[dt][0]), as_bf16x8(p_vec[0]), acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(v_vec[dt][1]), as_bf16x8(p_vec[1]), acc, 0, 0, 0);
-      o[dt] = acc;
     }
   }
 
-  // merge the four waves: lane (j, g) holds O^T[16dt + 4g + r, j]
-  run_sum += __shfl_xor(run_sum, 16, 64);
-  run_sum += __shfl_xor(run_sum, 32, 64);
-  if (g == 0) {
-    sm_m[wave][j] = run_max;
-    sm_l[wave][j] = run_sum;
-  }
+  // merge the four waves, one column tile after the other: lane (j, g) holds O^T[16dt + 4g + r, j]
 #pragma unroll
-  for (int dt = 0; dt < 2 * NS; ++dt)
-#pragma unroll
-    for (int r = 0; r < 4; ++r) sm_o[wave][j][16 * dt + 4 * g + r] = o[dt][r];
-  __syncthreads();
-  for (int e = threadIdx.x; e < 16 * HD; e += 256) {
-    const int col = e / HD, d = e % HD;
-    const int cc = tile * 16 + col;
-    if (cc >= n_cols) continue;
-    float top = fmaxf(fmaxf(sm_m[0][col], sm_m[1][col]), fmaxf(sm_m[2][col], sm_m[3][col]));
-    const float safe_top = (top == -INFINITY) ? 0.f : top;
-    float sum = 0.f, value = 0.f;
-#pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      const float f = exp2f(sm_m[v][col] - safe_top);
-      sum += sm_l[v][col] * f;
-      value += sm_o[v][col][d] * f;
+  for (int ct = 0; ct < CT; ++ct) {
+    const int tile = tile0 + ct;
+    if (tile * 16 >= n_cols) break;
+    float lane_sum = run_sum[ct];
+    lane_sum += __shfl_xor(lane_sum, 16, 64);
+    lane_sum += __shfl_xor(lane_sum, 32, 64);
+    if (ct > 0) __syncthreads();  // the previous tile's merge has read the buffers
+    if (g == 0) {
+      sm_m[wave][j] = run_max[ct];
+      sm_l[wave][j] = lane_sum;
     }
-    const size_t column = (size_t)(row0 + cc / G) * H + kvh * G + cc % G;
-    if (n_splits == 1) {
-      out[column * HD + d] = f32_to_bf16_bits(value / sum);
-    } else {
-      part_o[(column * n_splits + split) * HD + d] = value;
-      if (d == 0) {
-        part_ml[(column * n_splits + split) * 2] = top;
-        part_ml[(column * n_splits + split) * 2 + 1] = sum;
+#pragma unroll
+    for (int dt = 0; dt < 2 * NS; ++dt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) sm_o[wave][j][16 * dt + 4 * g + r] = o[ct][dt][r];
+    __syncthreads();
+    for (int e = threadIdx.x; e < 16 * HD; e += 256) {
+      const int col = e / HD, d = e % HD;
+      const int cc = tile * 16 + col;
+      if (cc >= n_cols) continue;
+      float top = fmaxf(fmaxf(sm_m[0][col], sm_m[1][col]), fmaxf(sm_m[2][col], sm_m[3][col]));
+      const float safe_top = (top == -INFINITY) ? 0.f : top;
+      float sum = 0.f, value = 0.f;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const float f = exp2f(sm_m[v][col] - safe_top);
+        sum += sm_l[v][col] * f;
+        value += sm_o[v][col][d] * f;
+      }
+      const size_t column = (size_t)(row0 + cc / G) * H + kvh * G + cc % G;
+      if (n_splits == 1) {
+        out[column * HD + d] = f32_to_bf16_bits(value / sum);
+      } else {
+        part_o[(column * n_splits + split) * HD + d] = value;
+        if (d == 0) {
+          part_ml[(column * n_splits + split) * 2] = top;
+          part_ml[(column * n_splits + split) * 2 + 1] = sum;
+        }
       }
     }
   }
@@ -268,14 +297,23 @@ extern "C" int bh_attention_bf16(const void* q, void* out, void* part_o, void* p
   const int tiles = (max_rows_per_seq * G + 15) / 16;
   const int pages = max_position / BH_PAGE + 1;
   const int per = (pages + n_splits - 1) / n_splits;
+  // several column tiles per workgroup when there are many (prefill): the cache is read that many times less
+  const int ct = (n_splits == 1 && hd <= 128 && (long)tiles * KVH * n_seqs >= 2048) ? 4
+               : (n_splits == 1 && (long)tiles * KVH * n_seqs >= 1024) ? 2 : 1;
   BH_REQUIRE((long)n_seqs * n_splits <= 65535 && KVH <= 65535, "attention_bf16: too many sequences x splits");
-  dim3 grid(tiles, KVH, n_seqs * n_splits), block(256);
+  dim3 grid((tiles + ct - 1) / ct, KVH, n_seqs * n_splits), block(256);
   const float scale_log2 = scale * 1.4426950408889634f;
-#define BH_ATT(NS)                                                                                              \
-  attention_mfma_kernel<NS><<<grid, block, 0, stream>>>(                                                        \
+#define BH_ATT_CT(NS, CT)                                                                                       \
+  attention_mfma_kernel<NS, CT><<<grid, block, 0, stream>>>(                                                    \
       (const uint16_t*)q, (uint16_t*)out, (float*)part_o, (float*)part_ml, (const uint16_t*)k_pages,            \
       (const uint16_t*)v_pages, page_table, table_stride, positions, seq_start, H, KVH, scale_log2, window,     \
       n_splits, per)
+#define BH_ATT(NS)                        \
+  do {                                    \
+    if (ct == 4) BH_ATT_CT(NS, 4);        \
+    else if (ct == 2) BH_ATT_CT(NS, 2);   \
+    else BH_ATT_CT(NS, 1);                \
+  } while (0)
   switch (hd / 32) {
     case 1: BH_ATT(1); break;
     case 2: BH_ATT(2); break;
@@ -287,6 +325,7 @@ extern "C" int bh_attention_bf16(const void* q, void* out, void* part_o, void* p
     default: BH_ATT(8); break;
   }
 #undef BH_ATT
+#undef BH_ATT_CT
   if (int status = bh_check_launch("attention_mfma")) return status;
   if (n_splits > 1) {
     attention_combine_kernel<<<dim3(n_rows * H), dim3(hd >= 128 ? 128 : 64), 0, stream>>>(
