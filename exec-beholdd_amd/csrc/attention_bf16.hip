@@ -156,24 +156,28 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
           acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(k_vec[t][s]), q_vec[ct][s], acc, 0, 0, 0);
         st[t] = acc;
       }
-      float local_max = -INFINITY;
+      // Online softmax with few instructions: the maximum is taken over the raw scores, the scale
+      // enters through one fused multiply-add per score, and the exponentials are bare v_exp_f32
+      // (arguments <= 0; results below the normal range may flush to zero).
+      if (mask_needed) {
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
+        for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float v = st[t][r] * scale_log2;
-          if (mask_needed) {
+          for (int r = 0; r < 4; ++r) {
             const int key = key0 + 32 * (t / 2) + 4 * (t % 2) + r;
-            if (key > pos[ct] || key < lo[ct]) v = -INFINITY;
+            if (key > pos[ct] || key < lo[ct]) st[t][r] = -INFINITY;
           }
-          st[t][r] = v;
-          local_max = fmaxf(local_max, v);
-        }
+      }
+      float local_max = fmaxf(fmaxf(st[0][0], st[0][1]), fmaxf(st[0][2], st[0][3]));
+#pragma unroll
+      for (int t = 1; t < 4; ++t)
+        local_max = fmaxf(local_max, fmaxf(fmaxf(st[t][0], st[t][1]), fmaxf(st[t][2], st[t][3])));
       local_max = fmaxf(local_max, __shfl_xor(local_max, 16, 64));
       local_max = fmaxf(local_max, __shfl_xor(local_max, 32, 64));
-      const float new_max = fmaxf(run_max[ct], local_max);
-      const float safe_max = (new_max == -INFINITY) ? 0.f : new_max;
-      const float alpha = exp2f(run_max[ct] - safe_max);  // 0 when nothing was seen before
+      const float new_max = fmaxf(run_max[ct], local_max);              // raw (unscaled) scores
+      const float shift = (new_max == -INFINITY) ? 0.f : -new_max * scale_log2;
+      // exactly 1 while the maximum stands still, 0 when nothing was seen before
+      const float alpha = (run_max[ct] == new_max) ? 1.0f : __builtin_amdgcn_exp2f((run_max[ct] - new_max) * scale_log2);
       float page_sum = 0.f;
       u32x4_t p_vec[2];
 #pragma unroll
@@ -181,14 +185,17 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
           const int t = 2 * u + half;
-          const float e0 = exp2f(st[t][0] - safe_max), e1 = exp2f(st[t][1] - safe_max);
-          const float e2 = exp2f(st[t][2] - safe_max), e3 = exp2f(st[t][3] - safe_max);
+          const float e0 = __builtin_amdgcn_exp2f(fmaf(st[t][0], scale_log2, shift));
+          const float e1 = __builtin_amdgcn_exp2f(fmaf(st[t][1], scale_log2, shift));
+          const float e2 = __builtin_amdgcn_exp2f(fmaf(st[t][2], scale_log2, shift));
+          const float e3 = __builtin_amdgcn_exp2f(fmaf(st[t][3], scale_log2, shift));
           page_sum += (e0 + e1) + (e2 + e3);
           p_vec[u][2 * half] = pack_bf16(e0, e1);
           p_vec[u][2 * half + 1] = pack_bf16(e2, e3);
         }
       run_sum[ct] = run_sum[ct] * alpha + page_sum;
       run_max[ct] = new_max;
+      const bool rescale = __any(alpha != 1.0f);   // after the first pages the maximum seldom moves
       if (ct == 0 && p * BH_PAGE + BH_PAGE - 1 > pos_max) {  // the page's tail was never written: zero it
         const int valid = pos_max + 1 - key0;
 #pragma unroll
@@ -197,9 +204,13 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
           v_vec[dt][1] = keep_first(v_vec[dt][1], valid - 32);
         }
       }
+      if (rescale) {
+#pragma unroll
+        for (int dt = 0; dt < 2 * NS; ++dt) o[ct][dt] = o[ct][dt] * alpha;
+      }
 #pragma unroll
       for (int dt = 0; dt < 2 * NS; ++dt) {
-        f32x4_t acc = o[ct][dt] * alpha;
+        f32x4_t acc = o[ct][dt];
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(v_vec[dt][0]), as_bf16x8(p_vec[0]), acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(v_vec[dt][1]), as_bf16x8(p_vec[1]), acc, 0, 0, 0);
         o[ct][dt] = acc;
@@ -217,7 +228,7 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
     lane_sum += __shfl_xor(lane_sum, 32, 64);
     if (ct > 0) __syncthreads();  // the previous tile's merge has read the buffers
     if (g == 0) {
-      sm_m[wave][j] = run_max[ct];
+      sm_m[wave][j] = run_max[ct] * scale_log2;   // in units of the base-2 exponent, as the merges use it
       sm_l[wave][j] = lane_sum;
     }
 #pragma unroll

@@ -16,8 +16,8 @@
 //     v_mfma_f32_16x16x32_bf16 with W as the row operand and the activations as the column
 //     operand; the waves' partial tiles are summed through LDS in a fixed order.
 //   tiled (M > 64, the prefill shapes): 128x128 output tile per workgroup of four waves, 64-wide
-//     k slices staged through padded LDS with the next slice's global loads in flight during
-//     the multiplies; v_mfma_f32_32x32x16_bf16, each wave a 64x64 quarter.  For SwiGLU a wave's
+//     k slices staged through padded LDS (one or two buffers) with the next slice's global loads in
+//     flight during the multiplies; v_mfma_f32_32x32x16_bf16, each wave a 64x64 quarter.  For SwiGLU a wave's
 //     two 32-column halves are the gate and the up columns of the same 32 outputs.
 // K must be a multiple of 8 (16-byte loads); other sizes are free.
 //
@@ -180,22 +180,28 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
 
 // ---- tiled -----------------------------------------------------------------------------------
 
-#define TB 128          // output tile edge
+#define TBN 128         // W rows (output columns, or gate+up rows) per tile
 #define TK 64           // k slice
 #define TPITCH (TK + 8) // LDS row pitch in elements: 144 bytes, so 16-byte reads of 16 rows hit 64 distinct banks
 
+// A workgroup of four waves (2 x 2) computes a (64 * WX) x 128 tile; a wave WX x 2 blocks of 32 x 32.
+// WX = 2 is what runs: WX = 4 (256 rows, fewer LDS reads per multiply) leaves room for one workgroup
+// per compute unit only and measured a third slower.
 // SWIGLU: the tile's 128 W rows are, per wave column half (32 outputs), 32 gate rows then the 32 up
 // rows of the same outputs; N counts outputs and the up rows start `N` rows (N/16 blocks) further on.
-template <bool TILES, bool SWIGLU, typename TC>
+template <bool TILES, bool SWIGLU, int WX, int BUFFERS, typename TC>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restrict__ a,
                                                          const uint16_t* __restrict__ w, TC* __restrict__ c,
                                                          int M, int N, int K, int accumulate) {
-  __shared__ __attribute__((aligned(16))) uint16_t as[2][TB * TPITCH];
-  __shared__ __attribute__((aligned(16))) uint16_t ws[2][TB * TPITCH];
+  constexpr int TBM = 64 * WX;
+  constexpr int A_PIECES = TBM / 32;   // 16-byte pieces of a slice that one thread stages: TBM rows x 8 / 256
+  constexpr int W_PIECES = TBN / 32;
+  __shared__ __attribute__((aligned(16))) uint16_t as[BUFFERS][TBM * TPITCH];
+  __shared__ __attribute__((aligned(16))) uint16_t ws[BUFFERS][TBN * TPITCH];
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
-  const int m0 = blockIdx.y * TB;
-  const int n0 = blockIdx.x * (SWIGLU ? TB / 2 : TB);   // first output column of the tile
-  const int wm = (wave / 2) * 64, wn = (wave % 2) * 64;  // this wave's quarter of the tile (in LDS rows)
+  const int m0 = blockIdx.y * TBM;
+  const int n0 = blockIdx.x * (SWIGLU ? TBN / 2 : TBN);      // first output column of the tile
+  const int wm = (wave / 2) * 32 * WX, wn = (wave % 2) * 64;  // this wave's part of the tile (in LDS rows)
   const int w_rows = SWIGLU ? 2 * N : N;
   const int w_blocks = (w_rows + 15) / 16;
 
@@ -206,21 +212,26 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
     return (inner < 32 ? 0 : N) + n0 + half * 32 + inner % 32;
   };
 
-  // global -> LDS staging: a slice is 128 rows x 8 pieces of 16 bytes; a thread moves 4 pieces per operand
-  int a_at[4], w_at[4], a_piece[4];
-  const uint16_t* a_src[4];
-  const uint16_t* w_src[4];
-  size_t w_step;
+  // global -> LDS staging: a slice is rows x 8 pieces of 16 bytes
+  int a_at[A_PIECES], w_at[W_PIECES], a_piece[A_PIECES], w_piece[W_PIECES];
+  const uint16_t* a_src[A_PIECES];
+  const uint16_t* w_src[W_PIECES];
 #pragma unroll
-  for (int s = 0; s < 4; ++s) {
+  for (int s = 0; s < A_PIECES; ++s) {
     const int e = tid + s * 256;
     const int row = e / 8, piece = e % 8;
     const int am = (m0 + row < M) ? m0 + row : M - 1;
     a_src[s] = a + (size_t)am * K + piece * 8;
     a_at[s] = row * TPITCH + piece * 8;
     a_piece[s] = piece;
+  }
+#pragma unroll
+  for (int s = 0; s < W_PIECES; ++s) {
+    const int e = tid + s * 256;
+    const int row = e / 8, piece = e % 8;
+    w_piece[s] = piece;
     if (TILES) {
-      // 8 blocks of 16 rows; inside a block piece p = u * 64 + l holds row l % 16, k 16 * (l / 16) + 8 * u
+      // blocks of 16 rows; inside a block piece p = u * 64 + l holds row l % 16, k 16 * (l / 16) + 8 * u
       const int block = e / 128, p = e % 128, u = p / 64, l = p % 64;
       int global_block = w_row_of(block * 16) / 16;
       if (global_block >= w_blocks) global_block = w_blocks - 1;
@@ -230,32 +241,30 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
       int wr = w_row_of(row);
       if (wr >= w_rows) wr = w_rows - 1;
       w_src[s] = w + (size_t)wr * K + piece * 8;
-      w_at[s] = a_at[s];
+      w_at[s] = row * TPITCH + piece * 8;
     }
   }
-  w_step = TILES ? 1024 : TK;
-  u32x4_t a_reg[4], w_reg[4];
+  const size_t w_step = TILES ? 1024 : TK;
+  u32x4_t a_reg[A_PIECES], w_reg[W_PIECES];
   const u32x4_t zero = {0u, 0u, 0u, 0u};
   auto fetch = [&](int slice) {
     const int k0 = slice * TK;
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      const bool inside = k0 + a_piece[s] * 8 < K;
-      a_reg[s] = inside ? load16(a_src[s] + k0) : zero;
-      w_reg[s] = (TILES || inside) ? load16(w_src[s] + (size_t)slice * w_step) : zero;
-    }
+    for (int s = 0; s < A_PIECES; ++s) a_reg[s] = (k0 + a_piece[s] * 8 < K) ? load16(a_src[s] + k0) : zero;
+#pragma unroll
+    for (int s = 0; s < W_PIECES; ++s)
+      w_reg[s] = (TILES || k0 + w_piece[s] * 8 < K) ? load16(w_src[s] + (size_t)slice * w_step) : zero;
   };
   auto stash = [&](int buffer) {
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      *reinterpret_cast<u32x4_t*>(&as[buffer][a_at[s]]) = a_reg[s];
-      *reinterpret_cast<u32x4_t*>(&ws[buffer][w_at[s]]) = w_reg[s];
-    }
+    for (int s = 0; s < A_PIECES; ++s) *reinterpret_cast<u32x4_t*>(&as[buffer][a_at[s]]) = a_reg[s];
+#pragma unroll
+    for (int s = 0; s < W_PIECES; ++s) *reinterpret_cast<u32x4_t*>(&ws[buffer][w_at[s]]) = w_reg[s];
   };
 
-  f32x16_t acc[2][2];
+  f32x16_t acc[WX][2];
 #pragma unroll
-  for (int x = 0; x < 2; ++x)
+  for (int x = 0; x < WX; ++x)
 #pragma unroll
     for (int y = 0; y < 2; ++y)
 #pragma unroll
@@ -267,29 +276,30 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
   __syncthreads();
   const int frag_row = lane % 32, frag_k = (lane / 32) * 8;
   for (int s = 0; s < slices; ++s) {
-    const int buffer = s & 1;
+    const int buffer = BUFFERS == 2 ? (s & 1) : 0;
     if (s + 1 < slices) fetch(s + 1);
 #pragma unroll
     for (int kk = 0; kk < TK; kk += 16) {
-      bf16x8_t af[2], wf[2];
+      bf16x8_t af[WX], wf[2];
 #pragma unroll
-      for (int x = 0; x < 2; ++x)
+      for (int x = 0; x < WX; ++x)
         af[x] = as_bf16x8(*reinterpret_cast<const u32x4_t*>(&as[buffer][(wm + x * 32 + frag_row) * TPITCH + kk + frag_k]));
 #pragma unroll
       for (int y = 0; y < 2; ++y)
         wf[y] = as_bf16x8(*reinterpret_cast<const u32x4_t*>(&ws[buffer][(wn + y * 32 + frag_row) * TPITCH + kk + frag_k]));
 #pragma unroll
-      for (int x = 0; x < 2; ++x)
+      for (int x = 0; x < WX; ++x)
 #pragma unroll
         for (int y = 0; y < 2; ++y)
           acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[x], wf[y], acc[x][y], 0, 0, 0);
     }
-    if (s + 1 < slices) stash(buffer ^ 1);
+    if (BUFFERS == 1) __syncthreads();   // one buffer: everyone has read the slice before it is overwritten
+    if (s + 1 < slices) stash(BUFFERS == 2 ? buffer ^ 1 : 0);
     __syncthreads();
   }
   // D of one 32x32 block: column (n) lane%32, rows (m) 8*(e/4) + 4*(lane/32) + e%4
 #pragma unroll
-  for (int x = 0; x < 2; ++x) {
+  for (int x = 0; x < WX; ++x) {
     if (SWIGLU) {
       const int n = n0 + (wave % 2) * 32 + lane % 32;
       if (n >= N) continue;
@@ -335,10 +345,17 @@ static void launch_skinny(const void* a, const void* w, void* c, int M, int N, i
 template <bool TILES, bool SWIGLU, typename TC>
 static void launch_tiled(const void* a, const void* w, void* c, int M, int N, int K, int accumulate,
                          hipStream_t stream) {
-  const int columns = SWIGLU ? TB / 2 : TB;
-  dim3 grid((N + columns - 1) / columns, (M + TB - 1) / TB), block(256);
-  gemm_tiled_kernel<TILES, SWIGLU, TC><<<grid, block, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, (TC*)c, M,
-                                                                   N, K, accumulate);
+  const int columns = SWIGLU ? TBN / 2 : TBN;
+  dim3 grid((N + columns - 1) / columns, (M + 127) / 128), block(256);
+  // Two LDS buffers let two workgroups per compute unit overlap loads and multiplies, which pays when
+  // there are several rounds of workgroups; with about one round, four smaller workgroups per compute
+  // unit (one buffer, a second barrier per slice) hide more latency.  Measured at the Qwen3-8B shapes.
+  if ((long)grid.x * grid.y >= 1024)
+    gemm_tiled_kernel<TILES, SWIGLU, 2, 2, TC><<<grid, block, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w,
+                                                                           (TC*)c, M, N, K, accumulate);
+  else
+    gemm_tiled_kernel<TILES, SWIGLU, 2, 1, TC><<<grid, block, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w,
+                                                                           (TC*)c, M, N, K, accumulate);
 }
 
 // layout: 0 = rows, 1 = tiles.  activation: 0 = none; 1 = SwiGLU (W has 2 * N rows: gate rows then up rows).
@@ -352,7 +369,7 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
   BH_REQUIRE(activation == 0 || activation == 1, "gemm_bf16: unknown activation %d", activation);
   BH_REQUIRE(activation == 0 || (N % 16 == 0 && !accumulate),
              "gemm_bf16: SwiGLU needs a multiple of 16 outputs (got %d) and no accumulation", N);
-  BH_REQUIRE((M + TB - 1) / TB <= 65535, "gemm_bf16: M=%d needs more than 65535 row tiles", M);
+  BH_REQUIRE((M + 127) / 128 <= 65535, "gemm_bf16: M=%d needs more than 65535 row tiles", M);
   const bool f32 = c_dtype == BH_F32;
 #define BH_PICK(FN, TILES, EXTRA, ...)                                             \
   do {                                                                              \
