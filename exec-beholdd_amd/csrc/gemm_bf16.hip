@@ -192,22 +192,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
 template <bool TILES, bool SWIGLU, int WX, int BUFFERS, typename TC>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restrict__ a,
                                                          const uint16_t* __restrict__ w, TC* __restrict__ c,
-                                                         int M, int N, int K, int accumulate, int m_tiles,
-                                                         int n_tiles) {
+                                                         int M, int N, int K, int accumulate) {
   constexpr int TBM = 64 * WX;
   constexpr int A_PIECES = TBM / 32;   // 16-byte pieces of a slice that one thread stages: TBM rows x 8 / 256
   constexpr int W_PIECES = TBN / 32;
   __shared__ __attribute__((aligned(16))) uint16_t as[BUFFERS][TBM * TPITCH];
   __shared__ __attribute__((aligned(16))) uint16_t ws[BUFFERS][TBN * TPITCH];
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
-  // Which tile: workgroups are handed to the 8 XCDs in turn, and each XCD has an L2 of its own, so
-  // the tiles are numbered such that one XCD gets a run of column tiles with all their row tiles one
-  // after the other: the workgroups that run together there read the same slices of W.
-  const int per_xcd = (m_tiles * n_tiles + 7) / 8;
-  const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-  if (logical >= m_tiles * n_tiles) return;
-  const int m0 = (logical % m_tiles) * TBM;
-  const int n0 = (logical / m_tiles) * (SWIGLU ? TBN / 2 : TBN);      // first output column of the tile
+  const int m0 = blockIdx.y * TBM;
+  const int n0 = blockIdx.x * (SWIGLU ? TBN / 2 : TBN);      // first output column of the tile
   const int wm = (wave / 2) * 32 * WX, wn = (wave % 2) * 64;  // this wave's part of the tile (in LDS rows)
   const int w_rows = SWIGLU ? 2 * N : N;
   const int w_blocks = (w_rows + 15) / 16;
@@ -353,18 +346,16 @@ template <bool TILES, bool SWIGLU, typename TC>
 static void launch_tiled(const void* a, const void* w, void* c, int M, int N, int K, int accumulate,
                          hipStream_t stream) {
   const int columns = SWIGLU ? TBN / 2 : TBN;
-  const int n_tiles = (N + columns - 1) / columns, m_tiles = (M + 127) / 128;
-  const long tiles = (long)n_tiles * m_tiles;
-  dim3 grid((unsigned)((tiles + 7) / 8 * 8)), block(256);
+  dim3 grid((N + columns - 1) / columns, (M + 127) / 128), block(256);
   // Two LDS buffers let two workgroups per compute unit overlap loads and multiplies, which pays when
   // there are several rounds of workgroups; with about one round, four smaller workgroups per compute
   // unit (one buffer, a second barrier per slice) hide more latency.  Measured at the Qwen3-8B shapes.
-  if (tiles >= 1024)
-    gemm_tiled_kernel<TILES, SWIGLU, 2, 2, TC><<<grid, block, 0, stream>>>(
-        (const uint16_t*)a, (const uint16_t*)w, (TC*)c, M, N, K, accumulate, m_tiles, n_tiles);
+  if ((long)grid.x * grid.y >= 1024)
+    gemm_tiled_kernel<TILES, SWIGLU, 2, 2, TC><<<grid, block, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w,
+                                                                           (TC*)c, M, N, K, accumulate);
   else
-    gemm_tiled_kernel<TILES, SWIGLU, 2, 1, TC><<<grid, block, 0, stream>>>(
-        (const uint16_t*)a, (const uint16_t*)w, (TC*)c, M, N, K, accumulate, m_tiles, n_tiles);
+    gemm_tiled_kernel<TILES, SWIGLU, 2, 1, TC><<<grid, block, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w,
+                                                                           (TC*)c, M, N, K, accumulate);
 }
 
 // layout: 0 = rows, 1 = tiles.  activation: 0 = none; 1 = SwiGLU (W has 2 * N rows: gate rows then up rows).
@@ -378,7 +369,7 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
   BH_REQUIRE(activation == 0 || activation == 1, "gemm_bf16: unknown activation %d", activation);
   BH_REQUIRE(activation == 0 || (N % 16 == 0 && !accumulate),
              "gemm_bf16: SwiGLU needs a multiple of 16 outputs (got %d) and no accumulation", N);
-  BH_REQUIRE((long)((M + 127) / 128) * ((N + 63) / 64) < 2000000000L, "gemm_bf16: M=%d x N=%d has too many tiles", M, N);
+  BH_REQUIRE((M + 127) / 128 <= 65535, "gemm_bf16: M=%d needs more than 65535 row tiles", M);
   const bool f32 = c_dtype == BH_F32;
 #define BH_PICK(FN, TILES, EXTRA, ...)                                             \
   do {                                                                              \
