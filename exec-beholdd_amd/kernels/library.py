@@ -76,23 +76,14 @@ class HipKernels:
             "bh_attention_generic": [p, p, i, p, p, p, i, p, p, i, i, i, i, f, i, p],
             "bh_swiglu": [p, p, i, i, i, p],
             "bh_sample": [p, p, p, p, p, p, p, i, i, p],
+            "bh_gemm_bf16": [p, p, p, i, i, i, i, i, i, i, p],
+            "bh_attention_bf16": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, i, i, f, i, i, i, p],
+            "bh_attention_bf16_splits": [i, i, i, i, i],
         }
         for name, argtypes in table.items():
             function = getattr(lib, name)
             function.argtypes = argtypes
             function.restype = i
-        self._optional = {}
-        for name, argtypes in {
-            "bh_gemm_bf16": [p, p, p, i, i, i, i, i, i, i, p],
-            "bh_attention_bf16": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, i, i, f, i, i, i, p],
-            "bh_attention_bf16_splits": [i, i, i, i, i],
-        }.items():
-            function = getattr(lib, name, None)
-            if function is not None:
-                function.argtypes = argtypes
-                function.restype = i
-                self._optional[name] = function
-
     # ---- helpers ----
     def _stream(self):
         return ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
@@ -145,8 +136,7 @@ class HipKernels:
     def pack_weight(self, w):
         """The form of a weight matrix that the matrix products read fastest: a `PackedWeight` for a
         bfloat16 matrix whose width is a multiple of 64, else the matrix itself."""
-        if (isinstance(w, torch.Tensor) and w.dim() == 2 and w.dtype == torch.bfloat16 and w.shape[1] % 64 == 0
-                and "bh_gemm_bf16" in self._optional):
+        if (isinstance(w, torch.Tensor) and w.dim() == 2 and w.dtype == torch.bfloat16 and w.shape[1] % 64 == 0):
             rows, cols = w.shape
             padded = -(-rows // 16) * 16
             if padded != rows:
@@ -158,9 +148,9 @@ class HipKernels:
 
     def _gemm_fast(self, a, w, out, accumulate, activation):
         """Launch the matrix-core product if it takes these operands; say whether it did."""
-        fast = self._optional.get("bh_gemm_bf16")
+        fast = self.lib.bh_gemm_bf16
         packed = isinstance(w, PackedWeight)
-        if fast is None or a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or a.shape[1] % 8:
+        if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or a.shape[1] % 8:
             if packed:
                 raise KernelError("gemm: a packed weight needs bfloat16 activations")
             return False
@@ -263,14 +253,14 @@ class HipKernels:
             raise KernelError("attention: positions and row_seq must have one entry per row")
         self._check_pages(k_pages, v_pages, page_table, n_kv_heads, head_dim, q.dtype, "attention")
         common = (self._ptr(q, "q"), self._ptr(out, "attention out"))
-        fast = self._optional.get("bh_attention_bf16")
-        if (fast is not None and q.dtype == torch.bfloat16 and layout is not None and head_dim % 32 == 0
+        fast = self.lib.bh_attention_bf16
+        if (q.dtype == torch.bfloat16 and layout is not None and head_dim % 32 == 0
                 and head_dim <= 256):
             n_seqs, max_rows = int(layout.n_seqs), int(layout.max_rows_per_seq)
             if layout.seq_start.shape != (n_seqs + 1,) or page_table.shape[0] < n_seqs:
                 raise KernelError("attention: seq_start must have one entry per sequence and one more, and the page "
                                   "table a row per sequence")
-            n_splits = int(self._optional["bh_attention_bf16_splits"](n_seqs, max_rows, n_heads, n_kv_heads,
+            n_splits = int(self.lib.bh_attention_bf16_splits(n_seqs, max_rows, n_heads, n_kv_heads,
                                                                       int(layout.max_position)))
             part_o = part_ml = None
             if n_splits > 1:   # partial results of the key splits: scratch for this call only

@@ -80,6 +80,27 @@ def test_every_cut_matches_the_plain_implementation(expected, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_one_layer_of_the_qwen3_8b_sizes(tmp_path_factory, dtype):
+    """The layer sizes of the benchmark model (hidden 4096, 32 query and 8 kv heads of 128, feed-forward
+    12288) in one layer with a small vocabulary: the kernels at the shapes they are tuned for, whole,
+    token by token and in a batch, against the plain implementation."""
+    import beholdd
+    config = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 1, "hidden_size": 4096,
+              "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128, "intermediate_size": 12288,
+              "vocab_size": 1000, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "max_position_embeddings": 8192,
+              "tie_word_embeddings": False}
+    folder = str(tmp_path_factory.mktemp("layer_8b"))
+    beholdd.write_random_model(folder, config, seed=1, dtype="bfloat16")
+    cfg, weights = plain.load_plain(folder)
+    requests = schedules.random_requests(cfg.vocab, [70, 9, 131], seed=5)
+    want = [plain.forward_logits(cfg, weights, r) for r in requests]
+    engine = engine_for(folder, dtype, max_tokens=1024)
+    check("whole", schedules.whole(engine, requests), want, TOLERANCE[dtype])
+    check("last 8 one by one", schedules.tail_one_by_one(engine, requests, tail=8), want, TOLERANCE[dtype])
+    check("batch", schedules.batches(engine, requests, batch_size=3, prompt_fraction=0.9), want, TOLERANCE[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_float32_storage_and_slot_reuse_in_a_small_cache(model_dirs, dtype):
     """Weights stored in 32-bit; a cache of three pages, so every request runs in pages and slots
     that earlier requests used."""
