@@ -180,36 +180,38 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
 
 // ---- tiled -----------------------------------------------------------------------------------
 
-#define TBN 128         // W rows (output columns, or gate+up rows) per tile
 #define TK 64           // k slice
 #define TPITCH (TK + 8) // LDS row pitch in elements: 144 bytes, so 16-byte reads of 16 rows hit 64 distinct banks
 
-// A workgroup of four waves (2 x 2) computes a (64 * WX) x 128 tile; a wave WX x 2 blocks of 32 x 32.
-// WX = 2 is what runs: WX = 4 (256 rows, fewer LDS reads per multiply) leaves room for one workgroup
-// per compute unit only and measured a third slower.
-// SWIGLU: the tile's 128 W rows are, per wave column half (32 outputs), 32 gate rows then the 32 up
-// rows of the same outputs; N counts outputs and the up rows start `N` rows (N/16 blocks) further on.
-template <bool TILES, bool SWIGLU, int WX, int BUFFERS, typename TC>
-__global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restrict__ a,
-                                                         const uint16_t* __restrict__ w, TC* __restrict__ c,
-                                                         int M, int N, int K, int accumulate) {
-  constexpr int TBM = 64 * WX;
-  constexpr int A_PIECES = TBM / 32;   // 16-byte pieces of a slice that one thread stages: TBM rows x 8 / 256
-  constexpr int W_PIECES = TBN / 32;
+// A workgroup of WM x WN waves computes a (32 WX WM) x (32 WY WN) tile; a wave WX x WY blocks of 32 x 32.
+// SWIGLU: a wave's 32 WY rows of W are the gate rows of its 16 WY outputs and then the up rows of the
+// same outputs; N counts outputs and the up rows start `N` rows (N/16 blocks) further on.
+template <bool TILES, bool SWIGLU, int WX, int WY, int WM, int WN, int BUFFERS, typename TC>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const uint16_t* __restrict__ a,
+                                                                   const uint16_t* __restrict__ w,
+                                                                   TC* __restrict__ c, int M, int N, int K,
+                                                                   int accumulate) {
+  constexpr int THREADS = 64 * WM * WN;
+  constexpr int TBM = 32 * WX * WM, TBN = 32 * WY * WN;
+  constexpr int A_PIECES = TBM * 8 / THREADS;   // 16-byte pieces of a slice that one thread stages
+  constexpr int W_PIECES = TBN * 8 / THREADS;
+  static_assert(TBM * 8 % THREADS == 0 && TBN * 8 % THREADS == 0, "the tile is staged in whole rounds of the workgroup");
+  static_assert(!SWIGLU || WY % 2 == 0, "gate and up blocks come in pairs");
   __shared__ __attribute__((aligned(16))) uint16_t as[BUFFERS][TBM * TPITCH];
   __shared__ __attribute__((aligned(16))) uint16_t ws[BUFFERS][TBN * TPITCH];
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int m0 = blockIdx.y * TBM;
   const int n0 = blockIdx.x * (SWIGLU ? TBN / 2 : TBN);      // first output column of the tile
-  const int wm = (wave / 2) * 32 * WX, wn = (wave % 2) * 64;  // this wave's part of the tile (in LDS rows)
+  const int wm = (wave / WN) * 32 * WX, wn = (wave % WN) * 32 * WY;  // this wave's part of the tile (in LDS rows)
   const int w_rows = SWIGLU ? 2 * N : N;
   const int w_blocks = (w_rows + 15) / 16;
 
   // LDS row r of the W tile -> row of W
   auto w_row_of = [&](int r) {
     if (!SWIGLU) return n0 + r;
-    const int half = r / 64, inner = r % 64;              // wave column half, then 32 gate rows + 32 up rows
-    return (inner < 32 ? 0 : N) + n0 + half * 32 + inner % 32;
+    constexpr int OUTS = 16 * WY;                          // outputs of one wave column
+    const int part = r / (2 * OUTS), inner = r % (2 * OUTS);
+    return (inner < OUTS ? 0 : N) + n0 + part * OUTS + inner % OUTS;
   };
 
   // global -> LDS staging: a slice is rows x 8 pieces of 16 bytes
@@ -218,7 +220,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
   const uint16_t* w_src[W_PIECES];
 #pragma unroll
   for (int s = 0; s < A_PIECES; ++s) {
-    const int e = tid + s * 256;
+    const int e = tid + s * THREADS;
     const int row = e / 8, piece = e % 8;
     const int am = (m0 + row < M) ? m0 + row : M - 1;
     a_src[s] = a + (size_t)am * K + piece * 8;
@@ -227,7 +229,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
   }
 #pragma unroll
   for (int s = 0; s < W_PIECES; ++s) {
-    const int e = tid + s * 256;
+    const int e = tid + s * THREADS;
     const int row = e / 8, piece = e % 8;
     w_piece[s] = piece;
     if (TILES) {
@@ -247,13 +249,21 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
   const size_t w_step = TILES ? 1024 : TK;
   u32x4_t a_reg[A_PIECES], w_reg[W_PIECES];
   const u32x4_t zero = {0u, 0u, 0u, 0u};
+  const bool whole_slices = K % TK == 0;   // then no piece of a slice lies beyond K and no load is predicated
   auto fetch = [&](int slice) {
     const int k0 = slice * TK;
+    if (whole_slices) {
 #pragma unroll
-    for (int s = 0; s < A_PIECES; ++s) a_reg[s] = (k0 + a_piece[s] * 8 < K) ? load16(a_src[s] + k0) : zero;
+      for (int s = 0; s < A_PIECES; ++s) a_reg[s] = load16(a_src[s] + k0);
 #pragma unroll
-    for (int s = 0; s < W_PIECES; ++s)
-      w_reg[s] = (TILES || k0 + w_piece[s] * 8 < K) ? load16(w_src[s] + (size_t)slice * w_step) : zero;
+      for (int s = 0; s < W_PIECES; ++s) w_reg[s] = load16(w_src[s] + (size_t)slice * w_step);
+    } else {
+#pragma unroll
+      for (int s = 0; s < A_PIECES; ++s) a_reg[s] = (k0 + a_piece[s] * 8 < K) ? load16(a_src[s] + k0) : zero;
+#pragma unroll
+      for (int s = 0; s < W_PIECES; ++s)
+        w_reg[s] = (TILES || k0 + w_piece[s] * 8 < K) ? load16(w_src[s] + (size_t)slice * w_step) : zero;
+    }
   };
   auto stash = [&](int buffer) {
 #pragma unroll
@@ -262,11 +272,11 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
     for (int s = 0; s < W_PIECES; ++s) *reinterpret_cast<u32x4_t*>(&ws[buffer][w_at[s]]) = w_reg[s];
   };
 
-  f32x16_t acc[WX][2];
+  f32x16_t acc[WX][WY];
 #pragma unroll
   for (int x = 0; x < WX; ++x)
 #pragma unroll
-    for (int y = 0; y < 2; ++y)
+    for (int y = 0; y < WY; ++y)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[x][y][e] = 0.f;
 
@@ -280,37 +290,40 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
     if (s + 1 < slices) fetch(s + 1);
 #pragma unroll
     for (int kk = 0; kk < TK; kk += 16) {
-      bf16x8_t af[WX], wf[2];
+      bf16x8_t af[WX], wf[WY];
 #pragma unroll
       for (int x = 0; x < WX; ++x)
         af[x] = as_bf16x8(*reinterpret_cast<const u32x4_t*>(&as[buffer][(wm + x * 32 + frag_row) * TPITCH + kk + frag_k]));
 #pragma unroll
-      for (int y = 0; y < 2; ++y)
+      for (int y = 0; y < WY; ++y)
         wf[y] = as_bf16x8(*reinterpret_cast<const u32x4_t*>(&ws[buffer][(wn + y * 32 + frag_row) * TPITCH + kk + frag_k]));
 #pragma unroll
       for (int x = 0; x < WX; ++x)
 #pragma unroll
-        for (int y = 0; y < 2; ++y)
+        for (int y = 0; y < WY; ++y)
           acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[x], wf[y], acc[x][y], 0, 0, 0);
     }
     if (BUFFERS == 1) __syncthreads();   // one buffer: everyone has read the slice before it is overwritten
-    if (s + 1 < slices) stash(BUFFERS == 2 ? buffer ^ 1 : 0);
+    if (s + 1 < slices) stash(BUFFERS == 2 ? buffer ^ 1 : 0);   // (writing it half-way through the multiplies measured slower)
     __syncthreads();
   }
   // D of one 32x32 block: column (n) lane%32, rows (m) 8*(e/4) + 4*(lane/32) + e%4
 #pragma unroll
   for (int x = 0; x < WX; ++x) {
     if (SWIGLU) {
-      const int n = n0 + (wave % 2) * 32 + lane % 32;
-      if (n >= N) continue;
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int m = m0 + wm + x * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
-        if (m < M) store_out<TC>(c, (size_t)m * N + n, silu_mul(acc[x][0][e], acc[x][1][e]), false);
+      for (int y = 0; y < WY / 2; ++y) {
+        const int n = n0 + (wave % WN) * 16 * WY + y * 32 + lane % 32;
+        if (n >= N) continue;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int m = m0 + wm + x * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
+          if (m < M) store_out<TC>(c, (size_t)m * N + n, silu_mul(acc[x][y][e], acc[x][y + WY / 2][e]), false);
+        }
       }
     } else {
 #pragma unroll
-      for (int y = 0; y < 2; ++y) {
+      for (int y = 0; y < WY; ++y) {
         const int n = n0 + wn + y * 32 + lane % 32;
         if (n >= N) continue;
 #pragma unroll
@@ -345,17 +358,24 @@ static void launch_skinny(const void* a, const void* w, void* c, int M, int N, i
 template <bool TILES, bool SWIGLU, typename TC>
 static void launch_tiled(const void* a, const void* w, void* c, int M, int N, int K, int accumulate,
                          hipStream_t stream) {
-  const int columns = SWIGLU ? TBN / 2 : TBN;
-  dim3 grid((N + columns - 1) / columns, (M + 127) / 128), block(256);
-  // Two LDS buffers let two workgroups per compute unit overlap loads and multiplies, which pays when
-  // there are several rounds of workgroups; with about one round, four smaller workgroups per compute
-  // unit (one buffer, a second barrier per slice) hide more latency.  Measured at the Qwen3-8B shapes.
-  if ((long)grid.x * grid.y >= 1024)
-    gemm_tiled_kernel<TILES, SWIGLU, 2, 2, TC><<<grid, block, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w,
-                                                                           (TC*)c, M, N, K, accumulate);
-  else
-    gemm_tiled_kernel<TILES, SWIGLU, 2, 1, TC><<<grid, block, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w,
-                                                                           (TC*)c, M, N, K, accumulate);
+#define BH_TILED(WX, WY, WM, WN, BUFFERS)                                                                 \
+  do {                                                                                                     \
+    const int columns = (SWIGLU ? 16 : 32) * WY * WN, rows = 32 * WX * WM;                                 \
+    dim3 grid((N + columns - 1) / columns, (M + rows - 1) / rows), block(64 * WM * WN);                    \
+    gemm_tiled_kernel<TILES, SWIGLU, WX, WY, WM, WN, BUFFERS, TC><<<grid, block, 0, stream>>>(             \
+        (const uint16_t*)a, (const uint16_t*)w, (TC*)c, M, N, K, accumulate);                              \
+  } while (0)
+  // Measured at the Qwen3-8B shapes (2,048 rows).  The multiplies of a 128 x 128 tile need as many LDS
+  // cycles (operand reads and the staging writes) as MFMA cycles, so LDS bounds them; a 256 x 256 tile
+  // of eight waves, each 64 x 128, reads a quarter less per multiply and wins once it still gives every
+  // compute unit three tiles.  Below that the smaller tile keeps more compute units busy: with two LDS
+  // buffers when there are several rounds of workgroups, with one (four workgroups per compute unit, a
+  // second barrier per slice) when there is about one round.
+  const long tiles_128 = (long)((N + (SWIGLU ? 63 : 127)) / (SWIGLU ? 64 : 128)) * ((M + 127) / 128);
+  if (tiles_128 >= 3072) BH_TILED(2, 4, 4, 2, 2);
+  else if (tiles_128 >= 1024) BH_TILED(2, 2, 2, 2, 2);
+  else BH_TILED(2, 2, 2, 2, 1);
+#undef BH_TILED
 }
 
 // layout: 0 = rows, 1 = tiles.  activation: 0 = none; 1 = SwiGLU (W has 2 * N rows: gate rows then up rows).

@@ -73,7 +73,8 @@ def test_rmsnorm(K, out_dtype, w_dtype, rows, width, eps):
                                              (torch.bfloat16, torch.float32)])
 @pytest.mark.parametrize("m,n,k", [(1, 96, 120), (7, 331, 200), (64, 130, 72), (65, 257, 1000), (200, 64, 48),
                                    (3, 1000, 4096), (130, 520, 264), (17, 40, 100), (33, 100, 2048), (48, 16, 8),
-                                   (8, 4096, 12288), (300, 1000, 1024), (1, 15, 64)])
+                                   (8, 4096, 12288), (300, 1000, 1024), (1, 15, 64),
+                                   (1030, 43700, 136)])      # the last: enough tiles for the largest tile shape
 def test_gemm(K, a_dtype, w_dtype, m, n, k):
     g = torch.Generator().manual_seed(m * 1000 + n)
     a = torch.randn(m, k, generator=g).to(a_dtype)
@@ -92,7 +93,8 @@ def test_gemm(K, a_dtype, w_dtype, m, n, k):
 
 @pytest.mark.parametrize("m,n,k", [(1, 96, 128), (8, 331, 192), (64, 130, 64), (65, 257, 1024), (200, 64, 448),
                                    (3, 1000, 4096), (130, 520, 256), (16, 24, 64), (33, 16, 2048),
-                                   (8, 4096, 12288), (300, 1000, 1024), (129, 129, 128)])
+                                   (8, 4096, 12288), (300, 1000, 1024), (129, 129, 128),
+                                   (1030, 43700, 192)])
 def test_gemm_with_packed_weights(K, m, n, k):
     """The same product from the regrouped (16 x 64 blocks) weight layout."""
     from beholdd.kernels import PackedWeight
@@ -118,7 +120,8 @@ def test_gemm_with_packed_weights(K, m, n, k):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("m,width,k", [(1, 16, 64), (8, 160, 128), (40, 896, 320), (64, 48, 192), (65, 64, 64),
-                                       (130, 208, 256), (300, 1000, 128), (7, 100, 64), (8, 12288, 4096), (5, 32, 72)])
+                                       (130, 208, 256), (300, 1000, 128), (7, 100, 64), (8, 12288, 4096), (5, 32, 72),
+                                       (650, 33008, 128)])
 def test_gemm_swiglu(K, dtype, packed, m, width, k):
     """silu(a Wg^T) * (a Wu^T) in one pass (or in two where the sizes do not allow one), from both layouts."""
     g = torch.Generator().manual_seed(m + width)
