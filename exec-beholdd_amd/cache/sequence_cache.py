@@ -4,8 +4,9 @@ Layout.  A *slot* is one sequence's handle: its length, its pages and its row in
 region.  Layers are sorted into *groups* by what they need (`CacheNeed`): every group has
 storage of its own.  A key/value group holds, for each of its cache entries (one per
 scheduled layer run that writes a cache), keys [pages, kv_heads, page_size, head_dim] and values
-[pages, kv_heads, head_dim, page_size] (transposed inside a page, the layout the matrix-core
-attention kernels load directly); a sequence's position p lives in page `table[p // page_size]`
+[pages, kv_heads, head_dim, page_size] (the order of one head's elements inside a page is the
+kernel library's: the kernel that writes them and the attention kernels agree on it, and the
+cache itself never looks inside); a sequence's position p lives in page `table[p // page_size]`
 at token `p % page_size`, and a
 group with a window gives pages back once every position in them has left the window.  A
 state group holds [entries, max_slots, *shape] and a slot's rows are zero when it starts.

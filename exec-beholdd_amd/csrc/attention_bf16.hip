@@ -32,6 +32,11 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 __device__ inline bf16x8_t as_bf16x8(u32x4_t v) { return __builtin_bit_cast(bf16x8_t, v); }
 __device__ inline u32x4_t load16(const uint16_t* p) { return *reinterpret_cast<const u32x4_t*>(p); }
+template <bool STREAM>
+__device__ inline u32x4_t load16_cache(const uint16_t* p) {   // STREAM: nobody else reads these bytes soon
+  if (STREAM) return __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+  return *reinterpret_cast<const u32x4_t*>(p);
+}
 
 __device__ inline int wave_max_int(int v) {
 #pragma unroll
@@ -65,7 +70,8 @@ __device__ inline u32x4_t keep_first(u32x4_t v, int n_valid) {
 
 // NS = head_dim / 32.  CT = column tiles (of 16 columns) per workgroup: every page a wave loads is
 // used for all CT tiles, which divides the cache traffic of a prefill by CT.
-template <int NS, int CT>
+// STREAM = one workgroup per (sequence, kv head, split): each cache byte is read once, past the caches.
+template <int NS, int CT, bool STREAM>
 __global__ __launch_bounds__(256) void attention_mfma_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages,
@@ -129,18 +135,15 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
     const uint16_t* kb = k_pages + ((size_t)page * KVH + kvh) * BH_PAGE * HD;
     const uint16_t* vb = v_pages + ((size_t)page * KVH + kvh) * HD * BH_PAGE;
     u32x4_t k_vec[4][NS], v_vec[2 * NS][2];
-    // every load instruction covers 64 contiguous bytes of each of its 16 rows (lane group g the g-th 16)
+    // the cache lies in pieces (BH_KV_PIECES): every load instruction covers 1 KB of contiguous memory
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const uint16_t* kr = kb + (size_t)(32 * (t / 2) + 4 * (t % 2) + 8 * (j / 4) + j % 4) * HD + 8 * g;
+    for (int t = 0; t < 4; ++t)
 #pragma unroll
-      for (int s = 0; s < NS; ++s) k_vec[t][s] = load16(kr + 32 * s);
-    }
+      for (int s = 0; s < NS; ++s) k_vec[t][s] = load16_cache<STREAM>(kb + ((t * NS + s) * 64 + lane) * 8);
 #pragma unroll
     for (int dt = 0; dt < 2 * NS; ++dt) {
-      const uint16_t* vr = vb + (size_t)(16 * dt + j) * BH_PAGE + 8 * g;
-      v_vec[dt][0] = load16(vr);
-      v_vec[dt][1] = load16(vr + 32);
+      v_vec[dt][0] = load16_cache<STREAM>(vb + ((dt * 2) * 64 + lane) * 8);
+      v_vec[dt][1] = load16_cache<STREAM>(vb + ((dt * 2 + 1) * 64 + lane) * 8);
     }
     const int key0 = p * BH_PAGE + 8 * g;  // lane (j, g) holds keys key0 + 32 * (t / 2) + 4 * (t % 2) + r
     const bool mask_needed = (p * BH_PAGE + BH_PAGE - 1 > pos_min) || (p * BH_PAGE < lo_max);
@@ -279,6 +282,12 @@ __global__ void attention_combine_kernel(const float* __restrict__ part_o, const
   }
 }
 
+// The order of a cache page's elements that the kernels of this library expect for a cache of the
+// given element type and head size: the writer, the attention for any size and this file's agree on it.
+extern "C" int bh_kv_order(int dtype, int hd) {
+  return (dtype == BH_BF16 && hd % 32 == 0 && hd >= 32 && hd <= 256) ? BH_KV_PIECES : BH_KV_ROWS;
+}
+
 // How many ways the keys are split for a given launch; the caller sizes the scratch from it.
 extern "C" int bh_attention_bf16_splits(int n_seqs, int max_rows_per_seq, int H, int KVH, int max_position) {
   if (n_seqs <= 0 || max_rows_per_seq <= 0 || H <= 0 || KVH <= 0 || H % KVH) return 1;
@@ -286,8 +295,10 @@ extern "C" int bh_attention_bf16_splits(int n_seqs, int max_rows_per_seq, int H,
   const long tiles = (long)((max_rows_per_seq * G + 15) / 16) * KVH * n_seqs;
   const int pages = max_position / BH_PAGE + 1;
   // about one workgroup per compute unit (256), every wave of a workgroup at least one page
-  if (tiles >= 256 || pages < 8) return 1;
-  long want = (256 + tiles - 1) / tiles;
+  const char* env = getenv("BH_ATT_TARGET");
+  const long target = env ? atol(env) : 256;
+  if (tiles >= target || pages < 8) return 1;
+  long want = (target + tiles - 1) / tiles;
   if (want > pages / 4) want = pages / 4;
   if (want < 1) want = 1;
   const int per = (int)((pages + want - 1) / want);
@@ -314,16 +325,17 @@ extern "C" int bh_attention_bf16(const void* q, void* out, void* part_o, void* p
   BH_REQUIRE((long)n_seqs * n_splits <= 65535 && KVH <= 65535, "attention_bf16: too many sequences x splits");
   dim3 grid((tiles + ct - 1) / ct, KVH, n_seqs * n_splits), block(256);
   const float scale_log2 = scale * 1.4426950408889634f;
-#define BH_ATT_CT(NS, CT)                                                                                       \
-  attention_mfma_kernel<NS, CT><<<grid, block, 0, stream>>>(                                                    \
+#define BH_ATT_CT(NS, CT, STREAM)                                                                               \
+  attention_mfma_kernel<NS, CT, STREAM><<<grid, block, 0, stream>>>(                                            \
       (const uint16_t*)q, (uint16_t*)out, (float*)part_o, (float*)part_ml, (const uint16_t*)k_pages,            \
       (const uint16_t*)v_pages, page_table, table_stride, positions, seq_start, H, KVH, scale_log2, window,     \
       n_splits, per)
-#define BH_ATT(NS)                        \
-  do {                                    \
-    if (ct == 4) BH_ATT_CT(NS, 4);        \
-    else if (ct == 2) BH_ATT_CT(NS, 2);   \
-    else BH_ATT_CT(NS, 1);                \
+#define BH_ATT(NS)                                 \
+  do {                                             \
+    if (ct == 4) BH_ATT_CT(NS, 4, false);          \
+    else if (ct == 2) BH_ATT_CT(NS, 2, false);     \
+    else if (grid.x == 1) BH_ATT_CT(NS, 1, true);  \
+    else BH_ATT_CT(NS, 1, false);                  \
   } while (0)
   switch (hd / 32) {
     case 1: BH_ATT(1); break;

@@ -226,7 +226,7 @@ extern "C" int bh_gemm_generic(const void* a, int a_dtype, const void* w, int w_
 // One wave per (row, head) of the fused projection row [q heads | k heads | v heads].
 // q head: optional RMSNorm over the head, rotation at the row's position, written to q_out.
 // k head: the same, written into the cache page of (sequence, position).
-// v head: copied into the cache (transposed within its page).  Rotation pairs are (i, i + rot/2) for i < rot/2; elements
+// v head: copied into the cache.  Where an element lies within its page follows `kv_order`.  Rotation pairs are (i, i + rot/2) for i < rot/2; elements
 // from rot to head_dim pass through.  With write_kv == 0 only the q heads are processed.
 
 template <typename T, typename TW>
@@ -235,7 +235,7 @@ __global__ __launch_bounds__(64) void qk_norm_rope_cache_kernel(
     const TW* __restrict__ k_weight, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, int rot, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ row_seq, T* __restrict__ k_pages, T* __restrict__ v_pages,
-    const int32_t* __restrict__ page_table, int table_stride, int H, int KVH, int hd) {
+    const int32_t* __restrict__ page_table, int table_stride, int H, int KVH, int hd, int kv_order) {
   const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int fused = (H + 2 * KVH) * hd;
   const T* src = qkv + (size_t)row * fused + (size_t)head * hd;
@@ -243,6 +243,7 @@ __global__ __launch_bounds__(64) void qk_norm_rope_cache_kernel(
 
   T* dst;
   const TW* weight;
+  int order = BH_KV_ROWS, token = 0;   // a q head is one row of its own
   if (head < H) {
     dst = q_out + ((size_t)row * H + head) * hd;
     weight = q_weight;
@@ -252,12 +253,14 @@ __global__ __launch_bounds__(64) void qk_norm_rope_cache_kernel(
     const int kv_head = (head - H) % KVH;
     const bool is_value = head >= H + KVH;
     weight = k_weight;
-    if (is_value) {  // values lie transposed in a page: [head_dim][token]
-      T* column = v_pages + ((size_t)page * KVH + kv_head) * BH_PAGE * hd + (pos % BH_PAGE);
-      for (int i = lane; i < hd; i += BH_WAVE) column[(size_t)i * BH_PAGE] = src[i];
+    order = kv_order;
+    token = pos % BH_PAGE;
+    if (is_value) {
+      T* block = v_pages + ((size_t)page * KVH + kv_head) * BH_PAGE * hd;
+      for (int i = lane; i < hd; i += BH_WAVE) block[bh_value_index(order, token, i, hd)] = src[i];
       return;
     }
-    dst = k_pages + (((size_t)page * KVH + kv_head) * BH_PAGE + (pos % BH_PAGE)) * hd;
+    dst = k_pages + ((size_t)page * KVH + kv_head) * BH_PAGE * hd;
   }
   float inv = 1.f;
   if (weight) {
@@ -281,13 +284,13 @@ __global__ __launch_bounds__(64) void qk_norm_rope_cache_kernel(
       c = cos_table[(size_t)pos * half + i];
       s = sin_table[(size_t)pos * half + i];
     }
-    dst[i] = from_f32<T>(a * c - b * s);
-    dst[i + half] = from_f32<T>(a * s + b * c);
+    dst[bh_key_index(order, token, i, hd)] = from_f32<T>(a * c - b * s);
+    dst[bh_key_index(order, token, i + half, hd)] = from_f32<T>(a * s + b * c);
   }
   for (int i = rot + lane; i < hd; i += BH_WAVE) {
     float a = to_f32(src[i]);
     if (weight) a = a * inv * to_f32(weight[i]);
-    dst[i] = from_f32<T>(a);
+    dst[bh_key_index(order, token, i, hd)] = from_f32<T>(a);
   }
 }
 
@@ -296,7 +299,7 @@ extern "C" int bh_qk_norm_rope_cache(const void* qkv, int dtype, void* q_out, co
                                      const float* sin_table, int table_positions, int rot,
                                      const int32_t* positions, const int32_t* row_seq, void* k_pages,
                                      void* v_pages, const int32_t* page_table, int table_stride, int n_rows,
-                                     int H, int KVH, int hd, int write_kv, int max_position,
+                                     int H, int KVH, int hd, int write_kv, int kv_order, int max_position,
                                      hipStream_t stream) {
   BH_REQUIRE(n_rows > 0 && H > 0 && KVH > 0 && hd > 0, "qk_norm_rope: sizes must be positive");
   BH_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0, "qk_norm_rope: rotary width %d must be even and at most %d", rot, hd);
@@ -304,12 +307,14 @@ extern "C" int bh_qk_norm_rope_cache(const void* qkv, int dtype, void* q_out, co
   BH_REQUIRE(cos_table == nullptr || max_position < table_positions,
              "qk_norm_rope: position %d is outside the rotation table of %d positions", max_position, table_positions);
   BH_REQUIRE(H + 2 * KVH <= 65535, "qk_norm_rope: too many heads");
+  BH_REQUIRE(kv_order == BH_KV_ROWS || (kv_order == BH_KV_PIECES && hd % 32 == 0),
+             "qk_norm_rope: cache order %d does not exist for head size %d", kv_order, hd);
   if (cos_table == nullptr) rot = 0;
   dim3 grid(n_rows, write_kv ? H + 2 * KVH : H), block(BH_WAVE);
 #define BH_QK(T, TW)                                                                                         \
   qk_norm_rope_cache_kernel<T, TW><<<grid, block, 0, stream>>>(                                              \
       (const T*)qkv, (T*)q_out, (const TW*)q_weight, (const TW*)k_weight, eps, cos_table, sin_table, rot,    \
-      positions, row_seq, (T*)k_pages, (T*)v_pages, page_table, table_stride, H, KVH, hd)
+      positions, row_seq, (T*)k_pages, (T*)v_pages, page_table, table_stride, H, KVH, hd, kv_order)
   if (dtype == BH_F32 && w_dtype == BH_F32) BH_QK(float, float);
   else if (dtype == BH_F32 && w_dtype == BH_BF16) BH_QK(float, bf16_t);
   else if (dtype == BH_BF16 && w_dtype == BH_F32) BH_QK(bf16_t, float);
@@ -331,7 +336,7 @@ template <typename T>
 __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
     const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int32_t* __restrict__ page_table, int table_stride, const int32_t* __restrict__ row_seq,
-    const int32_t* __restrict__ positions, int H, int KVH, int hd, float scale, int window) {
+    const int32_t* __restrict__ positions, int H, int KVH, int hd, float scale, int window, int kv_order) {
   extern __shared__ float smem[];
   float* qs = smem;                    // [hd]
   float* probs = qs + hd;              // [AG_THREADS]
@@ -359,9 +364,9 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
     float s = -INFINITY;
     if (j <= pos) {
       const int page = table[j / BH_PAGE];
-      const T* kr = k_pages + (((size_t)page * KVH + kv_head) * BH_PAGE + (j % BH_PAGE)) * hd;
+      const T* block = k_pages + ((size_t)page * KVH + kv_head) * BH_PAGE * hd;
       float dot = 0.f;
-      for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], to_f32(kr[d]), dot);
+      for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], to_f32(block[bh_key_index(kv_order, j % BH_PAGE, d, hd)]), dot);
       s = dot * scale;
     }
     const float chunk_max = block_max(s, scratch);
@@ -378,8 +383,8 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
       for (int jj = group; jj < n_keys; jj += n_groups) {
         const int key = c0 + jj;
         const int page = table[key / BH_PAGE];
-        const T* vr = v_pages + ((size_t)page * KVH + kv_head) * BH_PAGE * hd + (key % BH_PAGE);
-        acc = fmaf(probs[jj], to_f32(vr[(size_t)dim * BH_PAGE]), acc);
+        const T* block = v_pages + ((size_t)page * KVH + kv_head) * BH_PAGE * hd;
+        acc = fmaf(probs[jj], to_f32(block[bh_value_index(kv_order, key % BH_PAGE, dim, hd)]), acc);
       }
     }
     __syncthreads();  // probs[] is rewritten by the next chunk
@@ -396,22 +401,25 @@ __global__ __launch_bounds__(AG_THREADS) void attention_generic_kernel(
 extern "C" int bh_attention_generic(const void* q, void* out, int dtype, const void* k_pages,
                                     const void* v_pages, const int32_t* page_table, int table_stride,
                                     const int32_t* row_seq, const int32_t* positions, int n_rows, int H,
-                                    int KVH, int hd, float scale, int window, hipStream_t stream) {
+                                    int KVH, int hd, float scale, int window, int kv_order,
+                                    hipStream_t stream) {
   BH_REQUIRE(n_rows > 0 && H > 0 && KVH > 0 && hd > 0, "attention: sizes must be positive");
   BH_REQUIRE(H % KVH == 0, "attention: %d query heads do not group evenly into %d kv heads", H, KVH);
   BH_REQUIRE(hd <= AG_THREADS, "attention: head size %d is above the limit of %d", hd, AG_THREADS);
   BH_REQUIRE(H <= 65535, "attention: too many heads");
   BH_REQUIRE(window >= 0, "attention: window must not be negative");
+  BH_REQUIRE(kv_order == BH_KV_ROWS || (kv_order == BH_KV_PIECES && hd % 32 == 0),
+             "attention: cache order %d does not exist for head size %d", kv_order, hd);
   dim3 grid(n_rows, H), block(AG_THREADS);
   const size_t smem = (size_t)(hd + 2 * AG_THREADS) * sizeof(float);
   if (dtype == BH_F32)
     attention_generic_kernel<float><<<grid, block, smem, stream>>>(
         (const float*)q, (float*)out, (const float*)k_pages, (const float*)v_pages, page_table, table_stride,
-        row_seq, positions, H, KVH, hd, scale, window);
+        row_seq, positions, H, KVH, hd, scale, window, kv_order);
   else if (dtype == BH_BF16)
     attention_generic_kernel<bf16_t><<<grid, block, smem, stream>>>(
         (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_table,
-        table_stride, row_seq, positions, H, KVH, hd, scale, window);
+        table_stride, row_seq, positions, H, KVH, hd, scale, window, kv_order);
   else
     return bh_fail("attention: unknown dtype %d", dtype);
   return bh_check_launch("attention_generic");

@@ -72,13 +72,14 @@ class HipKernels:
             "bh_embed": [p, p, i, p, i, i, p],
             "bh_rmsnorm": [p, p, p, i, p, i, i, i, f, p],
             "bh_gemm_generic": [p, i, p, i, p, i, i, i, i, i, p],
-            "bh_qk_norm_rope_cache": [p, i, p, p, p, i, f, p, p, i, i, p, p, p, p, p, i, i, i, i, i, i, i, p],
-            "bh_attention_generic": [p, p, i, p, p, p, i, p, p, i, i, i, i, f, i, p],
+            "bh_qk_norm_rope_cache": [p, i, p, p, p, i, f, p, p, i, i, p, p, p, p, p, i, i, i, i, i, i, i, i, p],
+            "bh_attention_generic": [p, p, i, p, p, p, i, p, p, i, i, i, i, f, i, i, p],
             "bh_swiglu": [p, p, i, i, i, p],
             "bh_sample": [p, p, p, p, p, p, p, i, i, p],
             "bh_gemm_bf16": [p, p, p, i, i, i, i, i, i, i, p],
             "bh_attention_bf16": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, i, i, f, i, i, i, p],
             "bh_attention_bf16_splits": [i, i, i, i, i],
+            "bh_kv_order": [i, i],
         }
         for name, argtypes in table.items():
             function = getattr(lib, name)
@@ -223,7 +224,15 @@ class HipKernels:
             table_positions, rot, self._ptr(positions, "positions", (torch.int32,)),
             self._ptr(row_seq, "row_seq", (torch.int32,)), self._ptr(k_pages, "k_pages"), self._ptr(v_pages, "v_pages"),
             self._ptr(page_table, "page_table", (torch.int32,)), page_table.shape[1], n_rows, n_heads, n_kv_heads,
-            head_dim, int(bool(write_kv)), int(max_position), self._stream()))
+            head_dim, int(bool(write_kv)), self.kv_order(k_pages.dtype, head_dim), int(max_position), self._stream()))
+
+    def kv_order(self, dtype, head_dim) -> int:
+        """How the elements of one head lie within a cache page of this element type and head size:
+        0 = keys [token][dim] and values [dim][token]; 1 = regrouped in 16-byte pieces for the
+        matrix-core attention kernel (bfloat16, head sizes in steps of 32).  The kernel that writes
+        the cache and both attention kernels follow it, so a cache is only ever read the way it
+        was written; whoever fills or inspects pages directly has to follow it too."""
+        return int(self.lib.bh_kv_order(BF16 if dtype == torch.bfloat16 else F32, int(head_dim)))
 
     def _check_pages(self, k_pages, v_pages, page_table, n_kv_heads, head_dim, dtype, what):
         expected = (k_pages.shape[0], n_kv_heads, self.page_size, head_dim)
@@ -278,7 +287,8 @@ class HipKernels:
             *common, _code(q, "q"), self._ptr(k_pages, "k_pages"), self._ptr(v_pages, "v_pages"),
             self._ptr(page_table, "page_table", (torch.int32,)), page_table.shape[1],
             self._ptr(row_seq, "row_seq", (torch.int32,)), self._ptr(positions, "positions", (torch.int32,)),
-            n_rows, n_heads, n_kv_heads, head_dim, float(scale), int(window), self._stream()))
+            n_rows, n_heads, n_kv_heads, head_dim, float(scale), int(window), self.kv_order(k_pages.dtype, head_dim),
+            self._stream()))
 
     def swiglu(self, gate_up, out):
         """out[r, i] = silu(gate_up[r, i]) * gate_up[r, F + i]."""

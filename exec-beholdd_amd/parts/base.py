@@ -105,8 +105,9 @@ class LayerCache:
     """The storage of one cache entry as handed to a mixer for one step.
 
     kv need:    k_pages [pages, kv_heads, page_size, head_dim], v_pages [pages, kv_heads, head_dim,
-                page_size]; page_table int32
-                [n_seqs, width] for the sequences of this step, in batch order.
+                page_size], to be written and read through the kernel library only (it orders the
+                elements of a head inside a page as its attention kernels want them); page_table
+                int32 [n_seqs, width] for the sequences of this step, in batch order.
     state need: state [max_slots, *state_shape]; index it with ctx.seq_slot.
     `writes` is False when the schedule lets this layer read another layer's entry.
     """

@@ -161,6 +161,59 @@ def make_cache(n_seqs, lengths, kv_heads, head_dim, dtype, seed, extra_pages=3):
     return k_pages, v_pages, table, keys, values
 
 
+def piece_order(head_dim):
+    """Where key [token, dim] and value [dim, token] lie within one head's share of a page when the cache
+    is kept in 16-byte pieces: written from the description of that order, piece by piece, not from the
+    kernels' index arithmetic.  Piece (t * head_dim/32 + s) * 64 + lane of the keys holds token
+    32 (t/2) + 4 (t%2) + 8 (j/4) + j%4, dims 32 s + 8 g .. + 7 (lane = 16 g + j); piece (dt * 2 + u) * 64 +
+    lane of the values holds dim 16 dt + j, tokens 32 u + 8 g .. + 7."""
+    k_at = torch.full((PAGE, head_dim), -1, dtype=torch.long)
+    v_at = torch.full((head_dim, PAGE), -1, dtype=torch.long)
+    slices = head_dim // 32
+    for lane in range(64):
+        g, j = lane // 16, lane % 16
+        for t in range(4):
+            token = 32 * (t // 2) + 4 * (t % 2) + 8 * (j // 4) + j % 4
+            for s in range(slices):
+                piece = (t * slices + s) * 64 + lane
+                for e in range(8):
+                    k_at[token, 32 * s + 8 * g + e] = piece * 8 + e
+        for dt in range(head_dim // 16):
+            for u in range(2):
+                piece = (dt * 2 + u) * 64 + lane
+                for e in range(8):
+                    v_at[16 * dt + j, 32 * u + 8 * g + e] = piece * 8 + e
+    assert sorted(k_at.reshape(-1).tolist()) == list(range(PAGE * head_dim))       # a permutation
+    assert sorted(v_at.reshape(-1).tolist()) == list(range(PAGE * head_dim))
+    return k_at.reshape(-1), v_at.reshape(-1)
+
+
+def stored(K, k_pages, v_pages):
+    """Pages given as keys [.., token, dim] and values [.., dim, token], on the device in the order the
+    kernels keep them for this element type and head size."""
+    head_dim = k_pages.shape[-1]
+    if K.kv_order(k_pages.dtype, head_dim) == 0:
+        return dev(k_pages), dev(v_pages)
+    k_at, v_at = piece_order(head_dim)
+    lead = k_pages.shape[:2]
+    ks, vs = torch.empty_like(k_pages).reshape(*lead, -1), torch.empty_like(v_pages).reshape(*lead, -1)
+    ks[..., k_at] = k_pages.cpu().reshape(*lead, -1)
+    vs[..., v_at] = v_pages.cpu().reshape(*lead, -1)
+    return dev(ks.reshape(k_pages.shape)), dev(vs.reshape(v_pages.shape))
+
+
+def as_rows(K, k_stored, v_stored):
+    """The inverse of `stored`, on the CPU."""
+    head_dim = k_stored.shape[-1]
+    k_stored, v_stored = k_stored.cpu(), v_stored.cpu()
+    if K.kv_order(k_stored.dtype, head_dim) == 0:
+        return k_stored, v_stored
+    k_at, v_at = piece_order(head_dim)
+    lead = k_stored.shape[:2]
+    return (k_stored.reshape(*lead, -1)[..., k_at].reshape(k_stored.shape),
+            v_stored.reshape(*lead, -1)[..., v_at].reshape(v_stored.shape))
+
+
 def attention_reference(q, keys, values, pos, n_heads, kv_heads, head_dim, scale, window):
     group = n_heads // kv_heads
     first = max(0, pos - window + 1) if window else 0
@@ -198,7 +251,7 @@ def test_attention_decode_rows(K, dtype, n_heads, kv_heads, head_dim, window):
     out = torch.empty(len(lengths), n_heads * head_dim, dtype=dtype, device="cuda:0")
     scale = 1 / math.sqrt(head_dim)
     layout = Layout(True, dev(torch.arange(len(lengths) + 1, dtype=torch.int32)), len(lengths), 1, max(lengths) - 1)
-    K.attention(dev(q), out, dev(kp), dev(vp), dev(table), dev(row_seq), dev(positions), n_heads, kv_heads,
+    K.attention(dev(q), out, *stored(K, kp, vp), dev(table), dev(row_seq), dev(positions), n_heads, kv_heads,
                 head_dim, scale, window, layout=layout)
     for s, n in enumerate(lengths):
         want = attention_reference(q[s].reshape(n_heads, head_dim), keys[s], values[s], n - 1, n_heads, kv_heads,
@@ -226,7 +279,7 @@ def test_attention_decode_with_split_keys_and_garbage_beyond_the_end(K, n_heads,
     scale = 1 / math.sqrt(head_dim)
     layout = Layout(True, dev(torch.arange(len(lengths) + 1, dtype=torch.int32)), len(lengths), 1, max(lengths) - 1)
     assert K.lib.bh_attention_bf16_splits(len(lengths), 1, n_heads, kv_heads, max(lengths) - 1) > 1
-    K.attention(dev(q), out, dev(kp), dev(vp), dev(table), dev(row_seq), dev(positions), n_heads, kv_heads,
+    K.attention(dev(q), out, *stored(K, kp, vp), dev(table), dev(row_seq), dev(positions), n_heads, kv_heads,
                 head_dim, scale, 0, layout=layout)
     assert bool(torch.isfinite(out.float()).all())
     for s, n in enumerate(lengths):
@@ -250,7 +303,7 @@ def test_attention_prefill_rows_ragged(K, dtype, n_heads, kv_heads, head_dim):
     starts = torch.tensor(np.concatenate([[0], np.cumsum(news)]), dtype=torch.int32)
     out = torch.empty(n_rows, n_heads * head_dim, dtype=dtype, device="cuda:0")
     scale = 1 / math.sqrt(head_dim)
-    K.attention(dev(q), out, dev(kp), dev(vp), dev(table), dev(row_seq), dev(positions), n_heads, kv_heads,
+    K.attention(dev(q), out, *stored(K, kp, vp), dev(table), dev(row_seq), dev(positions), n_heads, kv_heads,
                 head_dim, scale, 0, layout=Layout(False, dev(starts), len(lengths), max(news), max(lengths) - 1))
     worst = 0.0
     for row in range(n_rows):
@@ -280,7 +333,7 @@ def test_attention_finds_one_far_key_among_hundreds(K, dtype, far):
     grouped = Layout(False, dev(torch.tensor([0, 2], dtype=torch.int32)), 1, 2, n - 1)
     for layout in (None, grouped):          # the kernel for any size, and the matrix-core kernel
         out = torch.empty(2, n_heads * head_dim, dtype=dtype, device="cuda:0")
-        K.attention(dev(q), out, dev(kp), dev(vp), dev(table), dev(row_seq), dev(positions), n_heads, kv_heads,
+        K.attention(dev(q), out, *stored(K, kp, vp), dev(table), dev(row_seq), dev(positions), n_heads, kv_heads,
                     head_dim, 1 / math.sqrt(head_dim), 0, layout=layout)
         got = out.float().cpu().reshape(2, n_heads, head_dim)
         for h in range(n_heads):
@@ -301,7 +354,7 @@ def test_attention_window_edge(K, dtype):
         kp[page, :, where % PAGE] = (direction * (40 if where == outside else 25)).to(dtype)
     q = (direction * 30).repeat(n_heads).reshape(1, -1).to(dtype)
     out = torch.empty(1, n_heads * head_dim, dtype=dtype, device="cuda:0")
-    args = (dev(kp), dev(vp), dev(table), dev(torch.zeros(1, dtype=torch.int32)), dev(torch.tensor([pos], dtype=torch.int32)),
+    args = (*stored(K, kp, vp), dev(table), dev(torch.zeros(1, dtype=torch.int32)), dev(torch.tensor([pos], dtype=torch.int32)),
             n_heads, kv_heads, head_dim, 1 / math.sqrt(head_dim))
     K.attention(dev(q), out, *args, window)
     assert torch.allclose(out.float().cpu().reshape(n_heads, head_dim)[0], values[0][inside, 0].float(), atol=2e-2)
@@ -332,7 +385,7 @@ def test_qk_norm_rope_cache(K, dtype, w_dtype, n_heads, kv_heads, head_dim, rot)
     sentinel = 768.0        # exact in bfloat16
     kp = torch.full((n_pages, kv_heads, PAGE, head_dim), sentinel).to(dtype)
     vp = torch.full((n_pages, kv_heads, head_dim, PAGE), sentinel).to(dtype)
-    kp_d, vp_d = dev(kp), dev(vp)
+    kp_d, vp_d = stored(K, kp, vp)
     q_out = torch.empty(n_rows, n_heads * head_dim, dtype=dtype, device="cuda:0")
     K.qk_norm_rope_cache(dev(qkv), q_out, dev(qw), dev(kw), eps, dev(cos), dev(sin), dev(positions), dev(row_seq),
                          kp_d, vp_d, dev(table), n_heads, kv_heads, head_dim, True, int(positions.max()))
@@ -345,6 +398,7 @@ def test_qk_norm_rope_cache(K, dtype, w_dtype, n_heads, kv_heads, head_dim, rot)
         return torch.cat([a * c - b * s, a * s + b * c, y[:, rot:]], dim=-1)
 
     written = torch.zeros(n_pages, PAGE, dtype=torch.bool)
+    kp_d, vp_d = as_rows(K, kp_d, vp_d)
     for row in range(n_rows):
         pos, seq = int(positions[row]), int(row_seq[row])
         x = qkv[row].double()
@@ -361,7 +415,7 @@ def test_qk_norm_rope_cache(K, dtype, w_dtype, n_heads, kv_heads, head_dim, rot)
     assert bool((kp_d.cpu().float()[untouched] == sentinel).all())
     assert bool((vp_d.cpu().float().transpose(2, 3)[untouched] == sentinel).all())
     # without weights and tables the heads pass through; without write_kv the cache stays as it is
-    kp2, vp2 = dev(kp), dev(vp)
+    kp2, vp2 = stored(K, kp, vp)
     K.qk_norm_rope_cache(dev(qkv), q_out, None, None, 0.0, None, None, dev(positions), dev(row_seq), kp2, vp2,
                          dev(table), n_heads, kv_heads, head_dim, False, int(positions.max()))
     assert torch.equal(q_out.cpu(), qkv[:, :n_heads * head_dim])
