@@ -295,10 +295,8 @@ extern "C" int bh_attention_bf16_splits(int n_seqs, int max_rows_per_seq, int H,
   const long tiles = (long)((max_rows_per_seq * G + 15) / 16) * KVH * n_seqs;
   const int pages = max_position / BH_PAGE + 1;
   // about one workgroup per compute unit (256), every wave of a workgroup at least one page
-  const char* env = getenv("BH_ATT_TARGET");
-  const long target = env ? atol(env) : 256;
-  if (tiles >= target || pages < 8) return 1;
-  long want = (target + tiles - 1) / tiles;
+  if (tiles >= 256 || pages < 8) return 1;
+  long want = (256 + tiles - 1) / tiles;
   if (want > pages / 4) want = pages / 4;
   if (want < 1) want = 1;
   const int per = (int)((pages + want - 1) / want);
