@@ -1,4 +1,6 @@
-// bfloat16 attention over the paged cache on the gfx950 matrix cores, for prefill and decode.
+// bfloat16 attention over the paged cache on the gfx950 matrix cores: the kernel for few columns per
+// sequence (decode, short steps) and the entry point, which hands steps with many columns per sequence
+// to the prefill kernel (attention_prefill_bf16.hip).
 //
 // A *column* is one (row, query head) pair.  A workgroup takes 16 columns that share a sequence
 // and a kv head (consecutive rows x the heads of one group) and a range of that sequence's cache
@@ -23,68 +25,26 @@
 // head_dim must be a multiple of 32, at most 256.  Masking is by position: column j sees keys
 // lo_j .. pos_j.  Rows of a page beyond the last written key are never multiplied in: their
 // probabilities are zero and their V values are zeroed before use.
-#include "common.h"
+#include "attention_bf16.h"
 
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
-typedef float f32x8_t __attribute__((ext_vector_type(8)));
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-
-__device__ inline bf16x8_t as_bf16x8(u32x4_t v) { return __builtin_bit_cast(bf16x8_t, v); }
-__device__ inline u32x4_t load16(const uint16_t* p) { return *reinterpret_cast<const u32x4_t*>(p); }
-template <bool STREAM>
-__device__ inline u32x4_t load16_cache(const uint16_t* p) {   // STREAM: nobody else reads these bytes soon
-  if (STREAM) return __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
-  return *reinterpret_cast<const u32x4_t*>(p);
-}
-
-__device__ inline int wave_max_int(int v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = max(v, __shfl_xor(v, off, 64));
-  return v;
-}
-__device__ inline int wave_min_int(int v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = min(v, __shfl_xor(v, off, 64));
-  return v;
-}
-
-typedef float f32x2_t __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-
-// two float32 values rounded to nearest-even bfloat16 and packed (one v_cvt_pk_bf16_f32)
-__device__ inline uint32_t pack_bf16(float lo, float hi) {
-  const f32x2_t v = {lo, hi};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
-}
-
-// keep the first `n_valid` (0..8) bfloat16 elements of a 16-byte vector, zero the rest
-__device__ inline u32x4_t keep_first(u32x4_t v, int n_valid) {
-#pragma unroll
-  for (int word = 0; word < 4; ++word) {
-    const uint32_t mask = (2 * word + 1 < n_valid) ? 0xffffffffu : (2 * word < n_valid ? 0x0000ffffu : 0u);
-    v[word] &= mask;
-  }
-  return v;
-}
-
-// NS = head_dim / 32.  CT = column tiles (of 16 columns) per workgroup: every page a wave loads is
-// used for all CT tiles, which divides the cache traffic of a prefill by CT.
+// NS = head_dim / 32.
 // STREAM = one workgroup per (sequence, kv head, split): each cache byte is read once, past the caches.
-template <int NS, int CT, bool STREAM>
+template <int NS, bool STREAM>
 __global__ __launch_bounds__(256) void attention_mfma_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages,
     const int32_t* __restrict__ page_table, int table_stride, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ seq_start, int H, int KVH, float scale_log2, int window, int n_splits,
-    int pages_per_split) {
+    int pages_per_split, int tile_groups) {
   constexpr int HD = 32 * NS;
+  constexpr int CT = 1;   // column tiles per workgroup
   __shared__ float sm_m[4][16];
   __shared__ float sm_l[4][16];
   __shared__ float sm_o[4][16][HD + 1];
 
-  const int tile0 = blockIdx.x * CT, kvh = blockIdx.y;
-  const int seq = blockIdx.z / n_splits, split = blockIdx.z % n_splits;
+  const int tile_group = blockIdx.x % tile_groups, unit = blockIdx.x / tile_groups;
+  const int tile0 = tile_group * CT, kvh = unit % KVH, z = unit / KVH;
+  const int seq = z / n_splits, split = z % n_splits;
   const int G = H / KVH;
   const int row0 = seq_start[seq];
   const int n_cols = (seq_start[seq + 1] - row0) * G;
@@ -317,23 +277,24 @@ extern "C" int bh_attention_bf16(const void* q, void* out, void* part_o, void* p
   const int tiles = (max_rows_per_seq * G + 15) / 16;
   const int pages = max_position / BH_PAGE + 1;
   const int per = (pages + n_splits - 1) / n_splits;
-  // several column tiles per workgroup when there are many (prefill): the cache is read that many times less
-  const int ct = (n_splits == 1 && hd <= 128 && (long)tiles * KVH * n_seqs >= 2048) ? 4
-               : (n_splits == 1 && (long)tiles * KVH * n_seqs >= 1024) ? 2 : 1;
-  BH_REQUIRE((long)n_seqs * n_splits <= 65535 && KVH <= 65535, "attention_bf16: too many sequences x splits");
-  dim3 grid((tiles + ct - 1) / ct, KVH, n_seqs * n_splits), block(256);
   const float scale_log2 = scale * 1.4426950408889634f;
-#define BH_ATT_CT(NS, CT, STREAM)                                                                               \
-  attention_mfma_kernel<NS, CT, STREAM><<<grid, block, 0, stream>>>(                                            \
+  BH_REQUIRE((long)tiles * KVH * n_seqs * n_splits < (1L << 31), "attention_bf16: too many workgroups");
+  if (n_splits == 1 && (long)tiles * KVH * n_seqs >= 1024) {   // many columns: the prefill kernel
+    bh_attention_prefill_launch(q, out, k_pages, v_pages, page_table, table_stride, positions, seq_start, n_seqs,
+                                tiles, H, KVH, hd, scale_log2, window, stream);
+    return bh_check_launch("attention_prefill_bf16");
+  }
+  const int tile_groups = tiles, z_count = n_seqs * n_splits;
+  dim3 grid(tile_groups * KVH * z_count), block(256);
+#define BH_ATT_ONE(NS, STREAM)                                                                                  \
+  attention_mfma_kernel<NS, STREAM><<<grid, block, 0, stream>>>(                                                \
       (const uint16_t*)q, (uint16_t*)out, (float*)part_o, (float*)part_ml, (const uint16_t*)k_pages,            \
       (const uint16_t*)v_pages, page_table, table_stride, positions, seq_start, H, KVH, scale_log2, window,     \
-      n_splits, per)
-#define BH_ATT(NS)                                 \
-  do {                                             \
-    if (ct == 4) BH_ATT_CT(NS, 4, false);          \
-    else if (ct == 2) BH_ATT_CT(NS, 2, false);     \
-    else if (grid.x == 1) BH_ATT_CT(NS, 1, true);  \
-    else BH_ATT_CT(NS, 1, false);                  \
+      n_splits, per, tile_groups)
+#define BH_ATT(NS)                               \
+  do {                                           \
+    if (tile_groups == 1) BH_ATT_ONE(NS, true);  \
+    else BH_ATT_ONE(NS, false);                  \
   } while (0)
   switch (hd / 32) {
     case 1: BH_ATT(1); break;
@@ -346,7 +307,7 @@ extern "C" int bh_attention_bf16(const void* q, void* out, void* part_o, void* p
     default: BH_ATT(8); break;
   }
 #undef BH_ATT
-#undef BH_ATT_CT
+#undef BH_ATT_ONE
   if (int status = bh_check_launch("attention_mfma")) return status;
   if (n_splits > 1) {
     attention_combine_kernel<<<dim3(n_rows * H), dim3(hd >= 128 ? 128 : 64), 0, stream>>>(

@@ -1,0 +1,265 @@
+// bfloat16 attention for steps with many rows per sequence (prefill), on the gfx950 matrix cores.
+//
+// The decode kernel (attention_bf16.hip) gives every wave of a workgroup different cache pages and the
+// same columns, and merges the waves at the end: right for few columns and long caches.  Here it is
+// the other way round.  A workgroup takes 64 * CTW columns of one (sequence, kv head); each of its
+// four waves owns CTW tiles of 16 columns for the whole kernel (its queries, running maximum and sum,
+// output accumulators), and all four walk over the same cache pages.  A page's keys and values are
+// brought into LDS once per workgroup (through registers, the next page while the current one is
+// multiplied) and every wave reads its matrix-core operands from there: the cache keeps a page in
+// 16-byte pieces in exactly the order the lanes take them (BH_KV_PIECES), so the copy is linear and
+// the LDS reads are conflict-free.  Nothing is merged at the end, a wave holds accumulators for its
+// own columns only, and two workgroups fit a compute unit at head size 128.
+//
+// Products, softmax and masking are those of the decode kernel:
+//     S^T[key, column] = K[key, :] . Q[column, :],   tile t, row i <-> key 32 (t/2) + 4 (t%2) + 8 (i/4) + i%4
+//     online softmax per column in float32, exponent base 2
+//     O^T[d, column] += V^T[d, key] . P^T[key, column]
+// A wave skips pages none of whose keys any of its columns may see.  Values beyond the last position
+// of the workgroup's columns are zeroed on their way into LDS (their probabilities are zero, but what
+// lies there may be anything).
+#include "attention_bf16.h"
+
+template <int NS, int CTW>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2 : 1))) void attention_prefill_kernel(
+    const uint16_t* __restrict__ q, uint16_t* __restrict__ out, const uint16_t* __restrict__ k_pages,
+    const uint16_t* __restrict__ v_pages, const int32_t* __restrict__ page_table, int table_stride,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_start, int H, int KVH,
+    float scale_log2, int window, int tile_groups, int n_seqs) {
+  constexpr int HD = 32 * NS;
+  constexpr int PIECES = BH_PAGE * HD / 8;        // 16-byte pieces of one head's keys (or values) in a page
+  constexpr int STAGE = 2 * PIECES / 256;         // pieces of a page (keys, then values) one thread copies
+  constexpr int GROUP_TILES = 4 * CTW;            // column tiles of a workgroup
+  __shared__ u32x4_t page_lds[2][2 * PIECES];
+
+  // Workgroups go to the eight XCDs in turn, each with an L2 of its own: when the number of
+  // (kv head, sequence) units allows it, all tile groups of a unit run on one XCD, one after the other,
+  // so that the unit's keys and values stay in that L2; and the groups with the most keys (the last
+  // rows of a causal prefill) start first.
+  int tile_group, unit;
+  const int units = KVH * n_seqs;
+  if (units % 8 == 0) {
+    const int xcd = blockIdx.x % 8, turn = blockIdx.x / 8;
+    tile_group = tile_groups - 1 - turn % tile_groups;
+    unit = (turn / tile_groups) * 8 + xcd;
+  } else {
+    tile_group = tile_groups - 1 - blockIdx.x % tile_groups;
+    unit = blockIdx.x / tile_groups;
+  }
+  const int kvh = unit % KVH, seq = unit / KVH;
+  const int G = H / KVH;
+  const int row0 = seq_start[seq];
+  const int n_cols = (seq_start[seq + 1] - row0) * G;
+  const int group_col0 = tile_group * GROUP_TILES * 16;
+  if (group_col0 >= n_cols) return;                // the whole workgroup: no barrier is left behind
+
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int j = lane % 16, g = lane / 16;
+
+  // rows of a sequence are consecutive and in position order: the workgroup's first and last row bound its keys
+  const int group_last_col = min(n_cols, group_col0 + GROUP_TILES * 16) - 1;
+  const int group_pos_max = positions[row0 + group_last_col / G];
+  const int group_pos_first = positions[row0 + group_col0 / G];
+  const int group_lo_min = (window > 0 && group_pos_first - window + 1 > 0) ? group_pos_first - window + 1 : 0;
+  const int begin = group_lo_min / BH_PAGE, last = group_pos_max / BH_PAGE;
+  const int32_t* table = page_table + (size_t)seq * table_stride;
+
+  // this wave's columns
+  const int wave_tile0 = tile_group * GROUP_TILES + wave * CTW;
+  const bool wave_active = wave_tile0 * 16 < n_cols;
+  int pos[CTW], lo[CTW];
+  bf16x8_t q_vec[CTW][NS];
+  int pos_max = 0, pos_min = 0x7fffffff, lo_min = 0x7fffffff, lo_max = 0;
+#pragma unroll
+  for (int ct = 0; ct < CTW; ++ct) {
+    const int wanted = (wave_tile0 + ct) * 16 + j;
+    const int c = wanted < n_cols ? wanted : n_cols - 1;
+    const int row = row0 + c / G, head = kvh * G + c % G;
+    pos[ct] = positions[row];
+    lo[ct] = (window > 0 && pos[ct] - window + 1 > 0) ? pos[ct] - window + 1 : 0;
+    pos_max = max(pos_max, pos[ct]);
+    pos_min = min(pos_min, pos[ct]);
+    lo_min = min(lo_min, lo[ct]);
+    lo_max = max(lo_max, lo[ct]);
+    const uint16_t* qp = q + ((size_t)row * H + head) * HD + 8 * g;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) q_vec[ct][s] = as_bf16x8(load16(qp + 32 * s));
+  }
+  pos_max = wave_max_int(pos_max);
+  pos_min = wave_min_int(pos_min);
+  lo_min = wave_min_int(lo_min);
+  lo_max = wave_max_int(lo_max);
+
+  f32x4_t o[CTW][2 * NS];
+  float run_max[CTW], run_sum[CTW];  // run_sum: this lane's share of the column's sum
+#pragma unroll
+  for (int ct = 0; ct < CTW; ++ct) {
+    run_max[ct] = -INFINITY;
+    run_sum[ct] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < 2 * NS; ++dt) o[ct][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+
+  // global -> registers -> LDS, piece by piece: thread `tid` copies pieces tid, tid + 256, ... of the
+  // page's keys and then of its values
+  u32x4_t stage[STAGE];
+  auto fetch = [&](int p) {
+    const int page = table[p];
+    const uint16_t* kb = k_pages + ((size_t)page * KVH + kvh) * BH_PAGE * HD;
+    const uint16_t* vb = v_pages + ((size_t)page * KVH + kvh) * HD * BH_PAGE;
+#pragma unroll
+    for (int i = 0; i < STAGE; ++i) {
+      const int piece = tid + i * 256;
+      stage[i] = load16(piece < PIECES ? kb + (size_t)piece * 8 : vb + (size_t)(piece - PIECES) * 8);
+    }
+  };
+  auto stash = [&](int p, int buffer) {
+    const bool tail = p * BH_PAGE + BH_PAGE - 1 > group_pos_max;   // the page's tail was never written
+#pragma unroll
+    for (int i = 0; i < STAGE; ++i) {
+      const int piece = tid + i * 256;
+      u32x4_t v = stage[i];
+      if (tail && piece >= PIECES) {
+        // value piece (dt * 2 + u) * 64 + l holds tokens 32 u + 8 (l / 16) .. + 7 of the page
+        const int pv = piece - PIECES;
+        const int first_token = p * BH_PAGE + 32 * ((pv / 64) % 2) + 8 * ((pv % 64) / 16);
+        v = keep_first(v, group_pos_max + 1 - first_token);
+      }
+      page_lds[buffer][piece] = v;
+    }
+  };
+
+  fetch(begin);
+  stash(begin, 0);
+  __syncthreads();
+  for (int p = begin; p <= last; ++p) {
+    const int buffer = (p - begin) & 1;
+    if (p < last) fetch(p + 1);
+    const u32x4_t* kl = page_lds[buffer];
+    const u32x4_t* vl = page_lds[buffer] + PIECES;
+    // a page none of whose keys this wave's columns may see changes nothing
+    const bool visible = wave_active && p * BH_PAGE <= pos_max && p * BH_PAGE + BH_PAGE - 1 >= lo_min;
+    if (visible) {
+      f32x4_t st[CTW][4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+#pragma unroll
+        for (int ct = 0; ct < CTW; ++ct) st[ct][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+          const bf16x8_t kf = as_bf16x8(kl[(t * NS + s) * 64 + lane]);
+#pragma unroll
+          for (int ct = 0; ct < CTW; ++ct)
+            st[ct][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, q_vec[ct][s], st[ct][t], 0, 0, 0);
+        }
+      }
+      const int key0 = p * BH_PAGE + 8 * g;  // lane (j, g) holds keys key0 + 32 * (t / 2) + 4 * (t % 2) + r
+      const bool mask_needed = (p * BH_PAGE + BH_PAGE - 1 > pos_min) || (p * BH_PAGE < lo_max);
+      u32x4_t p_vec[CTW][2];
+#pragma unroll
+      for (int ct = 0; ct < CTW; ++ct) {
+        if (mask_needed) {
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int key = key0 + 32 * (t / 2) + 4 * (t % 2) + r;
+              if (key > pos[ct] || key < lo[ct]) st[ct][t][r] = -INFINITY;
+            }
+        }
+        // Online softmax with few instructions: the maximum is taken over the raw scores, the scale
+        // enters through one fused multiply-add per score, and the exponentials are bare v_exp_f32
+        // (arguments <= 0; results below the normal range may flush to zero).
+        float local_max = fmaxf(fmaxf(st[ct][0][0], st[ct][0][1]), fmaxf(st[ct][0][2], st[ct][0][3]));
+#pragma unroll
+        for (int t = 1; t < 4; ++t)
+          local_max = fmaxf(local_max, fmaxf(fmaxf(st[ct][t][0], st[ct][t][1]), fmaxf(st[ct][t][2], st[ct][t][3])));
+        local_max = fmaxf(local_max, __shfl_xor(local_max, 16, 64));
+        local_max = fmaxf(local_max, __shfl_xor(local_max, 32, 64));
+        const float new_max = fmaxf(run_max[ct], local_max);              // raw (unscaled) scores
+        const float shift = (new_max == -INFINITY) ? 0.f : -new_max * scale_log2;
+        // exactly 1 while the maximum stands still, 0 when nothing was seen before
+        const float alpha =
+            (run_max[ct] == new_max) ? 1.0f : __builtin_amdgcn_exp2f((run_max[ct] - new_max) * scale_log2);
+        float page_sum = 0.f;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int half = 0; half < 2; ++half) {
+            const int t = 2 * u + half;
+            const float e0 = __builtin_amdgcn_exp2f(fmaf(st[ct][t][0], scale_log2, shift));
+            const float e1 = __builtin_amdgcn_exp2f(fmaf(st[ct][t][1], scale_log2, shift));
+            const float e2 = __builtin_amdgcn_exp2f(fmaf(st[ct][t][2], scale_log2, shift));
+            const float e3 = __builtin_amdgcn_exp2f(fmaf(st[ct][t][3], scale_log2, shift));
+            page_sum += (e0 + e1) + (e2 + e3);
+            p_vec[ct][u][2 * half] = pack_bf16(e0, e1);
+            p_vec[ct][u][2 * half + 1] = pack_bf16(e2, e3);
+          }
+        run_sum[ct] = run_sum[ct] * alpha + page_sum;
+        run_max[ct] = new_max;
+        if (__any(alpha != 1.0f)) {   // after the first pages the maximum seldom moves
+#pragma unroll
+          for (int dt = 0; dt < 2 * NS; ++dt) o[ct][dt] = o[ct][dt] * alpha;
+        }
+      }
+#pragma unroll
+      for (int dt = 0; dt < 2 * NS; ++dt) {
+        const bf16x8_t v0 = as_bf16x8(vl[(dt * 2) * 64 + lane]);
+        const bf16x8_t v1 = as_bf16x8(vl[(dt * 2 + 1) * 64 + lane]);
+#pragma unroll
+        for (int ct = 0; ct < CTW; ++ct) {
+          f32x4_t acc = o[ct][dt];
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v0, as_bf16x8(p_vec[ct][0]), acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v1, as_bf16x8(p_vec[ct][1]), acc, 0, 0, 0);
+          o[ct][dt] = acc;
+        }
+      }
+    }
+    if (p < last) stash(p + 1, buffer ^ 1);
+    __syncthreads();   // the next page is in place, and everyone is done with the one before it
+  }
+
+  // lane (j, g) holds O^T[16 dt + 4 g + r, column j] and its share of the column's sum
+#pragma unroll
+  for (int ct = 0; ct < CTW; ++ct) {
+    const int cc = (wave_tile0 + ct) * 16 + j;
+    float total = run_sum[ct];
+    total += __shfl_xor(total, 16, 64);
+    total += __shfl_xor(total, 32, 64);
+    if (cc >= n_cols) continue;
+    const float inv = 1.0f / total;
+    uint16_t* op = out + ((size_t)(row0 + cc / G) * H + kvh * G + cc % G) * HD + 4 * g;
+#pragma unroll
+    for (int dt = 0; dt < 2 * NS; ++dt) {
+      uint2 packed;
+      packed.x = pack_bf16(o[ct][dt][0] * inv, o[ct][dt][1] * inv);
+      packed.y = pack_bf16(o[ct][dt][2] * inv, o[ct][dt][3] * inv);
+      *reinterpret_cast<uint2*>(op + 16 * dt) = packed;
+    }
+  }
+}
+
+void bh_attention_prefill_launch(const void* q, void* out, const void* k_pages, const void* v_pages,
+                                 const int32_t* page_table, int table_stride, const int32_t* positions,
+                                 const int32_t* seq_start, int n_seqs, int tiles, int H, int KVH, int hd,
+                                 float scale_log2, int window, hipStream_t stream) {
+#define BH_PREFILL(NS, CTW)                                                                                  \
+  do {                                                                                                       \
+    const int tile_groups = (tiles + 4 * CTW - 1) / (4 * CTW);                                               \
+    attention_prefill_kernel<NS, CTW><<<dim3(tile_groups * KVH * n_seqs), dim3(256), 0, stream>>>(           \
+        (const uint16_t*)q, (uint16_t*)out, (const uint16_t*)k_pages, (const uint16_t*)v_pages, page_table,  \
+        table_stride, positions, seq_start, H, KVH, scale_log2, window, tile_groups, n_seqs);                \
+  } while (0)
+  // two column tiles per wave while the accumulators leave room for two workgroups per compute unit
+  switch (hd / 32) {
+    case 1: BH_PREFILL(1, 2); break;
+    case 2: BH_PREFILL(2, 2); break;
+    case 3: BH_PREFILL(3, 2); break;
+    case 4: BH_PREFILL(4, 2); break;
+    case 5: BH_PREFILL(5, 1); break;
+    case 6: BH_PREFILL(6, 1); break;
+    case 7: BH_PREFILL(7, 1); break;
+    default: BH_PREFILL(8, 1); break;
+  }
+#undef BH_PREFILL
+}

@@ -314,6 +314,55 @@ def test_attention_prefill_rows_ragged(K, dtype, n_heads, kv_heads, head_dim):
     assert worst < tol(dtype, 1e-5, 1.2e-2), worst
 
 
+def attention_reference_rows(q, keys, values, positions, n_heads, kv_heads, head_dim, scale, window):
+    """All rows of one sequence at once: q [rows, heads * head_dim], row r at position positions[r]."""
+    rows, group = q.shape[0], n_heads // kv_heads
+    qh = q.double().reshape(rows, kv_heads, group, head_dim)
+    scores = torch.einsum("rkgd,nkd->rkgn", qh, keys.double()) * scale
+    key_at = torch.arange(keys.shape[0])[None, :]
+    hidden = key_at > positions[:, None]
+    if window:
+        hidden |= key_at < positions[:, None] - window + 1
+    scores = scores.masked_fill(hidden[:, None, None, :], float("-inf"))
+    return torch.einsum("rkgn,nkd->rkgd", torch.softmax(scores, -1), values.double()).reshape(rows, n_heads * head_dim)
+
+
+@pytest.mark.parametrize("window", [0, 100])
+@pytest.mark.parametrize("n_heads,kv_heads,head_dim", [(32, 8, 128), (8, 2, 64), (6, 1, 96), (4, 4, 256), (2, 2, 32),
+                                                       (4, 2, 160)])
+def test_attention_prefill_many_columns(K, n_heads, kv_heads, head_dim, window):
+    """Steps wide enough for the kernel that keeps a page in LDS for four waves with columns of their own:
+    several sequences with pasts, ends that fill neither a tile nor a workgroup, NaN beyond the last key."""
+    dtype = torch.bfloat16
+    group = n_heads // kv_heads
+    longest = -(-1024 * 16 // (n_heads * 3)) + 40
+    pasts, news = [0, 70, 129], [longest, longest // 2 + 3, 65]
+    assert -(-max(news) * group // 16) * kv_heads * len(news) >= 1024      # what sends a step to that kernel
+    lengths = [p + n for p, n in zip(pasts, news)]
+    kp, vp, table, keys, values = make_cache(len(lengths), lengths, kv_heads, head_dim, dtype, seed=head_dim + n_heads)
+    for s, n in enumerate(lengths):
+        if n % PAGE:
+            page = int(table[s, (n - 1) // PAGE])
+            kp[page, :, n % PAGE:, :] = float("nan")
+            vp[page, :, :, n % PAGE:] = float("nan")
+    g = torch.Generator().manual_seed(13)
+    n_rows = sum(news)
+    q = torch.randn(n_rows, n_heads * head_dim, generator=g).to(dtype)
+    positions = torch.tensor([p + t for p, n in zip(pasts, news) for t in range(n)], dtype=torch.int32)
+    row_seq = torch.tensor([s for s, n in enumerate(news) for _ in range(n)], dtype=torch.int32)
+    starts = torch.tensor(np.concatenate([[0], np.cumsum(news)]), dtype=torch.int32)
+    out = torch.empty(n_rows, n_heads * head_dim, dtype=dtype, device="cuda:0")
+    scale = 1 / math.sqrt(head_dim)
+    K.attention(dev(q), out, *stored(K, kp, vp), dev(table), dev(row_seq), dev(positions), n_heads, kv_heads,
+                head_dim, scale, window, layout=Layout(False, dev(starts), len(lengths), max(news), max(lengths) - 1))
+    assert bool(torch.isfinite(out.float()).all())
+    for s in range(len(news)):
+        rows = slice(int(starts[s]), int(starts[s + 1]))
+        want = attention_reference_rows(q[rows], keys[s], values[s], positions[rows].long(), n_heads, kv_heads,
+                                        head_dim, scale, window)
+        assert rel(out[rows], want) < 1.2e-2, (s, rel(out[rows], want))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("far", [0, 63, 64, 127, 128, 300, 511, 640])
 def test_attention_finds_one_far_key_among_hundreds(K, dtype, far):
