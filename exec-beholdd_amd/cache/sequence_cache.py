@@ -244,6 +244,7 @@ class SequenceCache:
                     page = pages.pop()
                     if page >= 0:
                         g.free_pages.append(page)
+                g.pages_of[slot] = list(pages)   # a new list: whoever remembers the old one sees that entries went away
 
     # ---- what kernels and mixers get ----
     def page_table_rows(self, group: _Group, slots: list) -> list:

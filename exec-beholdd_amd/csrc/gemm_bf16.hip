@@ -59,12 +59,44 @@ __device__ inline float silu_mul(float gate, float up) { return gate / (1.0f + e
 // ---- skinny --------------------------------------------------------------------------------
 // RT = 1: plain product.  RT = 2: SwiGLU; the second row block lies `pair_blocks` blocks after the first.
 
+// An RMSNorm between two products can ride on them (struct SkinnyNorm):
+//   behind: the product that completes the float32 residual h also writes bfloat16(h[m][n] * g[n]) (the
+//           norm's output but for the row factor) and, per workgroup, the sum of h[m][n]^2 over its 16
+//           columns;
+//   ahead:  the product that consumes the norm's output takes those unscaled rows as its activations and
+//           multiplies its result by 1 / sqrt(sum of the partial sums / K + eps) of the row.
+// The row factor commutes with the product, so the result is the norm's up to the rounding of the
+// activations; the partial sums are added in a fixed order.
+struct SkinnyNorm {
+  const float* ahead_ss;   // [ahead_blocks][M] partial sums of squares for the rows of `a`, or null
+  int ahead_blocks;
+  float ahead_eps;
+  const void* behind_weight;  // [N] norm weight for the rows this product completes, or null
+  int behind_weight_f32;      // its element type: float32, else bfloat16
+  uint16_t* behind_rows;      // [M][N] bfloat16 out
+  float* behind_ss;           // [ceil(N / 16)][M] out
+};
+
 template <int MB, int WAVES, bool TILES, int RT, typename TC>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t* __restrict__ a,
                                                                  const uint16_t* __restrict__ w,
                                                                  TC* __restrict__ c, int M, int N, int K,
-                                                                 int accumulate, int pair_blocks) {
+                                                                 int accumulate, int pair_blocks,
+                                                                 SkinnyNorm norm) {
   __shared__ float partial[WAVES][RT][MB][256];
+  __shared__ float row_factor[MB * 16];
+  if (norm.ahead_ss) {
+    // 32 threads per row: each adds every 32nd partial sum, then the 32 are added pairwise
+    for (int r0 = 0; r0 < MB * 16; r0 += WAVES * 2) {
+      const int r = r0 + threadIdx.x / 32, part = threadIdx.x % 32;
+      float ss = 0.f;
+      if (r < M)
+        for (int block = part; block < norm.ahead_blocks; block += 32) ss += norm.ahead_ss[(size_t)block * M + r];
+#pragma unroll
+      for (int off = 16; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+      if (part == 0 && r < MB * 16) row_factor[r] = (r < M) ? 1.0f / sqrtf(ss / (float)K + norm.ahead_eps) : 0.f;
+    }
+  }
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int i = lane % 16, g = lane / 16;
   const int n0 = blockIdx.x * 16;
@@ -161,20 +193,42 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
 #pragma unroll
       for (int r = 0; r < 4; ++r) partial[wave][t][b][i * 16 + 4 * g + r] = acc[t][b][r];
   __syncthreads();
-  for (int e = threadIdx.x; e < MB * 256; e += WAVES * 64) {
+  for (int e = threadIdx.x; e < MB * 256; e += WAVES * 64) {   // whole waves enter or stay out
     const int b = e / 256, m = b * 16 + (e % 256) / 16, n = n0 + e % 16;
-    if (m >= M || n >= N) continue;
+    const bool valid = m < M && n < N;
     float sum[RT];
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
       sum[t] = 0.f;
 #pragma unroll
       for (int v = 0; v < WAVES; ++v) sum[t] += partial[v][t][b][e % 256];
+      if (norm.ahead_ss) sum[t] *= row_factor[m];
     }
-    if (RT == 2)
-      store_out<TC>(c, (size_t)m * N + n, silu_mul(sum[0], sum[RT - 1]), false);
-    else
-      store_out<TC>(c, (size_t)m * N + n, sum[0], accumulate != 0);
+    float value = 0.f;   // what the residual holds afterwards (norm.behind_weight: float32 output, RT == 1)
+    if (valid) {
+      if (RT == 2) {
+        store_out<TC>(c, (size_t)m * N + n, silu_mul(sum[0], sum[RT - 1]), false);
+      } else if (norm.behind_weight) {
+        float* cf = reinterpret_cast<float*>(c);
+        value = accumulate ? cf[(size_t)m * N + n] + sum[0] : sum[0];
+        cf[(size_t)m * N + n] = value;
+      } else {
+        store_out<TC>(c, (size_t)m * N + n, sum[0], accumulate != 0);
+      }
+    }
+    if (RT == 1 && norm.behind_weight) {
+      float sq = value * value;   // 0 where there is no element
+      sq += __shfl_xor(sq, 8, 64);   // the 16 columns of a row sit in 16 neighbouring lanes
+      sq += __shfl_xor(sq, 4, 64);
+      sq += __shfl_xor(sq, 2, 64);
+      sq += __shfl_xor(sq, 1, 64);
+      if (valid) {
+        const float g = norm.behind_weight_f32 ? reinterpret_cast<const float*>(norm.behind_weight)[n]
+                                               : bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(norm.behind_weight)[n]);
+        norm.behind_rows[(size_t)m * N + n] = f32_to_bf16_bits(value * g);
+        if (e % 16 == 0) norm.behind_ss[(size_t)blockIdx.x * M + m] = sq;
+      }
+    }
   }
 }
 
@@ -340,12 +394,12 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const uint16_t
 
 template <bool TILES, int RT, typename TC>
 static void launch_skinny(const void* a, const void* w, void* c, int M, int N, int K, int accumulate,
-                          int pair_blocks, hipStream_t stream) {
+                          int pair_blocks, const SkinnyNorm& norm, hipStream_t stream) {
   constexpr int WAVES = 8;
   dim3 grid((N + 15) / 16), block(WAVES * 64);
 #define BH_SKINNY(MB)                                                                                     \
   gemm_skinny_kernel<MB, WAVES, TILES, RT, TC><<<grid, block, 0, stream>>>(                               \
-      (const uint16_t*)a, (const uint16_t*)w, (TC*)c, M, N, K, accumulate, pair_blocks)
+      (const uint16_t*)a, (const uint16_t*)w, (TC*)c, M, N, K, accumulate, pair_blocks, norm)
   switch ((M + 15) / 16) {
     case 1: BH_SKINNY(1); break;
     case 2: BH_SKINNY(2); break;
@@ -379,8 +433,12 @@ static void launch_tiled(const void* a, const void* w, void* c, int M, int N, in
 }
 
 // layout: 0 = rows, 1 = tiles.  activation: 0 = none; 1 = SwiGLU (W has 2 * N rows: gate rows then up rows).
+// The `ahead_*` and `behind_*` arguments (null when unused) let an RMSNorm ride on the products before and
+// after it (struct SkinnyNorm); they exist for M <= 64 only.
 extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, int accumulate, int M, int N, int K,
-                            int layout, int activation, hipStream_t stream) {
+                            int layout, int activation, const float* ahead_ss, int ahead_blocks, float ahead_eps,
+                            const void* behind_weight, int behind_weight_dtype, void* behind_rows,
+                            float* behind_ss, hipStream_t stream) {
   BH_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_bf16: sizes M=%d N=%d K=%d must be positive", M, N, K);
   BH_REQUIRE(K % 8 == 0, "gemm_bf16: K=%d must be a multiple of 8", K);
   BH_REQUIRE(c_dtype == BH_F32 || c_dtype == BH_BF16, "gemm_bf16: unknown output dtype %d", c_dtype);
@@ -390,6 +448,15 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
   BH_REQUIRE(activation == 0 || (N % 16 == 0 && !accumulate),
              "gemm_bf16: SwiGLU needs a multiple of 16 outputs (got %d) and no accumulation", N);
   BH_REQUIRE((M + 127) / 128 <= 65535, "gemm_bf16: M=%d needs more than 65535 row tiles", M);
+  BH_REQUIRE((!ahead_ss && !behind_weight) || M <= 64,
+             "gemm_bf16: a norm rides on products of at most 64 rows only, not M=%d", M);
+  BH_REQUIRE(!ahead_ss || (ahead_blocks > 0 && ahead_eps > 0.f), "gemm_bf16: the norm ahead needs partial sums and an epsilon");
+  BH_REQUIRE(!behind_weight || (behind_rows && behind_ss && c_dtype == BH_F32 && activation == 0),
+             "gemm_bf16: the norm behind needs its outputs, a float32 product and no activation");
+  BH_REQUIRE(!behind_weight || behind_weight_dtype == BH_F32 || behind_weight_dtype == BH_BF16,
+             "gemm_bf16: unknown norm weight dtype %d", behind_weight_dtype);
+  const SkinnyNorm norm = {ahead_ss, ahead_blocks, ahead_eps, behind_weight, behind_weight_dtype == BH_F32,
+                           (uint16_t*)behind_rows, behind_ss};
   const bool f32 = c_dtype == BH_F32;
 #define BH_PICK(FN, TILES, EXTRA, ...)                                             \
   do {                                                                              \
@@ -399,11 +466,11 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
   if (M <= 64) {
     const int pair_blocks = N / 16;
     if (activation) {
-      if (layout) BH_PICK(launch_skinny, true, 2, a, w, c, M, N, K, 0, pair_blocks, stream);
-      else BH_PICK(launch_skinny, false, 2, a, w, c, M, N, K, 0, pair_blocks, stream);
+      if (layout) BH_PICK(launch_skinny, true, 2, a, w, c, M, N, K, 0, pair_blocks, norm, stream);
+      else BH_PICK(launch_skinny, false, 2, a, w, c, M, N, K, 0, pair_blocks, norm, stream);
     } else {
-      if (layout) BH_PICK(launch_skinny, true, 1, a, w, c, M, N, K, accumulate, 0, stream);
-      else BH_PICK(launch_skinny, false, 1, a, w, c, M, N, K, accumulate, 0, stream);
+      if (layout) BH_PICK(launch_skinny, true, 1, a, w, c, M, N, K, accumulate, 0, norm, stream);
+      else BH_PICK(launch_skinny, false, 1, a, w, c, M, N, K, accumulate, 0, norm, stream);
     }
     return bh_check_launch("gemm_skinny");
   }

@@ -50,6 +50,7 @@ class DecodeGraph:
         self.graph = None
         self.logits = None
         self.copied = None        # event: the last host-to-device copy of the step's numbers is done
+        self.known = {}           # kv group -> per row (the page list the host table row was written from, how far)
 
     def fill(self, entries, pasts):
         """Write this step's numbers into the static buffer (one host-to-device copy)."""
@@ -68,9 +69,20 @@ class DecodeGraph:
         at = self.n_meta
         for index in self.kv_groups:
             table = host[at:at + b * self.table_width].reshape(b, self.table_width)
-            table[:] = 0
-            for row, pages in enumerate(cache.page_table_rows(cache.groups[index], slots)):
-                table[row, :len(pages)] = pages
+            group = cache.groups[index]
+            known = self.known.setdefault(index, [(None, 0)] * b)
+            for row, slot in enumerate(slots):
+                pages = group.pages_of[slot]
+                before, count = known[row]
+                # a sequence's page list only grows while it lives (a window apart), so a row that was
+                # written for this very list needs its new pages only
+                if before is pages and count <= len(pages) and not group.need.window:
+                    for j in range(count, len(pages)):
+                        table[row, j] = pages[j]
+                else:
+                    table[row, :] = 0
+                    table[row, :len(pages)] = [max(page, 0) for page in pages]
+                known[row] = (pages, len(pages))
             at += b * self.table_width
         self.device.copy_(self.host, non_blocking=True)
         self.copied = torch.cuda.Event()

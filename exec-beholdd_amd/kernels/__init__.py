@@ -1,6 +1,6 @@
 """The gfx950 kernel library and its Python binding."""
 
-from .library import HipKernels, KernelError, PackedWeight
+from .library import HipKernels, KernelError, NormedRows, PackedWeight
 from . import build
 
-__all__ = ["HipKernels", "KernelError", "PackedWeight", "build"]
+__all__ = ["HipKernels", "KernelError", "NormedRows", "PackedWeight", "build"]

@@ -5,8 +5,8 @@ checks every argument on the host (device, dtype, contiguity, shapes) before a k
 launched: the kernels themselves trust their arguments.  There is no CPU path: without a GPU
 and the library, construction fails.
 
-Every method launches on torch's current HIP stream and returns nothing; results are written
-into the `out` tensors that the caller passes.
+Every method launches on torch's current HIP stream; results are written into the `out` tensors
+that the caller passes (`gemm` may besides return the prepared input of a following norm).
 """
 
 from __future__ import annotations
@@ -32,6 +32,23 @@ class PackedWeight:
 
     def __init__(self, data: torch.Tensor, rows: int, cols: int):
         self.data, self.shape, self.dtype = data, (rows, cols), data.dtype
+
+    def dim(self):
+        return 2
+
+
+class NormedRows:
+    """The output of an RMSNorm but for each row's factor: `rows` [n, width] bfloat16 holds x * weight and
+    `ss` [blocks, n] float32 partial sums of x^2 whose total over `blocks` gives the row's factor
+    1 / sqrt(total / width + eps).  Products (`gemm`, `gemm_swiglu`) take it in place of an activation
+    matrix and apply the factor to their result; one that cannot (other operand types) runs the norm
+    itself from `source`, which must still hold the norm's input then.  `shape` and `dtype` are those of
+    the matrix it stands for."""
+
+    def __init__(self, rows: torch.Tensor, ss: torch.Tensor, eps: float, source: torch.Tensor, weight: torch.Tensor):
+        self.rows, self.ss, self.eps = rows, ss, float(eps)
+        self.source, self.weight = source, weight       # the norm's input and weight, for a product that cannot take this form
+        self.shape, self.dtype, self.device = rows.shape, rows.dtype, rows.device
 
     def dim(self):
         return 2
@@ -76,7 +93,7 @@ class HipKernels:
             "bh_attention_generic": [p, p, i, p, p, p, i, p, p, i, i, i, i, f, i, i, p],
             "bh_swiglu": [p, p, i, i, i, p],
             "bh_sample": [p, p, p, p, p, p, p, i, i, p],
-            "bh_gemm_bf16": [p, p, p, i, i, i, i, i, i, i, p],
+            "bh_gemm_bf16": [p, p, p, i, i, i, i, i, i, i, p, i, f, p, i, p, p, p],
             "bh_attention_bf16": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, i, i, f, i, i, i, p],
             "bh_attention_bf16_splits": [i, i, i, i, i],
             "bh_kv_order": [i, i],
@@ -147,38 +164,73 @@ class HipKernels:
             return PackedWeight(data, rows, cols)
         return w
 
-    def _gemm_fast(self, a, w, out, accumulate, activation):
-        """Launch the matrix-core product if it takes these operands; say whether it did."""
+    SKINNY_ROWS = 64      # products of at most this many rows can carry a norm (csrc/gemm_bf16.hip)
+
+    def _gemm_fast(self, a, w, out, accumulate, activation, then_norm=None):
+        """Launch the matrix-core product if it takes these operands; say whether it did, and with
+        what prepared norm output (None if `then_norm` was not asked for or cannot ride on this product)."""
         fast = self.lib.bh_gemm_bf16
         packed = isinstance(w, PackedWeight)
+        ahead = a if isinstance(a, NormedRows) else None
         if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or a.shape[1] % 8:
             if packed:
                 raise KernelError("gemm: a packed weight needs bfloat16 activations")
-            return False
+            return False, None
         if activation and (out.shape[1] % 16 or accumulate):
-            return False
+            return False, None
         m, k = a.shape
-        self._check(fast(self._ptr(a, "gemm a"), self._ptr(w.data if packed else w, "gemm w"),
-                         self._ptr(out, "gemm out"), _code(out, "gemm out"), int(bool(accumulate)), m, out.shape[1], k,
-                         int(packed), int(activation), self._stream()))
-        return True
+        n = out.shape[1]
+        if ahead is not None and (m > self.SKINNY_ROWS or ahead.ss.shape[1] != m or ahead.ss.dtype != torch.float32):
+            raise KernelError(f"gemm: prepared norm rows of {m} rows do not fit (at most {self.SKINNY_ROWS}, one sum per row)")
+        behind = None
+        if (then_norm is not None and m <= self.SKINNY_ROWS and out.dtype == torch.float32 and not activation
+                and then_norm.weight.shape == (n,) and then_norm.weight.dtype in _CODES):
+            behind = NormedRows(torch.empty((m, n), dtype=torch.bfloat16, device=self.device),
+                                torch.empty((-(-n // 16), m), dtype=torch.float32, device=self.device), then_norm.eps,
+                                out, then_norm.weight)
+        a_rows = ahead.rows if ahead is not None else a
+        self._check(fast(
+            self._ptr(a_rows, "gemm a"), self._ptr(w.data if packed else w, "gemm w"), self._ptr(out, "gemm out"),
+            _code(out, "gemm out"), int(bool(accumulate)), m, n, k, int(packed), int(activation),
+            self._ptr(ahead.ss, "norm sums") if ahead is not None else None,
+            ahead.ss.shape[0] if ahead is not None else 0, ahead.eps if ahead is not None else 0.0,
+            self._ptr(then_norm.weight, "norm weight") if behind is not None else None,
+            _code(then_norm.weight, "norm weight") if behind is not None else 0,
+            self._ptr(behind.rows, "norm rows") if behind is not None else None,
+            self._ptr(behind.ss, "norm sums") if behind is not None else None, self._stream()))
+        return True, behind
 
-    def gemm(self, a, w, out, accumulate=False):
-        """out[M, N] (+)= a[M, K] @ w[N, K]^T with float32 accumulation; `w` may be a PackedWeight."""
+    def gemm(self, a, w, out, accumulate=False, then_norm=None):
+        """out[M, N] (+)= a[M, K] @ w[N, K]^T with float32 accumulation; `w` may be a PackedWeight and
+        `a` the NormedRows an earlier product prepared.  With `then_norm` (an object with `weight` [N] and
+        `eps`: an RMSNorm over the rows of `out` as they are after this product) the product may prepare that norm's
+        output on its way and return it as NormedRows; it returns None when it does not (then run the
+        norm as usual)."""
         if a.dim() != 2 or w.dim() != 2 or out.dim() != 2:
             raise KernelError("gemm: operands must be matrices")
         m, k = a.shape
         n = w.shape[0]
         if w.shape[1] != k or out.shape != (m, n):
             raise KernelError(f"gemm: shapes a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
-        if self._gemm_fast(a, w, out, accumulate, 0):
-            return
+        if isinstance(a, NormedRows) and (w.dtype != torch.bfloat16 or k % 8):
+            a = self._run_norm(a)
+        done, prepared = self._gemm_fast(a, w, out, accumulate, 0, then_norm)
+        if done:
+            return prepared
         self._check(self.lib.bh_gemm_generic(
             self._ptr(a, "gemm a"), _code(a, "gemm a"), self._ptr(w, "gemm w"), _code(w, "gemm w"),
             self._ptr(out, "gemm out"), _code(out, "gemm out"), int(bool(accumulate)), m, n, k, self._stream()))
+        return None
+
+    def _run_norm(self, prepared):
+        """The norm that `prepared` stands for, as a step of its own."""
+        out = torch.empty(tuple(prepared.shape), dtype=prepared.dtype, device=self.device)
+        self.rmsnorm(prepared.source, prepared.weight, prepared.eps, out)
+        return out
 
     def gemm_swiglu(self, a, w, out):
-        """out[M, F] = silu(a @ w[:F]^T) * (a @ w[F:]^T) for w [2F, K] = gate rows, then up rows."""
+        """out[M, F] = silu(a @ w[:F]^T) * (a @ w[F:]^T) for w [2F, K] = gate rows, then up rows; `a` may
+        be NormedRows."""
         if a.dim() != 2 or w.dim() != 2 or out.dim() != 2:
             raise KernelError("gemm_swiglu: operands must be matrices")
         m, k = a.shape
@@ -186,7 +238,7 @@ class HipKernels:
         if w.shape != (2 * width, k) or out.shape[0] != m or out.dtype != a.dtype:
             raise KernelError(f"gemm_swiglu: shapes a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} "
                               "do not fit")
-        if self._gemm_fast(a, w, out, False, 1):
+        if self._gemm_fast(a, w, out, False, 1)[0]:
             return
         both = torch.empty((m, 2 * width), dtype=a.dtype, device=self.device)
         self.gemm(a, w, both)

@@ -80,8 +80,10 @@ class DecoderModel:
         None); `want_rows` (int32 device tensor, may be empty) lists the rows whose logits are
         returned as float32 [len(want_rows), vocab]."""
         hidden = self.embedding.forward(ctx)
+        prepared = None      # the next block's first norm, when the block before could prepare it
         for run, (layer, _entry) in enumerate(self.schedule):
-            self.blocks[layer].forward(ctx, hidden, cache_for_run(run))
+            following = self.blocks[self.schedule[run + 1][0]] if run + 1 < len(self.schedule) else None
+            prepared = self.blocks[layer].forward(ctx, hidden, cache_for_run(run), prepared, following)
         if want_rows is None or want_rows.numel() == 0:
             return None
         return self.head.forward(ctx, self.final_norm.forward(ctx, hidden, rows=want_rows))

@@ -25,6 +25,8 @@ from .linear import Linear
 
 class GQAAttention:
     graph_safe = True      # forward reads only the step's device tensors
+    prepares_next_norm = True      # the output projection can carry the norm that follows
+    takes_prepared_input = True    # x goes to the q/k/v product untouched
     def __init__(self, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int, prefix: str, *,
                  position_encoding=None, qk_norm_eps: float | None = None, scale: float | None = None,
                  window: int = 0):
@@ -66,7 +68,7 @@ class GQAAttention:
     def cache_need(self):
         return CacheNeed(kind="kv", kv_heads=self.n_kv_heads, head_dim=self.head_dim, window=self.window)
 
-    def forward(self, ctx, x, hidden, cache):
+    def forward(self, ctx, x, hidden, cache, then_norm=None):
         k = ctx.kernels
         qkv = self.qkv.forward(ctx, x)
         q = ctx.new_activations(ctx.n_rows, self.n_heads * self.head_dim)
@@ -77,7 +79,7 @@ class GQAAttention:
         attended = ctx.new_activations(ctx.n_rows, self.n_heads * self.head_dim)
         k.attention(q, attended, cache.k_pages, cache.v_pages, cache.page_table, ctx.row_seq, ctx.positions,
                     self.n_heads, self.n_kv_heads, self.head_dim, self.scale, self.window, layout=ctx)
-        self.out.forward(ctx, attended, out=hidden, accumulate=True)
+        return self.out.add_into(ctx, attended, hidden, then_norm)
 
 
 @MIXERS.register("gqa_attention")

@@ -22,6 +22,16 @@ Feed-forward:
     forward(ctx, x, hidden)                adds its output into `hidden`
 Block:
     mixer, feed_forward attributes; forward(ctx, hidden, cache)
+A norm may ride on the products around it (optional, one flag per role):
+    norm.request() -> NormRequest          what the product that completes the norm's input needs
+    producer (mixer or feed-forward) with `prepares_next_norm = True`:
+        forward(..., then_norm=NormRequest) returns what its last product prepared (whatever
+        `kernels.gemm(..., then_norm=)` returned: the next part's input in the kernel library's own
+        form, or None when the product could not carry the norm)
+    consumer (mixer or feed-forward) with `takes_prepared_input = True`: its `x` may be that
+        prepared form; it hands `x` to the kernel library's products untouched.
+The block joins a producer and a consumer this way only when all three offer it, and runs the norm
+as a step of its own otherwise.
 A part may declare `graph_safe = True`: its forward uses only the device tensors of the step
 context (never the host_* lists, never a host-side decision that changes from step to step).
 Decode steps of a model whose parts all say so are captured and replayed as HIP graphs.
@@ -98,6 +108,13 @@ class StepContext:
 
     def new_f32(self, *shape) -> torch.Tensor:
         return torch.empty(shape, dtype=torch.float32, device=self.device)
+
+
+@dataclass
+class NormRequest:
+    """An RMSNorm (weight [width], eps) offered to the product that completes its input."""
+    weight: torch.Tensor
+    eps: float
 
 
 @dataclass

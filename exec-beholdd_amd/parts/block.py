@@ -37,9 +37,36 @@ class PreNormBlock:
     def cache_need(self):
         return self.mixer.cache_need()
 
-    def forward(self, ctx, hidden, cache):
-        self.mixer.forward(ctx, self.mixer_norm.forward(ctx, hidden), hidden, cache)
-        self.feed_forward.forward(ctx, self.feed_forward_norm.forward(ctx, hidden), hidden)
+    @staticmethod
+    def _joined(producer, norm, consumer):
+        """The request to hand `producer` so that its last product prepares `norm` for `consumer`, or None."""
+        if (getattr(producer, "prepares_next_norm", False) and getattr(consumer, "takes_prepared_input", False)
+                and hasattr(norm, "request")):
+            return norm.request()
+        return None
+
+    def entry_request(self, producer):
+        """What the part that runs before this block (`producer`) may prepare of this block's first norm."""
+        return self._joined(producer, self.mixer_norm, self.mixer)
+
+    def forward(self, ctx, hidden, cache, prepared=None, next_block=None):
+        """One layer.  `prepared`: the mixer's input if the block before has prepared it already;
+        `next_block`: the block that runs after this one, whose first norm this block's feed-forward
+        may prepare.  Returns that prepared input, or None."""
+        x = prepared if prepared is not None else self.mixer_norm.forward(ctx, hidden)
+        request = self._joined(self.mixer, self.feed_forward_norm, self.feed_forward)
+        if request is not None:
+            x = self.mixer.forward(ctx, x, hidden, cache, then_norm=request)
+        else:
+            self.mixer.forward(ctx, x, hidden, cache)
+            x = None
+        if x is None:
+            x = self.feed_forward_norm.forward(ctx, hidden)
+        request = next_block.entry_request(self.feed_forward) if hasattr(next_block, "entry_request") else None
+        if request is not None:
+            return self.feed_forward.forward(ctx, x, hidden, then_norm=request)
+        self.feed_forward.forward(ctx, x, hidden)
+        return None
 
 
 @BLOCKS.register("pre_norm")

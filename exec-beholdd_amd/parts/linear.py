@@ -58,3 +58,11 @@ class Linear:
             out = torch.empty((x.shape[0], self.out_features), dtype=out_dtype or ctx.act_dtype, device=x.device)
         ctx.kernels.gemm(x, self.weight, out, accumulate=accumulate)
         return out
+
+    def add_into(self, ctx, x, residual, then_norm=None):
+        """residual += W x.  With `then_norm` (a NormRequest for the norm that reads the residual next)
+        returns what the product prepared of that norm's output, or None."""
+        if then_norm is None:
+            ctx.kernels.gemm(x, self.weight, residual, accumulate=True)
+            return None
+        return ctx.kernels.gemm(x, self.weight, residual, accumulate=True, then_norm=then_norm)

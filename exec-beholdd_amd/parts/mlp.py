@@ -13,6 +13,8 @@ from .linear import Linear
 
 class SwiGLU:
     graph_safe = True      # forward reads only the step's device tensors
+    prepares_next_norm = True      # the down projection can carry the norm that follows
+    takes_prepared_input = True    # x goes to the gate/up product untouched
     def __init__(self, hidden: int, intermediate: int, prefix: str):
         self.hidden, self.intermediate = hidden, intermediate
         self.gate_up = Linear(hidden, [intermediate, intermediate],
@@ -30,10 +32,10 @@ class SwiGLU:
         self.gate_up.prepare(kernels)
         self.down.prepare(kernels)
 
-    def forward(self, ctx, x, hidden):
+    def forward(self, ctx, x, hidden, then_norm=None):
         activated = ctx.new_activations(x.shape[0], self.intermediate)
         ctx.kernels.gemm_swiglu(x, self.gate_up.weight, activated)     # both products and the gate in one pass
-        self.down.forward(ctx, activated, out=hidden, accumulate=True)
+        return self.down.add_into(ctx, activated, hidden, then_norm)
 
 
 @FEED_FORWARDS.register("swiglu")

@@ -10,7 +10,7 @@ from __future__ import annotations
 import torch
 
 from ..weights.binder import TensorSpec
-from .base import NORMS
+from .base import NORMS, NormRequest
 
 
 class RMSNorm:
@@ -32,6 +32,10 @@ class RMSNorm:
         out = ctx.new_activations(n, self.width)
         ctx.kernels.rmsnorm(hidden, self.weight, self.eps, out, rows=rows)
         return out
+
+    def request(self):
+        """This norm as the product that completes its input may prepare it."""
+        return NormRequest(self.weight, self.eps)
 
 
 @NORMS.register("rmsnorm")

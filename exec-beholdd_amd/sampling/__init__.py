@@ -65,8 +65,8 @@ class Sampler:
         n_rows = logits.shape[0]
         if not (len(params) == len(requests) == len(steps) == n_rows):
             raise ValueError("one sampling parameter set, request index and step per row")
-        tokens = torch.empty(n_rows, dtype=torch.int32, device=self.device)
-        bad = torch.empty(n_rows, dtype=torch.int32, device=self.device)
+        both = torch.empty((2, n_rows), dtype=torch.int32, device=self.device)   # one copy brings both back
+        tokens, bad = both[0], both[1]
         if all(p.greedy for p in params):
             self.kernels.sample(logits, tokens, bad)
         else:
@@ -76,7 +76,7 @@ class Sampler:
             top_k = torch.tensor([p.top_k for p in params], dtype=torch.int32).to(self.device)
             self.kernels.sample(logits, tokens, bad, temperature=columns[0], top_k=top_k, top_p=columns[1],
                                 uniform=columns[2])
-        result = torch.stack([tokens, bad]).cpu()
+        result = both.cpu()
         for row in range(n_rows):
             if int(result[1, row]):
                 raise SamplingError(f"request {requests[row]}, step {steps[row]}: a logit is not finite")

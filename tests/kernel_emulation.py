@@ -32,12 +32,13 @@ class TorchKernels:
             y = y * weight.float()
         out.copy_(y.to(out.dtype))
 
-    def gemm(self, a, w, out, accumulate=False):
+    def gemm(self, a, w, out, accumulate=False, then_norm=None):
         self.calls.append("gemm")
         product = (a.double() @ w.double().t()).float()
         if accumulate:
             product = product + out.float()
         out.copy_(product.to(out.dtype))
+        return None         # this double never prepares a following norm: the norm runs as a step of its own
 
     def qk_norm_rope_cache(self, qkv, q_out, q_weight, k_weight, eps, cos, sin, positions, row_seq,
                            k_pages, v_pages, page_table, n_heads, n_kv_heads, head_dim, write_kv, max_position):
