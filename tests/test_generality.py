@@ -56,3 +56,61 @@ def test_registering_twice_is_refused():
         beholdd.parts.MIXERS.register("gqa_attention", lambda *a: None)
     with pytest.raises(KeyError, match="gqa_attention"):
         beholdd.parts.MIXERS.get("no_such_mixer")
+
+
+def test_a_block_joins_a_norm_to_its_neighbours_only_when_all_three_offer_it():
+    """The block hands a norm to the part before it, and that part's result to the part after it, only if
+    the producer prepares norms, the consumer takes prepared input and the norm can describe itself."""
+    from beholdd.parts.block import PreNormBlock
+
+    calls = []
+
+    class Norm:
+        def __init__(self, name, describes=True):
+            self.name = name
+            if describes:
+                self.request = lambda: ("request", name)
+
+        def forward(self, ctx, hidden):
+            calls.append(("norm", self.name))
+            return ("normed", self.name)
+
+    class Part:
+        def __init__(self, name, prepares, takes):
+            self.name = name
+            if prepares:
+                self.prepares_next_norm = True
+            if takes:
+                self.takes_prepared_input = True
+
+        def forward(self, ctx, x, hidden, cache=None, then_norm=None):
+            calls.append((self.name, x, then_norm))
+            return ("prepared by", self.name) if then_norm is not None else None
+
+    class OldPart:          # the interface without the optional argument
+        def __init__(self, name):
+            self.name = name
+
+        def forward(self, ctx, x, hidden, cache=None):
+            calls.append((self.name, x, None))
+
+    # everything offers it: one norm call (the first), the rest rides
+    first = PreNormBlock(Norm("n1"), Part("mixer", True, True), Norm("n2"), Part("ff", True, True))
+    second = PreNormBlock(Norm("n3"), Part("mixer2", True, True), Norm("n4"), Part("ff2", True, True))
+    carried = first.forward(None, None, None, None, second)
+    assert carried == ("prepared by", "ff")
+    assert calls == [("norm", "n1"), ("mixer", ("normed", "n1"), ("request", "n2")),
+                     ("ff", ("prepared by", "mixer"), ("request", "n3"))]
+    calls.clear()
+    assert second.forward(None, None, None, carried, None) is None
+    assert calls == [("mixer2", ("prepared by", "ff"), ("request", "n4")), ("ff2", ("prepared by", "mixer2"), None)]
+
+    # a norm that cannot describe itself, an old-style part, consumers that do not take prepared input
+    calls.clear()
+    plain = PreNormBlock(Norm("n1"), Part("mixer", True, True), Norm("n2", describes=False), OldPart("ff"))
+    picky = PreNormBlock(Norm("n3"), Part("mixer2", True, False), Norm("n4"), Part("ff2", True, False))
+    last = PreNormBlock(Norm("n5"), Part("mixer3", True, False), Norm("n6"), Part("ff3", False, True))
+    assert plain.forward(None, None, None, None, picky) is None
+    assert picky.forward(None, None, None, None, last) is None
+    assert calls == [("norm", "n1"), ("mixer", ("normed", "n1"), None), ("norm", "n2"), ("ff", ("normed", "n2"), None),
+                     ("norm", "n3"), ("mixer2", ("normed", "n3"), None), ("norm", "n4"), ("ff2", ("normed", "n4"), None)]

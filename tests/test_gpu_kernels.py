@@ -117,6 +117,59 @@ def test_gemm_with_packed_weights(K, m, n, k):
     assert rel(acc, want + base.double()) < f32_bound
 
 
+@pytest.mark.parametrize("g_dtype", DTYPES)
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("m,n,k,n2", [(1, 192, 128, 48), (8, 4096, 256, 1000), (17, 200, 64, 64), (64, 320, 192, 130)])
+def test_norm_rides_on_the_products_around_it(K, g_dtype, packed, m, n, k, n2):
+    """The product that completes the residual prepares the following RMSNorm (rows times the norm weight,
+    partial sums of squares), and the product after it applies each row's factor to its result."""
+    from beholdd.kernels import NormedRows
+    from beholdd.parts.base import NormRequest
+    gen = torch.Generator().manual_seed(m * 31 + n)
+    a = torch.randn(m, k, generator=gen).to(torch.bfloat16)
+    w = (torch.randn(n, k, generator=gen) * 0.1).to(torch.bfloat16)
+    base = torch.randn(m, n, generator=gen) * 3
+    g = (1 + 0.3 * torch.randn(n, generator=gen)).to(g_dtype)
+    eps = 1e-5
+    residual = dev(base.clone())
+    w_dev = K.pack_weight(dev(w)) if packed else dev(w)
+    prepared = K.gemm(dev(a), w_dev, residual, accumulate=True, then_norm=NormRequest(dev(g), eps))
+    assert isinstance(prepared, NormedRows) and prepared.shape == (m, n)
+    want_residual = base.double() + a.double() @ w.double().t()
+    assert rel(residual, want_residual) < 4 * math.sqrt(k) * 2.0 ** -24
+    got_residual = residual.cpu().double()
+    assert rel(prepared.rows, got_residual * g.double()) < 4e-3                       # bfloat16 rounding
+    assert rel(prepared.ss.sum(0), (got_residual ** 2).sum(-1)) < 1e-5
+    assert prepared.ss.shape == (-(-n // 16), m)
+    normed = got_residual / torch.sqrt((got_residual ** 2).mean(-1, keepdim=True) + eps) * g.double()
+
+    w2 = (torch.randn(n2, n, generator=gen) * 0.1).to(torch.bfloat16)
+    w2_dev = K.pack_weight(dev(w2)) if packed else dev(w2)
+    for out_dtype in (torch.float32, torch.bfloat16):
+        out = torch.empty(m, n2, dtype=out_dtype, device="cuda:0")
+        assert K.gemm(prepared, w2_dev, out) is None
+        assert rel(out, normed @ w2.double().t()) < 8e-3, rel(out, normed @ w2.double().t())
+    # a product that cannot take the prepared form runs the norm itself, from the residual
+    out = torch.empty(m, n2, dtype=torch.float32, device="cuda:0")
+    K.gemm(prepared, dev(w2.float()), out)
+    assert rel(out, normed @ w2.double().t()) < 8e-3
+    if n2 % 2 == 0:
+        half = n2 // 2
+        act = torch.empty(m, half, dtype=torch.bfloat16, device="cuda:0")
+        K.gemm_swiglu(prepared, w2_dev, act)
+        gate, up = normed @ w2[:half].double().t(), normed @ w2[half:].double().t()
+        assert rel(act, gate / (1 + torch.exp(-gate)) * up) < 1.2e-2
+
+
+def test_norm_does_not_ride_on_wide_steps(K):
+    from beholdd.parts.base import NormRequest
+    a = torch.randn(65, 64).to(torch.bfloat16)
+    w = torch.randn(32, 64).to(torch.bfloat16)
+    residual = torch.zeros(65, 32, device="cuda:0")
+    assert K.gemm(dev(a), dev(w), residual, accumulate=True, then_norm=NormRequest(dev(torch.ones(32)), 1e-6)) is None
+    assert rel(residual, a.double() @ w.double().t()) < 1e-5
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("m,width,k", [(1, 16, 64), (8, 160, 128), (40, 896, 320), (64, 48, 192), (65, 64, 64),
