@@ -161,11 +161,105 @@ __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ lo
   }
 }
 
+// ---- argmax of long rows in two steps ---------------------------------------------------------
+// One block per row leaves all but a few compute units idle when there are few rows and a long
+// vocabulary.  Step one: a block per (row, chunk of AC elements) writes the chunk's largest value and its
+// lowest index, or index -1 if the chunk holds a non-finite value; step two: a wave per row takes the
+// best of the chunks (lowest index among equals, as chunks are in index order).
+
+#define AC 2048   // elements per chunk
+#define AT 256    // threads per chunk
+
+__global__ __launch_bounds__(AT) void argmax_chunk_kernel(const float* __restrict__ logits, float* __restrict__ part_val,
+                                                          int32_t* __restrict__ part_idx, int vocab, int chunks) {
+  __shared__ float val[AT];
+  __shared__ int idx[AT];
+  const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
+  const float* x = logits + (size_t)row * vocab;
+  const int end = min(vocab, (chunk + 1) * AC);
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  bool not_finite = false;
+  for (int i = chunk * AC + tid; i < end; i += AT) {
+    const float v = x[i];
+    if (!isfinite(v)) not_finite = true;
+    if (v > bv || bi == 0x7fffffff) {
+      bv = v;
+      bi = i;
+    }
+  }
+  val[tid] = bv;
+  idx[tid] = not_finite ? -1 : bi;
+  __syncthreads();
+  for (int stride = AT / 2; stride > 0; stride >>= 1) {
+    if (tid < stride) {
+      const float ov = val[tid + stride];
+      const int oi = idx[tid + stride];
+      // -1 (a non-finite value was seen) wins over everything
+      if (idx[tid] != -1 && (oi == -1 || ov > val[tid] || (ov == val[tid] && oi < idx[tid]))) {
+        val[tid] = ov;
+        idx[tid] = oi;
+      }
+    }
+    __syncthreads();
+  }
+  if (tid == 0) {
+    part_val[(size_t)row * chunks + chunk] = val[0];
+    part_idx[(size_t)row * chunks + chunk] = idx[0];
+  }
+}
+
+__global__ __launch_bounds__(BH_WAVE) void argmax_rows_kernel(const float* __restrict__ part_val,
+                                                              const int32_t* __restrict__ part_idx,
+                                                              int32_t* __restrict__ tokens, int32_t* __restrict__ bad,
+                                                              int chunks) {
+  const int row = blockIdx.x, lane = threadIdx.x;
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int c = lane; c < chunks; c += BH_WAVE) {
+    const float v = part_val[(size_t)row * chunks + c];
+    const int i = part_idx[(size_t)row * chunks + c];
+    if (bi != -1 && (i == -1 || v > bv || (v == bv && i < bi))) {
+      bv = v;
+      bi = i;
+    }
+  }
+#pragma unroll
+  for (int off = BH_WAVE / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, BH_WAVE);
+    const int oi = __shfl_xor(bi, off, BH_WAVE);
+    if (bi != -1 && (oi == -1 || ov > bv || (ov == bv && oi < bi))) {
+      bv = ov;
+      bi = oi;
+    }
+  }
+  if (lane == 0) {
+    tokens[row] = bi == -1 ? -1 : bi;
+    bad[row] = bi == -1 ? 1 : 0;
+  }
+}
+
+// Float-sized words of scratch that bh_sample wants for these rows when every row is greedy (0: none).
+extern "C" int bh_sample_scratch(int n_rows, int vocab) {
+  if (n_rows <= 0 || vocab < 4 * AC || n_rows >= 128) return 0;   // enough rows fill the compute units by themselves
+  return 2 * n_rows * ((vocab + AC - 1) / AC);
+}
+
 extern "C" int bh_sample(const float* logits, const float* temperature, const int32_t* top_k,
-                         const float* top_p, const float* uniform, int32_t* tokens, int32_t* bad, int n_rows,
-                         int vocab, hipStream_t stream) {
+                         const float* top_p, const float* uniform, int32_t* tokens, int32_t* bad, void* scratch,
+                         int n_rows, int vocab, hipStream_t stream) {
   BH_REQUIRE(n_rows > 0 && vocab > 0, "sample: rows %d and vocabulary %d must be positive", n_rows, vocab);
   BH_REQUIRE(temperature == nullptr || uniform != nullptr, "sample: temperature sampling needs uniform numbers");
+  if (temperature == nullptr && scratch != nullptr && bh_sample_scratch(n_rows, vocab) > 0) {
+    const int chunks = (vocab + AC - 1) / AC;
+    BH_REQUIRE(n_rows <= 65535, "sample: too many rows");
+    float* part_val = (float*)scratch;
+    int32_t* part_idx = (int32_t*)scratch + (size_t)n_rows * chunks;
+    argmax_chunk_kernel<<<dim3(chunks, n_rows), dim3(AT), 0, stream>>>(logits, part_val, part_idx, vocab, chunks);
+    if (int status = bh_check_launch("argmax_chunk")) return status;
+    argmax_rows_kernel<<<dim3(n_rows), dim3(BH_WAVE), 0, stream>>>(part_val, part_idx, tokens, bad, chunks);
+    return bh_check_launch("argmax_rows");
+  }
   sample_kernel<<<dim3(n_rows), dim3(SB), 0, stream>>>(logits, temperature, top_k, top_p, uniform, tokens, bad,
                                                        vocab);
   return bh_check_launch("sample");

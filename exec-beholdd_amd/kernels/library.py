@@ -92,7 +92,8 @@ class HipKernels:
             "bh_qk_norm_rope_cache": [p, i, p, p, p, i, f, p, p, i, i, p, p, p, p, p, i, i, i, i, i, i, i, i, p],
             "bh_attention_generic": [p, p, i, p, p, p, i, p, p, i, i, i, i, f, i, i, p],
             "bh_swiglu": [p, p, i, i, i, p],
-            "bh_sample": [p, p, p, p, p, p, p, i, i, p],
+            "bh_sample": [p, p, p, p, p, p, p, p, i, i, p],
+            "bh_sample_scratch": [i, i],
             "bh_gemm_bf16": [p, p, p, i, i, i, i, i, i, i, p, i, f, p, i, p, p, p],
             "bh_attention_bf16": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, i, i, f, i, i, i, p],
             "bh_attention_bf16_splits": [i, i, i, i, i],
@@ -363,8 +364,13 @@ class HipKernels:
                 raise KernelError(f"sample: {name} must be {dtype} [{n_rows}]")
         if temperature is not None and uniform is None:
             raise KernelError("sample: temperature sampling needs uniform numbers")
+        scratch = None
+        if temperature is None:      # greedy rows of a long vocabulary are searched chunk by chunk
+            words = int(self.lib.bh_sample_scratch(n_rows, vocab))
+            if words:
+                scratch = torch.empty(words, dtype=torch.float32, device=self.device)
         self._check(self.lib.bh_sample(
             self._ptr(logits, "logits", (torch.float32,)), self._ptr(temperature, "temperature", None, True),
             self._ptr(top_k, "top_k", None, True), self._ptr(top_p, "top_p", None, True),
             self._ptr(uniform, "uniform", None, True), self._ptr(tokens, "tokens"), self._ptr(bad, "bad"),
-            n_rows, vocab, self._stream()))
+            self._ptr(scratch, "sample scratch", None, True), n_rows, vocab, self._stream()))

@@ -535,7 +535,7 @@ def test_swiglu(K, dtype, rows, width):
     assert rel(out, gate / (1 + torch.exp(-gate)) * up) < tol(dtype, 2e-6, 4e-3)
 
 
-@pytest.mark.parametrize("vocab", [7, 331, 1024, 1500, 151936])
+@pytest.mark.parametrize("vocab", [7, 331, 1024, 1500, 8191, 8192, 8193, 10000, 151936])
 def test_argmax_ties_go_to_the_lowest_id(K, vocab):
     g = torch.Generator().manual_seed(vocab)
     logits = torch.randn(5, vocab, generator=g)
@@ -544,6 +544,7 @@ def test_argmax_ties_go_to_the_lowest_id(K, vocab):
     top = min(vocab - 1, 700)
     logits[3, top] = 60.0
     logits[3, top // 2] = 60.0               # a tie: the lower id wins
+    logits[3, vocab - 1] = 60.0              # ... also against one far away (another chunk of a long row)
     logits[4, :] = 1.25                      # all equal: id 0
     tokens = torch.empty(5, dtype=torch.int32, device="cuda:0")
     bad = torch.empty(5, dtype=torch.int32, device="cuda:0")
@@ -552,10 +553,11 @@ def test_argmax_ties_go_to_the_lowest_id(K, vocab):
     assert bad.cpu().tolist() == [0] * 5
 
 
-def test_sample_flags_rows_that_are_not_finite(K):
-    logits = torch.randn(3, 100)
-    logits[1, 40] = float("nan")
-    logits[2, 99] = float("inf")
+@pytest.mark.parametrize("vocab", [100, 20000])
+def test_sample_flags_rows_that_are_not_finite(K, vocab):
+    logits = torch.randn(3, vocab)
+    logits[1, (2 * vocab) // 5] = float("nan")
+    logits[2, vocab - 1] = float("inf")
     tokens = torch.empty(3, dtype=torch.int32, device="cuda:0")
     bad = torch.empty(3, dtype=torch.int32, device="cuda:0")
     K.sample(dev(logits), tokens, bad)
