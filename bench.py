@@ -63,23 +63,33 @@ def decode_run(engine, batch, context, steps, warmup, torch):
     from beholdd.engine import StepEntry
     from beholdd.sampling import SamplingParams
 
-    start = context - steps - warmup
+    start = context - steps - warmup - 1
     slots = [engine.alloc_slot() for _ in range(batch)]
     fill_cache(engine, slots, start, torch)
     greedy = [SamplingParams()] * batch
     tokens = [(7 * i + 3) % engine.model.vocab for i in range(batch)]
 
+    # The generation loop's own way of stepping (engine/generation.py): the next step is started with the
+    # tokens still on the device, then the host reads the tokens chosen before it.
+    requests = list(range(batch))
+    logits = engine.step([StepEntry(slot, [token], [0]) for slot, token in zip(slots, tokens)])
+    chosen = engine.select_async(logits, greedy, requests, [0] * batch)
+
     def one(step):
-        nonlocal tokens
-        logits = engine.step([StepEntry(slot, [token], [0]) for slot, token in zip(slots, tokens)])
-        tokens = engine.select(logits, greedy, list(range(batch)), [step] * batch)
+        nonlocal chosen
+        logits = engine.step([StepEntry(slot, [0], [0], fed_row=row) for slot, row in zip(slots, chosen.device_rows)])
+        ahead = engine.select_async(logits, greedy, requests, [step + 1] * batch)
+        chosen.result()
+        chosen = ahead
 
     for step in range(warmup):
         one(step)
+    chosen.result()
     torch.cuda.synchronize()
     begin = time.perf_counter()
     for step in range(steps):
         one(warmup + step)
+    chosen.result()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - begin
     lengths = [engine.cache.length(slot) for slot in slots]

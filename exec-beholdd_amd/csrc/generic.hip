@@ -30,25 +30,35 @@ extern "C" const char* bh_last_error() { return g_error; }
 extern "C" int bh_page_size() { return BH_PAGE; }
 
 // ---- embedding ---------------------------------------------------------------------------
-// hidden[row, :] = table[token[row], :], widened to float32.
+// hidden[row, :] = table[token[row], :], widened to float32.  A row's token is tokens[row], or, where
+// token_src is given and token_src[row] >= 0, fed[token_src[row]]: a token that an earlier kernel chose
+// and the host has not seen yet.  Such a token may be anything (the selection kernel writes -1 for a row
+// it refuses), so ids outside the table read row 0; the host finds out from the selection itself.
 
 template <typename T>
-__global__ void embed_kernel(const int32_t* __restrict__ tokens, const T* __restrict__ table,
-                             float* __restrict__ out, int width) {
+__global__ void embed_kernel(const int32_t* __restrict__ tokens, const int32_t* __restrict__ token_src,
+                             const int32_t* __restrict__ fed, const T* __restrict__ table,
+                             float* __restrict__ out, int width, int table_rows) {
   const int row = blockIdx.x;
-  const T* src = table + (size_t)tokens[row] * width;
+  int token = tokens[row];
+  if (token_src != nullptr && token_src[row] >= 0) token = fed[token_src[row]];
+  if (token < 0 || token >= table_rows) token = 0;
+  const T* src = table + (size_t)token * width;
   float* dst = out + (size_t)row * width;
   for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = to_f32(src[i]);
 }
 
-extern "C" int bh_embed(const int32_t* tokens, const void* table, int table_dtype, float* out,
-                        int n_rows, int width, hipStream_t stream) {
-  BH_REQUIRE(n_rows > 0 && width > 0, "embed: rows %d and width %d must be positive", n_rows, width);
+extern "C" int bh_embed(const int32_t* tokens, const int32_t* token_src, const int32_t* fed, const void* table,
+                        int table_dtype, float* out, int n_rows, int width, int table_rows, hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && width > 0 && table_rows > 0, "embed: rows %d, width %d and table rows %d must be positive",
+             n_rows, width, table_rows);
+  BH_REQUIRE((token_src == nullptr) == (fed == nullptr), "embed: fed tokens and their row indices come together");
   dim3 grid(n_rows), block(256);
   if (table_dtype == BH_F32)
-    embed_kernel<float><<<grid, block, 0, stream>>>(tokens, (const float*)table, out, width);
+    embed_kernel<float><<<grid, block, 0, stream>>>(tokens, token_src, fed, (const float*)table, out, width, table_rows);
   else if (table_dtype == BH_BF16)
-    embed_kernel<bf16_t><<<grid, block, 0, stream>>>(tokens, (const bf16_t*)table, out, width);
+    embed_kernel<bf16_t><<<grid, block, 0, stream>>>(tokens, token_src, fed, (const bf16_t*)table, out, width,
+                                                     table_rows);
   else
     return bh_fail("embed: unknown table dtype %d", table_dtype);
   return bh_check_launch("embed");

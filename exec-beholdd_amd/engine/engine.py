@@ -58,7 +58,8 @@ class Engine:
         self.cache = SequenceCache(model.entry_needs, max_tokens, self.dtype, self.device, kernels.page_size,
                                    max_slots=max_slots, max_position=model.max_position)
         self.cache_plan = self.cache.allocate(limit_bytes=memory_limit_bytes)
-        self.sampler = Sampler(kernels, self.device)
+        self.sampler = Sampler(kernels, self.device, capacity=self.cache.max_slots)
+        self._last_selection = None
         self.graphs = DecodeGraphs(self) if use_graphs and self.device.type == "cuda" else None
 
     # ---- what the generation loop needs of a stepper ----
@@ -85,7 +86,13 @@ class Engine:
         self.cache.free_slot(slot)
 
     def select(self, logits, params, requests, steps):
-        return self.sampler.select(logits, params, requests, steps)
+        return self.select_async(logits, params, requests, steps).result()
+
+    def select_async(self, logits, params, requests, steps):
+        """Start the selection and return at once: a `Selection` whose `result()` waits.  The step after
+        it may take its tokens on the device (`StepEntry.fed_row`) while the host has not read them."""
+        self._last_selection = self.sampler.select_async(logits, params, requests, steps)
+        return self._last_selection
 
     # ---- the step function ----
     def step(self, entries: list):
@@ -95,6 +102,12 @@ class Engine:
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
         if self.graphs is not None and entries and self.graphs.usable(entries):
             return self._graph_step(entries)
+        if any(e.fed_row is not None for e in entries):
+            # only the captured decode step reads tokens on the device; here the host waits for them
+            if self._last_selection is None:
+                raise ValueError("an entry takes its token from a selection, but nothing was selected yet")
+            entries = [e if e.fed_row is None
+                       else StepEntry(e.slot, [self._last_selection.token_at(e.fed_row)], e.want) for e in entries]
         ctx, want_rows, requests = build_step(self.kernels, self.dtype, self.device, self.cache, entries,
                                               self.model.vocab)
         self.cache.reserve(requests)

@@ -14,6 +14,16 @@ The loop decides on the host and talks to the model only through a *stepper*:
     stepper.alloc_slot() -> slot;  stepper.free_slot(slot)
     stepper.step(entries: list[StepEntry]) -> logits (one row per entry that wants one)
     stepper.select(logits, params, request_indices, steps) -> list[int]
+A stepper may also offer
+    stepper.select_async(logits, params, request_indices, steps) -> selection with `result() -> list[int]`,
+        `device_rows` and `take(positions)`
+    and take `StepEntry(slot, [0], [0], fed_row=r)`: the token at row r of the last selection, read on
+    the device.
+Then the loop runs one step ahead of what it knows: it starts the next step for every sequence that has
+tokens left to generate before it looks at the tokens just chosen, so the device never waits for the host.
+A sequence that turns out to have chosen a stop token has then been stepped once in vain; its slot is
+freed as always and what that step computed for it is dropped.  The tokens, their order and the finish
+reasons are those of the plain loop.
 """
 
 from __future__ import annotations
@@ -106,6 +116,8 @@ def generate(stepper, prompts: list, max_new_tokens, sampling=None, stop_token_i
 
 
 def _run_batch(stepper, batch, prompts, max_new, params, stops, on_token, control, results, on_logits):
+    if on_logits is None and hasattr(stepper, "select_async"):
+        return _run_batch_ahead(stepper, batch, prompts, max_new, params, stops, on_token, control, results)
     slots = {}
     try:
         for index in batch:
@@ -140,6 +152,55 @@ def _run_batch(stepper, batch, prompts, max_new, params, stops, on_token, contro
             if control is not None:
                 control()
             logits = stepper.step([StepEntry(slots[index], [token], [0]) for index, token in going])
+            step += 1
+    finally:
+        for slot in slots.values():
+            stepper.free_slot(slot)
+
+
+def _run_batch_ahead(stepper, batch, prompts, max_new, params, stops, on_token, control, results):
+    """`_run_batch` one step ahead of the host (see the module's text)."""
+    slots = {}
+    try:
+        for index in batch:
+            slots[index] = stepper.alloc_slot()
+        if control is not None:
+            control()
+        live = list(batch)
+        logits = stepper.step([StepEntry(slots[i], list(prompts[i]), [len(prompts[i]) - 1]) for i in live])
+        step = 0
+        chosen = stepper.select_async(logits, [params[i] for i in live], live, [step] * len(live))
+        while live:
+            # those that go on unless the token being chosen for them is a stop token: step them already
+            ahead = [at for at, index in enumerate(live) if len(results[index].token_ids) + 1 < max_new[index]]
+            chosen_ahead = None
+            if ahead:
+                if control is not None:
+                    control()
+                logits = stepper.step([StepEntry(slots[live[at]], [0], [0], fed_row=chosen.device_rows[at])
+                                       for at in ahead])
+                chosen_ahead = stepper.select_async(logits, [params[live[at]] for at in ahead],
+                                                    [live[at] for at in ahead], [step + 1] * len(ahead))
+            tokens = chosen.result()
+            going = set()
+            for index, token in zip(live, tokens):
+                result = results[index]
+                if token in stops:
+                    result.finish_reason, result.stop_token = FINISH_STOP, token
+                else:
+                    if on_token is not None:
+                        on_token(index, token)
+                    result.token_ids.append(token)
+                    if len(result.token_ids) < max_new[index]:
+                        going.add(index)
+                        continue
+                    result.finish_reason = FINISH_LENGTH
+                stepper.free_slot(slots.pop(index))    # the sequence has ended; its slot is free at once
+            if chosen_ahead is None:
+                break
+            kept = [position for position, at in enumerate(ahead) if live[at] in going]
+            live = [live[ahead[position]] for position in kept]
+            chosen = chosen_ahead.take(kept)
             step += 1
     finally:
         for slot in slots.values():

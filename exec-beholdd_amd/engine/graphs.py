@@ -28,12 +28,12 @@ class DecodeGraph:
         cache = engine.cache
         self.kv_groups = [index for index, g in enumerate(cache.groups) if g.need.kind == "kv"]
         b = n_seqs
-        self.n_meta = 7 * b + 1
+        self.n_meta = 8 * b + 1
         total = self.n_meta + len(self.kv_groups) * b * table_width
         self.host = torch.zeros(total, dtype=torch.int32).pin_memory()
         self.device = torch.zeros(total, dtype=torch.int32, device=engine.device)
         view, at = [], 0
-        for size in (b, b, b, b + 1, b, b, b):
+        for size in (b, b, b, b + 1, b, b, b, b):
             view.append(self.device[at:at + size])
             at += size
         self.tables = {}
@@ -45,8 +45,10 @@ class DecodeGraph:
             kernels=engine.kernels, act_dtype=engine.dtype, device=engine.device, n_rows=b, n_seqs=b,
             tokens=view[0], positions=view[1], row_seq=view[2], seq_start=view[3], seq_slot=view[4],
             seq_past=view[5], host_seq_start=None, host_seq_slot=None, host_seq_past=None, is_decode=True,
-            max_position=min(table_width * page, cache.max_position) - 1, max_rows_per_seq=1)
+            max_position=min(table_width * page, cache.max_position) - 1, max_rows_per_seq=1,
+            token_src=view[7], fed_tokens=engine.sampler.device_tokens)
         self.want_rows = view[6]
+        self.fed_buffer = engine.sampler.out       # the capture holds its address
         self.graph = None
         self.logits = None
         self.copied = None        # event: the last host-to-device copy of the step's numbers is done
@@ -59,7 +61,8 @@ class DecodeGraph:
             self.copied.synchronize()     # the pinned buffer may not change under a copy in flight
         host = self.host.numpy()
         slots = [e.slot for e in entries]
-        host[0:b] = [e.tokens[0] for e in entries]
+        host[0:b] = [e.tokens[0] if e.fed_row is None else 0 for e in entries]
+        host[7 * b + 1:8 * b + 1] = [-1 if e.fed_row is None else e.fed_row for e in entries]
         host[b:2 * b] = pasts
         host[2 * b:3 * b] = np.arange(b)
         host[3 * b:4 * b + 1] = np.arange(b + 1)
@@ -132,6 +135,8 @@ class DecodeGraphs:
         width = -(-pages // PAGE_BUCKET) * PAGE_BUCKET
         key = (len(entries), width)
         graph = self.graphs.pop(key, None)
+        if graph is not None and graph.fed_buffer is not self.engine.sampler.out:
+            graph = None                 # the sampler has a new buffer: what was captured reads the old one
         if graph is None:
             if len(self.graphs) >= self.limit:
                 self.graphs.pop(next(iter(self.graphs)))        # the least recently used

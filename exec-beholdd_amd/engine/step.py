@@ -28,6 +28,8 @@ class StepEntry:
     slot: int
     tokens: list
     want: list = field(default_factory=list)   # indices into `tokens` whose logits are returned
+    fed_row: int | None = None                 # the entry's one token is not `tokens[0]` (ignored then) but stands
+                                               # at this row of the sampler's device buffer, not yet seen by the host
 
 
 def check_entries(entries: list, cache, vocab: int) -> None:
@@ -39,7 +41,11 @@ def check_entries(entries: list, cache, vocab: int) -> None:
         if n_new == 0:
             raise StepError(f"entry {index} (slot {entry.slot}) brings no tokens")
         cache.length(entry.slot)       # raises for a slot that is not in use
-        for token in entry.tokens:
+        if entry.fed_row is not None:
+            if n_new != 1 or not isinstance(entry.fed_row, (int, np.integer)) or entry.fed_row < 0:
+                raise StepError(f"entry {index} (slot {entry.slot}): a token fed on the device is one token from a "
+                                f"row >= 0, got {n_new} tokens and row {entry.fed_row!r}")
+        for token in (entry.tokens if entry.fed_row is None else ()):
             if not isinstance(token, (int, np.integer)) or isinstance(token, bool) or not 0 <= token < vocab:
                 raise StepError(f"entry {index} (slot {entry.slot}): token {token!r} is outside the vocabulary "
                                 f"of {vocab}")

@@ -86,7 +86,7 @@ class HipKernels:
         lib.bh_last_error.restype = ctypes.c_char_p
         lib.bh_page_size.restype = i
         table = {
-            "bh_embed": [p, p, i, p, i, i, p],
+            "bh_embed": [p, p, p, p, i, p, i, i, i, p],
             "bh_rmsnorm": [p, p, p, i, p, i, i, i, f, p],
             "bh_gemm_generic": [p, i, p, i, p, i, i, i, i, i, p],
             "bh_qk_norm_rope_cache": [p, i, p, p, p, i, f, p, p, i, i, p, p, p, p, p, i, i, i, i, i, i, i, i, p],
@@ -126,16 +126,21 @@ class HipKernels:
         return ctypes.c_void_p(tensor.data_ptr())
 
     # ---- kernels ----
-    def embed(self, tokens, table, out):
-        """out[row] = table[tokens[row]] widened to float32; tokens int32 [T], table [V, D], out f32 [T, D]."""
+    def embed(self, tokens, table, out, token_src=None, fed_tokens=None):
+        """out[row] = table[token of the row] widened to float32; tokens int32 [T], table [V, D], out f32 [T, D].
+        With `token_src` (int32 [T]) and `fed_tokens` (int32, any length): where token_src[row] >= 0 the row's
+        token is fed_tokens[token_src[row]], read on the device."""
         n_rows, width = out.shape
         if tokens.shape != (n_rows,) or table.dim() != 2 or table.shape[1] != width:
             raise KernelError(f"embed: shapes tokens {tuple(tokens.shape)}, table {tuple(table.shape)}, "
                               f"out {tuple(out.shape)} do not fit")
+        if (token_src is None) != (fed_tokens is None) or (token_src is not None and token_src.shape != (n_rows,)):
+            raise KernelError("embed: fed tokens come with one source index per row")
         self._check(self.lib.bh_embed(
-            self._ptr(tokens, "embed tokens", (torch.int32,)), self._ptr(table, "embed table"),
+            self._ptr(tokens, "embed tokens", (torch.int32,)), self._ptr(token_src, "embed token_src", (torch.int32,), True),
+            self._ptr(fed_tokens, "embed fed tokens", (torch.int32,), True), self._ptr(table, "embed table"),
             _code(table, "embed table"), self._ptr(out, "embed out", (torch.float32,)), n_rows, width,
-            self._stream()))
+            table.shape[0], self._stream()))
 
     def rmsnorm(self, x, weight, eps, out, rows=None):
         """out[r] = x[rows[r] if rows is given else r] * inv_rms * weight; x f32 [*, D], out [n, D]."""

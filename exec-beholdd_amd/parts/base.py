@@ -101,6 +101,8 @@ class StepContext:
     is_decode: bool
     max_position: int                      # largest absolute position in this step
     max_rows_per_seq: int = 1              # most tokens any one sequence brings
+    token_src: torch.Tensor | None = None  # int32 [T]: >= 0 where a row's token is fed_tokens[token_src[row]]
+    fed_tokens: torch.Tensor | None = None # int32: tokens chosen on the device that the host has not read yet
     extras: dict = field(default_factory=dict)
 
     def new_activations(self, *shape) -> torch.Tensor:

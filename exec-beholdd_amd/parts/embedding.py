@@ -28,7 +28,10 @@ class Embedding:
 
     def forward(self, ctx):
         hidden = ctx.new_f32(ctx.n_rows, self.width)
-        ctx.kernels.embed(ctx.tokens, self.weight, hidden)
+        if ctx.token_src is not None:
+            ctx.kernels.embed(ctx.tokens, self.weight, hidden, token_src=ctx.token_src, fed_tokens=ctx.fed_tokens)
+        else:
+            ctx.kernels.embed(ctx.tokens, self.weight, hidden)
         return hidden
 
 

@@ -54,19 +54,74 @@ class SamplingError(RuntimeError):
     pass
 
 
+class Selection:
+    """Tokens that the selection kernel has chosen, or is still choosing, for some rows.
+
+    `result()` waits for them and returns them as a list (raising for a row whose logits were not
+    finite).  Until then, and afterwards, the tokens also stand in the sampler's device buffer:
+    element i at row `device_rows[i]`, where the next step can read them without the host
+    (`StepEntry.fed_row`).  A selection is good until the sampler has made a few more."""
+
+    def __init__(self, host, event, device_rows, requests, steps):
+        self._host, self._event = host, event
+        self.device_rows, self.requests, self.steps = list(device_rows), list(requests), list(steps)
+
+    def __len__(self):
+        return len(self.device_rows)
+
+    def take(self, positions):
+        """The selection restricted to some of its elements."""
+        return Selection(self._host, self._event, [self.device_rows[i] for i in positions],
+                         [self.requests[i] for i in positions], [self.steps[i] for i in positions])
+
+    def token_at(self, device_row: int) -> int:
+        """The token at a row of the device buffer, waited for; no check of the row's flag."""
+        if self._event is not None:
+            self._event.synchronize()
+        return int(self._host[0, device_row])
+
+    def result(self) -> list:
+        if self._event is not None:
+            self._event.synchronize()
+        tokens = []
+        for row, request, step in zip(self.device_rows, self.requests, self.steps):
+            if int(self._host[1, row]):
+                raise SamplingError(f"request {request}, step {step}: a logit is not finite")
+            tokens.append(int(self._host[0, row]))
+        return tokens
+
+
 class Sampler:
     """Runs the selection kernel on rows of float32 logits."""
 
-    def __init__(self, kernels, device):
-        self.kernels, self.device = kernels, torch.device(device)
+    RING = 4      # host buffers in turn: a selection stays readable while the next few are made
 
-    def select(self, logits: torch.Tensor, params: list, requests: list, steps: list) -> list:
-        """One token per row of `logits`; row i belongs to request `requests[i]` at step `steps[i]`."""
+    def __init__(self, kernels, device, capacity: int = 64):
+        self.kernels, self.device = kernels, torch.device(device)
+        self._allocate(int(capacity))
+
+    def _allocate(self, capacity):
+        self.capacity = capacity
+        # row 0: tokens, row 1: the not-finite flags.  Captured graphs read row 0, so the engine sizes the
+        # sampler once for its largest batch and this buffer is never replaced under it.
+        self.out = torch.zeros((2, capacity), dtype=torch.int32, device=self.device)
+        pin = self.device.type == "cuda"
+        self._hosts = [torch.zeros((2, capacity), dtype=torch.int32, pin_memory=pin) for _ in range(self.RING)]
+        self._turn = 0
+
+    @property
+    def device_tokens(self) -> torch.Tensor:
+        return self.out[0]
+
+    def select_async(self, logits: torch.Tensor, params: list, requests: list, steps: list) -> Selection:
+        """Start choosing one token per row of `logits` (row i belongs to request `requests[i]` at step
+        `steps[i]`) and bring them to the host without waiting for either."""
         n_rows = logits.shape[0]
         if not (len(params) == len(requests) == len(steps) == n_rows):
             raise ValueError("one sampling parameter set, request index and step per row")
-        both = torch.empty((2, n_rows), dtype=torch.int32, device=self.device)   # one copy brings both back
-        tokens, bad = both[0], both[1]
+        if n_rows > self.capacity:
+            self._allocate(n_rows)
+        tokens, bad = self.out[0, :n_rows], self.out[1, :n_rows]
         if all(p.greedy for p in params):
             self.kernels.sample(logits, tokens, bad)
         else:
@@ -76,8 +131,17 @@ class Sampler:
             top_k = torch.tensor([p.top_k for p in params], dtype=torch.int32).to(self.device)
             self.kernels.sample(logits, tokens, bad, temperature=columns[0], top_k=top_k, top_p=columns[1],
                                 uniform=columns[2])
-        result = both.cpu()
-        for row in range(n_rows):
-            if int(result[1, row]):
-                raise SamplingError(f"request {requests[row]}, step {steps[row]}: a logit is not finite")
-        return [int(t) for t in result[0]]
+        host = self._hosts[self._turn]
+        self._turn = (self._turn + 1) % self.RING
+        event = None
+        if self.device.type == "cuda":
+            host.copy_(self.out, non_blocking=True)
+            event = torch.cuda.Event()
+            event.record()
+        else:
+            host.copy_(self.out)
+        return Selection(host, event, range(n_rows), requests, steps)
+
+    def select(self, logits: torch.Tensor, params: list, requests: list, steps: list) -> list:
+        """One token per row of `logits`, on the host."""
+        return self.select_async(logits, params, requests, steps).result()

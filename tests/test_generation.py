@@ -185,3 +185,99 @@ def test_uniform_numbers_are_a_pure_function_of_seed_request_step():
     for bad in (dict(temperature=-1.0), dict(top_k=-1), dict(top_p=0.0), dict(top_p=1.5)):
         with pytest.raises(ValueError):
             SamplingParams(**bad)
+
+
+# ---- the loop that runs one step ahead of the host ------------------------------------------------
+
+class AheadStepper(ScriptedStepper):
+    """The scripted stepper with selections that the next step can read "on the device": an entry with
+    `fed_row` takes its token from that row of the last selection's buffer."""
+
+    class Selection:
+        def __init__(self, owner, buffer, device_rows, error=None):
+            self.owner, self.buffer, self.device_rows, self.error = owner, buffer, list(device_rows), error
+
+        def take(self, positions):
+            return AheadStepper.Selection(self.owner, self.buffer, [self.device_rows[i] for i in positions], self.error)
+
+        def result(self):
+            self.owner.results_read += 1
+            if self.error is not None:
+                raise self.error
+            return [self.buffer[row] for row in self.device_rows]
+
+    def __init__(self, *args, **kwargs):
+        super().__init__(*args, **kwargs)
+        self.buffer, self.results_read, self.wasted = [], 0, 0
+
+    def step(self, entries):
+        resolved = []
+        for e in entries:
+            if e.fed_row is not None:
+                assert e.tokens == [0] and e.want == [0]
+                e = type(e)(e.slot, [self.buffer[e.fed_row]], e.want)
+            resolved.append(e)
+        return super().step(resolved)
+
+    def select_async(self, logits, params, requests, steps):
+        self.buffer = self.select(logits, params, requests, steps)       # a new selection overwrites the buffer
+        return AheadStepper.Selection(self, self.buffer, range(len(self.buffer)))
+
+
+def both_loops(**kwargs):
+    return [ScriptedStepper(**kwargs), AheadStepper(**kwargs)]
+
+
+def test_the_loop_ahead_gives_the_same_tokens_reasons_and_callbacks():
+    prompts = [[1, 2, 3], [2, 2], [5], [7, 1]]
+    free_run = [expected_tokens(ScriptedStepper(), p, 9) for p in prompts]
+    for stop in (free_run[1][2], free_run[0][0], free_run[3][8], 49):
+        outcomes = []
+        for s in both_loops():
+            seen = []
+            results = generate(s, prompts, [9, 9, 4, 9], stop_token_ids=[stop], on_token=lambda i, t: seen.append((i, t)))
+            outcomes.append(([(r.token_ids, r.finish_reason, r.stop_token) for r in results], seen))
+            assert s.state == {} and sorted(s.free) == list(range(s.max_slots))       # every slot came back, once
+        assert outcomes[0] == outcomes[1]
+
+
+def test_the_loop_ahead_steps_a_stopped_sequence_once_in_vain_and_no_more():
+    prompts = [[1, 2, 3], [2, 2], [5]]
+    plain, ahead = both_loops()
+    free_run = [expected_tokens(plain, p, 6) for p in prompts]
+    stop = free_run[1][2]
+    generate(plain, prompts, 6, stop_token_ids=[stop])
+    generate(ahead, prompts, 6, stop_token_ids=[stop])
+    rows = lambda s: sum(len(slots) for _, slots in s.steps)
+    stopped = sum(1 for tokens in free_run if stop in tokens[:5])     # a stop at the last token costs no extra step
+    assert rows(ahead) == rows(plain) + stopped
+    # ends by length are known beforehand: nothing is stepped in vain
+    plain, ahead = both_loops()
+    generate(plain, [[1], [2], [3]], [2, 5, 3])
+    generate(ahead, [[1], [2], [3]], [2, 5, 3])
+    assert [len(slots) for _, slots in ahead.steps] == [len(slots) for _, slots in plain.steps] == [3, 3, 2, 1, 1]
+    assert [e for e in ahead.log if e[0] == "free"] == [("free", 0), ("free", 2), ("free", 1)]
+
+
+def test_the_loop_ahead_batches_errors_and_limits():
+    s = AheadStepper(max_slots=3)
+    prompts = [[i + 1] * (i + 1) for i in range(8)]
+    results = generate(s, prompts, 4)
+    assert [r.token_ids for r in results] == [expected_tokens(s, p, 4) for p in prompts]
+    assert s.peak_slots == 3 and s.state == {}
+    assert generate(AheadStepper(), [[1, 2], [3]], [0, 1])[1].completion_tokens == 1
+    assert generate(AheadStepper(max_position=10), [[1] * 10], 1)[0].completion_tokens == 1
+
+    def on_token(index, token):
+        if index == 1:
+            raise RuntimeError("consumer went away")
+
+    s = AheadStepper()
+    with pytest.raises(RuntimeError, match="went away"):
+        generate(s, [[1], [2], [3]], 4, on_token=on_token)
+    assert s.state == {}
+    # with a callback for logits the plain loop runs (the rows must still be there when the callback looks)
+    s = AheadStepper()
+    looked = []
+    generate(s, [[1], [2]], 3, on_logits=lambda i, step, row: looked.append((i, step)))
+    assert s.results_read == 0 and looked == [(0, 0), (1, 0), (0, 1), (1, 1), (0, 2), (1, 2)]

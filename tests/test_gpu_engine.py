@@ -216,8 +216,14 @@ def test_greedy_generation_through_the_entry_point(model_dirs):
             logits = plain.forward_logits(cfg, weights, tokens)[-1]
             assert logits[token] >= logits.max() - 2e-2 * np.abs(logits).max()
             tokens.append(token)
-    engine.cache.check_invariants()
-    assert engine.cache.live_slots() == []
+    # the loop that runs a step ahead of the host and the plain one (which a callback for logits selects) agree
+    for runner in (engine, engine16):
+        ahead = runner.generate(prompts, max_new_tokens=8, stop_token_ids=[stop])
+        plain_loop = runner.generate(prompts, max_new_tokens=8, stop_token_ids=[stop], on_logits=lambda *_: None)
+        assert [(r.token_ids, r.finish_reason, r.stop_token) for r in ahead] == \
+               [(r.token_ids, r.finish_reason, r.stop_token) for r in plain_loop]
+        runner.cache.check_invariants()
+        assert runner.cache.live_slots() == []
 
 
 def test_temperature_sampling_is_seeded_and_independent_of_the_batch(model_dirs):
