@@ -226,19 +226,37 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
   }
 }
 
+// One block per column.  Nothing here may wait for one split's numbers before asking for the next
+// one's: with 32 splits that is 32 trips to the L2 in a row.  So the lanes of a wave fetch the splits'
+// (maximum, sum) pairs side by side, and the partial outputs are fetched eight splits at a time.
 __global__ void attention_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                          uint16_t* __restrict__ out, int n_splits, int HD) {
   const size_t column = blockIdx.x;
   const float* ml = part_ml + column * n_splits * 2;
+  const int lane = threadIdx.x % BH_WAVE;
   float top = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) top = fmaxf(top, ml[2 * s]);
-  float sum = 0.f;
-  for (int s = 0; s < n_splits; ++s) sum += ml[2 * s + 1] * exp2f(ml[2 * s] - top);
+  for (int s = lane; s < n_splits; s += BH_WAVE) top = fmaxf(top, ml[2 * s]);
+#pragma unroll
+  for (int off = BH_WAVE / 2; off > 0; off >>= 1) top = fmaxf(top, __shfl_xor(top, off, BH_WAVE));
+  float sum = 0.f;   // in the order: each lane its splits upwards, then the lanes pairwise
+  for (int s = lane; s < n_splits; s += BH_WAVE) sum += ml[2 * s + 1] * exp2f(ml[2 * s] - top);
+#pragma unroll
+  for (int off = BH_WAVE / 2; off > 0; off >>= 1) sum += __shfl_xor(sum, off, BH_WAVE);
+  const float inv = 1.0f / sum;
   for (int d = threadIdx.x; d < HD; d += blockDim.x) {
     float value = 0.f;
-    for (int s = 0; s < n_splits; ++s)
-      value += part_o[(column * n_splits + s) * HD + d] * exp2f(ml[2 * s] - top);
-    out[column * HD + d] = f32_to_bf16_bits(value / sum);
+    for (int s0 = 0; s0 < n_splits; s0 += 8) {
+      float weight[8], part[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int s = s0 + u < n_splits ? s0 + u : n_splits - 1;
+        weight[u] = s0 + u < n_splits ? ml[2 * s] : -INFINITY;
+        part[u] = part_o[(column * n_splits + s) * HD + d];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) value += part[u] * exp2f(weight[u] - top);
+    }
+    out[column * HD + d] = f32_to_bf16_bits(value * inv);
   }
 }
 

@@ -85,16 +85,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
                                                                  SkinnyNorm norm) {
   __shared__ float partial[WAVES][RT][MB][256];
   __shared__ float row_factor[MB * 16];
+  // The norm ahead: 32 threads per row, each with every 32nd partial sum.  The first 256 of a row are asked
+  // for here and added up after the product's main loop, so that nobody waits for them.
+  constexpr int ROWS_PER_PASS = WAVES * 2, PASSES = (MB * 16 + ROWS_PER_PASS - 1) / ROWS_PER_PASS;
+  const int part = threadIdx.x % 32;
+  float early[PASSES][8];
   if (norm.ahead_ss) {
-    // 32 threads per row: each adds every 32nd partial sum, then the 32 are added pairwise
-    for (int r0 = 0; r0 < MB * 16; r0 += WAVES * 2) {
-      const int r = r0 + threadIdx.x / 32, part = threadIdx.x % 32;
-      float ss = 0.f;
-      if (r < M)
-        for (int block = part; block < norm.ahead_blocks; block += 32) ss += norm.ahead_ss[(size_t)block * M + r];
 #pragma unroll
-      for (int off = 16; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
-      if (part == 0 && r < MB * 16) row_factor[r] = (r < M) ? 1.0f / sqrtf(ss / (float)K + norm.ahead_eps) : 0.f;
+    for (int pass = 0; pass < PASSES; ++pass) {
+      const int r = pass * ROWS_PER_PASS + threadIdx.x / 32;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int block = part + 32 * u;
+        early[pass][u] = (r < M && block < norm.ahead_blocks) ? norm.ahead_ss[(size_t)block * M + r] : 0.f;
+      }
     }
   }
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
@@ -183,6 +187,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
         acc[t][b] = MFMA16(w0, x0, acc[t][b]);
         acc[t][b] = MFMA16(w1, x1, acc[t][b]);
       }
+    }
+  }
+  if (norm.ahead_ss) {
+#pragma unroll
+    for (int pass = 0; pass < PASSES; ++pass) {
+      const int r = pass * ROWS_PER_PASS + threadIdx.x / 32;
+      float ss = 0.f;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) ss += early[pass][u];
+      if (r < M)
+        for (int block = part + 256; block < norm.ahead_blocks; block += 32) ss += norm.ahead_ss[(size_t)block * M + r];
+#pragma unroll
+      for (int off = 16; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+      if (part == 0 && r < MB * 16) row_factor[r] = (r < M) ? 1.0f / sqrtf(ss / (float)K + norm.ahead_eps) : 0.f;
     }
   }
   // D: lane holds column (activation row) i and rows (W rows) 4g..4g+3; lay it out as [m][n]
