@@ -90,8 +90,10 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
     for (int dt = 0; dt < 2 * NS; ++dt) o[ct][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 
+  int page_ahead = (begin + wave < end) ? table[begin + wave] : 0;   // a page's number is asked for one page early
   for (int p = begin + wave; p < end; p += 4) {
-    const int page = table[p];
+    const int page = page_ahead;
+    if (p + 4 < end) page_ahead = table[p + 4];
     const uint16_t* kb = k_pages + ((size_t)page * KVH + kvh) * BH_PAGE * HD;
     const uint16_t* vb = v_pages + ((size_t)page * KVH + kvh) * HD * BH_PAGE;
     u32x4_t k_vec[4][NS], v_vec[2 * NS][2];

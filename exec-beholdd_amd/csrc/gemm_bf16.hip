@@ -408,6 +408,133 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const uint16_t
   }
 }
 
+// ---- tiled, whole tiles of the packed layout ---------------------------------------------------
+// The same product for the common case: W in the tiles layout, K a multiple of 64, N a multiple of 16, and
+// M and N at least a tile.  Then no load needs a bounds check: a tile that would stick out is moved back
+// inside (its last row or column on the matrix's last) and stores only what the tile it stands for owns.
+// Every thread's loads of a slice differ from one another by amounts that are the same for all threads,
+// so a thread keeps one offset for A and one for W instead of a pointer per load; with the registers this
+// frees, the compiler reads the next operand fragments from LDS while the current ones are multiplied.
+
+template <bool SWIGLU, int WX, int WY, int WM, int WN, int BUFFERS, typename TC>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_whole_kernel(const uint16_t* __restrict__ a,
+                                                                         const uint16_t* __restrict__ w,
+                                                                         TC* __restrict__ c, int M, int N, int K,
+                                                                         int accumulate) {
+  constexpr int THREADS = 64 * WM * WN;
+  constexpr int TBM = 32 * WX * WM, TBN = 32 * WY * WN;
+  constexpr int A_PIECES = TBM * 8 / THREADS, W_PIECES = TBN * 8 / THREADS;
+  constexpr int A_ROWS = THREADS / 8;      // rows of A that one round of the workgroup's loads covers
+  constexpr int W_BLOCKS = THREADS / 128;  // 16-row blocks of W per round
+  constexpr int OUTS = SWIGLU ? TBN / 2 : TBN;   // output columns of a tile
+  static_assert(TBM * 8 % THREADS == 0 && TBN * 8 % THREADS == 0, "the tile is staged in whole rounds of the workgroup");
+  static_assert(!SWIGLU || W_BLOCKS == WY, "a round of W loads is the gate half or the up half of one wave column");
+  __shared__ __attribute__((aligned(16))) uint16_t as[BUFFERS][TBM * TPITCH];
+  __shared__ __attribute__((aligned(16))) uint16_t ws[BUFFERS][TBN * TPITCH];
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int m_own = blockIdx.y * TBM, n_own = blockIdx.x * OUTS;   // what this tile stands for
+  const int m0 = min(m_own, M - TBM), n0 = min(n_own, N - OUTS);   // where it computes
+  const int wm = (wave / WN) * 32 * WX, wn = (wave % WN) * 32 * WY;
+
+  // A: piece e = tid + s * THREADS is row e / 8, 16 bytes e % 8 of the slice
+  const uint16_t* a_tile = a + (size_t)m0 * K;
+  const int a_off = (tid / 8) * K + (tid % 8) * 8;                 // + s * A_ROWS * K, the same for all threads
+  const int a_lds = (tid / 8) * TPITCH + (tid % 8) * 8;            // + s * A_ROWS * TPITCH
+  // W: piece e is block e / 128 of the tile's rows in LDS, piece p = e % 128 = u * 64 + l of that block's slice:
+  // row l % 16, k 16 * (l / 16) + 8 u.  LDS block b of round s holds W rows starting at
+  //   plain:  n0 + 16 (b + s * W_BLOCKS)
+  //   SwiGLU: wave column s / 2; s even: gate rows n0 + (s / 2) * 16 WY + 16 b; s odd: the up rows, N further on
+  const int w_block = tid / 128, w_p = tid % 128, w_l = w_p % 64, w_u = w_p / 64;
+  const size_t block_stride = (size_t)(K / 64) * 1024;             // elements from one 16-row block to the next
+  const uint16_t* w_tile = w + (size_t)(n0 / 16) * block_stride;
+  const int w_off = w_block * (int)block_stride + w_p * 8;         // + what round s adds, the same for all threads
+  const int w_lds = (w_block * 16 + w_l % 16) * TPITCH + 16 * (w_l / 16) + 8 * w_u;   // + s * W_BLOCKS * 16 * TPITCH
+  size_t w_round[W_PIECES];
+#pragma unroll
+  for (int s = 0; s < W_PIECES; ++s)
+    w_round[s] = SWIGLU ? ((size_t)(s / 2) * WY + (s % 2 ? (size_t)(N / 16) : 0)) * block_stride
+                        : (size_t)s * W_BLOCKS * block_stride;
+
+  u32x4_t a_reg[A_PIECES], w_reg[W_PIECES];
+  auto fetch = [&](int slice) {
+#pragma unroll
+    for (int s = 0; s < A_PIECES; ++s) a_reg[s] = load16(a_tile + (size_t)s * A_ROWS * K + slice * TK + a_off);
+#pragma unroll
+    for (int s = 0; s < W_PIECES; ++s) w_reg[s] = load16(w_tile + w_round[s] + (size_t)slice * 1024 + w_off);
+  };
+  auto stash = [&](int buffer) {
+#pragma unroll
+    for (int s = 0; s < A_PIECES; ++s)
+      *reinterpret_cast<u32x4_t*>(&as[buffer][a_lds + s * A_ROWS * TPITCH]) = a_reg[s];
+#pragma unroll
+    for (int s = 0; s < W_PIECES; ++s)
+      *reinterpret_cast<u32x4_t*>(&ws[buffer][w_lds + s * W_BLOCKS * 16 * TPITCH]) = w_reg[s];
+  };
+
+  f32x16_t acc[WX][WY];
+#pragma unroll
+  for (int x = 0; x < WX; ++x)
+#pragma unroll
+    for (int y = 0; y < WY; ++y)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[x][y][e] = 0.f;
+
+  const int slices = K / TK;
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  const int frag = (lane % 32) * TPITCH + (lane / 32) * 8;
+  for (int s = 0; s < slices; ++s) {
+    const int buffer = BUFFERS == 2 ? (s & 1) : 0;
+    if (s + 1 < slices) fetch(s + 1);
+#pragma unroll
+    for (int kk = 0; kk < TK; kk += 16) {
+      bf16x8_t af[WX], wf[WY];
+#pragma unroll
+      for (int x = 0; x < WX; ++x)
+        af[x] = as_bf16x8(*reinterpret_cast<const u32x4_t*>(&as[buffer][(wm + x * 32) * TPITCH + kk + frag]));
+#pragma unroll
+      for (int y = 0; y < WY; ++y)
+        wf[y] = as_bf16x8(*reinterpret_cast<const u32x4_t*>(&ws[buffer][(wn + y * 32) * TPITCH + kk + frag]));
+#pragma unroll
+      for (int x = 0; x < WX; ++x)
+#pragma unroll
+        for (int y = 0; y < WY; ++y)
+          acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[x], wf[y], acc[x][y], 0, 0, 0);
+    }
+    if (BUFFERS == 1) __syncthreads();   // one buffer: everyone has read the slice before it is overwritten
+    if (s + 1 < slices) stash(BUFFERS == 2 ? buffer ^ 1 : 0);
+    __syncthreads();
+  }
+  // D of one 32x32 block: column (n) lane%32, rows (m) 8*(e/4) + 4*(lane/32) + e%4
+#pragma unroll
+  for (int x = 0; x < WX; ++x) {
+    if (SWIGLU) {
+#pragma unroll
+      for (int y = 0; y < WY / 2; ++y) {
+        const int n = n0 + (wave % WN) * 16 * WY + y * 32 + lane % 32;
+        if (n < n_own) continue;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int m = m0 + wm + x * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
+          if (m >= m_own) store_out<TC>(c, (size_t)m * N + n, silu_mul(acc[x][y][e], acc[x][y + WY / 2][e]), false);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int y = 0; y < WY; ++y) {
+        const int n = n0 + wn + y * 32 + lane % 32;
+        if (n < n_own) continue;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int m = m0 + wm + x * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
+          if (m >= m_own) store_out<TC>(c, (size_t)m * N + n, acc[x][y][e], accumulate != 0);
+        }
+      }
+    }
+  }
+}
+
 // ---- entry -------------------------------------------------------------------------------------
 
 template <bool TILES, int RT, typename TC>
@@ -434,8 +561,12 @@ static void launch_tiled(const void* a, const void* w, void* c, int M, int N, in
   do {                                                                                                     \
     const int columns = (SWIGLU ? 16 : 32) * WY * WN, rows = 32 * WX * WM;                                 \
     dim3 grid((N + columns - 1) / columns, (M + rows - 1) / rows), block(64 * WM * WN);                    \
-    gemm_tiled_kernel<TILES, SWIGLU, WX, WY, WM, WN, BUFFERS, TC><<<grid, block, 0, stream>>>(             \
-        (const uint16_t*)a, (const uint16_t*)w, (TC*)c, M, N, K, accumulate);                              \
+    if (TILES && K % TK == 0 && N % 16 == 0 && M >= rows && N >= columns && (long)rows * K < (1L << 31))   \
+      gemm_tiled_whole_kernel<SWIGLU, WX, WY, WM, WN, BUFFERS, TC><<<grid, block, 0, stream>>>(            \
+          (const uint16_t*)a, (const uint16_t*)w, (TC*)c, M, N, K, accumulate);                            \
+    else                                                                                                   \
+      gemm_tiled_kernel<TILES, SWIGLU, WX, WY, WM, WN, BUFFERS, TC><<<grid, block, 0, stream>>>(           \
+          (const uint16_t*)a, (const uint16_t*)w, (TC*)c, M, N, K, accumulate);                            \
   } while (0)
   // Measured at the Qwen3-8B shapes (2,048 rows).  The multiplies of a 128 x 128 tile need as many LDS
   // cycles (operand reads and the staging writes) as MFMA cycles, so LDS bounds them; a 256 x 256 tile

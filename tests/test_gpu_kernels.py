@@ -94,7 +94,10 @@ def test_gemm(K, a_dtype, w_dtype, m, n, k):
 @pytest.mark.parametrize("m,n,k", [(1, 96, 128), (8, 331, 192), (64, 130, 64), (65, 257, 1024), (200, 64, 448),
                                    (3, 1000, 4096), (130, 520, 256), (16, 24, 64), (33, 16, 2048),
                                    (8, 4096, 12288), (300, 1000, 1024), (129, 129, 128),
-                                   (1030, 43700, 192)])
+                                   (1030, 43700, 192),
+                                   # whole tiles of the packed layout (N a multiple of 16), last tiles moved back inside
+                                   (300, 1008, 1024), (129, 144, 128), (128, 128, 64), (1030, 43712, 192),
+                                   (2048, 4096, 512)])
 def test_gemm_with_packed_weights(K, m, n, k):
     """The same product from the regrouped (16 x 64 blocks) weight layout."""
     from beholdd.kernels import PackedWeight
