@@ -484,9 +484,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_whole_kernel(const ui
   stash(0);
   __syncthreads();
   const int frag = (lane % 32) * TPITCH + (lane / 32) * 8;
-  for (int s = 0; s < slices; ++s) {
-    const int buffer = BUFFERS == 2 ? (s & 1) : 0;
-    if (s + 1 < slices) fetch(s + 1);
+  auto multiply = [&](int buffer) {
 #pragma unroll
     for (int kk = 0; kk < TK; kk += 16) {
       bf16x8_t af[WX], wf[WY];
@@ -502,10 +500,19 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_whole_kernel(const ui
         for (int y = 0; y < WY; ++y)
           acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[x], wf[y], acc[x][y], 0, 0, 0);
     }
+  };
+  // All slices but the last in a loop without a branch in its body: loads, multiplies and staging writes
+  // are one stretch of code that the compiler may interleave.
+  for (int s = 0; s + 1 < slices; ++s) {
+    const int buffer = BUFFERS == 2 ? (s & 1) : 0;
+    fetch(s + 1);
+    __builtin_amdgcn_sched_barrier(0);   // the loads go out first: a slice of multiplies is their time to land
+    multiply(buffer);
     if (BUFFERS == 1) __syncthreads();   // one buffer: everyone has read the slice before it is overwritten
-    if (s + 1 < slices) stash(BUFFERS == 2 ? buffer ^ 1 : 0);
+    stash(BUFFERS == 2 ? buffer ^ 1 : 0);
     __syncthreads();
   }
+  multiply(BUFFERS == 2 ? ((slices - 1) & 1) : 0);
   // D of one 32x32 block: column (n) lane%32, rows (m) 8*(e/4) + 4*(lane/32) + e%4
 #pragma unroll
   for (int x = 0; x < WX; ++x) {
