@@ -132,9 +132,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
   fetch(begin);
   stash(begin, 0);
   __syncthreads();
-  for (int p = begin; p <= last; ++p) {
-    const int buffer = (p - begin) & 1;
-    if (p < last) fetch(p + 1);
+  auto attend = [&](int p, int buffer) {
     const u32x4_t* kl = page_lds[buffer];
     const u32x4_t* vl = page_lds[buffer] + PIECES;
     // a page none of whose keys this wave's columns may see changes nothing
@@ -215,9 +213,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
         }
       }
     }
-    if (p < last) stash(p + 1, buffer ^ 1);
+  };
+  // all pages but the last in a loop whose body does not branch on the page count, so that the compiler may
+  // interleave the next page's loads and staging writes with this page's arithmetic
+  for (int p = begin; p < last; ++p) {
+    const int buffer = (p - begin) & 1;
+    fetch(p + 1);
+    __builtin_amdgcn_sched_barrier(0);   // the loads go out first
+    attend(p, buffer);
+    stash(p + 1, buffer ^ 1);
     __syncthreads();   // the next page is in place, and everyone is done with the one before it
   }
+  attend(last, (last - begin) & 1);
 
   // lane (j, g) holds O^T[16 dt + 4 g + r, column j] and its share of the column's sum
 #pragma unroll
