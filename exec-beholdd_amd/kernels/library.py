@@ -97,6 +97,8 @@ class HipKernels:
             "bh_gemm_bf16": [p, p, p, i, i, i, i, i, i, i, p, i, f, p, i, p, p, p],
             "bh_attention_bf16": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, i, i, f, i, i, i, p],
             "bh_attention_bf16_splits": [i, i, i, i, i],
+            "bh_attention_decode_fused": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, f, i, i, i, p, p, i, f, p, p, i, i,
+                                          i, p],
             "bh_kv_order": [i, i],
         }
         for name, argtypes in table.items():
@@ -347,6 +349,51 @@ class HipKernels:
             self._ptr(row_seq, "row_seq", (torch.int32,)), self._ptr(positions, "positions", (torch.int32,)),
             n_rows, n_heads, n_kv_heads, head_dim, float(scale), int(window), self.kv_order(k_pages.dtype, head_dim),
             self._stream()))
+
+    def attention_decode_fused(self, qkv, out, q_weight, k_weight, eps, cos, sin, positions, k_pages, v_pages,
+                               page_table, n_heads, n_kv_heads, head_dim, scale, window, write_kv, layout):
+        """`qk_norm_rope_cache` and `attention` in one launch for a step of one row per sequence, from
+        the fused projection rows `qkv` [n, (heads + 2 kv_heads) * head_dim].  Returns False, having done
+        nothing, where the one kernel that does it does not take the operands (then call the two)."""
+        n_rows = qkv.shape[0]
+        rot = 2 * cos.shape[1] if cos is not None else 0
+        if (qkv.dtype != torch.bfloat16 or k_pages.dtype != torch.bfloat16 or layout is None
+                or int(layout.max_rows_per_seq) != 1 or int(layout.n_seqs) != n_rows
+                or head_dim % 32 or head_dim > 256 or n_heads % n_kv_heads or n_heads // n_kv_heads > 16
+                or (cos is not None and (rot != head_dim or head_dim % 64))
+                or self.kv_order(k_pages.dtype, head_dim) != 1):
+            return False
+        if qkv.shape != (n_rows, (n_heads + 2 * n_kv_heads) * head_dim) or out.shape != (n_rows, n_heads * head_dim) \
+                or out.dtype != qkv.dtype:
+            raise KernelError(f"attention_decode_fused: shapes qkv {tuple(qkv.shape)}, out {tuple(out.shape)} do not fit "
+                              f"{n_heads}+2x{n_kv_heads} heads of {head_dim}")
+        if positions.shape != (n_rows,) or layout.seq_start.shape != (n_rows + 1,) or page_table.shape[0] < n_rows:
+            raise KernelError("attention_decode_fused: one position and one page-table row per sequence, and seq_start")
+        if (q_weight is None) != (k_weight is None) or (cos is None) != (sin is None):
+            raise KernelError("attention_decode_fused: norm weights come in pairs, and so do the rotation tables")
+        w_code = F32
+        if q_weight is not None:
+            if q_weight.shape != (head_dim,) or k_weight.shape != (head_dim,) or q_weight.dtype != k_weight.dtype:
+                raise KernelError("attention_decode_fused: norm weights must be [head_dim] and of one dtype")
+            w_code = _code(q_weight, "norm weight")
+        if cos is not None and (cos.shape != sin.shape or cos.dim() != 2):
+            raise KernelError("attention_decode_fused: cos and sin tables must be matrices of one shape")
+        self._check_pages(k_pages, v_pages, page_table, n_kv_heads, head_dim, qkv.dtype, "attention_decode_fused")
+        n_splits = int(self.lib.bh_attention_bf16_splits(n_rows, 1, n_heads, n_kv_heads, int(layout.max_position)))
+        part_o = part_ml = None
+        if n_splits > 1:
+            part_o = torch.empty(n_rows * n_heads * n_splits * head_dim, dtype=torch.float32, device=self.device)
+            part_ml = torch.empty(n_rows * n_heads * n_splits * 2, dtype=torch.float32, device=self.device)
+        self._check(self.lib.bh_attention_decode_fused(
+            self._ptr(qkv, "qkv"), self._ptr(out, "attention out"), self._ptr(part_o, "partial o", None, True),
+            self._ptr(part_ml, "partial sums", None, True), self._ptr(k_pages, "k_pages"), self._ptr(v_pages, "v_pages"),
+            self._ptr(page_table, "page_table", (torch.int32,)), page_table.shape[1],
+            self._ptr(positions, "positions", (torch.int32,)), self._ptr(layout.seq_start, "seq_start", (torch.int32,)),
+            n_rows, n_heads, n_kv_heads, head_dim, float(scale), int(window), int(layout.max_position), n_splits,
+            self._ptr(q_weight, "q_norm", None, True), self._ptr(k_weight, "k_norm", None, True), w_code, float(eps),
+            self._ptr(cos, "cos", (torch.float32,), True), self._ptr(sin, "sin", (torch.float32,), True),
+            cos.shape[0] if cos is not None else 0, rot, int(bool(write_kv)), self._stream()))
+        return True
 
     def swiglu(self, gate_up, out):
         """out[r, i] = silu(gate_up[r, i]) * gate_up[r, F + i]."""

@@ -419,6 +419,67 @@ def test_attention_prefill_many_columns(K, n_heads, kv_heads, head_dim, window):
         assert rel(out[rows], want) < 1.2e-2, (s, rel(out[rows], want))
 
 
+@pytest.mark.parametrize("window", [0, 70])
+@pytest.mark.parametrize("with_norm,with_rope,write_kv", [(True, True, True), (False, True, True), (True, False, True),
+                                                          (True, True, False)])
+@pytest.mark.parametrize("n_heads,kv_heads,head_dim", [(32, 8, 128), (8, 2, 64), (4, 4, 128), (6, 1, 256), (16, 1, 64)])
+def test_decode_attention_from_the_projection_rows(K, n_heads, kv_heads, head_dim, with_norm, with_rope, write_kv, window):
+    """Norm, rotation, cache write and attention of a decode step in one launch give what the two launches
+    give: the same output and the same cache, for sequences at a page's first and last slot, at position 0,
+    and long enough for split keys."""
+    dtype = torch.bfloat16
+    lengths = [1, 64, 65, 128, 131, 2500, 700]             # the new token stands at length - 1
+    n = len(lengths)
+    kp, vp, table, keys, values = make_cache(n, lengths, kv_heads, head_dim, dtype, seed=head_dim + n_heads)
+    gen = torch.Generator().manual_seed(5)
+    qkv = torch.randn(n, (n_heads + 2 * kv_heads) * head_dim, generator=gen).to(dtype)
+    qw = kw = cos = sin = None
+    if with_norm:
+        qw = dev((1 + 0.2 * torch.randn(head_dim, generator=gen)).to(dtype))
+        kw = dev((1 + 0.2 * torch.randn(head_dim, generator=gen)).to(dtype))
+    if with_rope:
+        freqs = 1.0 / 10000.0 ** (torch.arange(0, head_dim, 2, dtype=torch.float64) / head_dim)
+        angles = torch.arange(2600, dtype=torch.float64)[:, None] * freqs
+        cos, sin = dev(angles.cos().float()), dev(angles.sin().float())
+    positions = dev(torch.tensor([length - 1 for length in lengths], dtype=torch.int32))
+    row_seq = dev(torch.arange(n, dtype=torch.int32))
+    layout = Layout(True, dev(torch.arange(n + 1, dtype=torch.int32)), n, 1, max(lengths) - 1)
+    scale, eps = 1 / math.sqrt(head_dim), 1e-5
+
+    k_two, v_two = stored(K, kp, vp)
+    q = torch.empty(n, n_heads * head_dim, dtype=dtype, device="cuda:0")
+    out_two = torch.empty_like(q)
+    K.qk_norm_rope_cache(dev(qkv), q, qw, kw, eps, cos, sin, positions, row_seq, k_two, v_two, dev(table), n_heads,
+                         kv_heads, head_dim, write_kv, max(lengths) - 1)
+    K.attention(q, out_two, k_two, v_two, dev(table), row_seq, positions, n_heads, kv_heads, head_dim, scale, window,
+                layout=layout)
+
+    k_one, v_one = stored(K, kp, vp)
+    out_one = torch.empty_like(q)
+    took = K.attention_decode_fused(dev(qkv), out_one, qw, kw, eps, cos, sin, positions, k_one, v_one, dev(table),
+                                    n_heads, kv_heads, head_dim, scale, window, write_kv, layout)
+    assert took is True
+    assert bool(torch.isfinite(out_one.float()).all())
+    assert rel(out_one, out_two.double()) < 8e-3, rel(out_one, out_two.double())
+    assert torch.equal(v_one.cpu(), v_two.cpu())
+    assert rel(k_one, k_two.double()) < 8e-3                  # the same numbers but for the order of two float32 sums
+    assert (k_one.cpu() != k_two.cpu()).float().mean() < 1e-3
+    if not write_kv:
+        assert torch.equal(k_one.cpu(), stored(K, kp, vp)[0].cpu())
+
+
+def test_decode_attention_from_the_projection_rows_says_when_it_cannot(K):
+    dtype = torch.bfloat16
+    kp, vp, table, _, _ = make_cache(1, [10], 2, 48, dtype, seed=1)
+    qkv = dev(torch.randn(1, 8 * 48).to(dtype))
+    out = torch.empty(1, 4 * 48, dtype=dtype, device="cuda:0")
+    layout = Layout(True, dev(torch.tensor([0, 1], dtype=torch.int32)), 1, 1, 9)
+    positions = dev(torch.tensor([9], dtype=torch.int32))
+    k_pages, v_pages = stored(K, kp, vp)
+    assert K.attention_decode_fused(qkv, out, None, None, 0.0, None, None, positions, k_pages, v_pages, dev(table),
+                                    4, 2, 48, 0.1, 0, True, layout) is False          # head size 48
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("far", [0, 63, 64, 127, 128, 300, 511, 640])
 def test_attention_finds_one_far_key_among_hundreds(K, dtype, far):
