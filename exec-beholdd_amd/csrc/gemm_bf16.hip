@@ -578,13 +578,14 @@ static void launch_tiled(const void* a, const void* w, void* c, int M, int N, in
   // Measured at the Qwen3-8B shapes (2,048 rows).  The multiplies of a 128 x 128 tile need as many LDS
   // cycles (operand reads and the staging writes) as MFMA cycles, so LDS bounds them; a 256 x 256 tile
   // of eight waves, each 64 x 128, reads a quarter less per multiply and wins once it still gives every
-  // compute unit three tiles.  Below that the smaller tile keeps more compute units busy: with two LDS
-  // buffers when there are several rounds of workgroups, with one (four workgroups per compute unit, a
-  // second barrier per slice) when there is about one round.
+  // compute unit three tiles.  Below that the smaller tile keeps more compute units busy.  Two LDS buffers
+  // (one barrier per slice, two workgroups per compute unit) are the better choice unless a single one
+  // (four workgroups per compute unit) lets the whole grid run at once: between two and four tiles for
+  // each of the 256 compute units.
   const long tiles_128 = (long)((N + (SWIGLU ? 63 : 127)) / (SWIGLU ? 64 : 128)) * ((M + 127) / 128);
   if (tiles_128 >= 3072) BH_TILED(2, 4, 4, 2, 2);
-  else if (tiles_128 >= 1024) BH_TILED(2, 2, 2, 2, 2);
-  else BH_TILED(2, 2, 2, 2, 1);
+  else if (tiles_128 > 512 && tiles_128 <= 1024) BH_TILED(2, 2, 2, 2, 1);
+  else BH_TILED(2, 2, 2, 2, 2);
 #undef BH_TILED
 }
 
