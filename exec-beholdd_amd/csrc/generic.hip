@@ -304,6 +304,95 @@ __global__ __launch_bounds__(64) void qk_norm_rope_cache_kernel(
   }
 }
 
+// eight consecutive elements at an 8-element boundary, in one or two loads
+__device__ inline void load_eight(const float* p, float (&v)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ inline void load_eight(const bf16_t* p, float (&v)[8]) {
+  const uint4 q = *reinterpret_cast<const uint4*>(p);
+  const uint32_t words[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = bf16_bits_to_f32((uint16_t)(words[e / 2] >> (16 * (e % 2))));
+}
+
+// The same for many bfloat16 rows: a lane takes 8 consecutive elements of a head (16 bytes), LPH = head_dim / 8
+// lanes a head, 64 / LPH heads a wave, four waves a block.  The rotation spans the whole head or is absent, so
+// that an element's partner sits LPH / 2 lanes away.  Per head: one 16-byte load, one 16-byte store (values:
+// eight 2-byte stores, as their neighbours in memory are other tokens).
+template <typename TW, int LPH>
+__global__ __launch_bounds__(256) void qk_norm_rope_cache_rows_kernel(
+    const uint16_t* __restrict__ qkv, uint16_t* __restrict__ q_out, const TW* __restrict__ q_weight,
+    const TW* __restrict__ k_weight, float eps, const float* __restrict__ cos_table,
+    const float* __restrict__ sin_table, const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
+    uint16_t* __restrict__ k_pages, uint16_t* __restrict__ v_pages, const int32_t* __restrict__ page_table,
+    int table_stride, int H, int KVH, int kv_order, int n_rows, int n_heads) {
+  constexpr int HD = 8 * LPH, HPW = BH_WAVE / LPH;
+  const int waves_per_row = (n_heads + HPW - 1) / HPW;
+  const int wave = blockIdx.x * 4 + threadIdx.x / BH_WAVE, lane = threadIdx.x % BH_WAVE;
+  const int row = wave / waves_per_row;
+  if (row >= n_rows) return;   // whole waves leave; nothing below synchronises the block
+  const int wanted = (wave % waves_per_row) * HPW + lane / LPH, c = lane % LPH;
+  const bool active = wanted < n_heads;
+  const int head = active ? wanted : n_heads - 1;   // lanes without a head of their own follow the last one and store nothing
+  const bool is_q = head < H, is_value = head >= H + KVH;
+  const int pos = positions[row];
+  const uint16_t* src = qkv + ((size_t)row * (H + 2 * KVH) + head) * HD + 8 * c;
+  const uint4 raw = *reinterpret_cast<const uint4*>(src);
+  const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+  float x[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) x[e] = bf16_bits_to_f32((uint16_t)(words[e / 2] >> (16 * (e % 2))));
+  const TW* weight = is_q ? q_weight : k_weight;
+  if (!is_value) {
+    if (weight != nullptr) {
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
+#pragma unroll
+      for (int off = LPH / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, BH_WAVE);
+      const float inv = 1.0f / sqrtf(ss / (float)HD + eps);
+      float wv[8];
+      load_eight(weight + 8 * c, wv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] = x[e] * inv * wv[e];
+    }
+    if (cos_table != nullptr) {
+      constexpr int HALF = HD / 2;
+      const bool lower = c < LPH / 2;
+      float cs[8], sn[8];
+      load_eight(cos_table + (size_t)pos * HALF + 8 * (c % (LPH / 2)), cs);
+      load_eight(sin_table + (size_t)pos * HALF + 8 * (c % (LPH / 2)), sn);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float other = __shfl_xor(x[e], LPH / 2, BH_WAVE);
+        x[e] = lower ? x[e] * cs[e] - other * sn[e] : other * sn[e] + x[e] * cs[e];
+      }
+    }
+  }   // (all the lanes of a head take the same way through this: the exchanges stay within the head)
+  if (!active) return;
+  uint4 packed;
+  packed.x = (uint32_t)f32_to_bf16_bits(x[0]) | ((uint32_t)f32_to_bf16_bits(x[1]) << 16);
+  packed.y = (uint32_t)f32_to_bf16_bits(x[2]) | ((uint32_t)f32_to_bf16_bits(x[3]) << 16);
+  packed.z = (uint32_t)f32_to_bf16_bits(x[4]) | ((uint32_t)f32_to_bf16_bits(x[5]) << 16);
+  packed.w = (uint32_t)f32_to_bf16_bits(x[6]) | ((uint32_t)f32_to_bf16_bits(x[7]) << 16);
+  if (is_q) {
+    *reinterpret_cast<uint4*>(q_out + ((size_t)row * H + head) * HD + 8 * c) = packed;
+    return;
+  }
+  const int page = page_table[(size_t)row_seq[row] * table_stride + pos / BH_PAGE];
+  const int token = pos % BH_PAGE, kv_head = (head - H) % KVH;
+  if (!is_value) {
+    uint16_t* block = k_pages + ((size_t)page * KVH + kv_head) * BH_PAGE * HD;
+    *reinterpret_cast<uint4*>(block + bh_key_index(kv_order, token, 8 * c, HD)) = packed;   // 8 dims lie together in both orders
+  } else {
+    uint16_t* block = v_pages + ((size_t)page * KVH + kv_head) * BH_PAGE * HD;
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      block[bh_value_index(kv_order, token, 8 * c + e, HD)] = (uint16_t)(words[e / 2] >> (16 * (e % 2)));
+  }
+}
+
 extern "C" int bh_qk_norm_rope_cache(const void* qkv, int dtype, void* q_out, const void* q_weight,
                                      const void* k_weight, int w_dtype, float eps, const float* cos_table,
                                      const float* sin_table, int table_positions, int rot,
@@ -320,7 +409,30 @@ extern "C" int bh_qk_norm_rope_cache(const void* qkv, int dtype, void* q_out, co
   BH_REQUIRE(kv_order == BH_KV_ROWS || (kv_order == BH_KV_PIECES && hd % 32 == 0),
              "qk_norm_rope: cache order %d does not exist for head size %d", kv_order, hd);
   if (cos_table == nullptr) rot = 0;
-  dim3 grid(n_rows, write_kv ? H + 2 * KVH : H), block(BH_WAVE);
+  const int n_heads = write_kv ? H + 2 * KVH : H;
+  if (dtype == BH_BF16 && n_rows >= 64 && (hd == 64 || hd == 128 || hd == 256) && (rot == 0 || rot == hd)) {
+    const int lanes_per_head = hd / 8, waves = n_rows * ((n_heads + 64 / lanes_per_head - 1) / (64 / lanes_per_head));
+    dim3 wide_grid((waves + 3) / 4), wide_block(4 * BH_WAVE);
+#define BH_QK_ROWS(TW, LPH)                                                                                       \
+  qk_norm_rope_cache_rows_kernel<TW, LPH><<<wide_grid, wide_block, 0, stream>>>(                                   \
+      (const uint16_t*)qkv, (uint16_t*)q_out, (const TW*)q_weight, (const TW*)k_weight, eps,                        \
+      rot ? cos_table : nullptr, rot ? sin_table : nullptr,                                                          \
+      positions, row_seq, (uint16_t*)k_pages, (uint16_t*)v_pages, page_table, table_stride, H, KVH, kv_order,      \
+      n_rows, n_heads)
+#define BH_QK_ROWS_W(LPH)                              \
+  do {                                                 \
+    if (w_dtype == BH_F32) BH_QK_ROWS(float, LPH);     \
+    else BH_QK_ROWS(bf16_t, LPH);                      \
+  } while (0)
+    BH_REQUIRE(w_dtype == BH_F32 || w_dtype == BH_BF16, "qk_norm_rope: unknown weight dtype %d", w_dtype);
+    if (hd == 64) BH_QK_ROWS_W(8);
+    else if (hd == 128) BH_QK_ROWS_W(16);
+    else BH_QK_ROWS_W(32);
+#undef BH_QK_ROWS_W
+#undef BH_QK_ROWS
+    return bh_check_launch("qk_norm_rope_cache_rows");
+  }
+  dim3 grid(n_rows, n_heads), block(BH_WAVE);
 #define BH_QK(T, TW)                                                                                         \
   qk_norm_rope_cache_kernel<T, TW><<<grid, block, 0, stream>>>(                                              \
       (const T*)qkv, (T*)q_out, (const TW*)q_weight, (const TW*)k_weight, eps, cos_table, sin_table, rot,    \

@@ -531,11 +531,13 @@ def test_attention_window_edge(K, dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("w_dtype", DTYPES)
+@pytest.mark.parametrize("news", [[3, 5, 1], [70, 5, 1]])        # few rows, and enough for the kernel for many rows
 @pytest.mark.parametrize("n_heads,kv_heads,head_dim,rot", [(4, 2, 16, 16), (6, 2, 48, 48), (5, 1, 80, 32),
-                                                           (8, 2, 128, 128), (3, 3, 256, 256)])
-def test_qk_norm_rope_cache(K, dtype, w_dtype, n_heads, kv_heads, head_dim, rot):
+                                                           (8, 2, 128, 128), (3, 3, 256, 256), (5, 1, 64, 64),
+                                                           (5, 1, 128, 0), (7, 7, 128, 128), (4, 2, 128, 64)])
+def test_qk_norm_rope_cache(K, dtype, w_dtype, n_heads, kv_heads, head_dim, rot, news):
     g = torch.Generator().manual_seed(head_dim)
-    pasts, news = [0, 62, 130], [3, 5, 1]
+    pasts = [0, 62, 130]
     n_rows = sum(news)
     fused = (n_heads + 2 * kv_heads) * head_dim
     qkv = torch.randn(n_rows, fused, generator=g).to(dtype)
@@ -548,7 +550,7 @@ def test_qk_norm_rope_cache(K, dtype, w_dtype, n_heads, kv_heads, head_dim, rot)
     positions = torch.tensor([p + t for p, n in zip(pasts, news) for t in range(n)], dtype=torch.int32)
     row_seq = torch.tensor([s for s, n in enumerate(news) for _ in range(n)], dtype=torch.int32)
     n_pages = 9
-    table = torch.tensor([[4, 0, 0], [7, 2, 0], [1, 8, 3]], dtype=torch.int32)
+    table = torch.tensor([[4, 5, 0], [7, 2, 0], [1, 8, 3]], dtype=torch.int32)
     sentinel = 768.0        # exact in bfloat16
     kp = torch.full((n_pages, kv_heads, PAGE, head_dim), sentinel).to(dtype)
     vp = torch.full((n_pages, kv_heads, head_dim, PAGE), sentinel).to(dtype)
