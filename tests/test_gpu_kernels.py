@@ -53,7 +53,8 @@ def test_embed(K, dtype, rows, width, vocab):
 @pytest.mark.parametrize("out_dtype", DTYPES)
 @pytest.mark.parametrize("w_dtype", DTYPES)
 @pytest.mark.parametrize("rows,width,eps", [(1, 48, 1e-6), (33, 1000, 1e-5), (4, 5120, 1e-6), (3, 4097, 1e-2),
-                                            (300, 1000, 1e-5), (257, 4096, 1e-6), (256, 260, 1e-6), (301, 4098, 1e-6)])
+                                            (300, 1000, 1e-5), (257, 4096, 1e-6), (256, 260, 1e-6), (301, 4098, 1e-6),
+                                            (258, 256, 1e-6), (270, 2560, 1e-5), (259, 8192, 1e-6)])
 def test_rmsnorm(K, out_dtype, w_dtype, rows, width, eps):
     g = torch.Generator().manual_seed(width)
     x = torch.randn(rows, width, generator=g) * 3 + 0.5
