@@ -27,6 +27,7 @@
 //             rows 8*(i/4) + 4*(l/32) + i%4 for i = 0..15
 // Which 8 of the k values a lane group multiplies is free as long as both operands agree.
 #include "common.h"
+#include <type_traits>
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
@@ -68,13 +69,13 @@ __device__ inline float silu_mul(float gate, float up) { return gate / (1.0f + e
 // The row factor commutes with the product, so the result is the norm's up to the rounding of the
 // activations; the partial sums are added in a fixed order.
 struct SkinnyNorm {
-  const float* ahead_ss;   // [ahead_blocks][M] partial sums of squares for the rows of `a`, or null
+  const float* ahead_ss;   // [M][ahead_blocks] partial sums of squares for the rows of `a`, or null
   int ahead_blocks;
   float ahead_eps;
   const void* behind_weight;  // [N] norm weight for the rows this product completes, or null
   int behind_weight_f32;      // its element type: float32, else bfloat16
   uint16_t* behind_rows;      // [M][N] bfloat16 out
-  float* behind_ss;           // [ceil(N / 16)][M] out
+  float* behind_ss;           // [M][ceil(N / 16)] out
 };
 
 template <int MB, int WAVES, bool TILES, int RT, typename TC>
@@ -97,7 +98,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         const int block = part + 32 * u;
-        early[pass][u] = (r < M && block < norm.ahead_blocks) ? norm.ahead_ss[(size_t)block * M + r] : 0.f;
+        early[pass][u] = (r < M && block < norm.ahead_blocks) ? norm.ahead_ss[(size_t)r * norm.ahead_blocks + block] : 0.f;
       }
     }
   }
@@ -197,7 +198,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
 #pragma unroll
       for (int u = 0; u < 8; ++u) ss += early[pass][u];
       if (r < M)
-        for (int block = part + 256; block < norm.ahead_blocks; block += 32) ss += norm.ahead_ss[(size_t)block * M + r];
+        for (int block = part + 256; block < norm.ahead_blocks; block += 32) ss += norm.ahead_ss[(size_t)r * norm.ahead_blocks + block];
 #pragma unroll
       for (int off = 16; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
       if (part == 0 && r < MB * 16) row_factor[r] = (r < M) ? 1.0f / sqrtf(ss / (float)K + norm.ahead_eps) : 0.f;
@@ -244,10 +245,206 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
         const float g = norm.behind_weight_f32 ? reinterpret_cast<const float*>(norm.behind_weight)[n]
                                                : bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(norm.behind_weight)[n]);
         norm.behind_rows[(size_t)m * N + n] = f32_to_bf16_bits(value * g);
-        if (e % 16 == 0) norm.behind_ss[(size_t)blockIdx.x * M + m] = sq;
+        if (e % 16 == 0) norm.behind_ss[(size_t)m * gridDim.x + blockIdx.x] = sq;
       }
     }
   }
+}
+
+// ---- 17 to 64 rows ---------------------------------------------------------------------------
+// With more than 16 rows the skinny kernel's activations weigh more than its weights: every workgroup
+// reads all of them for 16 weight rows.  Here the eight waves of a workgroup take a block of 16 weight
+// rows each (of the packed layout, whatever they are: a SwiGLU's gate and up rows are just rows) and walk
+// over the same part of K together, 256 columns at a time: the activations of those columns go through
+// LDS once per workgroup, in the order in which the lanes take them, and every wave streams its own
+// weights.  K is cut into parts so that there are enough workgroups; the sums go to scratch memory as
+// [K part][row][weight row].  A second kernel adds the parts in order and does what the skinny kernel
+// does with its sums: the row factor of a norm ahead, SwiGLU, accumulation into the residual, a norm behind.
+
+#define MID_STAGE 4   // 64-wide chunks of K per stage
+
+template <int MB>
+__global__ __launch_bounds__(512) void gemm_mid_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ w,
+                                                       float* __restrict__ sums, int M, int w_rows, int K,
+                                                       int chunks_per_part) {
+  constexpr int WAVES = 8;
+  // activations of a stage as the multiplies take them: piece [chunk][row block][half][lane] holds row
+  // 16 b + lane % 16, columns 64 chunk + 16 (lane / 16) + 8 half .. + 7
+  static_assert(MID_STAGE * 128 == 512, "a thread stages one piece per row block and stage: 512 threads, 128 pieces per chunk and row block");
+  __shared__ u32x4_t xs[2][MID_STAGE][MB][2][64];
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int full = K / 64, n_blocks = (w_rows + 15) / 16;
+  const int block = blockIdx.x * WAVES + wave;
+  const bool own = block < n_blocks;                 // a wave beyond the last block repeats it and stores nothing
+  const uint16_t* wp = w + (size_t)min(block, n_blocks - 1) * full * 1024 + lane * 8;
+  const int first = blockIdx.y * chunks_per_part, end = min(full, first + chunks_per_part);
+
+  // what this thread brings into LDS for a stage: MB pieces
+  const uint16_t* x_src[MB];
+  int x_chunk[MB];
+#pragma unroll
+  for (int j = 0; j < MB; ++j) {
+    const int q = tid + 512 * j, l = q % 64, half = (q / 64) % 2, b = (q / 128) % MB, ch = q / (128 * MB);
+    const int row = min(b * 16 + l % 16, M - 1);
+    x_src[j] = a + (size_t)row * K + (l / 16) * 16 + half * 8;
+    x_chunk[j] = ch;
+  }
+  u32x4_t stage[MB];
+  auto fetch = [&](int c0) {   // chunks beyond the part are brought in as the part's last: they are not multiplied
+#pragma unroll
+    for (int j = 0; j < MB; ++j) stage[j] = load16(x_src[j] + (size_t)min(c0 + x_chunk[j], end - 1) * 64);
+  };
+  auto stash = [&](int buffer) {
+#pragma unroll
+    for (int j = 0; j < MB; ++j) (&xs[buffer][0][0][0][0])[tid + 512 * j] = stage[j];
+  };
+
+  f32x4_t acc[MB];
+#pragma unroll
+  for (int b = 0; b < MB; ++b) acc[b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  // weights of a stage, asked for one stage early (two register sets in turn)
+  u32x4_t wv[2][MID_STAGE][2];
+  auto fetch_w = [&](int c0, auto set_tag) {
+    constexpr int set = decltype(set_tag)::value;
+#pragma unroll
+    for (int ch = 0; ch < MID_STAGE; ++ch) {
+      const uint16_t* p = wp + (size_t)min(c0 + ch, end - 1) * 1024;
+      wv[set][ch][0] = load16_stream(p);
+      wv[set][ch][1] = load16_stream(p + 512);
+    }
+  };
+  auto multiply = [&](int c0, int buffer, auto set_tag) {
+    constexpr int set = decltype(set_tag)::value;
+#pragma unroll
+    for (int ch = 0; ch < MID_STAGE; ++ch) {
+      if (c0 + ch < end) {
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+          acc[b] = MFMA16(wv[set][ch][0], xs[buffer][ch][b][0][lane], acc[b]);
+          acc[b] = MFMA16(wv[set][ch][1], xs[buffer][ch][b][1][lane], acc[b]);
+        }
+      }
+    }
+  };
+  const std::integral_constant<int, 0> set0;
+  const std::integral_constant<int, 1> set1;
+  fetch_w(first, set0);
+  fetch(first);
+  stash(0);
+  __syncthreads();
+  for (int c0 = first; c0 < end; c0 += 2 * MID_STAGE) {
+    // even stage: from LDS buffer 0 and weight set 0, while the next stage's numbers come in
+    const bool more = c0 + MID_STAGE < end;
+    if (more) {   // activations first: they are waited for before this stage ends, the weights (behind them in the queue) are not
+      fetch(c0 + MID_STAGE);
+      fetch_w(c0 + MID_STAGE, set1);
+    }
+    multiply(c0, 0, set0);
+    if (more) stash(1);
+    __syncthreads();   // the next stage is in place, and everyone is done with this one
+    if (!more) break;
+    // odd stage
+    const bool further = c0 + 2 * MID_STAGE < end;
+    if (further) {
+      fetch(c0 + 2 * MID_STAGE);
+      fetch_w(c0 + 2 * MID_STAGE, set0);
+    }
+    multiply(c0 + MID_STAGE, 1, set1);
+    if (further) stash(0);
+    __syncthreads();
+  }
+  // D: lane holds column (activation row) i = lane % 16 and rows (W rows) 4g..4g+3 of the wave's block
+  if (!own) return;
+  const int i = lane % 16, g = lane / 16;
+  float* out = sums + (size_t)blockIdx.y * M * w_rows;
+#pragma unroll
+  for (int b = 0; b < MB; ++b) {
+    const int m = b * 16 + i;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int n = block * 16 + 4 * g + r;
+      if (m < M && n < w_rows) out[(size_t)m * w_rows + n] = acc[b][r];
+    }
+  }
+}
+
+// One block per 16 rows x 16 outputs: thread (r, col) = (tid / 16, tid % 16).  All of a thread's loads are asked
+// for before the first is used.
+#define MID_MAX_PARTS 16
+template <bool SWIGLU, typename TC>
+__global__ __launch_bounds__(256) void gemm_mid_finish_kernel(const float* __restrict__ sums, TC* __restrict__ c,
+                                                              int M, int N, int K, int parts, int accumulate,
+                                                              SkinnyNorm norm) {
+  const int w_rows = SWIGLU ? 2 * N : N;
+  const int col = threadIdx.x % 16, n = blockIdx.x * 16 + col, m = blockIdx.y * 16 + threadIdx.x / 16;
+  const bool valid = m < M && n < N;
+  float first_part[MID_MAX_PARTS], second_part[SWIGLU ? MID_MAX_PARTS : 1];
+#pragma unroll
+  for (int part = 0; part < MID_MAX_PARTS; ++part) {
+    const bool there = valid && part < parts;
+    const float* row = sums + ((size_t)(there ? part : 0) * M + (valid ? m : 0)) * w_rows;
+    first_part[part] = there ? row[n] : 0.f;
+    if (SWIGLU) second_part[part] = there ? row[N + n] : 0.f;
+  }
+  float factor = 1.f;
+  if (norm.ahead_ss) {   // 16 lanes share a row: each adds every 16th partial sum, then the 16 are added pairwise
+    float ss = 0.f;
+    for (int block0 = col; block0 < norm.ahead_blocks; block0 += 16 * 8) {
+      float piece[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int block = block0 + 16 * u;
+        piece[u] = (m < M && block < norm.ahead_blocks) ? norm.ahead_ss[(size_t)m * norm.ahead_blocks + block] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) ss += piece[u];
+    }
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+    factor = 1.0f / sqrtf(ss / (float)K + norm.ahead_eps);
+  }
+  float first = 0.f, second = 0.f;   // the output's sum over the parts, in their order; for SwiGLU the gate's and the up row's
+#pragma unroll
+  for (int part = 0; part < MID_MAX_PARTS; ++part) {
+    first += first_part[part];
+    if (SWIGLU) second += second_part[part];
+  }
+  first *= factor;
+  second *= factor;
+  float value = 0.f;   // what the residual holds afterwards (norm.behind_weight: float32 output, no SwiGLU)
+  if (valid) {
+    if (SWIGLU) {
+      store_out<TC>(c, (size_t)m * N + n, silu_mul(first, second), false);
+    } else if (norm.behind_weight) {
+      float* cf = reinterpret_cast<float*>(c);
+      value = accumulate ? cf[(size_t)m * N + n] + first : first;
+      cf[(size_t)m * N + n] = value;
+    } else {
+      store_out<TC>(c, (size_t)m * N + n, first, accumulate != 0);
+    }
+  }
+  if (!SWIGLU && norm.behind_weight) {
+    float sq = value * value;   // 0 where there is no element
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);   // the 16 columns of a row are 16 neighbouring lanes
+    if (valid) {
+      const float g = norm.behind_weight_f32 ? reinterpret_cast<const float*>(norm.behind_weight)[n]
+                                             : bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(norm.behind_weight)[n]);
+      norm.behind_rows[(size_t)m * N + n] = f32_to_bf16_bits(value * g);
+      if (col == 0) norm.behind_ss[(size_t)m * gridDim.x + blockIdx.x] = sq;
+    }
+  }
+}
+
+// How the 17-to-64-row path cuts K: the number of parts and the 64-wide chunks in each.
+static void mid_parts(int w_rows, int K, int* parts, int* chunks_per_part) {
+  const int full = K / 64, groups = ((w_rows + 15) / 16 + 7) / 8;   // workgroups along the weight rows
+  int p = 1;
+  while (groups * p < 256 && p < MID_MAX_PARTS && full / (p * 2) >= 2 * MID_STAGE) p *= 2;   // enough workgroups, and two stages each at least
+  int chunks = (full + p - 1) / p;
+  chunks = (chunks + MID_STAGE - 1) / MID_STAGE * MID_STAGE;          // whole stages
+  *chunks_per_part = chunks;
+  *parts = (full + chunks - 1) / chunks;
 }
 
 // ---- tiled -----------------------------------------------------------------------------------
@@ -590,12 +787,21 @@ static void launch_tiled(const void* a, const void* w, void* c, int M, int N, in
 }
 
 // layout: 0 = rows, 1 = tiles.  activation: 0 = none; 1 = SwiGLU (W has 2 * N rows: gate rows then up rows).
+// Bytes of scratch memory that bh_gemm_bf16 wants for this product (0: none).
+extern "C" long bh_gemm_bf16_scratch(int M, int N, int K, int layout, int activation) {
+  if (M <= 16 || M > 64 || layout != 1 || K % 64 != 0 || N <= 0) return 0;
+  int parts, chunks;
+  mid_parts(activation ? 2 * N : N, K, &parts, &chunks);
+  return (long)parts * M * (activation ? 2 * N : N) * (long)sizeof(float);
+}
+
 // The `ahead_*` and `behind_*` arguments (null when unused) let an RMSNorm ride on the products before and
-// after it (struct SkinnyNorm); they exist for M <= 64 only.
+// after it (struct SkinnyNorm); they exist for M <= 64 only.  `scratch`: bh_gemm_bf16_scratch() bytes, or
+// null (then products of 17 to 64 rows take the slower way without it).
 extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, int accumulate, int M, int N, int K,
                             int layout, int activation, const float* ahead_ss, int ahead_blocks, float ahead_eps,
                             const void* behind_weight, int behind_weight_dtype, void* behind_rows,
-                            float* behind_ss, hipStream_t stream) {
+                            float* behind_ss, void* scratch, hipStream_t stream) {
   BH_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_bf16: sizes M=%d N=%d K=%d must be positive", M, N, K);
   BH_REQUIRE(K % 8 == 0, "gemm_bf16: K=%d must be a multiple of 8", K);
   BH_REQUIRE(c_dtype == BH_F32 || c_dtype == BH_BF16, "gemm_bf16: unknown output dtype %d", c_dtype);
@@ -620,6 +826,26 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
     if (f32) FN<TILES, EXTRA, float>(__VA_ARGS__);                                  \
     else FN<TILES, EXTRA, bf16_t>(__VA_ARGS__);                                     \
   } while (0)
+  if (scratch != nullptr && bh_gemm_bf16_scratch(M, N, K, layout, activation) > 0) {
+    const int w_rows = activation ? 2 * N : N;
+    int parts, chunks;
+    mid_parts(w_rows, K, &parts, &chunks);
+    dim3 grid(((w_rows + 15) / 16 + 7) / 8, parts);
+    switch ((M + 15) / 16) {
+      case 2: gemm_mid_kernel<2><<<grid, 512, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, (float*)scratch, M, w_rows, K, chunks); break;
+      case 3: gemm_mid_kernel<3><<<grid, 512, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, (float*)scratch, M, w_rows, K, chunks); break;
+      default: gemm_mid_kernel<4><<<grid, 512, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, (float*)scratch, M, w_rows, K, chunks); break;
+    }
+    if (int status = bh_check_launch("gemm_mid")) return status;
+    dim3 finish_grid((N + 15) / 16, (M + 15) / 16);
+#define BH_FINISH(SWIGLU, TC)                                                                              \
+  gemm_mid_finish_kernel<SWIGLU, TC><<<finish_grid, 256, 0, stream>>>((const float*)scratch, (TC*)c, M, N, K, \
+                                                                       parts, accumulate, norm)
+    if (activation) { if (f32) BH_FINISH(true, float); else BH_FINISH(true, bf16_t); }
+    else { if (f32) BH_FINISH(false, float); else BH_FINISH(false, bf16_t); }
+#undef BH_FINISH
+    return bh_check_launch("gemm_mid_finish");
+  }
   if (M <= 64) {
     const int pair_blocks = N / 16;
     if (activation) {

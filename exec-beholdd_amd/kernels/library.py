@@ -39,7 +39,7 @@ class PackedWeight:
 
 class NormedRows:
     """The output of an RMSNorm but for each row's factor: `rows` [n, width] bfloat16 holds x * weight and
-    `ss` [blocks, n] float32 partial sums of x^2 whose total over `blocks` gives the row's factor
+    `ss` [n, blocks] float32 partial sums of x^2 whose total over `blocks` gives the row's factor
     1 / sqrt(total / width + eps).  Products (`gemm`, `gemm_swiglu`) take it in place of an activation
     matrix and apply the factor to their result; one that cannot (other operand types) runs the norm
     itself from `source`, which must still hold the norm's input then.  `shape` and `dtype` are those of
@@ -94,7 +94,7 @@ class HipKernels:
             "bh_swiglu": [p, p, i, i, i, p],
             "bh_sample": [p, p, p, p, p, p, p, p, i, i, p],
             "bh_sample_scratch": [i, i],
-            "bh_gemm_bf16": [p, p, p, i, i, i, i, i, i, i, p, i, f, p, i, p, p, p],
+            "bh_gemm_bf16": [p, p, p, i, i, i, i, i, i, i, p, i, f, p, i, p, p, p, p],
             "bh_attention_bf16": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, i, i, f, i, i, i, p],
             "bh_attention_bf16_splits": [i, i, i, i, i],
             "bh_attention_decode_fused": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, f, i, i, i, p, p, i, f, p, p, i, i,
@@ -105,6 +105,8 @@ class HipKernels:
             function = getattr(lib, name)
             function.argtypes = argtypes
             function.restype = i
+        lib.bh_gemm_bf16_scratch.argtypes = [i, i, i, i, i]
+        lib.bh_gemm_bf16_scratch.restype = ctypes.c_long
     # ---- helpers ----
     def _stream(self):
         return ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
@@ -188,24 +190,29 @@ class HipKernels:
             return False, None
         m, k = a.shape
         n = out.shape[1]
-        if ahead is not None and (m > self.SKINNY_ROWS or ahead.ss.shape[1] != m or ahead.ss.dtype != torch.float32):
+        if ahead is not None and (m > self.SKINNY_ROWS or ahead.ss.shape[0] != m or ahead.ss.dtype != torch.float32):
             raise KernelError(f"gemm: prepared norm rows of {m} rows do not fit (at most {self.SKINNY_ROWS}, one sum per row)")
         behind = None
         if (then_norm is not None and m <= self.SKINNY_ROWS and out.dtype == torch.float32 and not activation
                 and then_norm.weight.shape == (n,) and then_norm.weight.dtype in _CODES):
             behind = NormedRows(torch.empty((m, n), dtype=torch.bfloat16, device=self.device),
-                                torch.empty((-(-n // 16), m), dtype=torch.float32, device=self.device), then_norm.eps,
+                                torch.empty((m, -(-n // 16)), dtype=torch.float32, device=self.device), then_norm.eps,
                                 out, then_norm.weight)
         a_rows = ahead.rows if ahead is not None else a
+        scratch = None       # products of 17 to 64 rows add up parts of K through scratch memory
+        scratch_bytes = int(self.lib.bh_gemm_bf16_scratch(m, n, k, int(packed), int(activation)))
+        if scratch_bytes:
+            scratch = torch.empty(scratch_bytes // 4, dtype=torch.float32, device=self.device)
         self._check(fast(
             self._ptr(a_rows, "gemm a"), self._ptr(w.data if packed else w, "gemm w"), self._ptr(out, "gemm out"),
             _code(out, "gemm out"), int(bool(accumulate)), m, n, k, int(packed), int(activation),
             self._ptr(ahead.ss, "norm sums") if ahead is not None else None,
-            ahead.ss.shape[0] if ahead is not None else 0, ahead.eps if ahead is not None else 0.0,
+            ahead.ss.shape[1] if ahead is not None else 0, ahead.eps if ahead is not None else 0.0,
             self._ptr(then_norm.weight, "norm weight") if behind is not None else None,
             _code(then_norm.weight, "norm weight") if behind is not None else 0,
             self._ptr(behind.rows, "norm rows") if behind is not None else None,
-            self._ptr(behind.ss, "norm sums") if behind is not None else None, self._stream()))
+            self._ptr(behind.ss, "norm sums") if behind is not None else None,
+            self._ptr(scratch, "gemm scratch", None, True), self._stream()))
         return True, behind
 
     def gemm(self, a, w, out, accumulate=False, then_norm=None):

@@ -144,8 +144,8 @@ def test_norm_rides_on_the_products_around_it(K, g_dtype, packed, m, n, k, n2):
     assert rel(residual, want_residual) < 4 * math.sqrt(k) * 2.0 ** -24
     got_residual = residual.cpu().double()
     assert rel(prepared.rows, got_residual * g.double()) < 4e-3                       # bfloat16 rounding
-    assert rel(prepared.ss.sum(0), (got_residual ** 2).sum(-1)) < 1e-5
-    assert prepared.ss.shape == (-(-n // 16), m)
+    assert rel(prepared.ss.sum(1), (got_residual ** 2).sum(-1)) < 1e-5
+    assert prepared.ss.shape == (m, -(-n // 16))
     normed = got_residual / torch.sqrt((got_residual ** 2).mean(-1, keepdim=True) + eps) * g.double()
 
     w2 = (torch.randn(n2, n, generator=gen) * 0.1).to(torch.bfloat16)
