@@ -80,6 +80,24 @@ def test_every_cut_matches_the_plain_implementation(expected, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_batches_of_many_sequences(model_dirs, dtype):
+    """Twenty-odd and forty sequences decode together: steps of 17 to 64 rows take other matrix-product
+    kernels than steps of a few rows do, also inside the replayed graphs.  Configuration D has the sizes
+    that let every fast path run (widths in multiples of 64, head size 128)."""
+    folder = model_dirs("D", "bfloat16")
+    cfg, weights = plain.load_plain(folder)
+    lengths = [5 + (7 * i) % 23 for i in range(40)]
+    requests = schedules.random_requests(cfg.vocab, lengths, seed=3)
+    want = [plain.forward_logits(cfg, weights, r) for r in requests]
+    engine = engine_for(folder, dtype, max_tokens=8192)
+    for batch_size in (23, 40):
+        got = schedules.batches(engine, requests, batch_size=batch_size, prompt_fraction=0.4)
+        check(f"batches of {batch_size}", got, want, TOLERANCE[dtype])
+    engine.cache.check_invariants()
+    assert engine.cache.live_slots() == []
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_one_layer_of_the_qwen3_8b_sizes(tmp_path_factory, dtype):
     """The layer sizes of the benchmark model (hidden 4096, 32 query and 8 kv heads of 128, feed-forward
     12288) in one layer with a small vocabulary: the kernels at the shapes they are tuned for, whole,
