@@ -10,15 +10,19 @@
 // from HBM (decode) runs about a third faster from this layout than from strided rows.
 // Tiles need K % 64 == 0; rows beyond N in the last block are zero.
 //
-// Two kernels.
-//   skinny (M <= 64, the decode shapes): bound by reading W once.  A workgroup owns 16 rows of W
-//     (a gate block and its up block for SwiGLU); its 8 waves split K in 64-wide chunks and feed
-//     v_mfma_f32_16x16x32_bf16 with W as the row operand and the activations as the column
+// Three ways, by the number of rows M.
+//   skinny (M <= 16; up to 64 for row-major weights): bound by reading W once.  A workgroup owns 16
+//     rows of W (a gate block and its up block for SwiGLU); its 8 waves split K in 64-wide chunks and
+//     feed v_mfma_f32_16x16x32_bf16 with W as the row operand and the activations as the column
 //     operand; the waves' partial tiles are summed through LDS in a fixed order.
-//   tiled (M > 64, the prefill shapes): 128x128 output tile per workgroup of four waves, 64-wide
-//     k slices staged through padded LDS (one or two buffers) with the next slice's global loads in
-//     flight during the multiplies; v_mfma_f32_32x32x16_bf16, each wave a 64x64 quarter.  For SwiGLU a wave's
-//     two 32-column halves are the gate and the up columns of the same 32 outputs.
+//   mid (17 <= M <= 64, tiles layout): still bound by W, but the activations would be read once per 16
+//     rows of W.  Eight waves take 16 rows of W each and share the activations through LDS; K is cut
+//     into parts over workgroups and a finishing kernel adds the parts (needs scratch memory).
+//   tiled (M > 64, the prefill shapes): output tiles of 128 x 128 (four waves) or 256 x 256 (eight),
+//     64-wide k slices staged through padded LDS (one or two buffers) with the next slice's global
+//     loads in flight during the multiplies; v_mfma_f32_32x32x16_bf16.  For SwiGLU a wave's columns
+//     are the gate and the up columns of the same outputs.  `gemm_tiled_whole_kernel` is the variant
+//     for whole tiles of the tiles layout, `gemm_tiled_kernel` takes every shape and both layouts.
 // K must be a multiple of 8 (16-byte loads); other sizes are free.
 //
 // Operand layouts relied on (wave of 64 lanes, l = lane):
