@@ -22,7 +22,8 @@
 //     64-wide k slices staged through padded LDS (one or two buffers) with the next slice's global
 //     loads in flight during the multiplies; v_mfma_f32_32x32x16_bf16.  For SwiGLU a wave's columns
 //     are the gate and the up columns of the same outputs.  `gemm_tiled_whole_kernel` is the variant
-//     for whole tiles of the tiles layout, `gemm_tiled_kernel` takes every shape and both layouts.
+//     for whole tiles of the tiles layout (it can carry a norm, see struct RidingNorm), `gemm_tiled_kernel`
+//     takes every shape and both layouts.
 // K must be a multiple of 8 (16-byte loads); other sizes are free.
 //
 // Operand layouts relied on (wave of 64 lanes, l = lane):
@@ -64,22 +65,23 @@ __device__ inline float silu_mul(float gate, float up) { return gate / (1.0f + e
 // ---- skinny --------------------------------------------------------------------------------
 // RT = 1: plain product.  RT = 2: SwiGLU; the second row block lies `pair_blocks` blocks after the first.
 
-// An RMSNorm between two products can ride on them (struct SkinnyNorm):
+// An RMSNorm between two products can ride on them (struct RidingNorm):
 //   behind: the product that completes the float32 residual h also writes bfloat16(h[m][n] * g[n]) (the
-//           norm's output but for the row factor) and, per workgroup, the sum of h[m][n]^2 over its 16
-//           columns;
+//           norm's output but for the row factor) and, per workgroup, the sum of h[m][n]^2 over its
+//           columns (16 of them in the skinny and mid ways, a tile's width in whole tiles);
 //   ahead:  the product that consumes the norm's output takes those unscaled rows as its activations and
 //           multiplies its result by 1 / sqrt(sum of the partial sums / K + eps) of the row.
 // The row factor commutes with the product, so the result is the norm's up to the rounding of the
-// activations; the partial sums are added in a fixed order.
-struct SkinnyNorm {
+// activations; the partial sums are added in a fixed order.  The skinny and the mid way and whole tiles
+// do this; the tiled kernel for every shape does not.
+struct RidingNorm {
   const float* ahead_ss;   // [M][ahead_blocks] partial sums of squares for the rows of `a`, or null
   int ahead_blocks;
   float ahead_eps;
   const void* behind_weight;  // [N] norm weight for the rows this product completes, or null
   int behind_weight_f32;      // its element type: float32, else bfloat16
   uint16_t* behind_rows;      // [M][N] bfloat16 out
-  float* behind_ss;           // [M][ceil(N / 16)] out
+  float* behind_ss;           // [M][bh_gemm_bf16_norm_blocks()] out
 };
 
 template <int MB, int WAVES, bool TILES, int RT, typename TC>
@@ -87,7 +89,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
                                                                  const uint16_t* __restrict__ w,
                                                                  TC* __restrict__ c, int M, int N, int K,
                                                                  int accumulate, int pair_blocks,
-                                                                 SkinnyNorm norm) {
+                                                                 RidingNorm norm) {
   __shared__ float partial[WAVES][RT][MB][256];
   __shared__ float row_factor[MB * 16];
   // The norm ahead: 32 threads per row, each with every 32nd partial sum.  The first 256 of a row are asked
@@ -378,7 +380,7 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const uint16_t* __restric
 template <bool SWIGLU, typename TC>
 __global__ __launch_bounds__(256) void gemm_mid_finish_kernel(const float* __restrict__ sums, TC* __restrict__ c,
                                                               int M, int N, int K, int parts, int accumulate,
-                                                              SkinnyNorm norm) {
+                                                              RidingNorm norm) {
   const int w_rows = SWIGLU ? 2 * N : N;
   const int col = threadIdx.x % 16, n = blockIdx.x * 16 + col, m = blockIdx.y * 16 + threadIdx.x / 16;
   const bool valid = m < M && n < N;
@@ -621,9 +623,10 @@ template <bool SWIGLU, int WX, int WY, int WM, int WN, int BUFFERS, typename TC>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_whole_kernel(const uint16_t* __restrict__ a,
                                                                          const uint16_t* __restrict__ w,
                                                                          TC* __restrict__ c, int M, int N, int K,
-                                                                         int accumulate) {
+                                                                         int accumulate, RidingNorm norm) {
   constexpr int THREADS = 64 * WM * WN;
   constexpr int TBM = 32 * WX * WM, TBN = 32 * WY * WN;
+  static_assert(TBM <= THREADS, "one thread per row of the tile adds up the norm's partial sums");
   constexpr int A_PIECES = TBM * 8 / THREADS, W_PIECES = TBN * 8 / THREADS;
   constexpr int A_ROWS = THREADS / 8;      // rows of A that one round of the workgroup's loads covers
   constexpr int W_BLOCKS = THREADS / 128;  // 16-row blocks of W per round
@@ -632,6 +635,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_whole_kernel(const ui
   static_assert(!SWIGLU || W_BLOCKS == WY, "a round of W loads is the gate half or the up half of one wave column");
   __shared__ __attribute__((aligned(16))) uint16_t as[BUFFERS][TBM * TPITCH];
   __shared__ __attribute__((aligned(16))) uint16_t ws[BUFFERS][TBN * TPITCH];
+  __shared__ __attribute__((aligned(16))) float row_factor[TBM];   // norm ahead: what each row's result is multiplied by
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int m_own = blockIdx.y * TBM, n_own = blockIdx.x * OUTS;   // what this tile stands for
   const int m0 = min(m_own, M - TBM), n0 = min(n_own, N - OUTS);   // where it computes
@@ -682,6 +686,24 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_whole_kernel(const ui
 
   const int slices = K / TK;
   fetch(0);
+  if (norm.ahead_ss && tid < TBM) {   // while the first slice is on its way
+    const float* partial = norm.ahead_ss + (size_t)(m0 + tid) * norm.ahead_blocks;
+    float total = 0.f;
+    if (norm.ahead_blocks % 4 == 0) {   // 32 sums per round of loads, added in their order
+      const f32x4_t* four = reinterpret_cast<const f32x4_t*>(partial);
+      const int fours = norm.ahead_blocks / 4;
+      for (int b = 0; b < fours; b += 8) {
+        f32x4_t v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = b + i < fours ? four[b + i] : f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) total += v[i][0], total += v[i][1], total += v[i][2], total += v[i][3];
+      }
+    } else {
+      for (int b = 0; b < norm.ahead_blocks; ++b) total += partial[b];
+    }
+    row_factor[tid] = rsqrtf(total / (float)K + norm.ahead_eps);
+  }
   stash(0);
   __syncthreads();
   const int frag = (lane % 32) * TPITCH + (lane / 32) * 8;
@@ -715,6 +737,70 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_whole_kernel(const ui
   }
   multiply(BUFFERS == 2 ? ((slices - 1) & 1) : 0);
   // D of one 32x32 block: column (n) lane%32, rows (m) 8*(e/4) + 4*(lane/32) + e%4
+  if (norm.ahead_ss) {
+#pragma unroll
+    for (int x = 0; x < WX; ++x)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const f32x4_t f = *reinterpret_cast<const f32x4_t*>(&row_factor[wm + x * 32 + 8 * q + 4 * (lane / 32)]);
+#pragma unroll
+        for (int y = 0; y < WY; ++y)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[x][y][4 * q + i] *= f[i];
+      }
+  }
+  if constexpr (!SWIGLU && sizeof(TC) == 4) {
+    if (norm.behind_weight) {
+      // The residual's new values, the norm's unscaled output, and the sum of squares of each row over the
+      // columns this tile owns: within a wave by lane exchanges, across the WN waves of a row through LDS,
+      // always in the same order.
+      __syncthreads();   // the operand buffers are free now
+      float* partial = reinterpret_cast<float*>(&as[0][0]);   // [WN][TBM]
+      static_assert(WN * TBM * 4 <= (int)sizeof(as), "the partial sums fit in the A buffers");
+      float g[WY];
+#pragma unroll
+      for (int y = 0; y < WY; ++y) {
+        const int n = n0 + wn + y * 32 + lane % 32;
+        g[y] = norm.behind_weight_f32 ? reinterpret_cast<const float*>(norm.behind_weight)[n]
+                                      : bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(norm.behind_weight)[n]);
+      }
+#pragma unroll
+      for (int x = 0; x < WX; ++x) {
+        float sq[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) sq[e] = 0.f;
+#pragma unroll
+        for (int y = 0; y < WY; ++y) {
+          const int n = n0 + wn + y * 32 + lane % 32;
+          if (n < n_own) continue;
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int m = m0 + wm + x * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
+            if (m < m_own) continue;
+            const size_t at = (size_t)m * N + n;
+            const float value = accumulate ? c[at] + acc[x][y][e] : acc[x][y][e];
+            c[at] = value;
+            norm.behind_rows[at] = f32_to_bf16_bits(value * g[y]);
+            sq[e] += value * value;
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+#pragma unroll
+          for (int step = 16; step >= 1; step >>= 1) sq[e] += __shfl_xor(sq[e], step);
+          if (lane % 32 == 0) partial[(wave % WN) * TBM + wm + x * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4] = sq[e];
+        }
+      }
+      __syncthreads();
+      if (tid < TBM && m0 + tid >= m_own) {
+        float total = 0.f;
+#pragma unroll
+        for (int part = 0; part < WN; ++part) total += partial[part * TBM + tid];
+        norm.behind_ss[(size_t)(m0 + tid) * gridDim.x + blockIdx.x] = total;
+      }
+      return;
+    }
+  }
 #pragma unroll
   for (int x = 0; x < WX; ++x) {
     if (SWIGLU) {
@@ -747,7 +833,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_whole_kernel(const ui
 
 template <bool TILES, int RT, typename TC>
 static void launch_skinny(const void* a, const void* w, void* c, int M, int N, int K, int accumulate,
-                          int pair_blocks, const SkinnyNorm& norm, hipStream_t stream) {
+                          int pair_blocks, const RidingNorm& norm, hipStream_t stream) {
   constexpr int WAVES = 8;
   dim3 grid((N + 15) / 16), block(WAVES * 64);
 #define BH_SKINNY(MB)                                                                                     \
@@ -762,32 +848,66 @@ static void launch_skinny(const void* a, const void* w, void* c, int M, int N, i
 #undef BH_SKINNY
 }
 
+// Measured at the Qwen3-8B shapes (2,048 rows).  The multiplies of a 128 x 128 tile need as many LDS
+// cycles (operand reads and the staging writes) as MFMA cycles, so LDS bounds them; a 256 x 256 tile
+// of eight waves, each 64 x 128, reads a quarter less per multiply and wins once it still gives every
+// compute unit three tiles.  Below that the smaller tile keeps more compute units busy.  Two LDS buffers
+// (one barrier per slice, two workgroups per compute unit) are the better choice unless a single one
+// (four workgroups per compute unit) lets the whole grid run at once: between two and four tiles for
+// each of the 256 compute units.
+enum TiledConfig { TILED_256 = 0, TILED_128_ONE_BUFFER = 1, TILED_128 = 2 };
+static TiledConfig tiled_config(int M, int N, bool swiglu, int* rows, int* columns) {
+  const long tiles_128 = (long)((N + (swiglu ? 63 : 127)) / (swiglu ? 64 : 128)) * ((M + 127) / 128);
+  const bool big = tiles_128 >= 3072;
+  *rows = big ? 256 : 128;
+  *columns = (big ? 256 : 128) / (swiglu ? 2 : 1);
+  return big ? TILED_256 : tiles_128 > 512 && tiles_128 <= 1024 ? TILED_128_ONE_BUFFER : TILED_128;
+}
+// Whether the product runs as whole tiles (gemm_tiled_whole_kernel), the only tiled way a norm rides on.
+static bool tiled_whole(int M, int N, int K, int layout, int rows, int columns) {
+  return layout == 1 && K % TK == 0 && N % 16 == 0 && M >= rows && N >= columns && (long)rows * K < (1L << 31);
+}
+
 template <bool TILES, bool SWIGLU, typename TC>
 static void launch_tiled(const void* a, const void* w, void* c, int M, int N, int K, int accumulate,
-                         hipStream_t stream) {
+                         const RidingNorm& norm, hipStream_t stream) {
+  int rows, columns;
+  const TiledConfig config = tiled_config(M, N, SWIGLU, &rows, &columns);
+  const bool whole = tiled_whole(M, N, K, TILES ? 1 : 0, rows, columns);
+  dim3 grid((N + columns - 1) / columns, (M + rows - 1) / rows);
 #define BH_TILED(WX, WY, WM, WN, BUFFERS)                                                                 \
   do {                                                                                                     \
-    const int columns = (SWIGLU ? 16 : 32) * WY * WN, rows = 32 * WX * WM;                                 \
-    dim3 grid((N + columns - 1) / columns, (M + rows - 1) / rows), block(64 * WM * WN);                    \
-    if (TILES && K % TK == 0 && N % 16 == 0 && M >= rows && N >= columns && (long)rows * K < (1L << 31))   \
+    dim3 block(64 * WM * WN);                                                                              \
+    if (TILES && whole)                                                                                    \
       gemm_tiled_whole_kernel<SWIGLU, WX, WY, WM, WN, BUFFERS, TC><<<grid, block, 0, stream>>>(            \
-          (const uint16_t*)a, (const uint16_t*)w, (TC*)c, M, N, K, accumulate);                            \
+          (const uint16_t*)a, (const uint16_t*)w, (TC*)c, M, N, K, accumulate, norm);                      \
     else                                                                                                   \
       gemm_tiled_kernel<TILES, SWIGLU, WX, WY, WM, WN, BUFFERS, TC><<<grid, block, 0, stream>>>(           \
           (const uint16_t*)a, (const uint16_t*)w, (TC*)c, M, N, K, accumulate);                            \
   } while (0)
-  // Measured at the Qwen3-8B shapes (2,048 rows).  The multiplies of a 128 x 128 tile need as many LDS
-  // cycles (operand reads and the staging writes) as MFMA cycles, so LDS bounds them; a 256 x 256 tile
-  // of eight waves, each 64 x 128, reads a quarter less per multiply and wins once it still gives every
-  // compute unit three tiles.  Below that the smaller tile keeps more compute units busy.  Two LDS buffers
-  // (one barrier per slice, two workgroups per compute unit) are the better choice unless a single one
-  // (four workgroups per compute unit) lets the whole grid run at once: between two and four tiles for
-  // each of the 256 compute units.
-  const long tiles_128 = (long)((N + (SWIGLU ? 63 : 127)) / (SWIGLU ? 64 : 128)) * ((M + 127) / 128);
-  if (tiles_128 >= 3072) BH_TILED(2, 4, 4, 2, 2);
-  else if (tiles_128 > 512 && tiles_128 <= 1024) BH_TILED(2, 2, 2, 2, 1);
-  else BH_TILED(2, 2, 2, 2, 2);
+  switch (config) {
+    case TILED_256: BH_TILED(2, 4, 4, 2, 2); break;
+    case TILED_128_ONE_BUFFER: BH_TILED(2, 2, 2, 2, 1); break;
+    default: BH_TILED(2, 2, 2, 2, 2); break;
+  }
 #undef BH_TILED
+}
+
+// How many partial sums per row a product of these sizes writes when a norm rides behind it (0: it cannot
+// carry one), and whether it can take prepared norm rows as its activations.
+extern "C" int bh_gemm_bf16_norm_blocks(int M, int N, int K, int layout, int activation) {
+  if (activation || M <= 0 || N <= 0 || K % 8 != 0) return 0;
+  if (M <= 64) return (N + 15) / 16;
+  int rows, columns;
+  tiled_config(M, N, false, &rows, &columns);
+  return tiled_whole(M, N, K, layout, rows, columns) ? (N + columns - 1) / columns : 0;
+}
+extern "C" int bh_gemm_bf16_takes_norm(int M, int N, int K, int layout, int activation) {
+  if (M <= 0 || N <= 0 || K % 8 != 0 || (activation && N % 16 != 0)) return 0;
+  if (M <= 64) return 1;
+  int rows, columns;
+  tiled_config(M, N, activation != 0, &rows, &columns);
+  return tiled_whole(M, N, K, layout, rows, columns) ? 1 : 0;
 }
 
 // layout: 0 = rows, 1 = tiles.  activation: 0 = none; 1 = SwiGLU (W has 2 * N rows: gate rows then up rows).
@@ -800,7 +920,7 @@ extern "C" long bh_gemm_bf16_scratch(int M, int N, int K, int layout, int activa
 }
 
 // The `ahead_*` and `behind_*` arguments (null when unused) let an RMSNorm ride on the products before and
-// after it (struct SkinnyNorm); they exist for M <= 64 only.  `scratch`: bh_gemm_bf16_scratch() bytes, or
+// after it (struct RidingNorm) where bh_gemm_bf16_takes_norm / bh_gemm_bf16_norm_blocks say so.  `scratch`: bh_gemm_bf16_scratch() bytes, or
 // null (then products of 17 to 64 rows take the slower way without it).
 extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, int accumulate, int M, int N, int K,
                             int layout, int activation, const float* ahead_ss, int ahead_blocks, float ahead_eps,
@@ -815,14 +935,16 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
   BH_REQUIRE(activation == 0 || (N % 16 == 0 && !accumulate),
              "gemm_bf16: SwiGLU needs a multiple of 16 outputs (got %d) and no accumulation", N);
   BH_REQUIRE((M + 127) / 128 <= 65535, "gemm_bf16: M=%d needs more than 65535 row tiles", M);
-  BH_REQUIRE((!ahead_ss && !behind_weight) || M <= 64,
-             "gemm_bf16: a norm rides on products of at most 64 rows only, not M=%d", M);
+  BH_REQUIRE(!ahead_ss || bh_gemm_bf16_takes_norm(M, N, K, layout, activation),
+             "gemm_bf16: a product of M=%d N=%d K=%d cannot take prepared norm rows (bh_gemm_bf16_takes_norm)", M, N, K);
+  BH_REQUIRE(!behind_weight || bh_gemm_bf16_norm_blocks(M, N, K, layout, activation) > 0,
+             "gemm_bf16: a product of M=%d N=%d K=%d cannot carry a norm (bh_gemm_bf16_norm_blocks)", M, N, K);
   BH_REQUIRE(!ahead_ss || (ahead_blocks > 0 && ahead_eps > 0.f), "gemm_bf16: the norm ahead needs partial sums and an epsilon");
   BH_REQUIRE(!behind_weight || (behind_rows && behind_ss && c_dtype == BH_F32 && activation == 0),
              "gemm_bf16: the norm behind needs its outputs, a float32 product and no activation");
   BH_REQUIRE(!behind_weight || behind_weight_dtype == BH_F32 || behind_weight_dtype == BH_BF16,
              "gemm_bf16: unknown norm weight dtype %d", behind_weight_dtype);
-  const SkinnyNorm norm = {ahead_ss, ahead_blocks, ahead_eps, behind_weight, behind_weight_dtype == BH_F32,
+  const RidingNorm norm = {ahead_ss, ahead_blocks, ahead_eps, behind_weight, behind_weight_dtype == BH_F32,
                            (uint16_t*)behind_rows, behind_ss};
   const bool f32 = c_dtype == BH_F32;
 #define BH_PICK(FN, TILES, EXTRA, ...)                                             \
@@ -862,11 +984,11 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
     return bh_check_launch("gemm_skinny");
   }
   if (activation) {
-    if (layout) BH_PICK(launch_tiled, true, true, a, w, c, M, N, K, 0, stream);
-    else BH_PICK(launch_tiled, false, true, a, w, c, M, N, K, 0, stream);
+    if (layout) BH_PICK(launch_tiled, true, true, a, w, c, M, N, K, 0, norm, stream);
+    else BH_PICK(launch_tiled, false, true, a, w, c, M, N, K, 0, norm, stream);
   } else {
-    if (layout) BH_PICK(launch_tiled, true, false, a, w, c, M, N, K, accumulate, stream);
-    else BH_PICK(launch_tiled, false, false, a, w, c, M, N, K, accumulate, stream);
+    if (layout) BH_PICK(launch_tiled, true, false, a, w, c, M, N, K, accumulate, norm, stream);
+    else BH_PICK(launch_tiled, false, false, a, w, c, M, N, K, accumulate, norm, stream);
   }
 #undef BH_PICK
   return bh_check_launch("gemm_tiled");

@@ -14,17 +14,26 @@ declares `graph_safe = True`.
 
 from __future__ import annotations
 
+import gc
+import weakref
+
 import numpy as np
 import torch
 
 from ..parts.base import LayerCache, StepContext
+
+def _weakly(engine):
+    return engine if isinstance(engine, weakref.ProxyTypes) else weakref.proxy(engine)
+
 
 PAGE_BUCKET = 16      # page-table widths are rounded up to a multiple of this many pages
 
 
 class DecodeGraph:
     def __init__(self, engine, n_seqs: int, table_width: int):
-        self.engine, self.n_seqs, self.table_width = engine, n_seqs, table_width
+        # the engine owns its graphs; they point back weakly, so that an engine nobody holds any more is
+        # freed at once and not by a later garbage collection
+        self.engine, self.n_seqs, self.table_width = _weakly(engine), n_seqs, table_width
         cache = engine.cache
         self.kv_groups = [index for index, g in enumerate(cache.groups) if g.need.kind == "kv"]
         b = n_seqs
@@ -110,8 +119,16 @@ class DecodeGraph:
             self._forward()                      # once eagerly: loads every kernel before the capture
             torch.cuda.synchronize(self.engine.device)
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                self.logits = self._forward()
+            # No garbage collection while the stream is capturing: it could free another engine's graphs or
+            # memory there, and the runtime refuses such calls during a capture (the process aborts).
+            collecting = gc.isenabled()
+            gc.disable()
+            try:
+                with torch.cuda.graph(graph):
+                    self.logits = self._forward()
+            finally:
+                if collecting:
+                    gc.enable()
             self.graph = graph
         self.graph.replay()
         return self.logits
@@ -121,7 +138,7 @@ class DecodeGraphs:
     """The graphs of one engine, by (sequences, page-table width)."""
 
     def __init__(self, engine, limit: int = 48):
-        self.engine, self.limit = engine, limit
+        self.engine, self.limit = _weakly(engine), limit
         self.graphs: dict = {}
 
     def usable(self, ctx_entries) -> bool:

@@ -107,6 +107,8 @@ class HipKernels:
             function.restype = i
         lib.bh_gemm_bf16_scratch.argtypes = [i, i, i, i, i]
         lib.bh_gemm_bf16_scratch.restype = ctypes.c_long
+        for query in (lib.bh_gemm_bf16_norm_blocks, lib.bh_gemm_bf16_takes_norm):
+            query.argtypes, query.restype = [i, i, i, i, i], ctypes.c_int
     # ---- helpers ----
     def _stream(self):
         return ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
@@ -174,8 +176,6 @@ class HipKernels:
             return PackedWeight(data, rows, cols)
         return w
 
-    SKINNY_ROWS = 64      # products of at most this many rows can carry a norm (csrc/gemm_bf16.hip)
-
     def _gemm_fast(self, a, w, out, accumulate, activation, then_norm=None):
         """Launch the matrix-core product if it takes these operands; say whether it did, and with
         what prepared norm output (None if `then_norm` was not asked for or cannot ride on this product)."""
@@ -190,17 +190,21 @@ class HipKernels:
             return False, None
         m, k = a.shape
         n = out.shape[1]
-        if ahead is not None and (m > self.SKINNY_ROWS or ahead.ss.shape[0] != m or ahead.ss.dtype != torch.float32):
-            raise KernelError(f"gemm: prepared norm rows of {m} rows do not fit (at most {self.SKINNY_ROWS}, one sum per row)")
+        sizes = (m, n, k, int(packed), int(activation))
+        if ahead is not None and (ahead.ss.shape[0] != m or ahead.ss.dtype != torch.float32
+                                  or not self.lib.bh_gemm_bf16_takes_norm(*sizes)):
+            raise KernelError(f"gemm: a product of {m} x {n} x {k} does not take these prepared norm rows")
         behind = None
-        if (then_norm is not None and m <= self.SKINNY_ROWS and out.dtype == torch.float32 and not activation
+        if (then_norm is not None and out.dtype == torch.float32 and not activation
                 and then_norm.weight.shape == (n,) and then_norm.weight.dtype in _CODES):
-            behind = NormedRows(torch.empty((m, n), dtype=torch.bfloat16, device=self.device),
-                                torch.empty((m, -(-n // 16)), dtype=torch.float32, device=self.device), then_norm.eps,
-                                out, then_norm.weight)
+            blocks = int(self.lib.bh_gemm_bf16_norm_blocks(*sizes))      # 0: this product carries no norm
+            if blocks:
+                behind = NormedRows(torch.empty((m, n), dtype=torch.bfloat16, device=self.device),
+                                    torch.empty((m, blocks), dtype=torch.float32, device=self.device), then_norm.eps,
+                                    out, then_norm.weight)
         a_rows = ahead.rows if ahead is not None else a
         scratch = None       # products of 17 to 64 rows add up parts of K through scratch memory
-        scratch_bytes = int(self.lib.bh_gemm_bf16_scratch(m, n, k, int(packed), int(activation)))
+        scratch_bytes = int(self.lib.bh_gemm_bf16_scratch(*sizes))
         if scratch_bytes:
             scratch = torch.empty(scratch_bytes // 4, dtype=torch.float32, device=self.device)
         self._check(fast(
@@ -227,7 +231,7 @@ class HipKernels:
         n = w.shape[0]
         if w.shape[1] != k or out.shape != (m, n):
             raise KernelError(f"gemm: shapes a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
-        if isinstance(a, NormedRows) and (w.dtype != torch.bfloat16 or k % 8):
+        if isinstance(a, NormedRows) and not self._takes_norm(a, w, n, 0):
             a = self._run_norm(a)
         done, prepared = self._gemm_fast(a, w, out, accumulate, 0, then_norm)
         if done:
@@ -236,6 +240,12 @@ class HipKernels:
             self._ptr(a, "gemm a"), _code(a, "gemm a"), self._ptr(w, "gemm w"), _code(w, "gemm w"),
             self._ptr(out, "gemm out"), _code(out, "gemm out"), int(bool(accumulate)), m, n, k, self._stream()))
         return None
+
+    def _takes_norm(self, a, w, n, activation):
+        """Whether the matrix-core product of these operands applies the row factors of prepared norm rows."""
+        m, k = a.shape
+        return bool(w.dtype == torch.bfloat16 and k % 8 == 0 and (not activation or n % 16 == 0)
+                    and self.lib.bh_gemm_bf16_takes_norm(m, n, k, int(isinstance(w, PackedWeight)), int(activation)))
 
     def _run_norm(self, prepared):
         """The norm that `prepared` stands for, as a step of its own."""
@@ -253,6 +263,8 @@ class HipKernels:
         if w.shape != (2 * width, k) or out.shape[0] != m or out.dtype != a.dtype:
             raise KernelError(f"gemm_swiglu: shapes a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} "
                               "do not fit")
+        if isinstance(a, NormedRows) and width % 16 == 0 and not self._takes_norm(a, w, width, 1):
+            a = self._run_norm(a)
         if self._gemm_fast(a, w, out, False, 1)[0]:
             return
         both = torch.empty((m, 2 * width), dtype=a.dtype, device=self.device)

@@ -160,6 +160,33 @@ def test_first_tokens_of_a_sequence(model_dirs, name, dtype):
         check(f"one by one {length}", schedules.tail_one_by_one(engine, [tokens], tail=length), [want], TOLERANCE[dtype])
 
 
+def test_capture_is_safe_from_the_garbage_collector(model_dirs):
+    """No garbage collection runs while a stream is capturing (freeing another engine's graphs there is
+    refused by the runtime), and an engine that nobody holds is freed at once, with no collection."""
+    import gc
+    import weakref
+    from beholdd.engine import Engine, StepEntry
+    engine = Engine(model_dirs("A", "bfloat16"), dtype="bfloat16", max_tokens=256)
+    seen, forward = [], engine.model.forward
+
+    def watched(*args, **kwargs):
+        seen.append((torch.cuda.is_current_stream_capturing(), gc.isenabled()))
+        return forward(*args, **kwargs)
+
+    engine.model.forward = watched
+    slot = engine.alloc_slot()
+    engine.step([StepEntry(slot, [1, 2, 3], [2])])
+    engine.step([StepEntry(slot, [4], [0])])
+    engine.step([StepEntry(slot, [5], [0])])
+    assert gc.isenabled()
+    assert (True, False) in seen and not any(capturing and collecting for capturing, collecting in seen), seen
+    engine.model.forward = forward
+    del watched, forward
+    alive = weakref.ref(engine)
+    del engine
+    assert alive() is None
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_graph_replays_equal_eager_steps(model_dirs, dtype):
     """Decode steps replayed from captured HIP graphs against the same steps launched one kernel at

@@ -166,6 +166,45 @@ def test_norm_rides_on_the_products_around_it(K, g_dtype, packed, m, n, k, n2):
         assert rel(act, gate / (1 + torch.exp(-gate)) * up) < 1.2e-2
 
 
+@pytest.mark.parametrize("m,n,k,n2,g_dtype", [(200, 320, 192, 130, torch.float32), (200, 320, 192, 144, torch.bfloat16),
+                                              (300, 4096, 128, 256, torch.float32), (128, 128, 64, 128, torch.bfloat16),
+                                              (3072, 16384, 64, 256, torch.float32)])
+def test_norm_rides_on_wide_products(K, m, n, k, n2, g_dtype):
+    """The same for the products of many rows: whole tiles of a packed weight carry the norm (partial sums
+    per tile column, edge tiles counting only what they own); other wide products leave it alone."""
+    from beholdd.kernels import NormedRows
+    from beholdd.parts.base import NormRequest
+    gen = torch.Generator().manual_seed(m + n)
+    a = torch.randn(m, k, generator=gen).to(torch.bfloat16)
+    w = (torch.randn(n, k, generator=gen) * 0.1).to(torch.bfloat16)
+    base = torch.randn(m, n, generator=gen) * 3
+    g = (1 + 0.3 * torch.randn(n, generator=gen)).to(g_dtype)
+    eps = 1e-5
+    on = lambda t: t.double().to("cuda:0")      # the references of these sizes are computed on the device, by torch
+    residual = dev(base.clone())
+    assert K.gemm(dev(a), dev(w), residual.clone(), accumulate=True, then_norm=NormRequest(dev(g), eps)) is None
+    prepared = K.gemm(dev(a), K.pack_weight(dev(w)), residual, accumulate=True, then_norm=NormRequest(dev(g), eps))
+    assert isinstance(prepared, NormedRows) and prepared.shape == (m, n) and prepared.ss.shape[0] == m
+    want_residual = on(base) + on(a) @ on(w).t()
+    assert rel(residual, want_residual.cpu()) < 4 * math.sqrt(k) * 2.0 ** -24
+    got_residual = residual.double()
+    assert rel(prepared.rows, (got_residual * on(g)).cpu()) < 4e-3
+    assert rel(prepared.ss.sum(1), (got_residual ** 2).sum(-1).cpu()) < 1e-5
+    normed = got_residual / torch.sqrt((got_residual ** 2).mean(-1, keepdim=True) + eps) * on(g)
+    w2 = (torch.randn(n2, n, generator=gen) * 0.1).to(torch.bfloat16)
+    want = (normed @ on(w2).t()).cpu()
+    for w2_dev in (K.pack_weight(dev(w2)), dev(w2)):        # the second runs the norm itself, from the residual
+        for out_dtype in (torch.float32, torch.bfloat16):
+            out = torch.empty(m, n2, dtype=out_dtype, device="cuda:0")
+            assert K.gemm(prepared, w2_dev, out) is None
+            assert rel(out, want) < 8e-3, rel(out, want)
+    half = n2 // 2
+    act = torch.empty(m, half, dtype=torch.bfloat16, device="cuda:0")
+    K.gemm_swiglu(prepared, K.pack_weight(dev(w2)), act)
+    gate, up = want[:, :half], want[:, half:]
+    assert rel(act, gate / (1 + torch.exp(-gate)) * up) < 1.2e-2
+
+
 def test_norm_does_not_ride_on_wide_steps(K):
     from beholdd.parts.base import NormRequest
     a = torch.randn(65, 64).to(torch.bfloat16)
