@@ -98,7 +98,8 @@ class Engine:
     def step(self, entries: list):
         """Run the given tokens of each entry's sequence from the cache; return float32 logits
         [wanted, vocab] in the order of the entries and of their `want` lists (None if nothing is
-        wanted).  On an error no sequence's length changes."""
+        wanted).  On an error no sequence's length changes.  The logits of a decode step stand in memory
+        that the next decode step of the same shape writes again: copy what has to outlive it."""
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
         if self.graphs is not None and entries and self.graphs.usable(entries):
             return self._graph_step(entries)
