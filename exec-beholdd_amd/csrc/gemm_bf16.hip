@@ -10,20 +10,18 @@
 // from HBM (decode) runs about a third faster from this layout than from strided rows.
 // Tiles need K % 64 == 0; rows beyond N in the last block are zero.
 //
-// Three ways, by the number of rows M.
-//   skinny (M <= 16; up to 64 for row-major weights): bound by reading W once.  A workgroup owns 16
-//     rows of W (a gate block and its up block for SwiGLU); its 8 waves split K in 64-wide chunks and
-//     feed v_mfma_f32_16x16x32_bf16 with W as the row operand and the activations as the column
-//     operand; the waves' partial tiles are summed through LDS in a fixed order.
-//   mid (17 <= M <= 64, tiles layout): still bound by W, but the activations would be read once per 16
-//     rows of W.  Eight waves take 16 rows of W each and share the activations through LDS; K is cut
-//     into parts over workgroups and a finishing kernel adds the parts (needs scratch memory).
-//   tiled (M > 64, the prefill shapes): output tiles of 128 x 128 (four waves) or 256 x 256 (eight),
-//     64-wide k slices staged through padded LDS (one or two buffers) with the next slice's global
-//     loads in flight during the multiplies; v_mfma_f32_32x32x16_bf16.  For SwiGLU a wave's columns
-//     are the gate and the up columns of the same outputs.  `gemm_tiled_whole_kernel` is the variant
-//     for whole tiles of the tiles layout (it can carry a norm, see struct RidingNorm), `gemm_tiled_kernel`
-//     takes every shape and both layouts.
+// Two ways, by the number of rows M.
+//   skinny (M <= 16; up to 64 where the tiled way below does not take the shape): bound by reading W once.
+//     A workgroup owns 16 rows of W (a gate block and its up block for SwiGLU); its 8 waves split K in
+//     64-wide chunks and feed v_mfma_f32_16x16x32_bf16 with W as the row operand and the activations as the
+//     column operand; the waves' partial tiles are summed through LDS in a fixed order.
+//   tiled (M > 16): output tiles of 32 x 128, 64 x 128, 128 x 128 (four waves) or 256 x 256 (eight), 64-wide
+//     k slices staged through padded LDS (one or two buffers) with the next slice's global loads in flight
+//     during the multiplies; v_mfma_f32_32x32x16_bf16.  For SwiGLU a wave's columns are the gate and the up
+//     columns of the same outputs.  `gemm_tiled_whole_kernel` is the variant for whole tiles of the tiles
+//     layout: it can carry a norm (struct RidingNorm), and where the tiles are too few to fill the chip
+//     (17 to about 512 rows at these widths) it cuts K into parts over workgroups and a finishing kernel adds
+//     them (needs scratch memory).  `gemm_tiled_kernel` takes every shape and both layouts.
 // K must be a multiple of 8 (16-byte loads); other sizes are free.
 //
 // Operand layouts relied on (wave of 64 lanes, l = lane):
@@ -32,6 +30,7 @@
 //             rows 8*(i/4) + 4*(l/32) + i%4 for i = 0..15
 // Which 8 of the k values a lane group multiplies is free as long as both operands agree.
 #include "common.h"
+#include <algorithm>
 #include <type_traits>
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -68,12 +67,12 @@ __device__ inline float silu_mul(float gate, float up) { return gate / (1.0f + e
 // An RMSNorm between two products can ride on them (struct RidingNorm):
 //   behind: the product that completes the float32 residual h also writes bfloat16(h[m][n] * g[n]) (the
 //           norm's output but for the row factor) and, per workgroup, the sum of h[m][n]^2 over its
-//           columns (16 of them in the skinny and mid ways, a tile's width in whole tiles);
+//           columns (16 of them in the skinny kernel and the finishing kernel, a tile's width in whole tiles);
 //   ahead:  the product that consumes the norm's output takes those unscaled rows as its activations and
 //           multiplies its result by 1 / sqrt(sum of the partial sums / K + eps) of the row.
 // The row factor commutes with the product, so the result is the norm's up to the rounding of the
-// activations; the partial sums are added in a fixed order.  The skinny and the mid way and whole tiles
-// do this; the tiled kernel for every shape does not.
+// activations; the partial sums are added in a fixed order.  The skinny kernel and whole tiles (with or
+// without the finishing kernel) do this; the tiled kernel for every shape does not.
 struct RidingNorm {
   const float* ahead_ss;   // [M][ahead_blocks] partial sums of squares for the rows of `a`, or null
   int ahead_blocks;
@@ -257,136 +256,24 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
   }
 }
 
-// ---- 17 to 64 rows ---------------------------------------------------------------------------
-// With more than 16 rows the skinny kernel's activations weigh more than its weights: every workgroup
-// reads all of them for 16 weight rows.  Here the eight waves of a workgroup take a block of 16 weight
-// rows each (of the packed layout, whatever they are: a SwiGLU's gate and up rows are just rows) and walk
-// over the same part of K together, 256 columns at a time: the activations of those columns go through
-// LDS once per workgroup, in the order in which the lanes take them, and every wave streams its own
-// weights.  K is cut into parts so that there are enough workgroups; the sums go to scratch memory as
-// [K part][row][weight row].  A second kernel adds the parts in order and does what the skinny kernel
-// does with its sums: the row factor of a norm ahead, SwiGLU, accumulation into the residual, a norm behind.
-
-#define MID_STAGE 4   // 64-wide chunks of K per stage
-
-template <int MB>
-__global__ __launch_bounds__(512) void gemm_mid_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ w,
-                                                       float* __restrict__ sums, int M, int w_rows, int K,
-                                                       int chunks_per_part) {
-  constexpr int WAVES = 8;
-  // activations of a stage as the multiplies take them: piece [chunk][row block][half][lane] holds row
-  // 16 b + lane % 16, columns 64 chunk + 16 (lane / 16) + 8 half .. + 7
-  static_assert(MID_STAGE * 128 == 512, "a thread stages one piece per row block and stage: 512 threads, 128 pieces per chunk and row block");
-  __shared__ u32x4_t xs[2][MID_STAGE][MB][2][64];
-  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
-  const int full = K / 64, n_blocks = (w_rows + 15) / 16;
-  const int block = blockIdx.x * WAVES + wave;
-  const bool own = block < n_blocks;                 // a wave beyond the last block repeats it and stores nothing
-  const uint16_t* wp = w + (size_t)min(block, n_blocks - 1) * full * 1024 + lane * 8;
-  const int first = blockIdx.y * chunks_per_part, end = min(full, first + chunks_per_part);
-
-  // what this thread brings into LDS for a stage: MB pieces
-  const uint16_t* x_src[MB];
-  int x_chunk[MB];
-#pragma unroll
-  for (int j = 0; j < MB; ++j) {
-    const int q = tid + 512 * j, l = q % 64, half = (q / 64) % 2, b = (q / 128) % MB, ch = q / (128 * MB);
-    const int row = min(b * 16 + l % 16, M - 1);
-    x_src[j] = a + (size_t)row * K + (l / 16) * 16 + half * 8;
-    x_chunk[j] = ch;
-  }
-  u32x4_t stage[MB];
-  auto fetch = [&](int c0) {   // chunks beyond the part are brought in as the part's last: they are not multiplied
-#pragma unroll
-    for (int j = 0; j < MB; ++j) stage[j] = load16(x_src[j] + (size_t)min(c0 + x_chunk[j], end - 1) * 64);
-  };
-  auto stash = [&](int buffer) {
-#pragma unroll
-    for (int j = 0; j < MB; ++j) (&xs[buffer][0][0][0][0])[tid + 512 * j] = stage[j];
-  };
-
-  f32x4_t acc[MB];
-#pragma unroll
-  for (int b = 0; b < MB; ++b) acc[b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  // weights of a stage, asked for one stage early (two register sets in turn)
-  u32x4_t wv[2][MID_STAGE][2];
-  auto fetch_w = [&](int c0, auto set_tag) {
-    constexpr int set = decltype(set_tag)::value;
-#pragma unroll
-    for (int ch = 0; ch < MID_STAGE; ++ch) {
-      const uint16_t* p = wp + (size_t)min(c0 + ch, end - 1) * 1024;
-      wv[set][ch][0] = load16_stream(p);
-      wv[set][ch][1] = load16_stream(p + 512);
-    }
-  };
-  auto multiply = [&](int c0, int buffer, auto set_tag) {
-    constexpr int set = decltype(set_tag)::value;
-#pragma unroll
-    for (int ch = 0; ch < MID_STAGE; ++ch) {
-      if (c0 + ch < end) {
-#pragma unroll
-        for (int b = 0; b < MB; ++b) {
-          acc[b] = MFMA16(wv[set][ch][0], xs[buffer][ch][b][0][lane], acc[b]);
-          acc[b] = MFMA16(wv[set][ch][1], xs[buffer][ch][b][1][lane], acc[b]);
-        }
-      }
-    }
-  };
-  const std::integral_constant<int, 0> set0;
-  const std::integral_constant<int, 1> set1;
-  fetch_w(first, set0);
-  fetch(first);
-  stash(0);
-  __syncthreads();
-  for (int c0 = first; c0 < end; c0 += 2 * MID_STAGE) {
-    // even stage: from LDS buffer 0 and weight set 0, while the next stage's numbers come in
-    const bool more = c0 + MID_STAGE < end;
-    if (more) {   // activations first: they are waited for before this stage ends, the weights (behind them in the queue) are not
-      fetch(c0 + MID_STAGE);
-      fetch_w(c0 + MID_STAGE, set1);
-    }
-    multiply(c0, 0, set0);
-    if (more) stash(1);
-    __syncthreads();   // the next stage is in place, and everyone is done with this one
-    if (!more) break;
-    // odd stage
-    const bool further = c0 + 2 * MID_STAGE < end;
-    if (further) {
-      fetch(c0 + 2 * MID_STAGE);
-      fetch_w(c0 + 2 * MID_STAGE, set0);
-    }
-    multiply(c0 + MID_STAGE, 1, set1);
-    if (further) stash(0);
-    __syncthreads();
-  }
-  // D: lane holds column (activation row) i = lane % 16 and rows (W rows) 4g..4g+3 of the wave's block
-  if (!own) return;
-  const int i = lane % 16, g = lane / 16;
-  float* out = sums + (size_t)blockIdx.y * M * w_rows;
-#pragma unroll
-  for (int b = 0; b < MB; ++b) {
-    const int m = b * 16 + i;
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int n = block * 16 + 4 * g + r;
-      if (m < M && n < w_rows) out[(size_t)m * w_rows + n] = acc[b][r];
-    }
-  }
-}
-
+// ---- K in parts: the finishing kernel ---------------------------------------------------------
+// Whole tiles that are too few to fill the chip cut K into parts over workgroups (gemm_tiled_whole_kernel
+// with `parts_out`); the bare sums go to scratch memory as [K part][row][weight row].  This kernel adds the
+// parts in order and does what the other kernels do with their sums: the row factor of a norm ahead,
+// SwiGLU, accumulation into the residual, a norm behind.
 // One block per 16 rows x 16 outputs: thread (r, col) = (tid / 16, tid % 16).  All of a thread's loads are asked
 // for before the first is used.
-#define MID_MAX_PARTS 16
+#define MAX_PARTS 16
 template <bool SWIGLU, typename TC>
-__global__ __launch_bounds__(256) void gemm_mid_finish_kernel(const float* __restrict__ sums, TC* __restrict__ c,
+__global__ __launch_bounds__(256) void gemm_parts_finish_kernel(const float* __restrict__ sums, TC* __restrict__ c,
                                                               int M, int N, int K, int parts, int accumulate,
                                                               RidingNorm norm) {
   const int w_rows = SWIGLU ? 2 * N : N;
   const int col = threadIdx.x % 16, n = blockIdx.x * 16 + col, m = blockIdx.y * 16 + threadIdx.x / 16;
   const bool valid = m < M && n < N;
-  float first_part[MID_MAX_PARTS], second_part[SWIGLU ? MID_MAX_PARTS : 1];
+  float first_part[MAX_PARTS], second_part[SWIGLU ? MAX_PARTS : 1];
 #pragma unroll
-  for (int part = 0; part < MID_MAX_PARTS; ++part) {
+  for (int part = 0; part < MAX_PARTS; ++part) {
     const bool there = valid && part < parts;
     const float* row = sums + ((size_t)(there ? part : 0) * M + (valid ? m : 0)) * w_rows;
     first_part[part] = there ? row[n] : 0.f;
@@ -411,7 +298,7 @@ __global__ __launch_bounds__(256) void gemm_mid_finish_kernel(const float* __res
   }
   float first = 0.f, second = 0.f;   // the output's sum over the parts, in their order; for SwiGLU the gate's and the up row's
 #pragma unroll
-  for (int part = 0; part < MID_MAX_PARTS; ++part) {
+  for (int part = 0; part < MAX_PARTS; ++part) {
     first += first_part[part];
     if (SWIGLU) second += second_part[part];
   }
@@ -440,17 +327,6 @@ __global__ __launch_bounds__(256) void gemm_mid_finish_kernel(const float* __res
       if (col == 0) norm.behind_ss[(size_t)m * gridDim.x + blockIdx.x] = sq;
     }
   }
-}
-
-// How the 17-to-64-row path cuts K: the number of parts and the 64-wide chunks in each.
-static void mid_parts(int w_rows, int K, int* parts, int* chunks_per_part) {
-  const int full = K / 64, groups = ((w_rows + 15) / 16 + 7) / 8;   // workgroups along the weight rows
-  int p = 1;
-  while (groups * p < 256 && p < MID_MAX_PARTS && full / (p * 2) >= 2 * MID_STAGE) p *= 2;   // enough workgroups, and two stages each at least
-  int chunks = (full + p - 1) / p;
-  chunks = (chunks + MID_STAGE - 1) / MID_STAGE * MID_STAGE;          // whole stages
-  *chunks_per_part = chunks;
-  *parts = (full + chunks - 1) / chunks;
 }
 
 // ---- tiled -----------------------------------------------------------------------------------
@@ -623,7 +499,9 @@ template <bool SWIGLU, int WX, int WY, int WM, int WN, int BUFFERS, typename TC>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_whole_kernel(const uint16_t* __restrict__ a,
                                                                          const uint16_t* __restrict__ w,
                                                                          TC* __restrict__ c, int M, int N, int K,
-                                                                         int accumulate, RidingNorm norm) {
+                                                                         int accumulate, RidingNorm norm,
+                                                                         float* __restrict__ parts_out,
+                                                                         int slices_per_part) {
   constexpr int THREADS = 64 * WM * WN;
   constexpr int TBM = 32 * WX * WM, TBN = 32 * WY * WN;
   static_assert(TBM <= THREADS, "one thread per row of the tile adds up the norm's partial sums");
@@ -638,13 +516,21 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_whole_kernel(const ui
   __shared__ __attribute__((aligned(16))) float row_factor[TBM];   // norm ahead: what each row's result is multiplied by
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int m_own = blockIdx.y * TBM, n_own = blockIdx.x * OUTS;   // what this tile stands for
-  const int m0 = min(m_own, M - TBM), n0 = min(n_own, N - OUTS);   // where it computes
+  // Tiles of 32 or 64 rows (WX == 1) also take fewer rows than a tile: loads repeat the last row, and
+  // nothing beyond it is stored.
+  constexpr bool SHORT = WX == 1;
+  const int m0 = SHORT && M < TBM ? 0 : min(m_own, M - TBM), n0 = min(n_own, N - OUTS);   // where it computes
   const int wm = (wave / WN) * 32 * WX, wn = (wave % WN) * 32 * WY;
 
   // A: piece e = tid + s * THREADS is row e / 8, 16 bytes e % 8 of the slice
   const uint16_t* a_tile = a + (size_t)m0 * K;
   const int a_off = (tid / 8) * K + (tid % 8) * 8;                 // + s * A_ROWS * K, the same for all threads
   const int a_lds = (tid / 8) * TPITCH + (tid % 8) * 8;            // + s * A_ROWS * TPITCH
+  int a_short[SHORT ? A_PIECES : 1];                               // short tiles: an offset per round, rows clamped
+  if (SHORT) {
+#pragma unroll
+    for (int s = 0; s < A_PIECES; ++s) a_short[s] = min(tid / 8 + s * A_ROWS, M - 1 - m0) * K + (tid % 8) * 8;
+  }
   // W: piece e is block e / 128 of the tile's rows in LDS, piece p = e % 128 = u * 64 + l of that block's slice:
   // row l % 16, k 16 * (l / 16) + 8 u.  LDS block b of round s holds W rows starting at
   //   plain:  n0 + 16 (b + s * W_BLOCKS)
@@ -663,7 +549,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_whole_kernel(const ui
   u32x4_t a_reg[A_PIECES], w_reg[W_PIECES];
   auto fetch = [&](int slice) {
 #pragma unroll
-    for (int s = 0; s < A_PIECES; ++s) a_reg[s] = load16(a_tile + (size_t)s * A_ROWS * K + slice * TK + a_off);
+    for (int s = 0; s < A_PIECES; ++s)
+      a_reg[s] = load16(a_tile + (SHORT ? (size_t)a_short[s] : (size_t)s * A_ROWS * K + a_off) + slice * TK);
 #pragma unroll
     for (int s = 0; s < W_PIECES; ++s) w_reg[s] = load16(w_tile + w_round[s] + (size_t)slice * 1024 + w_off);
   };
@@ -684,10 +571,13 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_whole_kernel(const ui
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[x][y][e] = 0.f;
 
-  const int slices = K / TK;
-  fetch(0);
-  if (norm.ahead_ss && tid < TBM) {   // while the first slice is on its way
-    const float* partial = norm.ahead_ss + (size_t)(m0 + tid) * norm.ahead_blocks;
+  // K in parts (parts_out): workgroup z multiplies its part of the slices and leaves the bare sums to
+  // gemm_parts_finish_kernel.
+  const int first_slice = parts_out ? blockIdx.z * slices_per_part : 0;
+  const int end_slice = parts_out ? min(K / TK, first_slice + slices_per_part) : K / TK;
+  fetch(first_slice);
+  if (norm.ahead_ss && !parts_out && tid < TBM) {   // while the first slice is on its way
+    const float* partial = norm.ahead_ss + (size_t)min(m0 + tid, M - 1) * norm.ahead_blocks;
     float total = 0.f;
     if (norm.ahead_blocks % 4 == 0) {   // 32 sums per round of loads, added in their order
       const f32x4_t* four = reinterpret_cast<const f32x4_t*>(partial);
@@ -726,8 +616,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_whole_kernel(const ui
   };
   // All slices but the last in a loop without a branch in its body: loads, multiplies and staging writes
   // are one stretch of code that the compiler may interleave.
-  for (int s = 0; s + 1 < slices; ++s) {
-    const int buffer = BUFFERS == 2 ? (s & 1) : 0;
+  for (int s = first_slice; s + 1 < end_slice; ++s) {
+    const int buffer = BUFFERS == 2 ? ((s - first_slice) & 1) : 0;
     fetch(s + 1);
     __builtin_amdgcn_sched_barrier(0);   // the loads go out first: a slice of multiplies is their time to land
     multiply(buffer);
@@ -735,8 +625,26 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_whole_kernel(const ui
     stash(BUFFERS == 2 ? buffer ^ 1 : 0);
     __syncthreads();
   }
-  multiply(BUFFERS == 2 ? ((slices - 1) & 1) : 0);
+  multiply(BUFFERS == 2 ? ((end_slice - 1 - first_slice) & 1) : 0);
   // D of one 32x32 block: column (n) lane%32, rows (m) 8*(e/4) + 4*(lane/32) + e%4
+  if (parts_out) {   // [part][row][weight row]; a SwiGLU's up rows lie N after its gate rows
+    const int w_rows = SWIGLU ? 2 * N : N;
+    float* out = parts_out + (size_t)blockIdx.z * M * w_rows;
+#pragma unroll
+    for (int x = 0; x < WX; ++x)
+#pragma unroll
+      for (int y = 0; y < WY; ++y) {
+        const int n = SWIGLU ? n0 + (wave % WN) * 16 * WY + (y % (WY / 2)) * 32 + lane % 32 : n0 + wn + y * 32 + lane % 32;
+        if (n < n_own) continue;
+        const int w_row = SWIGLU && y >= WY / 2 ? N + n : n;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int m = m0 + wm + x * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
+          if (m >= m_own && m < M) out[(size_t)m * w_rows + w_row] = acc[x][y][e];
+        }
+      }
+    return;
+  }
   if (norm.ahead_ss) {
 #pragma unroll
     for (int x = 0; x < WX; ++x)
@@ -776,7 +684,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_whole_kernel(const ui
 #pragma unroll
           for (int e = 0; e < 16; ++e) {
             const int m = m0 + wm + x * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
-            if (m < m_own) continue;
+            if (m < m_own || m >= M) continue;
             const size_t at = (size_t)m * N + n;
             const float value = accumulate ? c[at] + acc[x][y][e] : acc[x][y][e];
             c[at] = value;
@@ -792,7 +700,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_whole_kernel(const ui
         }
       }
       __syncthreads();
-      if (tid < TBM && m0 + tid >= m_own) {
+      if (tid < TBM && m0 + tid >= m_own && m0 + tid < M) {
         float total = 0.f;
 #pragma unroll
         for (int part = 0; part < WN; ++part) total += partial[part * TBM + tid];
@@ -811,7 +719,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_whole_kernel(const ui
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
           const int m = m0 + wm + x * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
-          if (m >= m_own) store_out<TC>(c, (size_t)m * N + n, silu_mul(acc[x][y][e], acc[x][y + WY / 2][e]), false);
+          if (m >= m_own && m < M) store_out<TC>(c, (size_t)m * N + n, silu_mul(acc[x][y][e], acc[x][y + WY / 2][e]), false);
         }
       }
     } else {
@@ -822,7 +730,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_whole_kernel(const ui
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
           const int m = m0 + wm + x * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
-          if (m >= m_own) store_out<TC>(c, (size_t)m * N + n, acc[x][y][e], accumulate != 0);
+          if (m >= m_own && m < M) store_out<TC>(c, (size_t)m * N + n, acc[x][y][e], accumulate != 0);
         }
       }
     }
@@ -855,32 +763,82 @@ static void launch_skinny(const void* a, const void* w, void* c, int M, int N, i
 // (one barrier per slice, two workgroups per compute unit) are the better choice unless a single one
 // (four workgroups per compute unit) lets the whole grid run at once: between two and four tiles for
 // each of the 256 compute units.
-enum TiledConfig { TILED_256 = 0, TILED_128_ONE_BUFFER = 1, TILED_128 = 2 };
+// Fewer than 128 rows (decode steps of many sequences, short prompts) are still bound by reading W: tiles
+// of 64 rows, or of 32 for up to 32 rows, which the kernel also takes when there are fewer rows than a tile.
+enum TiledConfig { TILED_256 = 0, TILED_128_ONE_BUFFER = 1, TILED_128 = 2, TILED_64_ROWS = 3, TILED_32_ROWS = 4 };
 static TiledConfig tiled_config(int M, int N, bool swiglu, int* rows, int* columns) {
+  if (M <= 32) {
+    *rows = 32;
+    *columns = 128;
+    return TILED_32_ROWS;
+  }
+  if (M < 128) {
+    *rows = 64;
+    *columns = swiglu ? 64 : 128;
+    return TILED_64_ROWS;
+  }
   const long tiles_128 = (long)((N + (swiglu ? 63 : 127)) / (swiglu ? 64 : 128)) * ((M + 127) / 128);
   const bool big = tiles_128 >= 3072;
   *rows = big ? 256 : 128;
   *columns = (big ? 256 : 128) / (swiglu ? 2 : 1);
   return big ? TILED_256 : tiles_128 > 512 && tiles_128 <= 1024 ? TILED_128_ONE_BUFFER : TILED_128;
 }
-// Whether the product runs as whole tiles (gemm_tiled_whole_kernel), the only tiled way a norm rides on.
+// Whether the product runs as whole tiles (gemm_tiled_whole_kernel): the way that cuts K into parts and
+// the only tiled way a norm rides on.  Up to 16 rows belong to the skinny kernel.
 static bool tiled_whole(int M, int N, int K, int layout, int rows, int columns) {
-  return layout == 1 && K % TK == 0 && N % 16 == 0 && M >= rows && N >= columns && (long)rows * K < (1L << 31);
+  return layout == 1 && K % TK == 0 && N % 16 == 0 && M > 16 && (M >= rows || rows <= 64) && N >= columns &&
+         (long)rows * K < (1L << 31);
+}
+
+// Whole tiles that are too few to fill the chip cut K into parts (gemm_parts_finish_kernel adds them): the
+// number of parts and the 64-wide slices in each; one part means no cut.
+// Measured at the Qwen3-8B shapes.  128 to 1,024 rows: up to half a tile per compute unit the cut pays
+// (M = 512: o 50 -> 40 us, down 146 -> 82 us; M = 128: qkv 52 -> 27, o 50 -> 22, down 136 -> 34 us), at one
+// tile per compute unit it no longer does; one workgroup per compute unit is enough (more parts only add
+// scratch traffic) unless a part would still be longer than 64 slices.  Fewer than 128 rows (bound by
+// reading W, little scratch traffic): about 384 workgroups, whatever the number of tiles, was the best of
+// 256 to 2,048 in decode steps of 17 to 64 sequences.
+#define TILED_FEW_TILES 128
+#define TILED_SHORT_WORKGROUPS 384
+static void tiled_parts(int M, int N, int K, int layout, bool swiglu, int* parts, int* slices_per_part) {
+  int rows, columns;
+  tiled_config(M, N, swiglu, &rows, &columns);
+  *parts = 1;
+  *slices_per_part = K / TK;
+  if (!tiled_whole(M, N, K, layout, rows, columns)) return;
+  const long tiles = (long)((N + columns - 1) / columns) * ((M + rows - 1) / rows);
+  const int slices = K / TK;
+  int p;
+  if (rows <= 64) {
+    p = (int)((TILED_SHORT_WORKGROUPS + tiles - 1) / tiles);
+  } else {
+    if (tiles > TILED_FEW_TILES) return;
+    p = (int)(2 * TILED_FEW_TILES / tiles);
+    if (slices / p > 64) p *= 2;
+  }
+  p = std::min(std::min(p, MAX_PARTS), slices / 4);    // at least four slices each
+  if (p < 2) return;
+  *slices_per_part = (slices + p - 1) / p;
+  *parts = (slices + *slices_per_part - 1) / *slices_per_part;
 }
 
 template <bool TILES, bool SWIGLU, typename TC>
 static void launch_tiled(const void* a, const void* w, void* c, int M, int N, int K, int accumulate,
-                         const RidingNorm& norm, hipStream_t stream) {
+                         const RidingNorm& norm, float* parts_out, hipStream_t stream) {
   int rows, columns;
   const TiledConfig config = tiled_config(M, N, SWIGLU, &rows, &columns);
   const bool whole = tiled_whole(M, N, K, TILES ? 1 : 0, rows, columns);
-  dim3 grid((N + columns - 1) / columns, (M + rows - 1) / rows);
+  int parts = 1, slices_per_part = 0;
+  if (parts_out) tiled_parts(M, N, K, TILES ? 1 : 0, SWIGLU, &parts, &slices_per_part);
+  if (parts == 1) parts_out = nullptr;
+  dim3 grid((N + columns - 1) / columns, (M + rows - 1) / rows, parts);
 #define BH_TILED(WX, WY, WM, WN, BUFFERS)                                                                 \
   do {                                                                                                     \
     dim3 block(64 * WM * WN);                                                                              \
     if (TILES && whole)                                                                                    \
       gemm_tiled_whole_kernel<SWIGLU, WX, WY, WM, WN, BUFFERS, TC><<<grid, block, 0, stream>>>(            \
-          (const uint16_t*)a, (const uint16_t*)w, (TC*)c, M, N, K, accumulate, norm);                      \
+          (const uint16_t*)a, (const uint16_t*)w, (TC*)c, M, N, K, accumulate, norm, parts_out,            \
+          slices_per_part);                                                                                \
     else                                                                                                   \
       gemm_tiled_kernel<TILES, SWIGLU, WX, WY, WM, WN, BUFFERS, TC><<<grid, block, 0, stream>>>(           \
           (const uint16_t*)a, (const uint16_t*)w, (TC*)c, M, N, K, accumulate);                            \
@@ -888,6 +846,11 @@ static void launch_tiled(const void* a, const void* w, void* c, int M, int N, in
   switch (config) {
     case TILED_256: BH_TILED(2, 4, 4, 2, 2); break;
     case TILED_128_ONE_BUFFER: BH_TILED(2, 2, 2, 2, 1); break;
+    case TILED_64_ROWS: BH_TILED(1, 2, 2, 2, 1); break;   // one LDS buffer: more workgroups per compute unit, more loads in flight
+    case TILED_32_ROWS:
+      if constexpr (SWIGLU) BH_TILED(1, 2, 1, 4, 1);
+      else BH_TILED(1, 1, 1, 4, 1);
+      break;
     default: BH_TILED(2, 2, 2, 2, 2); break;
   }
 #undef BH_TILED
@@ -897,10 +860,11 @@ static void launch_tiled(const void* a, const void* w, void* c, int M, int N, in
 // carry one), and whether it can take prepared norm rows as its activations.
 extern "C" int bh_gemm_bf16_norm_blocks(int M, int N, int K, int layout, int activation) {
   if (activation || M <= 0 || N <= 0 || K % 8 != 0) return 0;
-  if (M <= 64) return (N + 15) / 16;
-  int rows, columns;
+  int rows, columns, parts, each;
   tiled_config(M, N, false, &rows, &columns);
-  return tiled_whole(M, N, K, layout, rows, columns) ? (N + columns - 1) / columns : 0;
+  if (!tiled_whole(M, N, K, layout, rows, columns)) return M <= 64 ? (N + 15) / 16 : 0;   // the skinny kernel's blocks
+  tiled_parts(M, N, K, layout, false, &parts, &each);
+  return parts > 1 ? (N + 15) / 16 : (N + columns - 1) / columns;   // the finishing kernel's blocks, or the tiles'
 }
 extern "C" int bh_gemm_bf16_takes_norm(int M, int N, int K, int layout, int activation) {
   if (M <= 0 || N <= 0 || K % 8 != 0 || (activation && N % 16 != 0)) return 0;
@@ -913,15 +877,15 @@ extern "C" int bh_gemm_bf16_takes_norm(int M, int N, int K, int layout, int acti
 // layout: 0 = rows, 1 = tiles.  activation: 0 = none; 1 = SwiGLU (W has 2 * N rows: gate rows then up rows).
 // Bytes of scratch memory that bh_gemm_bf16 wants for this product (0: none).
 extern "C" long bh_gemm_bf16_scratch(int M, int N, int K, int layout, int activation) {
-  if (M <= 16 || M > 64 || layout != 1 || K % 64 != 0 || N <= 0) return 0;
-  int parts, chunks;
-  mid_parts(activation ? 2 * N : N, K, &parts, &chunks);
-  return (long)parts * M * (activation ? 2 * N : N) * (long)sizeof(float);
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  int parts, each;
+  tiled_parts(M, N, K, layout, activation != 0, &parts, &each);
+  return parts == 1 ? 0 : (long)parts * M * (activation ? 2 * N : N) * (long)sizeof(float);
 }
 
 // The `ahead_*` and `behind_*` arguments (null when unused) let an RMSNorm ride on the products before and
 // after it (struct RidingNorm) where bh_gemm_bf16_takes_norm / bh_gemm_bf16_norm_blocks say so.  `scratch`: bh_gemm_bf16_scratch() bytes, or
-// null (then products of 17 to 64 rows take the slower way without it).
+// null (then K is not cut into parts where that would be faster).
 extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, int accumulate, int M, int N, int K,
                             int layout, int activation, const float* ahead_ss, int ahead_blocks, float ahead_eps,
                             const void* behind_weight, int behind_weight_dtype, void* behind_rows,
@@ -952,27 +916,28 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
     if (f32) FN<TILES, EXTRA, float>(__VA_ARGS__);                                  \
     else FN<TILES, EXTRA, bf16_t>(__VA_ARGS__);                                     \
   } while (0)
-  if (scratch != nullptr && bh_gemm_bf16_scratch(M, N, K, layout, activation) > 0) {
-    const int w_rows = activation ? 2 * N : N;
-    int parts, chunks;
-    mid_parts(w_rows, K, &parts, &chunks);
-    dim3 grid(((w_rows + 15) / 16 + 7) / 8, parts);
-    switch ((M + 15) / 16) {
-      case 2: gemm_mid_kernel<2><<<grid, 512, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, (float*)scratch, M, w_rows, K, chunks); break;
-      case 3: gemm_mid_kernel<3><<<grid, 512, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, (float*)scratch, M, w_rows, K, chunks); break;
-      default: gemm_mid_kernel<4><<<grid, 512, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, (float*)scratch, M, w_rows, K, chunks); break;
-    }
-    if (int status = bh_check_launch("gemm_mid")) return status;
+  const bool in_parts = scratch != nullptr && bh_gemm_bf16_scratch(M, N, K, layout, activation) > 0;
+  BH_REQUIRE(in_parts || !behind_weight || bh_gemm_bf16_scratch(M, N, K, layout, activation) == 0,
+             "gemm_bf16: a product of M=%d N=%d K=%d carries a norm through its finishing kernel and needs scratch memory", M, N, K);
+  if (in_parts) {   // K in parts, then the finishing kernel
+    int parts, each;
+    tiled_parts(M, N, K, layout, activation != 0, &parts, &each);
+    const RidingNorm none = {};
+    if (activation) launch_tiled<true, true, float>(a, w, nullptr, M, N, K, 0, none, (float*)scratch, stream);
+    else launch_tiled<true, false, float>(a, w, nullptr, M, N, K, 0, none, (float*)scratch, stream);
+    if (int status = bh_check_launch("gemm_tiled")) return status;
     dim3 finish_grid((N + 15) / 16, (M + 15) / 16);
-#define BH_FINISH(SWIGLU, TC)                                                                              \
-  gemm_mid_finish_kernel<SWIGLU, TC><<<finish_grid, 256, 0, stream>>>((const float*)scratch, (TC*)c, M, N, K, \
-                                                                       parts, accumulate, norm)
+#define BH_FINISH(SWIGLU, TC)                                                                                \
+  gemm_parts_finish_kernel<SWIGLU, TC><<<finish_grid, 256, 0, stream>>>((const float*)scratch, (TC*)c, M, N, K, \
+                                                                         parts, accumulate, norm)
     if (activation) { if (f32) BH_FINISH(true, float); else BH_FINISH(true, bf16_t); }
     else { if (f32) BH_FINISH(false, float); else BH_FINISH(false, bf16_t); }
 #undef BH_FINISH
-    return bh_check_launch("gemm_mid_finish");
+    return bh_check_launch("gemm_parts_finish");
   }
-  if (M <= 64) {
+  int tile_rows, tile_columns;
+  tiled_config(M, N, activation != 0, &tile_rows, &tile_columns);
+  if (M <= 64 && !tiled_whole(M, N, K, layout, tile_rows, tile_columns)) {
     const int pair_blocks = N / 16;
     if (activation) {
       if (layout) BH_PICK(launch_skinny, true, 2, a, w, c, M, N, K, 0, pair_blocks, norm, stream);
@@ -984,11 +949,11 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
     return bh_check_launch("gemm_skinny");
   }
   if (activation) {
-    if (layout) BH_PICK(launch_tiled, true, true, a, w, c, M, N, K, 0, norm, stream);
-    else BH_PICK(launch_tiled, false, true, a, w, c, M, N, K, 0, norm, stream);
+    if (layout) BH_PICK(launch_tiled, true, true, a, w, c, M, N, K, 0, norm, nullptr, stream);
+    else BH_PICK(launch_tiled, false, true, a, w, c, M, N, K, 0, norm, nullptr, stream);
   } else {
-    if (layout) BH_PICK(launch_tiled, true, false, a, w, c, M, N, K, accumulate, norm, stream);
-    else BH_PICK(launch_tiled, false, false, a, w, c, M, N, K, accumulate, norm, stream);
+    if (layout) BH_PICK(launch_tiled, true, false, a, w, c, M, N, K, accumulate, norm, nullptr, stream);
+    else BH_PICK(launch_tiled, false, false, a, w, c, M, N, K, accumulate, norm, nullptr, stream);
   }
 #undef BH_PICK
   return bh_check_launch("gemm_tiled");

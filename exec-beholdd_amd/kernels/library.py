@@ -203,7 +203,7 @@ class HipKernels:
                                     torch.empty((m, blocks), dtype=torch.float32, device=self.device), then_norm.eps,
                                     out, then_norm.weight)
         a_rows = ahead.rows if ahead is not None else a
-        scratch = None       # products of 17 to 64 rows add up parts of K through scratch memory
+        scratch = None       # products of few tiles add up parts of K through scratch memory
         scratch_bytes = int(self.lib.bh_gemm_bf16_scratch(*sizes))
         if scratch_bytes:
             scratch = torch.empty(scratch_bytes // 4, dtype=torch.float32, device=self.device)

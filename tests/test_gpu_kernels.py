@@ -99,7 +99,11 @@ def test_gemm(K, a_dtype, w_dtype, m, n, k):
                                    (1030, 43700, 192),
                                    # whole tiles of the packed layout (N a multiple of 16), last tiles moved back inside
                                    (300, 1008, 1024), (129, 144, 128), (128, 128, 64), (1030, 43712, 192),
-                                   (2048, 4096, 512)])
+                                   (2048, 4096, 512),
+                                   # few whole tiles: K in parts (equal and unequal ones) and a finishing kernel
+                                   (200, 320, 832), (512, 4096, 4096), (128, 128, 4096),
+                                   # 65 to 127 rows: whole tiles of 64 rows
+                                   (100, 256, 1024), (127, 4096, 512), (65, 128, 64)])
 def test_gemm_with_packed_weights(K, m, n, k):
     """The same product from the regrouped (16 x 64 blocks) weight layout."""
     from beholdd.kernels import PackedWeight
@@ -145,7 +149,7 @@ def test_norm_rides_on_the_products_around_it(K, g_dtype, packed, m, n, k, n2):
     got_residual = residual.cpu().double()
     assert rel(prepared.rows, got_residual * g.double()) < 4e-3                       # bfloat16 rounding
     assert rel(prepared.ss.sum(1), (got_residual ** 2).sum(-1)) < 1e-5
-    assert prepared.ss.shape == (m, -(-n // 16))
+    assert prepared.ss.shape[0] == m and prepared.ss.dim() == 2
     normed = got_residual / torch.sqrt((got_residual ** 2).mean(-1, keepdim=True) + eps) * g.double()
 
     w2 = (torch.randn(n2, n, generator=gen) * 0.1).to(torch.bfloat16)
@@ -168,7 +172,9 @@ def test_norm_rides_on_the_products_around_it(K, g_dtype, packed, m, n, k, n2):
 
 @pytest.mark.parametrize("m,n,k,n2,g_dtype", [(200, 320, 192, 130, torch.float32), (200, 320, 192, 144, torch.bfloat16),
                                               (300, 4096, 128, 256, torch.float32), (128, 128, 64, 128, torch.bfloat16),
-                                              (3072, 16384, 64, 256, torch.float32)])
+                                              (3072, 16384, 64, 256, torch.float32),
+                                              (200, 320, 832, 144, torch.float32), (256, 1024, 512, 1024, torch.bfloat16),
+                                              (100, 320, 832, 144, torch.float32), (65, 128, 64, 128, torch.bfloat16)])
 def test_norm_rides_on_wide_products(K, m, n, k, n2, g_dtype):
     """The same for the products of many rows: whole tiles of a packed weight carry the norm (partial sums
     per tile column, edge tiles counting only what they own); other wide products leave it alone."""
@@ -218,7 +224,8 @@ def test_norm_does_not_ride_on_wide_steps(K):
 @pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("m,width,k", [(1, 16, 64), (8, 160, 128), (40, 896, 320), (64, 48, 192), (65, 64, 64),
                                        (130, 208, 256), (300, 1000, 128), (7, 100, 64), (8, 12288, 4096), (5, 32, 72),
-                                       (650, 33008, 128)])
+                                       (650, 33008, 128), (130, 208, 832), (256, 512, 1024), (100, 256, 512),
+                                       (127, 64, 64)])
 def test_gemm_swiglu(K, dtype, packed, m, width, k):
     """silu(a Wg^T) * (a Wu^T) in one pass (or in two where the sizes do not allow one), from both layouts."""
     g = torch.Generator().manual_seed(m + width)
