@@ -67,7 +67,7 @@ __device__ inline float silu_mul(float gate, float up) { return gate / (1.0f + e
 // An RMSNorm between two products can ride on them (struct RidingNorm):
 //   behind: the product that completes the float32 residual h also writes bfloat16(h[m][n] * g[n]) (the
 //           norm's output but for the row factor) and, per workgroup, the sum of h[m][n]^2 over its
-//           columns (16 of them in the skinny kernel and the finishing kernel, a tile's width in whole tiles);
+//           columns (16 of them in the skinny kernel, 64 in the finishing kernel, a tile's width in whole tiles);
 //   ahead:  the product that consumes the norm's output takes those unscaled rows as its activations and
 //           multiplies its result by 1 / sqrt(sum of the partial sums / K + eps) of the row.
 // The row factor commutes with the product, so the result is the norm's up to the rounding of the
@@ -261,23 +261,27 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
 // with `parts_out`); the bare sums go to scratch memory as [K part][row][weight row].  This kernel adds the
 // parts in order and does what the other kernels do with their sums: the row factor of a norm ahead,
 // SwiGLU, accumulation into the residual, a norm behind.
-// One block per 16 rows x 16 outputs: thread (r, col) = (tid / 16, tid % 16).  All of a thread's loads are asked
-// for before the first is used.
+// One block per 16 rows x 64 outputs: thread (r, col) = (tid / 16, tid % 16) has the four outputs
+// 64 * blockIdx.x + 4 col .. + 3 of row 16 * blockIdx.y + r (N is a multiple of 16 here).  All of a thread's
+// loads are asked for before the first is used.  A norm behind gets one partial sum per row and block.
 #define MAX_PARTS 16
+#define FINISH_COLUMNS 64
+typedef uint16_t u16x4_t __attribute__((ext_vector_type(4)));
 template <bool SWIGLU, typename TC>
 __global__ __launch_bounds__(256) void gemm_parts_finish_kernel(const float* __restrict__ sums, TC* __restrict__ c,
-                                                              int M, int N, int K, int parts, int accumulate,
-                                                              RidingNorm norm) {
+                                                                int M, int N, int K, int parts, int accumulate,
+                                                                RidingNorm norm) {
   const int w_rows = SWIGLU ? 2 * N : N;
-  const int col = threadIdx.x % 16, n = blockIdx.x * 16 + col, m = blockIdx.y * 16 + threadIdx.x / 16;
+  const int col = threadIdx.x % 16, n = blockIdx.x * FINISH_COLUMNS + 4 * col, m = blockIdx.y * 16 + threadIdx.x / 16;
   const bool valid = m < M && n < N;
-  float first_part[MAX_PARTS], second_part[SWIGLU ? MAX_PARTS : 1];
+  const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+  f32x4_t first_part[MAX_PARTS], second_part[SWIGLU ? MAX_PARTS : 1];
 #pragma unroll
   for (int part = 0; part < MAX_PARTS; ++part) {
     const bool there = valid && part < parts;
     const float* row = sums + ((size_t)(there ? part : 0) * M + (valid ? m : 0)) * w_rows;
-    first_part[part] = there ? row[n] : 0.f;
-    if (SWIGLU) second_part[part] = there ? row[N + n] : 0.f;
+    first_part[part] = there ? *reinterpret_cast<const f32x4_t*>(row + n) : zero;
+    if (SWIGLU) second_part[part] = there ? *reinterpret_cast<const f32x4_t*>(row + N + n) : zero;
   }
   float factor = 1.f;
   if (norm.ahead_ss) {   // 16 lanes share a row: each adds every 16th partial sum, then the 16 are added pairwise
@@ -296,7 +300,7 @@ __global__ __launch_bounds__(256) void gemm_parts_finish_kernel(const float* __r
     for (int off = 8; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
     factor = 1.0f / sqrtf(ss / (float)K + norm.ahead_eps);
   }
-  float first = 0.f, second = 0.f;   // the output's sum over the parts, in their order; for SwiGLU the gate's and the up row's
+  f32x4_t first = zero, second = zero;   // the outputs' sums over the parts, in their order; for SwiGLU the gates' and the up rows'
 #pragma unroll
   for (int part = 0; part < MAX_PARTS; ++part) {
     first += first_part[part];
@@ -304,28 +308,48 @@ __global__ __launch_bounds__(256) void gemm_parts_finish_kernel(const float* __r
   }
   first *= factor;
   second *= factor;
-  float value = 0.f;   // what the residual holds afterwards (norm.behind_weight: float32 output, no SwiGLU)
+  const size_t at = (size_t)(valid ? m : 0) * N + (valid ? n : 0);
+  f32x4_t value = zero;   // what the outputs hold afterwards; 0 where there is no element
   if (valid) {
     if (SWIGLU) {
-      store_out<TC>(c, (size_t)m * N + n, silu_mul(first, second), false);
-    } else if (norm.behind_weight) {
-      float* cf = reinterpret_cast<float*>(c);
-      value = accumulate ? cf[(size_t)m * N + n] + first : first;
-      cf[(size_t)m * N + n] = value;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) value[i] = silu_mul(first[i], second[i]);
     } else {
-      store_out<TC>(c, (size_t)m * N + n, first, accumulate != 0);
+      value = first;
+      if (accumulate) {
+        if constexpr (sizeof(TC) == 4) {
+          value += *reinterpret_cast<const f32x4_t*>(reinterpret_cast<const float*>(c) + at);
+        } else {
+          const u16x4_t old = *reinterpret_cast<const u16x4_t*>(reinterpret_cast<const uint16_t*>(c) + at);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) value[i] += bf16_bits_to_f32(old[i]);
+        }
+      }
+    }
+    if constexpr (sizeof(TC) == 4) {
+      *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(c) + at) = value;
+    } else {
+      u16x4_t packed;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) packed[i] = f32_to_bf16_bits(value[i]);
+      *reinterpret_cast<u16x4_t*>(reinterpret_cast<uint16_t*>(c) + at) = packed;
     }
   }
-  if (!SWIGLU && norm.behind_weight) {
-    float sq = value * value;   // 0 where there is no element
+  if (!SWIGLU && norm.behind_weight) {   // float32 output
+    float sq = value[0] * value[0] + value[1] * value[1] + value[2] * value[2] + value[3] * value[3];
 #pragma unroll
-    for (int off = 8; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);   // the 16 columns of a row are 16 neighbouring lanes
+    for (int off = 8; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);   // the 64 columns of a row are 16 neighbouring lanes
     if (valid) {
-      const float g = norm.behind_weight_f32 ? reinterpret_cast<const float*>(norm.behind_weight)[n]
-                                             : bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(norm.behind_weight)[n]);
-      norm.behind_rows[(size_t)m * N + n] = f32_to_bf16_bits(value * g);
-      if (col == 0) norm.behind_ss[(size_t)m * gridDim.x + blockIdx.x] = sq;
+      u16x4_t rows;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float g = norm.behind_weight_f32 ? reinterpret_cast<const float*>(norm.behind_weight)[n + i]
+                                               : bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(norm.behind_weight)[n + i]);
+        rows[i] = f32_to_bf16_bits(value[i] * g);
+      }
+      *reinterpret_cast<u16x4_t*>(norm.behind_rows + at) = rows;
     }
+    if (col == 0 && m < M) norm.behind_ss[(size_t)m * gridDim.x + blockIdx.x] = sq;
   }
 }
 
@@ -864,7 +888,7 @@ extern "C" int bh_gemm_bf16_norm_blocks(int M, int N, int K, int layout, int act
   tiled_config(M, N, false, &rows, &columns);
   if (!tiled_whole(M, N, K, layout, rows, columns)) return M <= 64 ? (N + 15) / 16 : 0;   // the skinny kernel's blocks
   tiled_parts(M, N, K, layout, false, &parts, &each);
-  return parts > 1 ? (N + 15) / 16 : (N + columns - 1) / columns;   // the finishing kernel's blocks, or the tiles'
+  return parts > 1 ? (N + FINISH_COLUMNS - 1) / FINISH_COLUMNS : (N + columns - 1) / columns;   // the finishing kernel's blocks, or the tiles'
 }
 extern "C" int bh_gemm_bf16_takes_norm(int M, int N, int K, int layout, int activation) {
   if (M <= 0 || N <= 0 || K % 8 != 0 || (activation && N % 16 != 0)) return 0;
@@ -920,13 +944,15 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
   BH_REQUIRE(in_parts || !behind_weight || bh_gemm_bf16_scratch(M, N, K, layout, activation) == 0,
              "gemm_bf16: a product of M=%d N=%d K=%d carries a norm through its finishing kernel and needs scratch memory", M, N, K);
   if (in_parts) {   // K in parts, then the finishing kernel
+    BH_REQUIRE(((uintptr_t)c | (uintptr_t)scratch | (uintptr_t)behind_rows) % 16 == 0,
+               "gemm_bf16: output, scratch memory and norm rows must be 16-byte aligned");
     int parts, each;
     tiled_parts(M, N, K, layout, activation != 0, &parts, &each);
     const RidingNorm none = {};
     if (activation) launch_tiled<true, true, float>(a, w, nullptr, M, N, K, 0, none, (float*)scratch, stream);
     else launch_tiled<true, false, float>(a, w, nullptr, M, N, K, 0, none, (float*)scratch, stream);
     if (int status = bh_check_launch("gemm_tiled")) return status;
-    dim3 finish_grid((N + 15) / 16, (M + 15) / 16);
+    dim3 finish_grid((N + FINISH_COLUMNS - 1) / FINISH_COLUMNS, (M + 15) / 16);
 #define BH_FINISH(SWIGLU, TC)                                                                                \
   gemm_parts_finish_kernel<SWIGLU, TC><<<finish_grid, 256, 0, stream>>>((const float*)scratch, (TC*)c, M, N, K, \
                                                                          parts, accumulate, norm)
