@@ -802,7 +802,8 @@ static TiledConfig tiled_config(int M, int N, bool swiglu, int* rows, int* colum
     return TILED_64_ROWS;
   }
   const long tiles_128 = (long)((N + (swiglu ? 63 : 127)) / (swiglu ? 64 : 128)) * ((M + 127) / 128);
-  const bool big = tiles_128 >= 3072;
+  const long tiles_256 = (long)((N + (swiglu ? 127 : 255)) / (swiglu ? 128 : 256)) * ((M + 255) / 256);
+  const bool big = tiles_256 >= 512;
   *rows = big ? 256 : 128;
   *columns = (big ? 256 : 128) / (swiglu ? 2 : 1);
   return big ? TILED_256 : tiles_128 > 512 && tiles_128 <= 1024 ? TILED_128_ONE_BUFFER : TILED_128;
