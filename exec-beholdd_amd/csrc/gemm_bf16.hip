@@ -817,14 +817,15 @@ static bool tiled_whole(int M, int N, int K, int layout, int rows, int columns) 
 
 // Whole tiles that are too few to fill the chip cut K into parts (gemm_parts_finish_kernel adds them): the
 // number of parts and the 64-wide slices in each; one part means no cut.
-// Measured at the Qwen3-8B shapes.  128 to 1,024 rows: up to half a tile per compute unit the cut pays
-// (M = 512: o 50 -> 40 us, down 146 -> 82 us; M = 128: qkv 52 -> 27, o 50 -> 22, down 136 -> 34 us), at one
-// tile per compute unit it no longer does; one workgroup per compute unit is enough (more parts only add
-// scratch traffic) unless a part would still be longer than 64 slices.  Fewer than 128 rows (bound by
-// reading W, little scratch traffic): about 384 workgroups, whatever the number of tiles, was the best of
-// 256 to 2,048 in decode steps of 17 to 64 sequences.
+// Measured at the Qwen3-8B shapes.  Up to 512 rows (much of the time still goes to reading W, and there is
+// little scratch traffic): about 384 workgroups, whatever the number of tiles, was the best of 256 to 2,048
+// in decode steps of 17 to 64 sequences and in prompts of 128 to 512 tokens (512 tokens, per layer: o 70 ->
+// 40 us, down 250 -> 82 us).  Beyond that the cut pays up to half a tile per compute unit and no longer at
+// one; one workgroup per compute unit is then enough (more parts only add scratch traffic) unless a part
+// would still be longer than 64 slices.
+#define TILED_FEW_ROWS 512
+#define TILED_FEW_ROWS_WORKGROUPS 384
 #define TILED_FEW_TILES 128
-#define TILED_SHORT_WORKGROUPS 384
 static void tiled_parts(int M, int N, int K, int layout, bool swiglu, int* parts, int* slices_per_part) {
   int rows, columns;
   tiled_config(M, N, swiglu, &rows, &columns);
@@ -834,8 +835,8 @@ static void tiled_parts(int M, int N, int K, int layout, bool swiglu, int* parts
   const long tiles = (long)((N + columns - 1) / columns) * ((M + rows - 1) / rows);
   const int slices = K / TK;
   int p;
-  if (rows <= 64) {
-    p = (int)((TILED_SHORT_WORKGROUPS + tiles - 1) / tiles);
+  if (M <= TILED_FEW_ROWS) {
+    p = (int)((TILED_FEW_ROWS_WORKGROUPS + tiles - 1) / tiles);
   } else {
     if (tiles > TILED_FEW_TILES) return;
     p = (int)(2 * TILED_FEW_TILES / tiles);
