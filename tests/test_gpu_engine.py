@@ -98,24 +98,28 @@ def test_batches_of_many_sequences(model_dirs, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_one_layer_of_the_qwen3_8b_sizes(tmp_path_factory, dtype):
+def test_two_layers_of_the_qwen3_8b_sizes(tmp_path_factory, dtype):
     """The layer sizes of the benchmark model (hidden 4096, 32 query and 8 kv heads of 128, feed-forward
-    12288) in one layer with a small vocabulary: the kernels at the shapes they are tuned for, whole,
-    token by token and in a batch, against the plain implementation."""
+    12288) in two layers with a small vocabulary: the kernels at the shapes they are tuned for (steps of 1,
+    9, 24, 70, 131 and 300 rows take different matrix-product kernels and tile shapes), whole, token by
+    token and in batches, against the plain implementation."""
     import beholdd
-    config = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 1, "hidden_size": 4096,
+    config = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 4096,
               "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128, "intermediate_size": 12288,
               "vocab_size": 1000, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "max_position_embeddings": 8192,
               "tie_word_embeddings": False}
-    folder = str(tmp_path_factory.mktemp("layer_8b"))
+    folder = str(tmp_path_factory.mktemp("layers_8b"))
     beholdd.write_random_model(folder, config, seed=1, dtype="bfloat16")
     cfg, weights = plain.load_plain(folder)
-    requests = schedules.random_requests(cfg.vocab, [70, 9, 131], seed=5)
+    requests = schedules.random_requests(cfg.vocab, [70, 9, 131, 300], seed=5)
     want = [plain.forward_logits(cfg, weights, r) for r in requests]
-    engine = engine_for(folder, dtype, max_tokens=1024)
+    engine = engine_for(folder, dtype, max_tokens=4096)
     check("whole", schedules.whole(engine, requests), want, TOLERANCE[dtype])
     check("last 8 one by one", schedules.tail_one_by_one(engine, requests, tail=8), want, TOLERANCE[dtype])
-    check("batch", schedules.batches(engine, requests, batch_size=3, prompt_fraction=0.9), want, TOLERANCE[dtype])
+    check("batch", schedules.batches(engine, requests[:3], batch_size=3, prompt_fraction=0.9), want[:3], TOLERANCE[dtype])
+    many = schedules.random_requests(cfg.vocab, [3 + i % 9 for i in range(24)], seed=6)
+    want_many = [plain.forward_logits(cfg, weights, r) for r in many]
+    check("24 together", schedules.batches(engine, many, batch_size=24, prompt_fraction=0.5), want_many, TOLERANCE[dtype])
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
