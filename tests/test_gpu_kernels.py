@@ -434,14 +434,17 @@ def attention_reference_rows(q, keys, values, positions, n_heads, kv_heads, head
 @pytest.mark.parametrize("window", [0, 100])
 @pytest.mark.parametrize("n_heads,kv_heads,head_dim", [(32, 8, 128), (8, 2, 64), (6, 1, 96), (4, 4, 256), (2, 2, 32),
                                                        (4, 2, 160)])
-def test_attention_prefill_many_columns(K, n_heads, kv_heads, head_dim, window):
+@pytest.mark.parametrize("copies", [1, 5])
+def test_attention_prefill_many_columns(K, n_heads, kv_heads, head_dim, window, copies):
     """Steps wide enough for the kernel that keeps a page in LDS for four waves with columns of their own:
-    several sequences with pasts, ends that fill neither a tile nor a workgroup, NaN beyond the last key."""
+    several sequences with pasts, ends that fill neither a tile nor a workgroup, NaN beyond the last key.
+    Five copies of the sequences make enough workgroups for two column tiles per wave, one copy runs with one."""
     dtype = torch.bfloat16
     group = n_heads // kv_heads
     longest = -(-1024 * 16 // (n_heads * 3)) + 40
-    pasts, news = [0, 70, 129], [longest, longest // 2 + 3, 65]
-    assert -(-max(news) * group // 16) * kv_heads * len(news) >= 1024      # what sends a step to that kernel
+    pasts, news = [0, 70, 129] * copies, [longest, longest // 2 + 3, 65] * copies
+    assert -(-max(news) * group // 16) * kv_heads * 3 >= 1024      # what sends a step to that kernel
+    assert (-(-max(news) * group // 128) * kv_heads * len(news) >= 512) == (copies == 5)
     lengths = [p + n for p, n in zip(pasts, news)]
     kp, vp, table, keys, values = make_cache(len(lengths), lengths, kv_heads, head_dim, dtype, seed=head_dim + n_heads)
     for s, n in enumerate(lengths):
