@@ -97,28 +97,48 @@ def test_batches_of_many_sequences(model_dirs, dtype):
     assert engine.cache.live_slots() == []
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_two_layers_of_the_qwen3_8b_sizes(tmp_path_factory, dtype):
-    """The layer sizes of the benchmark model (hidden 4096, 32 query and 8 kv heads of 128, feed-forward
-    12288) in two layers with a small vocabulary: the kernels at the shapes they are tuned for (steps of 1,
-    9, 24, 70, 131 and 300 rows take different matrix-product kernels and tile shapes), whole, token by
-    token and in batches, against the plain implementation."""
+# (layers, hidden, query heads, kv heads, feed-forward width, prompt lengths)
+LARGE_SHAPES = {"8b": (2, 4096, 32, 8, 12288, [70, 9, 131, 300]), "14b": (1, 5120, 40, 8, 17408, [70, 9, 131]),
+                "32b": (1, 5120, 64, 8, 25600, [70, 9, 131])}
+
+
+@pytest.fixture(scope="module")
+def large_expected(tmp_path_factory):
+    """Per shape: the model folder, the requests and the plain implementation's logits, made once."""
     import beholdd
-    config = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 4096,
-              "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128, "intermediate_size": 12288,
-              "vocab_size": 1000, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "max_position_embeddings": 8192,
-              "tie_word_embeddings": False}
-    folder = str(tmp_path_factory.mktemp("layers_8b"))
-    beholdd.write_random_model(folder, config, seed=1, dtype="bfloat16")
-    cfg, weights = plain.load_plain(folder)
-    requests = schedules.random_requests(cfg.vocab, [70, 9, 131, 300], seed=5)
-    want = [plain.forward_logits(cfg, weights, r) for r in requests]
+    cache = {}
+
+    def get(shape):
+        if shape not in cache:
+            layers, hidden, heads, kv_heads, intermediate, lengths = LARGE_SHAPES[shape]
+            config = {"architectures": ["Qwen3ForCausalLM"], "num_hidden_layers": layers, "hidden_size": hidden,
+                      "num_attention_heads": heads, "num_key_value_heads": kv_heads, "head_dim": 128,
+                      "intermediate_size": intermediate, "vocab_size": 1000, "rope_theta": 1000000.0,
+                      "rms_norm_eps": 1e-6, "max_position_embeddings": 8192, "tie_word_embeddings": False}
+            folder = str(tmp_path_factory.mktemp(f"layers_{shape}"))
+            beholdd.write_random_model(folder, config, seed=1, dtype="bfloat16")
+            cfg, weights = plain.load_plain(folder)
+            requests = schedules.random_requests(cfg.vocab, lengths, seed=5)
+            many = schedules.random_requests(cfg.vocab, [3 + i % 9 for i in range(24)], seed=6)
+            cache[shape] = (folder, requests, [plain.forward_logits(cfg, weights, r) for r in requests],
+                            many, [plain.forward_logits(cfg, weights, r) for r in many])
+        return cache[shape]
+
+    return get
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", ["8b", "14b", "32b"])
+def test_layers_of_the_large_models_sizes(large_expected, shape, dtype):
+    """The layer sizes of Qwen3-8B, 14B and 32B (five and eight query heads per kv head, heads that do not
+    add up to the width) in one or two layers with a small vocabulary: the kernels at the shapes they are
+    tuned for (steps of 1, 9, 24, 70, 131 and 300 rows take different matrix-product kernels and tile
+    shapes), whole, token by token and in batches, against the plain implementation."""
+    folder, requests, want, many, want_many = large_expected(shape)
     engine = engine_for(folder, dtype, max_tokens=4096)
     check("whole", schedules.whole(engine, requests), want, TOLERANCE[dtype])
     check("last 8 one by one", schedules.tail_one_by_one(engine, requests, tail=8), want, TOLERANCE[dtype])
     check("batch", schedules.batches(engine, requests[:3], batch_size=3, prompt_fraction=0.9), want[:3], TOLERANCE[dtype])
-    many = schedules.random_requests(cfg.vocab, [3 + i % 9 for i in range(24)], seed=6)
-    want_many = [plain.forward_logits(cfg, weights, r) for r in many]
     check("24 together", schedules.batches(engine, many, batch_size=24, prompt_fraction=0.5), want_many, TOLERANCE[dtype])
 
 
