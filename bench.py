@@ -1,6 +1,6 @@
 """Decode and prefill throughput of the Qwen3-8B shape with random bfloat16 weights on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C] [--shape 8b|14b|32b]
 
 A step is one decode step of the batch: every live sequence's next token through the whole
 model, logits of each and a greedy choice.  The sequences' caches are filled with random keys
@@ -28,12 +28,19 @@ QWEN3_8B = {
 }
 
 
+# The other shapes of the family, for measurements beside the default one (--shape).
+QWEN3_14B = dict(QWEN3_8B, num_hidden_layers=40, hidden_size=5120, num_attention_heads=40, intermediate_size=17408)
+QWEN3_32B = dict(QWEN3_8B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, intermediate_size=25600)
+SHAPES = {"8b": ("Qwen3-8B shape", QWEN3_8B), "14b": ("Qwen3-14B shape", QWEN3_14B), "32b": ("Qwen3-32B shape", QWEN3_32B)}
+
+
 def parse():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=32)
     parser.add_argument("--warmup", type=int, default=4)
-    parser.add_argument("--layers", type=int, default=QWEN3_8B["num_hidden_layers"])
+    parser.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes; the default is the benchmark's")
+    parser.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has")
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--context", type=int, default=8192)
     parser.add_argument("--prefill-tokens", type=int, default=2048)
@@ -124,7 +131,8 @@ def main():
     import beholdd
     from beholdd.engine import Engine, random_model_on_device
 
-    config = dict(QWEN3_8B, num_hidden_layers=args.layers)
+    shape_name, shape = SHAPES[args.shape]
+    config = dict(shape, num_hidden_layers=args.layers or shape["num_hidden_layers"])
     device = "cuda:0"
     dtype_tag = "bf16" if args.dtype == "bfloat16" else "fp32"
     element = 2 if args.dtype == "bfloat16" else 4
@@ -158,12 +166,12 @@ def main():
             points[f"decode_b{batch}"] = round(batch / s, 2)
 
     line = {
-        "metric": "decode tok/s @ batch 8 (Qwen3-8B shape, context 8192)", "value": round(value, 2), "unit": "tok/s",
+        "metric": f"decode tok/s @ batch {args.batch} ({shape_name}, context {args.context})", "value": round(value, 2), "unit": "tok/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(seconds * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype_tag,
         "data": "synthetic: seeded random weights, random token ids, caches filled with random keys and values",
         "config": {
-            "model": "Qwen3-8B shape", "layers": cfg.n_layers, "layers_of_full_model": QWEN3_8B["num_hidden_layers"],
+            "model": shape_name, "layers": cfg.n_layers, "layers_of_full_model": shape["num_hidden_layers"],
             "hidden_size": cfg.hidden, "num_attention_heads": cfg.n_heads, "num_key_value_heads": cfg.n_kv_heads,
             "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate, "vocab_size": cfg.vocab,
             "rope_theta": cfg.rope_theta, "rms_norm_eps": cfg.rms_eps, "tie_word_embeddings": cfg.tie_word_embeddings,
