@@ -5,8 +5,8 @@
 // the other way round.  A workgroup takes 64 * CTW columns of one (sequence, kv head); each of its
 // four waves owns CTW tiles of 16 columns for the whole kernel (its queries, running maximum and sum,
 // output accumulators), and all four walk over the same cache pages.  A page's keys and values are
-// brought into LDS once per workgroup (through registers, the next page while the current one is
-// multiplied) and every wave reads its matrix-core operands from there: the cache keeps a page in
+// brought into LDS once per workgroup (by loads that write LDS directly, the next page while the current
+// one is multiplied) and every wave reads its matrix-core operands from there: the cache keeps a page in
 // 16-byte pieces in exactly the order the lanes take them (BH_KV_PIECES), so the copy is linear and
 // the LDS reads are conflict-free.  Nothing is merged at the end, a wave holds accumulators for its
 // own columns only, and two workgroups fit a compute unit at head size 128.
@@ -16,8 +16,8 @@
 //     online softmax per column in float32, exponent base 2
 //     O^T[d, column] += V^T[d, key] . P^T[key, column]
 // A wave skips pages none of whose keys any of its columns may see.  Values beyond the last position
-// of the workgroup's columns are zeroed on their way into LDS (their probabilities are zero, but what
-// lies there may be anything).
+// of the workgroup's columns are zeroed in LDS before the last page is used (their probabilities are
+// zero, but what lies there may be anything).
 #include "attention_bf16.h"
 
 template <int NS, int CTW>
@@ -100,37 +100,40 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
     for (int dt = 0; dt < 2 * NS; ++dt) o[ct][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 
-  // global -> registers -> LDS, piece by piece: thread `tid` copies pieces tid, tid + 256, ... of the
-  // page's keys and then of its values
-  u32x4_t stage[STAGE];
-  auto fetch = [&](int p) {
+  // global -> LDS directly (16-byte loads that write LDS at the wave's base + 16 * lane), piece by piece:
+  // thread `tid` brings pieces tid, tid + 256, ... of the page's keys and then of its values, which is their
+  // order in LDS too.  The loads are waited for (vmcnt) before the barrier that hands the page over.
+  auto fetch = [&](int p, int buffer) {
     const int page = table[p];
     const uint16_t* kb = k_pages + ((size_t)page * KVH + kvh) * BH_PAGE * HD;
     const uint16_t* vb = v_pages + ((size_t)page * KVH + kvh) * HD * BH_PAGE;
 #pragma unroll
     for (int i = 0; i < STAGE; ++i) {
       const int piece = tid + i * 256;
-      stage[i] = load16(piece < PIECES ? kb + (size_t)piece * 8 : vb + (size_t)(piece - PIECES) * 8);
+      const uint16_t* src = piece < PIECES ? kb + (size_t)piece * 8 : vb + (size_t)(piece - PIECES) * 8;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)&page_lds[buffer][i * 256 + wave * 64],
+                                       16, 0, 0);
     }
   };
-  auto stash = [&](int p, int buffer) {
-    const bool tail = p * BH_PAGE + BH_PAGE - 1 > group_pos_max;   // the page's tail was never written
+  // The last page's tail was never written: what lies there may be anything, and although its probabilities
+  // are zero its values must be too.  Once the page is in LDS, every thread clears that part of its pieces.
+  auto clear_tail = [&](int p, int buffer) {
+    if (p * BH_PAGE + BH_PAGE - 1 <= group_pos_max) return;   // the same for the whole workgroup
 #pragma unroll
     for (int i = 0; i < STAGE; ++i) {
       const int piece = tid + i * 256;
-      u32x4_t v = stage[i];
-      if (tail && piece >= PIECES) {
-        // value piece (dt * 2 + u) * 64 + l holds tokens 32 u + 8 (l / 16) .. + 7 of the page
-        const int pv = piece - PIECES;
-        const int first_token = p * BH_PAGE + 32 * ((pv / 64) % 2) + 8 * ((pv % 64) / 16);
-        v = keep_first(v, group_pos_max + 1 - first_token);
-      }
-      page_lds[buffer][piece] = v;
+      if (piece < PIECES) continue;
+      // value piece (dt * 2 + u) * 64 + l holds tokens 32 u + 8 (l / 16) .. + 7 of the page
+      const int pv = piece - PIECES;
+      const int first_token = p * BH_PAGE + 32 * ((pv / 64) % 2) + 8 * ((pv % 64) / 16);
+      page_lds[buffer][piece] = keep_first(page_lds[buffer][piece], group_pos_max + 1 - first_token);
     }
+    __syncthreads();
   };
 
-  fetch(begin);
-  stash(begin, 0);
+  fetch(begin, 0);
+  __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   auto attend = [&](int p, int buffer) {
     const u32x4_t* kl = page_lds[buffer];
@@ -218,12 +221,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
   // interleave the next page's loads and staging writes with this page's arithmetic
   for (int p = begin; p < last; ++p) {
     const int buffer = (p - begin) & 1;
-    fetch(p + 1);
-    __builtin_amdgcn_sched_barrier(0);   // the loads go out first
+    fetch(p + 1, buffer ^ 1);   // everyone was done with that buffer at the last barrier
     attend(p, buffer);
-    stash(p + 1, buffer ^ 1);
+    __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();   // the next page is in place, and everyone is done with the one before it
   }
+  clear_tail(last, (last - begin) & 1);
   attend(last, (last - begin) & 1);
 
   // lane (j, g) holds O^T[16 dt + 4 g + r, column j] and its share of the column's sum
