@@ -46,6 +46,8 @@ def parse():
     parser.add_argument("--prefill-tokens", type=int, default=2048)
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
+    parser.add_argument("--hbm-ceiling", action="store_true",
+                        help="measure what a plain streaming read and a copy of 8 GB reach on this GPU, print it and exit")
     return parser.parse_args()
 
 
@@ -121,12 +123,32 @@ def prefill_run(engine, n_tokens, torch, repeats=3):
     return min(times[1:])
 
 
+def hbm_ceiling(torch):
+    """What library kernels that only stream memory reach here: a sum over 8 GB (read) and a copy of 8 GB
+    (read + write).  Not part of the product path; a yardstick for the roofline fractions."""
+    x = torch.empty(2 << 30, dtype=torch.float32, device="cuda:0").normal_()
+    y = torch.empty_like(x)
+    out = {}
+    for name, run, moved in (("read", lambda: x.sum(), x.numel() * 4), ("copy", lambda: y.copy_(x), 2 * x.numel() * 4)):
+        run()
+        torch.cuda.synchronize()
+        begin = time.perf_counter()
+        for _ in range(10):
+            run()
+        torch.cuda.synchronize()
+        out[f"hbm_{name}_GBs"] = round(moved * 10 / (time.perf_counter() - begin) / 1e9, 1)
+    return out
+
+
 def main():
     args = parse()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU library")
         return 2
     import torch
+    if args.hbm_ceiling:
+        print(json.dumps(hbm_ceiling(torch)))
+        return 0
 
     import beholdd
     from beholdd.engine import Engine, random_model_on_device
