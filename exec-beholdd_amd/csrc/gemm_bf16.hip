@@ -30,6 +30,7 @@
 //             rows 8*(i/4) + 4*(l/32) + i%4 for i = 0..15
 // Which 8 of the k values a lane group multiplies is free as long as both operands agree.
 #include "common.h"
+#include "gemm_bf16_turns.h"
 #include <algorithm>
 #include <type_traits>
 
@@ -908,6 +909,7 @@ extern "C" int bh_gemm_bf16_takes_norm(int M, int N, int K, int layout, int acti
 // Bytes of scratch memory that bh_gemm_bf16 wants for this product (0: none).
 extern "C" long bh_gemm_bf16_scratch(int M, int N, int K, int layout, int activation) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
+  if (gemm_turns_blocks(M, N, K, layout, activation)) return 0;
   int parts, each;
   tiled_parts(M, N, K, layout, activation != 0, &parts, &each);
   return parts == 1 ? 0 : (long)parts * M * (activation ? 2 * N : N) * (long)sizeof(float);
@@ -941,6 +943,10 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
   const RidingNorm norm = {ahead_ss, ahead_blocks, ahead_eps, behind_weight, behind_weight_dtype == BH_F32,
                            (uint16_t*)behind_rows, behind_ss};
   const bool f32 = c_dtype == BH_F32;
+  if (!ahead_ss && !behind_weight && (f32 || !accumulate)) {   // many rows: the kernel whose wave groups take turns
+    if (const int blocks = gemm_turns_blocks(M, N, K, layout, activation))
+      return gemm_turns_launch(a, w, c, c_dtype, accumulate, M, N, K, activation, blocks, stream);
+  }
 #define BH_PICK(FN, TILES, EXTRA, ...)                                             \
   do {                                                                              \
     if (f32) FN<TILES, EXTRA, float>(__VA_ARGS__);                                  \

@@ -95,6 +95,7 @@ class HipKernels:
             "bh_sample": [p, p, p, p, p, p, p, p, i, i, p],
             "bh_sample_scratch": [i, i],
             "bh_gemm_bf16": [p, p, p, i, i, i, i, i, i, i, p, i, f, p, i, p, p, p, p],
+            "bh_gemm_bf16_turns": [p, p, p, i, i, i, i, i, i, i, p],
             "bh_attention_bf16": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, i, i, f, i, i, i, p],
             "bh_attention_bf16_splits": [i, i, i, i, i],
             "bh_attention_decode_fused": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, f, i, i, i, p, p, i, f, p, p, i, i,
@@ -107,7 +108,7 @@ class HipKernels:
             function.restype = i
         lib.bh_gemm_bf16_scratch.argtypes = [i, i, i, i, i]
         lib.bh_gemm_bf16_scratch.restype = ctypes.c_long
-        for query in (lib.bh_gemm_bf16_norm_blocks, lib.bh_gemm_bf16_takes_norm):
+        for query in (lib.bh_gemm_bf16_norm_blocks, lib.bh_gemm_bf16_takes_norm, lib.bh_gemm_bf16_turns_blocks):
             query.argtypes, query.restype = [i, i, i, i, i], ctypes.c_int
     # ---- helpers ----
     def _stream(self):
@@ -240,6 +241,24 @@ class HipKernels:
             self._ptr(a, "gemm a"), _code(a, "gemm a"), self._ptr(w, "gemm w"), _code(w, "gemm w"),
             self._ptr(out, "gemm out"), _code(out, "gemm out"), int(bool(accumulate)), m, n, k, self._stream()))
         return None
+
+    def gemm_turns(self, a, w, out, blocks, accumulate=False, swiglu=False):
+        """The product for many rows whose wave groups take turns, at a given tile width (`blocks` of 16
+        weight rows per wave: 8, 6 or 4), whatever `gemm` would choose for these sizes: out[M, N] (+)= a @ w^T,
+        or with `swiglu` out[M, F] = silu(a @ w[:F]^T) * (a @ w[F:]^T).  `w` is a PackedWeight."""
+        if not isinstance(w, PackedWeight) or a.dim() != 2 or out.dim() != 2 or a.dtype != torch.bfloat16:
+            raise KernelError("gemm_turns: bfloat16 activations [M, K] and a packed weight")
+        m, k = a.shape
+        n = out.shape[1]
+        if w.shape[1] != k or w.shape[0] != (2 * n if swiglu else n) or out.shape[0] != m:
+            raise KernelError(f"gemm_turns: shapes a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
+        self._check(self.lib.bh_gemm_bf16_turns(
+            self._ptr(a, "gemm a"), self._ptr(w.data, "gemm w"), self._ptr(out, "gemm out"), _code(out, "gemm out"),
+            int(bool(accumulate)), m, n, k, int(bool(swiglu)), int(blocks), self._stream()))
+
+    def gemm_turns_blocks(self, m, n, k, swiglu=False):
+        """The tile width `gemm` uses for a packed product of these sizes (0: another kernel runs it)."""
+        return int(self.lib.bh_gemm_bf16_turns_blocks(m, n, k, 1, int(bool(swiglu))))
 
     def _takes_norm(self, a, w, n, activation):
         """Whether the matrix-core product of these operands applies the row factors of prepared norm rows."""

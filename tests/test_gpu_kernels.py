@@ -225,6 +225,82 @@ def test_norm_does_not_ride_on_wide_steps(K):
     assert rel(residual, a.double() @ w.double().t()) < 1e-5
 
 
+@pytest.mark.parametrize("blocks", [8, 6, 4])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (300, 400, 384), (520, 1040, 256), (257, 272, 1152),
+                                   (1024, 768, 2048)])
+def test_gemm_whose_wave_groups_take_turns(K, blocks, m, n, k):
+    """The product for many rows at each of its tile widths: whole tiles, tiles moved back inside at both
+    edges, one and many k steps; float32 with and without accumulation, bfloat16, SwiGLU."""
+    g = torch.Generator().manual_seed(m + n + blocks)
+    a = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(2 * n, k, generator=g) * 0.05).to(torch.bfloat16)
+    plain, both = K.pack_weight(dev(w[:n].contiguous())), K.pack_weight(dev(w))
+    want = a.double() @ w[:n].double().t()
+    f32_bound = 4 * math.sqrt(k) * 2.0 ** -24
+    out = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
+    K.gemm_turns(dev(a), plain, out, blocks)
+    assert rel(out, want) < f32_bound, rel(out, want)
+    base = torch.randn(m, n, generator=g)
+    acc = dev(base.clone())
+    K.gemm_turns(dev(a), plain, acc, blocks, accumulate=True)
+    assert rel(acc, want + base.double()) < f32_bound
+    out16 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda:0")
+    K.gemm_turns(dev(a), plain, out16, blocks)
+    assert rel(out16, want) < 4e-3, rel(out16, want)
+    if n >= 16 * blocks:
+        up = a.double() @ w[n:].double().t()
+        want_act = want / (1 + torch.exp(-want)) * up
+        act = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda:0")
+        K.gemm_turns(dev(a), both, act, blocks, swiglu=True)
+        assert rel(act, want_act) < 6e-3, rel(act, want_act)
+
+
+def test_gemm_with_turns_refuses_what_it_cannot_do(K):
+    from beholdd.kernels import KernelError
+    a = dev(torch.zeros(256, 192, dtype=torch.bfloat16))
+    w = K.pack_weight(dev(torch.zeros(256, 192, dtype=torch.bfloat16)))
+    out = torch.empty(256, 256, dtype=torch.float32, device="cuda:0")
+    with pytest.raises(KernelError, match="multiple of 128"):
+        K.gemm_turns(a, w, out, 8)                                     # K = 192
+    a, w = dev(torch.zeros(200, 256, dtype=torch.bfloat16)), K.pack_weight(dev(torch.zeros(256, 256, dtype=torch.bfloat16)))
+    with pytest.raises(KernelError, match="M >= 256"):
+        K.gemm_turns(a, w, torch.empty(200, 256, dtype=torch.float32, device="cuda:0"), 8)
+    a = dev(torch.zeros(256, 256, dtype=torch.bfloat16))
+    with pytest.raises(KernelError, match="blocks per wave"):
+        K.gemm_turns(a, w, out, 5)
+    with pytest.raises(KernelError, match="bfloat16 without accumulation"):
+        K.gemm_turns(a, w, torch.empty(256, 256, dtype=torch.bfloat16, device="cuda:0"), 8, accumulate=True)
+
+
+@pytest.mark.parametrize("m,n,k,swiglu,blocks", [(2048, 6144, 256, False, 6), (2048, 12288, 128, True, 8),
+                                                 (2048, 4096, 256, False, 4), (4000, 4096, 128, False, 8),
+                                                 (500, 12288, 128, True, 6), (300, 4096, 128, False, 0),
+                                                 (256, 12288, 128, True, 0), (2048, 4096, 12288, False, 0)])
+def test_gemm_chooses_the_turns_kernel_where_it_fills_the_chip(K, m, n, k, swiglu, blocks):
+    """Which products go to the kernel whose wave groups take turns, and that `gemm` gives the right result there."""
+    assert K.gemm_turns_blocks(m, n, k, swiglu) == blocks
+    if k > 1024:
+        return
+    g = torch.Generator().manual_seed(m + n)
+    a = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(2 * n if swiglu else n, k, generator=g) * 0.05).to(torch.bfloat16)
+    packed = K.pack_weight(dev(w))
+    if swiglu:
+        gate, up = a.double() @ w[:n].double().t(), a.double() @ w[n:].double().t()
+        out = torch.empty(m, n, dtype=torch.bfloat16, device="cuda:0")
+        K.gemm_swiglu(dev(a), packed, out)
+        assert rel(out, gate / (1 + torch.exp(-gate)) * up) < 6e-3
+    else:
+        want = a.double() @ w.double().t()
+        base = torch.randn(m, n, generator=g)
+        acc = dev(base.clone())
+        K.gemm(dev(a), packed, acc, accumulate=True)
+        assert rel(acc, want + base.double()) < 4 * math.sqrt(k) * 2.0 ** -24
+        out = torch.empty(m, n, dtype=torch.bfloat16, device="cuda:0")
+        K.gemm(dev(a), packed, out)
+        assert rel(out, want) < 4e-3
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("m,width,k", [(1, 16, 64), (8, 160, 128), (40, 896, 320), (64, 48, 192), (65, 64, 64),
