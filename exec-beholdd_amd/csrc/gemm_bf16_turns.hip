@@ -6,17 +6,31 @@
 // in registers), the other reads its next operands from LDS and asks for data that is three steps ahead; a
 // barrier ends every turn.  So the matrix cores always have one wave per SIMD that does nothing but multiply,
 // and no wave waits for memory in the middle of its multiplies.  A step is half a 64-wide k slice: the 32 k
-// values that one 16x16x32 MFMA takes, in the order in which the tiles layout holds them.
+// values that one 16x16x32 MFMA takes.
 //
 // Global memory goes to LDS directly (16-byte loads that write LDS at the wave's base + 16 * lane): 1 KB per
 // load, which is one operand of 16 rows x 32 k in lane order, so that reading it back is one conflict-free
-// 16-byte read per lane.  W's tiles layout already is that order (contiguous 1 KB loads); for A a lane loads
-// its 16 bytes from its row.  LDS holds four steps (4 x (16 + 2 YB) KB); a step's region is loaded again as
-// soon as both groups have read it, which is five to six turns before it is read next: time enough for
-// loads that miss every cache.
+// 16-byte read per lane.  Four lanes bring 64 consecutive bytes of a row of A, or 256 bytes of a block of W.
+// LDS holds four steps (4 x (16 + 2 YB) KB); a step's region is loaded again as soon as both groups have read
+// it, which is five to six turns before it is read next.
 //
-// Measured at the Qwen3-8B shapes, 2,048 rows: gate/up with SwiGLU 404 -> 330 us (1.25 PFLOP/s), qkv
-// 132 -> 104 us with tiles of 192 weight rows (256 of them, one per compute unit), o 102 -> 83 us with 128.
+// Measured at the Qwen3-8B shapes, 2,048 rows, each product alone: gate/up with SwiGLU 404 -> 330 us
+// (1.25 PFLOP/s), qkv 132 -> 104 us with tiles of 192 weight rows (256 of them, one per compute unit), o 102 ->
+// 84 us with 128; in the whole model 381 -> 338, 115 -> 101 and 87 -> 94 us (o is kept: with the tile order
+// below the whole prefill is the faster for it).
+// What bounds it: the loads alone (no multiplies) take 0.9 of the whole kernel's time, the multiplies alone
+// 0.6.  It is not the loads' latency (five or six steps in LDS instead of four changed nothing; touching the
+// lines three slices ahead with 4-byte loads made it slower, 0.9 PFLOP/s for gate/up: loads retire in order, so
+// the loads for LDS waited behind the touches), not LDS (a compute unit reads 256 bytes per clock from it and
+// needs a third of that) and not memory beyond L2 (87 % of the L2 requests hit; 0.3 to 0.6 GB come from beyond
+// it).  The 32 compute units of an XCD ask its L2 for 1 MB per step, which at the matrix cores' full speed
+// would be all that its 16 channels of 64 bytes per clock can give; a compute unit alone gets at most about
+// 43 bytes per clock out of L1 and L2 (loads only, to LDS or to registers alike), and a tile of 256 x 128 asks
+// for 47 where 256 x 256 asks for 32, which is why the narrower tiles lose.
+// Tried for the products with 4,096 weight rows, which have only 128 tiles of 256 x 256: a tile of 256 x 128
+// in which the two groups divide the k steps between them (every wave 64 x 128, sums exchanged through LDS at
+// the end) ran like the 128-wide tile (0.8 PFLOP/s); A brought in whole 128-byte lines and kept permuted in
+// LDS was slower (its slice buffer is free only four turns before it is read again).
 #include "gemm_bf16_turns.h"
 #include <type_traits>
 
@@ -42,6 +56,18 @@ __device__ inline float silu_mul(float gate, float up) { return gate / (1.0f + e
     __builtin_amdgcn_sched_barrier(0);    \
   } while (0)
 
+// Which tile a workgroup takes.  Workgroups go to the eight XCDs in turn (workgroup i to XCD i % 8), and each
+// XCD has an L2 of its own: neighbours in the order below are workgroups of one XCD, and they take the
+// row tiles of one weight tile one after the other, so that an XCD fetches a weight tile once for all of
+// them and the rows' slices while they are recent (measured: L2 delivers 26 TB/s to the compute units,
+// what lies beyond it 7).  Only speed depends on where the workgroups really run.
+__device__ inline void tile_of_workgroup(int n_tiles, int m_tiles, int* tile_n, int* tile_m) {
+  const int total = n_tiles * m_tiles, xcd = blockIdx.x % 8, each = total / 8, more = total % 8;
+  const int v = xcd * each + min(xcd, more) + blockIdx.x / 8;
+  *tile_n = v / m_tiles;
+  *tile_m = v % m_tiles;
+}
+
 // MODE 0: bfloat16 output.  1: float32 output, optionally added to what is there.  2: SwiGLU, bfloat16 output
 // (N outputs; W has 2 N rows, gate rows then up rows; a wave's weight rows are the gate and the up rows of
 // the same outputs).  YB: blocks of 16 weight rows per wave.
@@ -52,38 +78,43 @@ __global__ __launch_bounds__(512) void gemm_turns_kernel(const uint16_t* __restr
   constexpr int OUTS = MODE == 2 ? 16 * YB : 32 * YB;
   constexpr int CHUNKS = 16 + 2 * YB;
   constexpr int WL = YB / 2;   // W chunks per loading wave
-  __shared__ __attribute__((aligned(16))) u32x4_t lds[4][CHUNKS][64];   // [region][16 A blocks, then 2 YB W blocks][lane]
+  constexpr int R = 4;                 // steps that LDS holds (with five or six of them it ran no faster)
+  __shared__ __attribute__((aligned(16))) u32x4_t lds[R * CHUNKS * 64];   // [region][16 A blocks, then 2 YB W blocks][lane]
   const int tid = threadIdx.x, lane = tid % 64;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const int g = wave / 4, i4 = wave % 4;
-  const int n_tiles = (N + OUTS - 1) / OUTS;
-  const int tile_n = blockIdx.x % n_tiles, tile_m = blockIdx.x / n_tiles;
+  int tile_n, tile_m;
+  tile_of_workgroup((N + OUTS - 1) / OUTS, (M + 255) / 256, &tile_n, &tile_m);
   const int m_own = tile_m * 256, n_own = tile_n * OUTS;
   const int m0 = min(m_own, M - 256), n0 = min(n_own, N - OUTS);
   const int J = K / 32;   // half slices; K % 128 == 0
 
   // The first group brings A (four blocks of 16 rows per wave), the second W (YB / 2 blocks per wave).
-  const uint16_t* a_src = a + (size_t)(m0 + 64 * i4 + lane % 16) * K + 16 * (lane / 16);
+  // A step takes 32 consecutive k: lane (row r = lane % 16, group q = lane / 16) holds k 8 q .. 8 q + 7 of them,
+  // so four lanes bring 64 consecutive bytes of a row.  In W's tiles layout those are the 16-byte pieces
+  // 4 v + q of the row (v: first or second step of the slice), piece p at half p % 2, lane 16 (p / 2) + r.
+  const uint16_t* a_src = a + (size_t)(m0 + 64 * i4 + lane % 16) * K + 8 * (lane / 16);
+  const int w_lane = ((lane / 16) % 2) * 512 + (16 * (lane / 32) + lane % 16) * 8;   // + 256 elements for the second step
   const uint16_t* w_src[WL];
 #pragma unroll
   for (int b = 0; b < WL; ++b) {
     const int rb = i4 * WL + b, gg = rb / YB, y = rb % YB;
     const int nb = MODE == 2 ? (y < YB / 2 ? 0 : N / 16) + n0 / 16 + (YB / 2) * gg + y % (YB / 2) : n0 / 16 + rb;
-    w_src[b] = w + (size_t)nb * (K / 64) * 1024 + lane * 8;
+    w_src[b] = w + (size_t)nb * (K / 64) * 1024 + w_lane;
   }
-  auto fetch_a = [&](int j, int region) {
+  auto fetch_a = [&](int j, int region) {   // step j = half u of slice s
     const int s = j >> 1, u = j & 1;
 #pragma unroll
     for (int b = 0; b < 4; ++b)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_src + (size_t)b * 16 * K + s * 64 + u * 8),
-                                       (__attribute__((address_space(3))) void*)&lds[region][4 * i4 + b][0], 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_src + (size_t)b * 16 * K + s * 64 + u * 32),
+                                       (__attribute__((address_space(3))) void*)&lds[(region * CHUNKS + 4 * i4 + b) * 64], 16, 0, 0);
   };
   auto fetch_w = [&](int j, int region) {
     const int s = j >> 1, u = j & 1;
 #pragma unroll
     for (int b = 0; b < WL; ++b)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(w_src[b] + (size_t)s * 1024 + u * 512),
-                                       (__attribute__((address_space(3))) void*)&lds[region][16 + i4 * WL + b][0], 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(w_src[b] + (size_t)s * 1024 + u * 256),
+                                       (__attribute__((address_space(3))) void*)&lds[(region * CHUNKS + 16 + i4 * WL + b) * 64], 16, 0, 0);
   };
 
   f32x4_t acc[4][YB];
@@ -95,9 +126,9 @@ __global__ __launch_bounds__(512) void gemm_turns_kernel(const uint16_t* __restr
 
   auto read_operands = [&](int region) {
 #pragma unroll
-    for (int x = 0; x < 4; ++x) af[x] = lds[region][4 * i4 + x][lane];
+    for (int x = 0; x < 4; ++x) af[x] = lds[(region * CHUNKS + 4 * i4 + x) * 64 + lane];
 #pragma unroll
-    for (int y = 0; y < YB; ++y) wf[y] = lds[region][16 + YB * g + y][lane];
+    for (int y = 0; y < YB; ++y) wf[y] = lds[(region * CHUNKS + 16 + YB * g + y) * 64 + lane];
   };
   auto multiply = [&]() {
     __builtin_amdgcn_s_setprio(1);
@@ -109,56 +140,56 @@ __global__ __launch_bounds__(512) void gemm_turns_kernel(const uint16_t* __restr
     __builtin_amdgcn_s_setprio(0);
   };
 
+  // Step j lies in region j % R.  A wave asks for step j + R - 1 while it reads step j (into the region that
+  // step j - 1 has left); before the turn in which the first group reads step j + 1, all that was asked for
+  // it must have landed: what may still be on its way are the loads of the steps after it.
+  auto wait_for_next = [&](int j, int per_step, bool with_lds) {   // per_step: this wave's loads per step
+    const int later = min(R - 2, J - 2 - j);   // steps after j + 1 that have been asked for
+    (void)with_lds;
+    if (per_step == 4) {
+      if (later >= 4) WAIT_VM_LGKM0(16); else if (later == 3) WAIT_VM_LGKM0(12); else if (later == 2) WAIT_VM_LGKM0(8);
+      else if (later == 1) WAIT_VM_LGKM0(4); else WAIT_VM_LGKM0(0);
+    } else if (per_step == 3) {
+      if (later >= 4) WAIT_VM_LGKM0(12); else if (later == 3) WAIT_VM_LGKM0(9); else if (later == 2) WAIT_VM_LGKM0(6);
+      else if (later == 1) WAIT_VM_LGKM0(3); else WAIT_VM_LGKM0(0);
+    } else {
+      if (later >= 4) WAIT_VM_LGKM0(8); else if (later == 3) WAIT_VM_LGKM0(6); else if (later == 2) WAIT_VM_LGKM0(4);
+      else if (later == 1) WAIT_VM_LGKM0(2); else WAIT_VM_LGKM0(0);
+    }
+  };
+  static_assert(R - 2 <= 4, "wait_for_next knows up to four steps on their way after the next");
   if (g == 0) {
-    fetch_a(0, 0); fetch_a(1, 1); fetch_a(2, 2);
+    for (int j = 0; j < R - 1 && j < J; ++j) fetch_a(j, j);
     WAIT_VM_LGKM0(0);
     TICK();
-    auto step = [&](auto fetch, auto pending, int j, int region) {
-      if (fetch.value) fetch_a(j + 3, (region + 3) % 4);
+    int region = 0;
+    for (int j = 0; j < J; ++j) {
+      if (j + R - 1 < J) fetch_a(j + R - 1, region == 0 ? R - 1 : region - 1);
       read_operands(region);
       WAIT_LGKM0();
       TICK();
       multiply();
-      // half slice j + 1 must have landed before the next tick, in which this group reads it
-      WAIT_VM_LGKM0(4 * pending.value);
+      wait_for_next(j, 4, false);
       TICK();
-    };
-    using std::integral_constant;
-    typedef integral_constant<bool, true> yes;
-    typedef integral_constant<bool, false> no;
-    int j = 0;
-    for (; j + 4 < J; j += 4) {
-      step(yes(), integral_constant<int, 2>(), j, 0); step(yes(), integral_constant<int, 2>(), j + 1, 1);
-      step(yes(), integral_constant<int, 2>(), j + 2, 2); step(yes(), integral_constant<int, 2>(), j + 3, 3);
+      region = region == R - 1 ? 0 : region + 1;
     }
-    step(yes(), integral_constant<int, 2>(), j, 0); step(no(), integral_constant<int, 1>(), j + 1, 1);
-    step(no(), integral_constant<int, 0>(), j + 2, 2); step(no(), integral_constant<int, 0>(), j + 3, 3);
     TICK();
   } else {
-    fetch_w(0, 0); fetch_w(1, 1); fetch_w(2, 2);
+    for (int j = 0; j < R - 1 && j < J; ++j) fetch_w(j, j);
     WAIT_VM_LGKM0(0);
     TICK();
     TICK();   // the second group runs one tick behind
-    auto step = [&](auto fetch, auto pending, int j, int region) {
-      if (fetch.value) fetch_w(j + 3, (region + 3) % 4);
+    int region = 0;
+    for (int j = 0; j < J; ++j) {
+      if (j + R - 1 < J) fetch_w(j + R - 1, region == 0 ? R - 1 : region - 1);
       read_operands(region);
-      WAIT_VM_LGKM0(WL * pending.value);
+      wait_for_next(j, WL, true);
       TICK();
       multiply();
       TICK();
-    };
-    using std::integral_constant;
-    typedef integral_constant<bool, true> yes;
-    typedef integral_constant<bool, false> no;
-    int j = 0;
-    for (; j + 4 < J; j += 4) {
-      step(yes(), integral_constant<int, 2>(), j, 0); step(yes(), integral_constant<int, 2>(), j + 1, 1);
-      step(yes(), integral_constant<int, 2>(), j + 2, 2); step(yes(), integral_constant<int, 2>(), j + 3, 3);
+      region = region == R - 1 ? 0 : region + 1;
     }
-    step(yes(), integral_constant<int, 2>(), j, 0); step(no(), integral_constant<int, 1>(), j + 1, 1);
-    step(no(), integral_constant<int, 0>(), j + 2, 2); step(no(), integral_constant<int, 0>(), j + 3, 3);
   }
-
   // acc[x][y][i]: row 64 i4 + 16 x + lane % 16 of the tile, weight row 16 (YB g + y) + 4 (lane / 16) + i
   const int m = m0 + 64 * i4 + lane % 16;
   if (MODE == 2) {
@@ -244,7 +275,7 @@ int gemm_turns_blocks(int M, int N, int K, int layout, int activation) {
     const long tiles = (long)((N + outs - 1) / outs) * ((M + 255) / 256);
     const long rounds = (tiles + 255) / 256;
     const double cost = blocks == 8 ? 1.0 : blocks == 6 ? 1.12 : 1.39;
-    const double rate = 1250.0 * work / ((double)rounds * 256 * 256 * 32 * blocks * cost);   // TFLOP/s, roughly
+    const double rate = 1250.0 * work / ((double)rounds * 256 * 256 * (activation ? 2 : 1) * outs * cost);   // TFLOP/s, roughly
     if (rate > best_rate) best_rate = rate, best = blocks;
   }
   const double others = K <= 8192 ? 800.0 : 950.0;
