@@ -910,6 +910,8 @@ extern "C" int bh_gemm_bf16_takes_norm(int M, int N, int K, int layout, int acti
 extern "C" long bh_gemm_bf16_scratch(int M, int N, int K, int layout, int activation) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
   if (gemm_turns_blocks(M, N, K, layout, activation)) return 0;
+  if (const int turns_parts = gemm_turns_parts(M, N, K, layout, activation); turns_parts > 1)
+    return (long)turns_parts * M * N * (long)sizeof(float);
   int parts, each;
   tiled_parts(M, N, K, layout, activation != 0, &parts, &each);
   return parts == 1 ? 0 : (long)parts * M * (activation ? 2 * N : N) * (long)sizeof(float);
@@ -959,11 +961,16 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
     BH_REQUIRE(((uintptr_t)c | (uintptr_t)scratch | (uintptr_t)behind_rows) % 16 == 0,
                "gemm_bf16: output, scratch memory and norm rows must be 16-byte aligned");
     int parts, each;
-    tiled_parts(M, N, K, layout, activation != 0, &parts, &each);
-    const RidingNorm none = {};
-    if (activation) launch_tiled<true, true, float>(a, w, nullptr, M, N, K, 0, none, (float*)scratch, stream);
-    else launch_tiled<true, false, float>(a, w, nullptr, M, N, K, 0, none, (float*)scratch, stream);
-    if (int status = bh_check_launch("gemm_tiled")) return status;
+    if (const int turns_parts = gemm_turns_parts(M, N, K, layout, activation); turns_parts > 1) {
+      parts = turns_parts;
+      if (int status = gemm_turns_launch_parts(a, w, (float*)scratch, M, N, K, parts, stream)) return status;
+    } else {
+      tiled_parts(M, N, K, layout, activation != 0, &parts, &each);
+      const RidingNorm none = {};
+      if (activation) launch_tiled<true, true, float>(a, w, nullptr, M, N, K, 0, none, (float*)scratch, stream);
+      else launch_tiled<true, false, float>(a, w, nullptr, M, N, K, 0, none, (float*)scratch, stream);
+      if (int status = bh_check_launch("gemm_tiled")) return status;
+    }
     dim3 finish_grid((N + FINISH_COLUMNS - 1) / FINISH_COLUMNS, (M + 15) / 16);
 #define BH_FINISH(SWIGLU, TC)                                                                                \
   gemm_parts_finish_kernel<SWIGLU, TC><<<finish_grid, 256, 0, stream>>>((const float*)scratch, (TC*)c, M, N, K, \

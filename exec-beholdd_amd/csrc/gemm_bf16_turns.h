@@ -10,3 +10,7 @@ bool gemm_turns_can(int M, int N, int K, int layout, int activation, int blocks)
 // c_dtype BH_F32 (accumulate allowed) or BH_BF16 (no accumulate); activation 1 = SwiGLU, bfloat16 output only.
 int gemm_turns_launch(const void* a, const void* w, void* c, int c_dtype, int accumulate, int M, int N, int K,
                       int activation, int blocks, hipStream_t stream);
+// In how many parts of K the widest tile multiplies a product that would otherwise leave compute units idle
+// (1: not this way), and that multiplication: bare sums [part][M][N] for gemm_parts_finish_kernel.
+int gemm_turns_parts(int M, int N, int K, int layout, int activation);
+int gemm_turns_launch_parts(const void* a, const void* w, float* sums, int M, int N, int K, int parts, hipStream_t stream);

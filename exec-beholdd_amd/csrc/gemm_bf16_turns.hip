@@ -87,20 +87,23 @@ __global__ __launch_bounds__(512) void gemm_turns_kernel(const uint16_t* __restr
   tile_of_workgroup((N + OUTS - 1) / OUTS, (M + 255) / 256, &tile_n, &tile_m);
   const int m_own = tile_m * 256, n_own = tile_n * OUTS;
   const int m0 = min(m_own, M - 256), n0 = min(n_own, N - OUTS);
-  const int J = K / 32;   // half slices; K % 128 == 0
+  // K in parts (blockIdx.y, MODE 1 only): part p multiplies its share of k and leaves the bare sums at
+  // c + p * M * N for the finishing kernel of gemm_bf16.hip; one part is the whole product.
+  const int k_part = K / gridDim.y, k_first = blockIdx.y * k_part;
+  const int J = k_part / 32;   // steps: half slices; k_part % 128 == 0
 
   // The first group brings A (four blocks of 16 rows per wave), the second W (YB / 2 blocks per wave).
   // A step takes 32 consecutive k: lane (row r = lane % 16, group q = lane / 16) holds k 8 q .. 8 q + 7 of them,
   // so four lanes bring 64 consecutive bytes of a row.  In W's tiles layout those are the 16-byte pieces
   // 4 v + q of the row (v: first or second step of the slice), piece p at half p % 2, lane 16 (p / 2) + r.
-  const uint16_t* a_src = a + (size_t)(m0 + 64 * i4 + lane % 16) * K + 8 * (lane / 16);
+  const uint16_t* a_src = a + (size_t)(m0 + 64 * i4 + lane % 16) * K + k_first + 8 * (lane / 16);
   const int w_lane = ((lane / 16) % 2) * 512 + (16 * (lane / 32) + lane % 16) * 8;   // + 256 elements for the second step
   const uint16_t* w_src[WL];
 #pragma unroll
   for (int b = 0; b < WL; ++b) {
     const int rb = i4 * WL + b, gg = rb / YB, y = rb % YB;
     const int nb = MODE == 2 ? (y < YB / 2 ? 0 : N / 16) + n0 / 16 + (YB / 2) * gg + y % (YB / 2) : n0 / 16 + rb;
-    w_src[b] = w + (size_t)nb * (K / 64) * 1024 + w_lane;
+    w_src[b] = w + ((size_t)nb * (K / 64) + k_first / 64) * 1024 + w_lane;
   }
   auto fetch_a = [&](int j, int region) {   // step j = half u of slice s
     const int s = j >> 1, u = j & 1;
@@ -218,7 +221,7 @@ __global__ __launch_bounds__(512) void gemm_turns_kernel(const uint16_t* __restr
         const int n = n0 + 16 * YB * g + 16 * y + 4 * (lane / 16);
         if (n < n_own) continue;
         if (MODE == 1) {
-          f32x4_t* at = reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(c) + (size_t)row * N + n);
+          f32x4_t* at = reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(c) + ((size_t)blockIdx.y * M + row) * N + n);
           f32x4_t v = acc[x][y];
           if (accumulate) v += *at;
           *at = v;
@@ -239,9 +242,10 @@ __global__ __launch_bounds__(512) void gemm_turns_kernel(const uint16_t* __restr
 #undef TICK
 
 template <int MODE>
-void launch(const void* a, const void* w, void* c, int blocks, int M, int N, int K, int accumulate, hipStream_t stream) {
+void launch(const void* a, const void* w, void* c, int blocks, int M, int N, int K, int accumulate, hipStream_t stream,
+            int parts = 1) {
   const int outs = (MODE == 2 ? 16 : 32) * blocks;
-  dim3 grid(((N + outs - 1) / outs) * ((M + 255) / 256));
+  dim3 grid(((N + outs - 1) / outs) * ((M + 255) / 256), parts);
 #define BH_TURNS(YB) \
   gemm_turns_kernel<MODE, YB><<<grid, 512, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, c, M, N, K, accumulate)
   if (blocks == 8) BH_TURNS(8);
@@ -280,6 +284,24 @@ int gemm_turns_blocks(int M, int N, int K, int layout, int activation) {
   }
   const double others = K <= 8192 ? 800.0 : 950.0;
   return best_rate >= others ? best : 0;
+}
+
+// Products with so few of the widest tiles that half the compute units would idle, and a long K: K in two
+// parts over twice the workgroups, each leaving its bare sums in scratch memory ([part][row][weight row],
+// float32) for the finishing kernel.  Measured at 2,048 rows x 4,096 weight rows x 12,288: see gemm_turns_blocks.
+int gemm_turns_parts(int M, int N, int K, int layout, int activation) {
+  if (activation || M <= 256 || K < 8192 || K % 256 || !gemm_turns_can(M, N, K, layout, 0, 8)) return 1;
+  if (gemm_turns_blocks(M, N, K, layout, 0)) return 1;   // a tile of its own fills the chip
+  const long tiles = (long)((N + 255) / 256) * ((M + 255) / 256);
+  return tiles > 64 && tiles <= 128 ? 2 : 1;
+}
+
+int gemm_turns_launch_parts(const void* a, const void* w, float* sums, int M, int N, int K, int parts, hipStream_t stream) {
+  BH_REQUIRE(parts >= 1 && K % (128 * parts) == 0 && gemm_turns_can(M, N, K / parts, 1, 0, 8),
+             "gemm_turns: M=%d N=%d K=%d cannot be multiplied in %d parts of K", M, N, K, parts);
+  BH_REQUIRE(((uintptr_t)a | (uintptr_t)w | (uintptr_t)sums) % 16 == 0, "gemm_turns: operands must be 16-byte aligned");
+  launch<1>(a, w, sums, 8, M, N, K, 0, stream, parts);
+  return bh_check_launch("gemm_turns");
 }
 
 int gemm_turns_launch(const void* a, const void* w, void* c, int c_dtype, int accumulate, int M, int N, int K,

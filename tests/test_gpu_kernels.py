@@ -102,6 +102,8 @@ def test_gemm(K, a_dtype, w_dtype, m, n, k):
                                    (2048, 4096, 512),
                                    # few whole tiles: K in parts (equal and unequal ones) and a finishing kernel
                                    (200, 320, 832), (512, 4096, 4096), (128, 128, 4096),
+                                   # many rows, few of the widest tiles, long K: K in two parts of the kernel whose wave groups take turns
+                                   (1100, 4096, 8192),
                                    # 65 to 127 rows: whole tiles of 64 rows
                                    (100, 256, 1024), (127, 4096, 512), (65, 128, 64)])
 def test_gemm_with_packed_weights(K, m, n, k):
