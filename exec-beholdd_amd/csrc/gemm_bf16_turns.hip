@@ -264,10 +264,11 @@ bool gemm_turns_can(int M, int N, int K, int layout, int activation, int blocks)
 }
 
 // Which tile, if any.  A tile of YB blocks per wave costs a compute unit YB x cost(YB) units of time, where
-// cost is what the narrower tiles lose (more LDS reads and loads per multiply: measured 1.25, 1.11 and 0.90
-// PFLOP/s for 8, 6 and 4 with the chip full), and the chip works in rounds of 256 tiles.  The estimate is
-// compared with what the other tiled kernels reach (about 0.85 PFLOP/s at their best, less for short K,
-// where their start and end of a tile weigh more).
+// cost is what the narrower tiles lose (measured 1.25, 1.11 and 0.90 PFLOP/s for 8, 6 and 4 with the chip
+// full), and the chip works in rounds of 256 tiles.  The estimate is compared with what the other ways reach
+// (the other tiled kernels about 0.85 PFLOP/s at their best; K in two parts of the widest tile, see
+// gemm_turns_parts, about 1.0: in the whole model it beat the 128-wide tile for the o projection too, prefill
+// of 2,048 tokens 31.8 -> 30.5 ms, though the two run alike alone).
 int gemm_turns_blocks(int M, int N, int K, int layout, int activation) {
   if (M <= 256) return 0;   // up to there a norm may ride on the product, which this kernel does not carry
   int best = 0;
@@ -282,18 +283,21 @@ int gemm_turns_blocks(int M, int N, int K, int layout, int activation) {
     const double rate = 1250.0 * work / ((double)rounds * 256 * 256 * (activation ? 2 : 1) * outs * cost);   // TFLOP/s, roughly
     if (rate > best_rate) best_rate = rate, best = blocks;
   }
-  const double others = K <= 8192 ? 800.0 : 950.0;
+  const double others = 950.0;
   return best_rate >= others ? best : 0;
 }
 
-// Products with so few of the widest tiles that half the compute units would idle, and a long K: K in two
-// parts over twice the workgroups, each leaving its bare sums in scratch memory ([part][row][weight row],
-// float32) for the finishing kernel.  Measured at 2,048 rows x 4,096 weight rows x 12,288: see gemm_turns_blocks.
+// Products with so few of the widest tiles that half the compute units or more would idle: K in two or four
+// parts over as many times the workgroups, each leaving its bare sums in scratch memory ([part][row][weight row],
+// float32) for the finishing kernel.  Measured at 2,048 rows x 4,096 weight rows x 12,288 (the down projection
+// of the Qwen3-8B shape): 240 -> 199 us with the finishing kernel's 23 us.
 int gemm_turns_parts(int M, int N, int K, int layout, int activation) {
-  if (activation || M <= 256 || K < 8192 || K % 256 || !gemm_turns_can(M, N, K, layout, 0, 8)) return 1;
+  if (activation || M <= 256 || !gemm_turns_can(M, N, K, layout, 0, 8)) return 1;
   if (gemm_turns_blocks(M, N, K, layout, 0)) return 1;   // a tile of its own fills the chip
   const long tiles = (long)((N + 255) / 256) * ((M + 255) / 256);
-  return tiles > 64 && tiles <= 128 ? 2 : 1;
+  const int parts = tiles <= 64 ? 4 : 2;                 // two or four parts: more only add scratch traffic
+  if (tiles * parts <= 192 || tiles * parts > 256) return 1;   // worth it from three quarters of the chip on
+  return K / parts >= 1024 && K % (128 * parts) == 0 ? parts : 1;
 }
 
 int gemm_turns_launch_parts(const void* a, const void* w, float* sums, int M, int N, int K, int parts, hipStream_t stream) {
