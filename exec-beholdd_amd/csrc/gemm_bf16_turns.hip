@@ -263,16 +263,25 @@ bool gemm_turns_can(int M, int N, int K, int layout, int activation, int blocks)
          (long)M * K < (1L << 31) && (long)((N + outs - 1) / outs) * ((M + 255) / 256) < (1L << 31);
 }
 
-// Which tile, if any.  A tile of YB blocks per wave costs a compute unit YB x cost(YB) units of time, where
-// cost is what the narrower tiles lose (measured 1.25, 1.11 and 0.90 PFLOP/s for 8, 6 and 4 with the chip
-// full), and the chip works in rounds of 256 tiles.  The estimate is compared with what the other ways reach
-// (the other tiled kernels about 0.85 PFLOP/s at their best; K in two parts of the widest tile, see
-// gemm_turns_parts, about 1.0: in the whole model it beat the 128-wide tile for the o projection too, prefill
-// of 2,048 tokens 31.8 -> 30.5 ms, though the two run alike alone).
-int gemm_turns_blocks(int M, int N, int K, int layout, int activation) {
-  if (M <= 256) return 0;   // up to there a norm may ride on the product, which this kernel does not carry
-  int best = 0;
-  double best_rate = 0.0;
+// Which way, if any.  A tile of YB blocks per wave costs a compute unit YB x cost(YB) units of time, where cost
+// is what the narrower tiles lose (measured 1.25, 1.11 and 0.90 PFLOP/s for 8, 6 and 4 with the chip full), and
+// the chip works in rounds of 256 tiles.  Products with so few of the widest tiles that a quarter of the compute
+// units or more would idle can instead cut K into two or four parts over as many times the workgroups, each
+// leaving its bare sums in scratch memory ([part][row][weight row], float32) for the finishing kernel of
+// gemm_bf16.hip; that costs about 0.85 of the tile's rate (measured at 2,048 rows x 4,096 weight rows x 12,288,
+// the down projection of the Qwen3-8B shape: 240 -> 199 us with the finishing kernel's 21 us; for its o
+// projection the parts and the 128-wide tile run alike alone, but the whole prefill of 2,048 tokens went
+// 31.8 -> 30.5 ms with the parts).  The better estimate wins if it beats what the other tiled kernels reach
+// (about 0.8 PFLOP/s at their best).
+namespace {
+struct TurnsPlan {
+  int blocks;   // tile width for the product in one launch, or 0
+  int parts;    // parts of K with the widest tile, or 1
+};
+TurnsPlan turns_plan(int M, int N, int K, int layout, int activation) {
+  TurnsPlan plan = {0, 1};
+  if (M <= 256) return plan;   // up to there a norm may ride on the product, which this kernel does not carry
+  double best_rate = 800.0;    // TFLOP/s, roughly: what the other kernels reach
   const double work = (double)M * (activation ? 2.0 * N : (double)N);   // rows x weight rows
   for (int blocks = 8; blocks >= 4; blocks -= 2) {
     if (!gemm_turns_can(M, N, K, layout, activation, blocks)) continue;
@@ -280,24 +289,26 @@ int gemm_turns_blocks(int M, int N, int K, int layout, int activation) {
     const long tiles = (long)((N + outs - 1) / outs) * ((M + 255) / 256);
     const long rounds = (tiles + 255) / 256;
     const double cost = blocks == 8 ? 1.0 : blocks == 6 ? 1.12 : 1.39;
-    const double rate = 1250.0 * work / ((double)rounds * 256 * 256 * (activation ? 2 : 1) * outs * cost);   // TFLOP/s, roughly
-    if (rate > best_rate) best_rate = rate, best = blocks;
+    const double rate = 1250.0 * work / ((double)rounds * 256 * 256 * (activation ? 2 : 1) * outs * cost);
+    if (rate >= best_rate) best_rate = rate, plan.blocks = blocks;
   }
-  const double others = 950.0;
-  return best_rate >= others ? best : 0;
+  if (!activation && gemm_turns_can(M, N, K, layout, 0, 8)) {
+    const long tiles = (long)((N + 255) / 256) * ((M + 255) / 256);
+    const int parts = tiles <= 64 ? 4 : 2;   // more parts only add scratch traffic
+    if (tiles * parts > 192 && tiles * parts <= 256 && K / parts >= 1024 && K % (128 * parts) == 0) {
+      const double rate = 0.85 * 1250.0 * work / (256.0 * 256 * 256 / parts);
+      if (rate > best_rate) best_rate = rate, plan.blocks = 0, plan.parts = parts;
+    }
+  }
+  return plan;
 }
+}  // namespace
 
-// Products with so few of the widest tiles that half the compute units or more would idle: K in two or four
-// parts over as many times the workgroups, each leaving its bare sums in scratch memory ([part][row][weight row],
-// float32) for the finishing kernel.  Measured at 2,048 rows x 4,096 weight rows x 12,288 (the down projection
-// of the Qwen3-8B shape): 240 -> 199 us with the finishing kernel's 23 us.
+int gemm_turns_blocks(int M, int N, int K, int layout, int activation) {
+  return turns_plan(M, N, K, layout, activation).blocks;
+}
 int gemm_turns_parts(int M, int N, int K, int layout, int activation) {
-  if (activation || M <= 256 || !gemm_turns_can(M, N, K, layout, 0, 8)) return 1;
-  if (gemm_turns_blocks(M, N, K, layout, 0)) return 1;   // a tile of its own fills the chip
-  const long tiles = (long)((N + 255) / 256) * ((M + 255) / 256);
-  const int parts = tiles <= 64 ? 4 : 2;                 // two or four parts: more only add scratch traffic
-  if (tiles * parts <= 192 || tiles * parts > 256) return 1;   // worth it from three quarters of the chip on
-  return K / parts >= 1024 && K % (128 * parts) == 0 ? parts : 1;
+  return turns_plan(M, N, K, layout, activation).parts;
 }
 
 int gemm_turns_launch_parts(const void* a, const void* w, float* sums, int M, int N, int K, int parts, hipStream_t stream) {
