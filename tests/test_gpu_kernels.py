@@ -54,7 +54,9 @@ def test_embed(K, dtype, rows, width, vocab):
 @pytest.mark.parametrize("w_dtype", DTYPES)
 @pytest.mark.parametrize("rows,width,eps", [(1, 48, 1e-6), (33, 1000, 1e-5), (4, 5120, 1e-6), (3, 4097, 1e-2),
                                             (300, 1000, 1e-5), (257, 4096, 1e-6), (256, 260, 1e-6), (301, 4098, 1e-6),
-                                            (258, 256, 1e-6), (270, 2560, 1e-5), (259, 8192, 1e-6)])
+                                            (258, 256, 1e-6), (270, 2560, 1e-5), (259, 8192, 1e-6),
+                                            # many rows and a width that is a multiple of 4: 16 bytes per load
+                                            (100, 5120, 1e-6), (64, 16384, 1e-6), (65, 17408, 1e-6), (80, 12, 1e-5)])
 def test_rmsnorm(K, out_dtype, w_dtype, rows, width, eps):
     g = torch.Generator().manual_seed(width)
     x = torch.randn(rows, width, generator=g) * 3 + 0.5
@@ -69,6 +71,11 @@ def test_rmsnorm(K, out_dtype, w_dtype, rows, width, eps):
     K.rmsnorm(dev(x), None, eps, out2, rows=dev(index))
     want2 = (x.double() / torch.sqrt((x.double() ** 2).mean(-1, keepdim=True) + eps))[index.long()]
     assert rel(out2, want2) < tol(out_dtype, 2e-6, 4e-3)
+    if rows >= 64:      # many gathered rows, with a weight
+        index = torch.randint(0, rows, (rows + 5,), generator=g, dtype=torch.int32)
+        out3 = torch.empty(rows + 5, width, dtype=out_dtype, device="cuda:0")
+        K.rmsnorm(dev(x), dev(w), eps, out3, rows=dev(index))
+        assert rel(out3, want[index.long()]) < tol(out_dtype, 2e-6, 4e-3)
 
 
 @pytest.mark.parametrize("a_dtype,w_dtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
