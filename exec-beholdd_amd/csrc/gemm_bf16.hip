@@ -266,6 +266,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
 // 64 * blockIdx.x + 4 col .. + 3 of row 16 * blockIdx.y + r (N is a multiple of 16 here).  All of a thread's
 // loads are asked for before the first is used.  A norm behind gets one partial sum per row and block.
 #define MAX_PARTS 16
+#define MAX_TURNS_PARTS 4   // what gemm_turns_parts cuts K into at most
 #define FINISH_COLUMNS 64
 typedef uint16_t u16x4_t __attribute__((ext_vector_type(4)));
 template <bool SWIGLU, typename TC>
@@ -355,6 +356,58 @@ __global__ __launch_bounds__(256) void gemm_parts_finish_kernel(const float* __r
 }
 
 // ---- tiled -----------------------------------------------------------------------------------
+
+// The same for a product that completes the float32 residual right before an RMSNorm reads it, with many rows
+// (the parts come from the kernel whose wave groups take turns): a block owns a whole row, so it can finish the
+// norm itself and the norm needs no launch and no second pass over the residual.  Thread t has the groups of
+// four columns t, t + 256, ...; the parts are added in their order, then the residual's old values, as the kernel
+// above does; the row's sum of squares is added up as rmsnorm does it for this width.
+#define FINISH_NORM_GROUPS 8   // groups of four columns per thread: rows of up to 8,192
+__global__ __launch_bounds__(256) void gemm_parts_finish_norm_kernel(const float* __restrict__ sums, float* __restrict__ c,
+                                                                     int M, int N, int parts, const void* __restrict__ weight,
+                                                                     int weight_f32, float eps, uint16_t* __restrict__ normed) {
+  __shared__ float scratch[4];
+  const int row = blockIdx.x, fours = N / 4;
+  f32x4_t* residual = reinterpret_cast<f32x4_t*>(c + (size_t)row * N);
+  f32x4_t value[FINISH_NORM_GROUPS];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < FINISH_NORM_GROUPS; ++j) {
+    const int i = threadIdx.x + j * 256;
+    value[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    if (i >= fours) continue;
+    f32x4_t part[MAX_TURNS_PARTS];
+    const f32x4_t old = residual[i];
+#pragma unroll
+    for (int p = 0; p < MAX_TURNS_PARTS; ++p)
+      part[p] = p < parts ? reinterpret_cast<const f32x4_t*>(sums + ((size_t)p * M + row) * N)[i] : f32x4_t{0.f, 0.f, 0.f, 0.f};
+    f32x4_t sum = part[0];
+#pragma unroll
+    for (int p = 1; p < MAX_TURNS_PARTS; ++p) sum += part[p];
+    value[j] = sum + old;
+    residual[i] = value[j];
+    ss += value[j][0] * value[j][0] + value[j][1] * value[j][1] + value[j][2] * value[j][2] + value[j][3] * value[j][3];
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)N + eps);
+#pragma unroll
+  for (int j = 0; j < FINISH_NORM_GROUPS; ++j) {
+    const int i = threadIdx.x + j * 256;
+    if (i >= fours) continue;
+    f32x4_t g;
+    if (weight_f32) {
+      g = reinterpret_cast<const f32x4_t*>(weight)[i];
+    } else {
+      const u16x4_t raw = reinterpret_cast<const u16x4_t*>(weight)[i];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) g[e] = bf16_bits_to_f32(raw[e]);
+    }
+    u16x4_t bits;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) bits[e] = f32_to_bf16_bits(value[j][e] * inv * g[e]);
+    reinterpret_cast<u16x4_t*>(normed + (size_t)row * N)[i] = bits;
+  }
+}
 
 #define TK 64           // k slice
 #define TPITCH (TK + 8) // LDS row pitch in elements: 144 bytes, so 16-byte reads of 16 rows hit 64 distinct banks
@@ -1002,4 +1055,29 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
   }
 #undef BH_PICK
   return bh_check_launch("gemm_tiled");
+}
+
+// residual[M, N] += A W^T and normed = RMSNorm(residual; weight, eps) as bfloat16, in one go: for the products of
+// many rows whose K the turns kernel multiplies in parts (bh_gemm_bf16_finishes_norm says which), whose finishing
+// kernel streams the residual anyway.  `scratch`: bh_gemm_bf16_scratch() bytes.
+extern "C" int bh_gemm_bf16_finishes_norm(int M, int N, int K, int layout) {
+  if (M <= 0 || N <= 0 || K <= 0 || N % 4 != 0 || N > 4 * 256 * FINISH_NORM_GROUPS) return 0;
+  const int parts = gemm_turns_parts(M, N, K, layout, 0);
+  return parts > 1 && parts <= MAX_TURNS_PARTS ? 1 : 0;
+}
+extern "C" int bh_gemm_bf16_then_norm(const void* a, const void* w, float* residual, int M, int N, int K, int layout,
+                                      const void* norm_weight, int norm_weight_dtype, float eps, void* normed,
+                                      void* scratch, hipStream_t stream) {
+  BH_REQUIRE(bh_gemm_bf16_finishes_norm(M, N, K, layout),
+             "gemm_bf16_then_norm: a product of M=%d N=%d K=%d does not finish a norm (bh_gemm_bf16_finishes_norm)", M, N, K);
+  BH_REQUIRE(a && w && residual && norm_weight && normed && scratch, "gemm_bf16_then_norm: every operand is needed");
+  BH_REQUIRE(norm_weight_dtype == BH_F32 || norm_weight_dtype == BH_BF16, "gemm_bf16_then_norm: unknown norm weight dtype %d", norm_weight_dtype);
+  BH_REQUIRE(eps >= 0.f, "gemm_bf16_then_norm: eps must not be negative");
+  BH_REQUIRE(((uintptr_t)a | (uintptr_t)w | (uintptr_t)residual | (uintptr_t)normed | (uintptr_t)scratch | (uintptr_t)norm_weight) % 16 == 0,
+             "gemm_bf16_then_norm: operands must be 16-byte aligned");
+  const int parts = gemm_turns_parts(M, N, K, layout, 0);
+  if (int status = gemm_turns_launch_parts(a, w, (float*)scratch, M, N, K, parts, stream)) return status;
+  gemm_parts_finish_norm_kernel<<<M, 256, 0, stream>>>((const float*)scratch, residual, M, N, parts, norm_weight,
+                                                       norm_weight_dtype == BH_F32, eps, (uint16_t*)normed);
+  return bh_check_launch("gemm_parts_finish_norm");
 }

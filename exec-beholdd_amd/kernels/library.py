@@ -96,6 +96,8 @@ class HipKernels:
             "bh_sample_scratch": [i, i],
             "bh_gemm_bf16": [p, p, p, i, i, i, i, i, i, i, p, i, f, p, i, p, p, p, p],
             "bh_gemm_bf16_turns": [p, p, p, i, i, i, i, i, i, i, p],
+            "bh_gemm_bf16_then_norm": [p, p, p, i, i, i, i, p, i, f, p, p, p],
+            "bh_gemm_bf16_finishes_norm": [i, i, i, i],
             "bh_attention_bf16": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, i, i, f, i, i, i, p],
             "bh_attention_bf16_splits": [i, i, i, i, i],
             "bh_attention_decode_fused": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, f, i, i, i, p, p, i, f, p, p, i, i,
@@ -195,6 +197,17 @@ class HipKernels:
         if ahead is not None and (ahead.ss.shape[0] != m or ahead.ss.dtype != torch.float32
                                   or not self.lib.bh_gemm_bf16_takes_norm(*sizes)):
             raise KernelError(f"gemm: a product of {m} x {n} x {k} does not take these prepared norm rows")
+        if (then_norm is not None and ahead is None and accumulate and packed and out.dtype == torch.float32
+                and not activation and then_norm.weight.shape == (n,) and then_norm.weight.dtype in _CODES
+                and self.lib.bh_gemm_bf16_finishes_norm(m, n, k, 1)):
+            # many rows, K in parts: the finishing kernel owns whole rows and finishes the norm itself
+            normed = torch.empty((m, n), dtype=torch.bfloat16, device=self.device)
+            scratch = torch.empty(int(self.lib.bh_gemm_bf16_scratch(*sizes)) // 4, dtype=torch.float32, device=self.device)
+            self._check(self.lib.bh_gemm_bf16_then_norm(
+                self._ptr(a, "gemm a"), self._ptr(w.data, "gemm w"), self._ptr(out, "gemm out", (torch.float32,)), m, n, k, 1,
+                self._ptr(then_norm.weight, "norm weight"), _code(then_norm.weight, "norm weight"), float(then_norm.eps),
+                self._ptr(normed, "norm rows"), self._ptr(scratch, "gemm scratch"), self._stream()))
+            return True, normed
         behind = None
         if (then_norm is not None and out.dtype == torch.float32 and not activation
                 and then_norm.weight.shape == (n,) and then_norm.weight.dtype in _CODES):
@@ -224,8 +237,8 @@ class HipKernels:
         """out[M, N] (+)= a[M, K] @ w[N, K]^T with float32 accumulation; `w` may be a PackedWeight and
         `a` the NormedRows an earlier product prepared.  With `then_norm` (an object with `weight` [N] and
         `eps`: an RMSNorm over the rows of `out` as they are after this product) the product may prepare that norm's
-        output on its way and return it as NormedRows; it returns None when it does not (then run the
-        norm as usual)."""
+        output on its way and return it, as NormedRows or, where it finishes the norm itself, as the bfloat16
+        matrix the norm would have given; it returns None when it does neither (then run the norm as usual)."""
         if a.dim() != 2 or w.dim() != 2 or out.dim() != 2:
             raise KernelError("gemm: operands must be matrices")
         m, k = a.shape

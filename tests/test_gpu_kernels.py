@@ -225,6 +225,35 @@ def test_norm_rides_on_wide_products(K, m, n, k, n2, g_dtype):
     assert rel(act, gate / (1 + torch.exp(-gate)) * up) < 1.2e-2
 
 
+@pytest.mark.parametrize("g_dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", [(2048, 4096, 4096), (1000, 4096, 2048 * 4), (1800, 5120 - 1024, 2048)])
+def test_product_in_parts_of_many_rows_finishes_the_norm(K, g_dtype, m, n, k):
+    """Beyond 256 rows, where K goes through the turns kernel in parts, the finishing kernel owns whole rows and
+    writes the norm's output itself: `gemm(..., then_norm=)` returns it as a plain bfloat16 matrix."""
+    from beholdd.parts.base import NormRequest
+    gen = torch.Generator().manual_seed(m + n)
+    a = (torch.randn(m, k, generator=gen) * 0.5).to(torch.bfloat16)
+    w = (torch.randn(n, k, generator=gen) * 0.05).to(torch.bfloat16)
+    base = torch.randn(m, n, generator=gen) * 3
+    g = (1 + 0.3 * torch.randn(n, generator=gen)).to(g_dtype)
+    eps = 1e-5
+    on = lambda t: t.double().to("cuda:0")
+    packed = K.pack_weight(dev(w))
+    plain = dev(base.clone())
+    assert K.gemm(dev(a), packed, plain, accumulate=True) is None
+    residual = dev(base.clone())
+    normed = K.gemm(dev(a), packed, residual, accumulate=True, then_norm=NormRequest(dev(g), eps))
+    assert isinstance(normed, torch.Tensor) and normed.dtype == torch.bfloat16 and normed.shape == (m, n)
+    assert torch.equal(residual, plain)            # the same sums in the same order as without the norm
+    assert rel(residual, (on(base) + on(a) @ on(w).t()).cpu()) < 4 * math.sqrt(k) * 2.0 ** -24
+    got = residual.double()
+    want = got / torch.sqrt((got ** 2).mean(-1, keepdim=True) + eps) * on(g)
+    assert rel(normed, want.cpu()) < 4e-3
+    reference = torch.empty(m, n, dtype=torch.bfloat16, device="cuda:0")
+    K.rmsnorm(residual, dev(g), eps, reference)
+    assert (normed.float() - reference.float()).abs().max() <= 2.0 ** -7 * reference.float().abs().max()
+
+
 def test_norm_does_not_ride_on_wide_steps(K):
     from beholdd.parts.base import NormRequest
     a = torch.randn(65, 64).to(torch.bfloat16)
