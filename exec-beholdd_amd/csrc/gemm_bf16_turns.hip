@@ -146,21 +146,14 @@ __global__ __launch_bounds__(512) void gemm_turns_kernel(const uint16_t* __restr
   // Step j lies in region j % R.  A wave asks for step j + R - 1 while it reads step j (into the region that
   // step j - 1 has left); before the turn in which the first group reads step j + 1, all that was asked for
   // it must have landed: what may still be on its way are the loads of the steps after it.
-  auto wait_for_next = [&](int j, int per_step, bool with_lds) {   // per_step: this wave's loads per step
+  auto wait_for_next = [&](int j, auto per_step) {   // per_step: this wave's loads per step
+    constexpr int each = decltype(per_step)::value;
     const int later = min(R - 2, J - 2 - j);   // steps after j + 1 that have been asked for
-    (void)with_lds;
-    if (per_step == 4) {
-      if (later >= 4) WAIT_VM_LGKM0(16); else if (later == 3) WAIT_VM_LGKM0(12); else if (later == 2) WAIT_VM_LGKM0(8);
-      else if (later == 1) WAIT_VM_LGKM0(4); else WAIT_VM_LGKM0(0);
-    } else if (per_step == 3) {
-      if (later >= 4) WAIT_VM_LGKM0(12); else if (later == 3) WAIT_VM_LGKM0(9); else if (later == 2) WAIT_VM_LGKM0(6);
-      else if (later == 1) WAIT_VM_LGKM0(3); else WAIT_VM_LGKM0(0);
-    } else {
-      if (later >= 4) WAIT_VM_LGKM0(8); else if (later == 3) WAIT_VM_LGKM0(6); else if (later == 2) WAIT_VM_LGKM0(4);
-      else if (later == 1) WAIT_VM_LGKM0(2); else WAIT_VM_LGKM0(0);
-    }
+    if (later >= 2) WAIT_VM_LGKM0(2 * each);
+    else if (later == 1) WAIT_VM_LGKM0(each);
+    else WAIT_VM_LGKM0(0);
   };
-  static_assert(R - 2 <= 4, "wait_for_next knows up to four steps on their way after the next");
+  static_assert(R == 4, "wait_for_next knows of two steps on their way after the next");
   if (g == 0) {
     for (int j = 0; j < R - 1 && j < J; ++j) fetch_a(j, j);
     WAIT_VM_LGKM0(0);
@@ -172,7 +165,7 @@ __global__ __launch_bounds__(512) void gemm_turns_kernel(const uint16_t* __restr
       WAIT_LGKM0();
       TICK();
       multiply();
-      wait_for_next(j, 4, false);
+      wait_for_next(j, std::integral_constant<int, 4>());
       TICK();
       region = region == R - 1 ? 0 : region + 1;
     }
@@ -186,7 +179,7 @@ __global__ __launch_bounds__(512) void gemm_turns_kernel(const uint16_t* __restr
     for (int j = 0; j < J; ++j) {
       if (j + R - 1 < J) fetch_w(j + R - 1, region == 0 ? R - 1 : region - 1);
       read_operands(region);
-      wait_for_next(j, WL, true);
+      wait_for_next(j, std::integral_constant<int, WL>());
       TICK();
       multiply();
       TICK();
