@@ -266,7 +266,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
 // 64 * blockIdx.x + 4 col .. + 3 of row 16 * blockIdx.y + r (N is a multiple of 16 here).  All of a thread's
 // loads are asked for before the first is used.  A norm behind gets one partial sum per row and block.
 #define MAX_PARTS 16
-#define MAX_TURNS_PARTS 4   // what gemm_turns_parts cuts K into at most
+#define MAX_TURNS_PARTS 8   // what gemm_turns_parts cuts K into at most
 #define FINISH_COLUMNS 64
 typedef uint16_t u16x4_t __attribute__((ext_vector_type(4)));
 template <bool SWIGLU, typename TC>

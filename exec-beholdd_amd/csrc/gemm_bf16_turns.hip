@@ -258,14 +258,12 @@ bool gemm_turns_can(int M, int N, int K, int layout, int activation, int blocks)
 
 // Which way, if any.  A tile of YB blocks per wave costs a compute unit YB x cost(YB) units of time, where cost
 // is what the narrower tiles lose (measured 1.25, 1.11 and 0.90 PFLOP/s for 8, 6 and 4 with the chip full), and
-// the chip works in rounds of 256 tiles.  Products with so few of the widest tiles that a quarter of the compute
-// units or more would idle can instead cut K into two or four parts over as many times the workgroups, each
-// leaving its bare sums in scratch memory ([part][row][weight row], float32) for the finishing kernel of
-// gemm_bf16.hip; that costs about 0.85 of the tile's rate (measured at 2,048 rows x 4,096 weight rows x 12,288,
-// the down projection of the Qwen3-8B shape: 240 -> 199 us with the finishing kernel's 21 us; for its o
-// projection the parts and the 128-wide tile run alike alone, but the whole prefill of 2,048 tokens went
-// 31.8 -> 30.5 ms with the parts).  The better estimate wins if it beats what the other tiled kernels reach
-// (about 0.8 PFLOP/s at their best).
+// the chip works in rounds of 256 tiles; a tile of its own is taken if that estimate beats what the other tiled
+// kernels reach at their best (about 0.8 PFLOP/s).  Products with so few of the widest tiles that much of the
+// chip would idle can instead cut K into parts over as many times the workgroups, each leaving its bare sums in
+// scratch memory ([part][row][weight row], float32) for a finishing kernel of gemm_bf16.hip; that costs about
+// 0.85 of the tile's rate (for the o projection of the Qwen3-8B shape at 2,048 rows the parts and the 128-wide
+// tile run alike alone, but the whole prefill went 31.8 -> 30.5 ms with the parts).
 namespace {
 struct TurnsPlan {
   int blocks;   // tile width for the product in one launch, or 0
@@ -274,7 +272,8 @@ struct TurnsPlan {
 TurnsPlan turns_plan(int M, int N, int K, int layout, int activation) {
   TurnsPlan plan = {0, 1};
   if (M <= 256) return plan;   // up to there a norm may ride on the product, which this kernel does not carry
-  double best_rate = 800.0;    // TFLOP/s, roughly: what the other kernels reach
+  double best_rate = 800.0;    // TFLOP/s, roughly: what the other kernels reach at their best
+  double direct_rate = 0.0;
   const double work = (double)M * (activation ? 2.0 * N : (double)N);   // rows x weight rows
   for (int blocks = 8; blocks >= 4; blocks -= 2) {
     if (!gemm_turns_can(M, N, K, layout, activation, blocks)) continue;
@@ -283,14 +282,20 @@ TurnsPlan turns_plan(int M, int N, int K, int layout, int activation) {
     const long rounds = (tiles + 255) / 256;
     const double cost = blocks == 8 ? 1.0 : blocks == 6 ? 1.12 : 1.39;
     const double rate = 1250.0 * work / ((double)rounds * 256 * 256 * (activation ? 2 : 1) * outs * cost);
-    if (rate >= best_rate) best_rate = rate, plan.blocks = blocks;
+    if (rate >= best_rate) best_rate = direct_rate = rate, plan.blocks = blocks;
   }
-  if (!activation && gemm_turns_can(M, N, K, layout, 0, 8)) {
+  if (!activation && M >= 512 && gemm_turns_can(M, N, K, layout, 0, 8)) {
+    // As many parts (8, 4 or 2) as keep the workgroups within one round and every part at least 1,024 long; worth
+    // it from about five eighths of the chip on.  Measured at the Qwen3-8B widths against the other kernels, us:
+    // 512 rows: down in 8 parts 88 -> 72 (o in 4 parts, half the chip, 41 -> 45: left alone); 768 rows: o 71 -> 53,
+    // down 195 -> 102 in 4; 1,024 rows: o 72 -> 57, down 196 -> 111 in 4; 1,536 rows: o 93 -> 77, down 219 -> 173 in 2;
+    // 2,048 rows: down 240 -> 199 in 2; 384 rows: slower for qkv and o, so not below 512.
     const long tiles = (long)((N + 255) / 256) * ((M + 255) / 256);
-    const int parts = tiles <= 64 ? 4 : 2;   // more parts only add scratch traffic
-    if (tiles * parts > 192 && tiles * parts <= 256 && K / parts >= 1024 && K % (128 * parts) == 0) {
+    int parts = 8;
+    while (parts > 1 && (tiles * parts > 256 || K / parts < 1024 || K % (128 * parts) != 0)) parts /= 2;
+    if (parts > 1 && tiles * parts >= 160) {
       const double rate = 0.85 * 1250.0 * work / (256.0 * 256 * 256 / parts);
-      if (rate > best_rate) best_rate = rate, plan.blocks = 0, plan.parts = parts;
+      if (rate > direct_rate) plan.blocks = 0, plan.parts = parts;
     }
   }
   return plan;
