@@ -46,6 +46,11 @@ def parse():
     parser.add_argument("--prefill-tokens", type=int, default=2048)
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
+    parser.add_argument("--workload", action="store_true",
+                        help="instead of the step timings, generate through the engine's own loop for the batch the shape's "
+                             "benchmark configuration names (8b: 8 prompts of 256 to 1,024 tokens up to the context; 14b: 16 "
+                             "prompts of 64 to 4,096 tokens, 256 greedy tokens each; 32b: 32 prompts of 128 to 8,192 tokens, "
+                             "128 tokens each at temperature 1) and print its tokens per second")
     parser.add_argument("--hbm-ceiling", action="store_true",
                         help="measure what a plain streaming read and a copy of 8 GB reach on this GPU, print it and exit")
     return parser.parse_args()
@@ -123,6 +128,31 @@ def prefill_run(engine, n_tokens, torch, repeats=3):
     return min(times[1:])
 
 
+# Batches of the benchmark configurations: (prompts, shortest, longest, new tokens, temperature, context).
+WORKLOADS = {"8b": (8, 256, 1024, 256, 0.0, 8192), "14b": (16, 64, 4096, 256, 0.0, 8192),
+             "32b": (32, 128, 8192, 128, 1.0, 16384)}
+
+
+def workload_run(engine, shape, torch):
+    """Unequal prompts through `Engine.generate` (prompts in one step, then a token each, sequences that end
+    give their slots back): what a user of the library gets, host loop and sampling included."""
+    import random
+    count, shortest, longest, new_tokens, temperature, _ = WORKLOADS[shape]
+    rng = random.Random(0)
+    lengths = [rng.randint(shortest, longest) for _ in range(count)]
+    prompts = [[rng.randrange(engine.model.vocab) for _ in range(n)] for n in lengths]
+    engine.generate([prompts[0][:64]], max_new_tokens=4)          # warms up: graphs are captured per batch size as they come
+    torch.cuda.synchronize()
+    begin = time.perf_counter()
+    results = engine.generate(prompts, max_new_tokens=new_tokens, temperature=temperature, seed=1)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - begin
+    generated = sum(len(r.token_ids) for r in results)
+    return {"prompts": count, "prompt_tokens": sum(lengths), "generated_tokens": generated,
+            "seconds": round(elapsed, 3), "generated_tok_per_s": round(generated / elapsed, 1),
+            "all_tok_per_s": round((generated + sum(lengths)) / elapsed, 1), "temperature": temperature}
+
+
 def hbm_ceiling(torch):
     """What library kernels that only stream memory reach here: a sum over 8 GB (read) and a copy of 8 GB
     (read + write).  Not part of the product path; a yardstick for the roofline fractions."""
@@ -160,6 +190,16 @@ def main():
     element = 2 if args.dtype == "bfloat16" else 4
     model = random_model_on_device(config, seed=0, dtype=args.dtype, device=device)
     biggest = 1 if args.no_points else 64
+    if args.workload:
+        count, _, longest, new_tokens, _, context = WORKLOADS[args.shape]
+        engine = Engine(model=model, dtype=args.dtype, max_tokens=count * (-(-(longest + new_tokens) // 64) * 64),
+                        max_slots=count, device=device)
+        line = {"metric": f"generation of the {shape_name} batch", "unit": "tok/s", "dtype": dtype_tag,
+                "layers": config["num_hidden_layers"], "layers_of_full_model": shape["num_hidden_layers"], "context": context}
+        line.update(workload_run(engine, args.shape, torch))
+        line["value"] = line["generated_tok_per_s"]
+        print(json.dumps(line))
+        return 0
     max_tokens = max(args.batch, biggest) * (-(-args.context // 64) * 64)
     engine = Engine(model=model, dtype=args.dtype, max_tokens=max_tokens, max_slots=max(args.batch, biggest, 64),
                     device=device)
