@@ -142,6 +142,24 @@ def test_layers_of_the_large_models_sizes(large_expected, shape, dtype):
     check("24 together", schedules.batches(engine, many, batch_size=24, prompt_fraction=0.5), want_many, TOLERANCE[dtype])
 
 
+def test_prompts_of_many_rows(large_expected):
+    """Steps of 400 to 2,200 rows at the Qwen3-8B layer sizes, where the bfloat16 products go to the kernel whose
+    wave groups take turns (a tile of its own, K in parts, the finishing kernel that also finishes the norm):
+    three prompts in one step and each alone, against the float32 engine, which the test above holds to
+    the plain implementation at these sizes."""
+    folder = large_expected("8b")[0]
+    requests = schedules.random_requests(1000, [700, 1100, 400], seed=9)
+    engine32 = engine_for(folder, "float32", max_tokens=4096)
+    want = schedules.whole(engine32, requests)
+    del engine32
+    engine = engine_for(folder, "bfloat16", max_tokens=4096)
+    alone = schedules.whole(engine, requests)
+    check("each alone", alone, want, TOLERANCE["bfloat16"])
+    together = schedules.batches(engine, requests, batch_size=3, prompt_fraction=1.0)
+    check("one step of 2,200 rows", together, want, TOLERANCE["bfloat16"])
+    check("together against alone", together, alone, TOLERANCE["bfloat16"] / 2)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_float32_storage_and_slot_reuse_in_a_small_cache(model_dirs, dtype):
     """Weights stored in 32-bit; a cache of three pages, so every request runs in pages and slots
