@@ -16,8 +16,9 @@
 //
 // Measured at the Qwen3-8B shapes, 2,048 rows, each product alone: gate/up with SwiGLU 404 -> 330 us
 // (1.25 PFLOP/s), qkv 132 -> 104 us with tiles of 192 weight rows (256 of them, one per compute unit), o 102 ->
-// 84 us with 128; in the whole model 381 -> 338, 115 -> 101 and 87 -> 94 us (o is kept: with the tile order
-// below the whole prefill is the faster for it).
+// 84 us with 128; in the whole model 381 -> 338, 115 -> 101 and 87 -> 94 us (which is why the o and down
+// projections there go through K in parts of the widest tile instead, see turns_plan: 77 us for o, finishing
+// kernel included).
 // What bounds it: the loads alone (no multiplies) take 0.9 of the whole kernel's time, the multiplies alone
 // 0.6.  It is not the loads' latency (five or six steps in LDS instead of four changed nothing; touching the
 // lines three slices ahead with 4-byte loads made it slower, 0.9 PFLOP/s for gate/up: loads retire in order, so
