@@ -313,6 +313,7 @@ def test_gemm_with_turns_refuses_what_it_cannot_do(K):
 @pytest.mark.parametrize("m,n,k,swiglu,blocks", [(2048, 6144, 256, False, 6), (2048, 12288, 128, True, 8),
                                                  (2048, 4096, 256, False, 4), (4000, 4096, 128, False, 8),
                                                  (500, 12288, 128, True, 6), (300, 4096, 128, False, 0),
+                                                 (512, 151936, 128, False, 8),      # a head over many wanted rows
                                                  (256, 12288, 128, True, 0), (2048, 4096, 12288, False, 0)])
 def test_gemm_chooses_the_turns_kernel_where_it_fills_the_chip(K, m, n, k, swiglu, blocks):
     """Which products go to the kernel whose wave groups take turns, and that `gemm` gives the right result there."""
