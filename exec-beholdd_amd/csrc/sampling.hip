@@ -7,7 +7,9 @@
 //                     number in [0, 1).  Sums run in a fixed order, so a row's result does not
 //                     depend on the other rows.
 // A row with a non-finite logit sets bad[row] = 1 and selects nothing (token -1).
-#include "common.h"
+#include "sampling.h"
+
+#include <mutex>
 
 #define SB 1024  // threads per block
 
@@ -263,4 +265,54 @@ extern "C" int bh_sample(const float* logits, const float* temperature, const in
   sample_kernel<<<dim3(n_rows), dim3(SB), 0, stream>>>(logits, temperature, top_k, top_p, uniform, tokens, bad,
                                                        vocab);
   return bh_check_launch("sample");
+}
+
+// ---- greedy selection without an allocation ----------------------------------------------------
+// The per-chunk maxima of the two-step argmax in a fixed array of the library's own.  In host code the
+// array's name is only a handle: its address on the current GPU comes from hipGetSymbolAddress, once per
+// device, and that address is what the kernels get.
+
+static __device__ __align__(256) float greedy_scratch[BH_GREEDY_STATIC_WORDS];
+
+#define BH_MAX_DEVICES 64
+static float* greedy_scratch_at[BH_MAX_DEVICES];   // the array's address on each device, null until asked
+static std::mutex greedy_scratch_lock;
+
+static int greedy_scratch_here(float** out) {
+  int device = -1;
+  hipError_t status = hipGetDevice(&device);
+  if (status != hipSuccess) return bh_fail("sample: no current device: %s", hipGetErrorString(status));
+  BH_REQUIRE(device >= 0 && device < BH_MAX_DEVICES, "sample: device %d is beyond the %d this library keeps scratch for",
+             device, BH_MAX_DEVICES);
+  std::lock_guard<std::mutex> guard(greedy_scratch_lock);
+  if (greedy_scratch_at[device] == nullptr) {
+    void* address = nullptr;
+    status = hipGetSymbolAddress(&address, HIP_SYMBOL(greedy_scratch));
+    if (status != hipSuccess || address == nullptr)
+      return bh_fail("sample: the address of the static scratch on device %d is not known: %s", device,
+                     hipGetErrorString(status));
+    greedy_scratch_at[device] = (float*)address;
+  }
+  *out = greedy_scratch_at[device];
+  return 0;
+}
+
+extern "C" int bh_sample_greedy_static(const float* logits, int32_t* tokens, int32_t* bad, int n_rows, int vocab,
+                                       hipStream_t stream) {
+  BH_REQUIRE(logits != nullptr && tokens != nullptr && bad != nullptr, "sample: logits, tokens and flags are required");
+  BH_REQUIRE(n_rows > 0 && vocab > 0, "sample: rows %d and vocabulary %d must be positive", n_rows, vocab);
+  BH_REQUIRE(n_rows <= 65535, "sample: too many rows");
+  const long chunks = ((long)vocab + AC - 1) / AC;
+  BH_REQUIRE(2 * (long)n_rows * chunks <= BH_GREEDY_STATIC_WORDS,
+             "sample: %d rows of %d logits need %ld words of scratch, the static array holds %d "
+             "(2 x rows x ceil(vocabulary / %d) words)", n_rows, vocab, 2 * (long)n_rows * chunks,
+             BH_GREEDY_STATIC_WORDS, AC);
+  float* scratch = nullptr;
+  if (int status = greedy_scratch_here(&scratch)) return status;
+  float* part_val = scratch;
+  int32_t* part_idx = (int32_t*)scratch + (size_t)n_rows * chunks;
+  argmax_chunk_kernel<<<dim3((int)chunks, n_rows), dim3(AT), 0, stream>>>(logits, part_val, part_idx, vocab, (int)chunks);
+  if (int status = bh_check_launch("argmax_chunk")) return status;
+  argmax_rows_kernel<<<dim3(n_rows), dim3(BH_WAVE), 0, stream>>>(part_val, part_idx, tokens, bad, (int)chunks);
+  return bh_check_launch("argmax_rows");
 }
