@@ -222,8 +222,10 @@ def load_plain(model_dir):
     return cfg, weights
 
 
-def attention_block(cfg, w, prefix, hidden):
-    """The attention half of a layer: h + Wo * Attn(...).
+def attention_block(cfg, w, prefix, hidden, first_position=0):
+    """The attention half of a layer: h + Wo * Attn(...).  Row t stands at position first_position + t
+    and sees the rows before it (the reference's chunk at `position_start`, forward.rs:1164-1189, with
+    nothing in the cache before it).
 
     crates/beholdd-model/src/qwen3moe/forward.rs:1075-1252: input RMSNorm; q, k, v
     projections; per-head RMSNorm of q and k with one [head_dim] weight each and the same
@@ -241,7 +243,7 @@ def attention_block(cfg, w, prefix, hidden):
     k = rmsnorm(k, w[prefix + "self_attn.k_norm.weight"], cfg.eps)
     freqs = rope_frequencies(cfg.theta, hd)
     for t in range(t_len):
-        cos, sin = rope_cos_sin(freqs, t)
+        cos, sin = rope_cos_sin(freqs, first_position + t)
         q[t] = rope_split_half(q[t], cos, sin)
         k[t] = rope_split_half(k[t], cos, sin)
     scale = F32(1.0) / np.sqrt(F32(hd))
@@ -262,13 +264,13 @@ def mlp_block(cfg, w, prefix, hidden):
     return (hidden + out).astype(F32)
 
 
-def layer(cfg, w, index, hidden):
+def layer(cfg, w, index, hidden, first_position=0):
     """h = h + Attn(RMSNorm(h)); h = h + MLP(RMSNorm(h)).
 
     crates/beholdd-model/src/qwen3moe/forward.rs:1022-1414.
     """
     prefix = f"model.layers.{index}."
-    hidden = attention_block(cfg, w, prefix, hidden)
+    hidden = attention_block(cfg, w, prefix, hidden, first_position)
     return mlp_block(cfg, w, prefix, hidden)
 
 
@@ -283,14 +285,14 @@ def head(cfg, w, hidden):
     return linear(xl, out)
 
 
-def forward_logits(cfg, w, tokens):
+def forward_logits(cfg, w, tokens, first_position=0):
     """Logits [T, vocab] of every position of one whole sequence.
 
     crates/beholdd-model/src/qwen3moe/forward.rs:412-436 (the non-cached forward).
     """
     hidden = embed(tokens, w["model.embed_tokens.weight"])
     for index in range(cfg.n_layers):
-        hidden = layer(cfg, w, index, hidden)
+        hidden = layer(cfg, w, index, hidden, first_position)
     return head(cfg, w, hidden)
 
 

@@ -252,26 +252,6 @@ def test_hand_checkable_model_logits_equal_hidden_over_rms():
     assert np.allclose(logits, expected, atol=1e-5)
 
 
-def test_qk_norm_comes_before_rotation_and_uses_its_own_weights():
-    # q_norm scaled by c scales every score of the layer by c; were the norm applied after the
-    # rotation with a non-uniform weight, or the weights swapped, the logits would differ.
-    cfg = _cfg(num_hidden_layers=1)
-    w = _tiny_weights(cfg, np.random.default_rng(8))
-    base = plain.forward_logits(cfg, w, [1, 2, 3, 4])
-    w2 = dict(w)
-    w2["model.layers.0.self_attn.q_norm.weight"] = w["model.layers.0.self_attn.q_norm.weight"] * 2
-    w2["model.layers.0.self_attn.k_norm.weight"] = w["model.layers.0.self_attn.k_norm.weight"] / 2
-    assert np.allclose(plain.forward_logits(cfg, w2, [1, 2, 3, 4]), base, atol=1e-5)
-    # a non-uniform norm weight does not commute with the rotation
-    hd = cfg.head_dim
-    x = np.arange(1, hd + 1, dtype=np.float32)
-    wq = np.array([1, 2, 3, 4], np.float32)
-    freqs = plain.rope_frequencies(cfg.theta, hd)
-    cs = plain.rope_cos_sin(freqs, 3)
-    assert not np.allclose(plain.rope_split_half(plain.rmsnorm(x, wq, 1e-6), *cs),
-                           plain.rmsnorm(plain.rope_split_half(x, *cs), wq, 1e-6), atol=1e-3)
-
-
 def test_greedy_generate_stop_token_is_not_emitted():
     cfg = _cfg()
     w = _tiny_weights(cfg, np.random.default_rng(9))
