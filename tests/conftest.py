@@ -62,12 +62,12 @@ def model_dirs(tmp_path_factory):
 
     made = {}
 
-    def get(name: str, dtype: str = "bfloat16", seed: int = 0):
-        key = (name, dtype, seed)
+    def get(name: str, dtype: str = "bfloat16", seed: int = 0, std: float = 0.02):
+        key = (name, dtype, seed, std)
         if key not in made:
             folder = tmp_path_factory.mktemp(f"tiny_{name}_{dtype}_{seed}")
             config = CONFIGS[name]
-            beholdd.write_random_model(str(folder), dict(config), seed=seed, dtype=dtype)
+            beholdd.write_random_model(str(folder), dict(config), seed=seed, dtype=dtype, std=std)
             made[key] = str(folder)
         return made[key]
 

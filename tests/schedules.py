@@ -79,6 +79,34 @@ def batches(engine, requests, batch_size, prompt_fraction=0.6):
     return out
 
 
+def portions(engine, requests, sizes=(2, 62, 1, 64, 2, 63, 1, 1, 65, 3, 61), rest_every=4):
+    """All requests together, every one fed in portions of unequal sizes: steps of several tokens onto a cache
+    that already holds some (also ending exactly at a page's end, one before and one after), portions of one
+    token beside portions of many in the same step, and now and then a request that rests for a step while its
+    batch-mates advance.  A request ends when its tokens are used up; the others go on."""
+    slots = [engine.alloc_slot() for _ in requests]
+    done = [0] * len(requests)
+    rows = [[] for _ in requests]
+    live = list(range(len(requests)))
+    step = 0
+    while live:
+        resting = [i for i in live if (step + i) % rest_every == rest_every - 1]
+        moving = [i for i in live if i not in resting] or live
+        counts = {i: min(sizes[(step + 3 * i) % len(sizes)], len(requests[i]) - done[i]) for i in moving}
+        logits = _rows(engine.step([StepEntry(slots[i], list(requests[i][done[i]:done[i] + counts[i]]),
+                                              list(range(counts[i]))) for i in moving]))
+        at = 0
+        for i in moving:
+            rows[i].append(logits[at:at + counts[i]])
+            at += counts[i]
+            done[i] += counts[i]
+            if done[i] == len(requests[i]):
+                engine.free_slot(slots[i])
+                live.remove(i)
+        step += 1
+    return [np.concatenate(r, axis=0) for r in rows]
+
+
 def relative_error(got, want):
     """max |got - want| / max |want|: the measure the acceptance tolerance is stated in."""
     return float(np.abs(got.astype(np.float64) - want.astype(np.float64)).max() / np.abs(want).max())

@@ -26,7 +26,8 @@ def test_every_cut_matches_the_plain_implementation(model_dirs, name, lengths):
     engine = make_engine(folder)
     for label, got in (("whole", schedules.whole(engine, requests)),
                        ("tail", schedules.tail_one_by_one(engine, requests, tail=32)),
-                       ("batches", schedules.batches(engine, requests, batch_size=3))):
+                       ("batches", schedules.batches(engine, requests, batch_size=3)),
+                       ("portions", schedules.portions(engine, requests))):
         for i, (g, e) in enumerate(zip(got, expected)):
             assert g.shape == e.shape, (label, i)
             assert schedules.relative_error(g, e) < 1e-4, (label, i, schedules.relative_error(g, e))
