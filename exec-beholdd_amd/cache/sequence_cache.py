@@ -104,6 +104,7 @@ class SequenceCache:
         heapq.heapify(self._free_slots)
         self._length: dict = {}      # live slot -> committed length
         self._allocated = False
+        self._state_before: list = []    # (group, slot indices, their state rows) as they were before the running step
 
     # ---- accounting and allocation ----
     def plan(self) -> CachePlan:
@@ -213,9 +214,18 @@ class SequenceCache:
                 pages = g.pages_of[slot]
                 while len(pages) * self.page_size < self._length[slot] + n_new:
                     pages.append(g.free_pages.pop())
+        # State regions are updated in place while the step runs; keep what the step's slots held, so that a
+        # failed step can put it back (the key/value pages need no such copy: rows beyond a sequence's length are
+        # never read).
+        self._state_before = []
+        for g in self.groups:
+            if g.need.kind == "state" and g.state is not None:
+                index = torch.tensor([slot for slot, _ in requests], dtype=torch.long, device=self.device)
+                self._state_before.append((g, index, g.state.index_select(1, index)))
 
     def commit(self, requests: list) -> None:
         """The step succeeded: the new tokens become part of their sequences."""
+        self._state_before = []
         for slot, n_new in requests:
             self._length[slot] += n_new
         for g in self.groups:
@@ -231,7 +241,11 @@ class SequenceCache:
                         pages[index] = -1
 
     def rollback(self, requests: list) -> None:
-        """The step failed: give back pages that `reserve` took beyond the committed lengths."""
+        """The step failed: give back pages that `reserve` took beyond the committed lengths, and put back
+        the state that the step's sequences held before it."""
+        for g, index, before in self._state_before:
+            g.state.index_copy_(1, index, before)
+        self._state_before = []
         for g in self.groups:
             if g.need.kind != "kv":
                 continue
@@ -247,19 +261,32 @@ class SequenceCache:
                 g.pages_of[slot] = list(pages)   # a new list: whoever remembers the old one sees that entries went away
 
     # ---- what kernels and mixers get ----
-    def page_table_rows(self, group: _Group, slots: list) -> list:
-        return [[max(page, 0) for page in group.pages_of[slot]] for slot in slots]
+    def kv_group_indices(self) -> list:
+        """The indices (into `groups`) of the groups that hold keys and values."""
+        return [index for index, g in enumerate(self.groups) if g.need.kind == "kv"]
+
+    def pages_held(self, group: int, slot: int) -> int:
+        return len(self.groups[group].pages_of[slot])
+
+    def write_page_table(self, group: int, slots: list, out) -> None:
+        """Write the page ids of `slots` into `out` [len(slots), width] (a host array): a row per sequence in
+        position order, 0 where a page was given back or none is held yet."""
+        g = self.groups[group]
+        for row, slot in enumerate(slots):
+            pages = g.pages_of[slot]
+            out[row, :] = 0
+            out[row, :len(pages)] = [max(page, 0) for page in pages]
 
     def page_tables(self, slots: list, min_width: int = 1) -> dict:
         """For each key/value group, an int32 device tensor [len(slots), width] of page ids."""
+        import numpy as np
+
         tables = {}
-        for index, g in enumerate(self.groups):
-            if g.need.kind != "kv":
-                continue
-            rows = self.page_table_rows(g, slots)
-            width = max(min_width, max(len(r) for r in rows))
-            flat = [r + [0] * (width - len(r)) for r in rows]
-            tables[index] = torch.tensor(flat, dtype=torch.int32).to(self.device, non_blocking=False)
+        for index in self.kv_group_indices():
+            width = max(min_width, max(self.pages_held(index, slot) for slot in slots))
+            host = np.zeros((len(slots), width), dtype=np.int32)
+            self.write_page_table(index, slots, host)
+            tables[index] = torch.from_numpy(host).to(self.device, non_blocking=False)
         return tables
 
     def layer_cache(self, entry: int, writes: bool, tables: dict) -> LayerCache:

@@ -19,7 +19,7 @@ from ..weights.binder import bind
 from ..weights.random_init import random_tensor_on_device
 from . import generation
 from .graphs import DecodeGraphs
-from .step import StepEntry, build_step, check_entries
+from .step import StepEntry, build_step, cache_for_runs, check_entries
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
 
@@ -109,22 +109,12 @@ class Engine:
                 raise ValueError("an entry takes its token from a selection, but nothing was selected yet")
             entries = [e if e.fed_row is None
                        else StepEntry(e.slot, [self._last_selection.token_at(e.fed_row)], e.want) for e in entries]
-        ctx, want_rows, requests = build_step(self.kernels, self.dtype, self.device, self.cache, entries,
-                                              self.model.vocab)
+        check_entries(entries, self.cache, self.model.vocab)
+        requests = [(e.slot, len(e.tokens)) for e in entries]
         self.cache.reserve(requests)
         try:
-            tables = self.cache.page_tables([slot for slot, _ in requests])
-            runs = self.model.schedule
-            writes = self.model.run_writes
-            entry_needs = self.model.entry_needs
-
-            def cache_for_run(run):
-                entry = runs[run][1]
-                if entry not in entry_needs or self.model.blocks[runs[run][0]].cache_need() is None:
-                    return None
-                return self.cache.layer_cache(entry, writes[run], tables)
-
-            logits = self.model.forward(ctx, cache_for_run, want_rows)
+            ctx, want_rows, tables = build_step(self.kernels, self.dtype, self.device, self.cache, entries)
+            logits = self.model.forward(ctx, cache_for_runs(self.model, self.cache, tables), want_rows)
         except BaseException:
             self.cache.rollback(requests)
             raise

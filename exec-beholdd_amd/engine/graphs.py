@@ -17,10 +17,10 @@ from __future__ import annotations
 import gc
 import weakref
 
-import numpy as np
 import torch
 
-from ..parts.base import LayerCache, StepContext
+from .step import StepLayout, cache_for_runs
+
 
 def _weakly(engine):
     return engine if isinstance(engine, weakref.ProxyTypes) else weakref.proxy(engine)
@@ -35,28 +35,17 @@ class DecodeGraph:
         # freed at once and not by a later garbage collection
         self.engine, self.n_seqs, self.table_width = _weakly(engine), n_seqs, table_width
         cache = engine.cache
-        self.kv_groups = [index for index, g in enumerate(cache.groups) if g.need.kind == "kv"]
-        b = n_seqs
-        self.n_meta = 8 * b + 1
-        total = self.n_meta + len(self.kv_groups) * b * table_width
-        self.host = torch.zeros(total, dtype=torch.int32).pin_memory()
-        self.device = torch.zeros(total, dtype=torch.int32, device=engine.device)
-        view, at = [], 0
-        for size in (b, b, b, b + 1, b, b, b, b):
-            view.append(self.device[at:at + size])
-            at += size
-        self.tables = {}
-        for index in self.kv_groups:
-            self.tables[index] = self.device[at:at + b * table_width].view(b, table_width)
-            at += b * table_width
-        page = cache.page_size
-        self.ctx = StepContext(
-            kernels=engine.kernels, act_dtype=engine.dtype, device=engine.device, n_rows=b, n_seqs=b,
-            tokens=view[0], positions=view[1], row_seq=view[2], seq_start=view[3], seq_slot=view[4],
-            seq_past=view[5], host_seq_start=None, host_seq_slot=None, host_seq_past=None, is_decode=True,
-            max_position=min(table_width * page, cache.max_position) - 1, max_rows_per_seq=1,
-            token_src=view[7], fed_tokens=engine.sampler.device_tokens)
-        self.want_rows = view[6]
+        self.layout = StepLayout(n_seqs, n_seqs, n_seqs, cache.kv_group_indices(), table_width)
+        self.host = torch.zeros(self.layout.total, dtype=torch.int32).pin_memory()
+        self.device = torch.zeros(self.layout.total, dtype=torch.int32, device=engine.device)
+        self.host_views = self.layout.views(self.host.numpy())
+        views = self.layout.views(self.device)
+        self.tables = views["tables"]
+        self.ctx = self.layout.context(
+            views, engine.kernels, engine.dtype, engine.device, max_rows_per_seq=1,
+            max_position=min(table_width * cache.page_size, cache.max_position) - 1,
+            fed_tokens=engine.sampler.device_tokens)
+        self.want_rows = views["want_rows"]
         self.fed_buffer = engine.sampler.out       # the capture holds its address
         self.graph = None
         self.logits = None
@@ -65,24 +54,16 @@ class DecodeGraph:
 
     def fill(self, entries, pasts):
         """Write this step's numbers into the static buffer (one host-to-device copy)."""
-        b, cache = self.n_seqs, self.engine.cache
+        cache = self.engine.cache
         if self.copied is not None:
             self.copied.synchronize()     # the pinned buffer may not change under a copy in flight
-        host = self.host.numpy()
+        host = self.host_views
+        self.layout.fill(host, [_every_row_wanted(e) for e in entries], pasts)
         slots = [e.slot for e in entries]
-        host[0:b] = [e.tokens[0] if e.fed_row is None else 0 for e in entries]
-        host[7 * b + 1:8 * b + 1] = [-1 if e.fed_row is None else e.fed_row for e in entries]
-        host[b:2 * b] = pasts
-        host[2 * b:3 * b] = np.arange(b)
-        host[3 * b:4 * b + 1] = np.arange(b + 1)
-        host[4 * b + 1:5 * b + 1] = slots
-        host[5 * b + 1:6 * b + 1] = pasts
-        host[6 * b + 1:7 * b + 1] = np.arange(b)
-        at = self.n_meta
-        for index in self.kv_groups:
-            table = host[at:at + b * self.table_width].reshape(b, self.table_width)
+        for index in self.layout.kv_groups:
+            table = host["tables"][index]
             group = cache.groups[index]
-            known = self.known.setdefault(index, [(None, 0)] * b)
+            known = self.known.setdefault(index, [(None, 0)] * self.n_seqs)
             for row, slot in enumerate(slots):
                 pages = group.pages_of[slot]
                 before, count = known[row]
@@ -92,31 +73,23 @@ class DecodeGraph:
                     for j in range(count, len(pages)):
                         table[row, j] = pages[j]
                 else:
-                    table[row, :] = 0
-                    table[row, :len(pages)] = [max(page, 0) for page in pages]
+                    cache.write_page_table(index, [slot], table[row:row + 1])
                 known[row] = (pages, len(pages))
-            at += b * self.table_width
         self.device.copy_(self.host, non_blocking=True)
         self.copied = torch.cuda.Event()
         self.copied.record()
 
     def _forward(self):
         engine = self.engine
-        model, cache = engine.model, engine.cache
-        runs, writes = model.schedule, model.run_writes
-
-        def cache_for_run(run):
-            entry = runs[run][1]
-            if entry not in model.entry_needs or model.blocks[runs[run][0]].cache_need() is None:
-                return None
-            return cache.layer_cache(entry, writes[run], self.tables)
-
-        return model.forward(self.ctx, cache_for_run, self.want_rows)
+        return engine.model.forward(self.ctx, cache_for_runs(engine.model, engine.cache, self.tables), self.want_rows)
 
     def run(self):
-        """Replay (capturing first if need be); the logits tensor is reused by the next run."""
+        """This step's logits.  The first step of a shape runs kernel by kernel (which also loads every kernel
+        before the capture) and is then captured without being run again: a part that keeps state advances it
+        once per step, whether the step was launched or replayed.  Later steps replay the capture; their logits
+        tensor is reused by the next replay."""
         if self.graph is None:
-            self._forward()                      # once eagerly: loads every kernel before the capture
+            logits = self._forward()
             torch.cuda.synchronize(self.engine.device)
             graph = torch.cuda.CUDAGraph()
             # No garbage collection while the stream is capturing: it could free another engine's graphs or
@@ -130,8 +103,17 @@ class DecodeGraph:
                 if collecting:
                     gc.enable()
             self.graph = graph
+            return logits
         self.graph.replay()
         return self.logits
+
+
+class _every_row_wanted:
+    """An entry of a captured step as the layout sees it: the capture computes every row's logits, and the
+    engine picks the wanted ones afterwards."""
+
+    def __init__(self, entry):
+        self.slot, self.tokens, self.fed_row, self.want = entry.slot, entry.tokens, entry.fed_row, (0,)
 
 
 class DecodeGraphs:

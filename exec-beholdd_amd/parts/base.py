@@ -32,6 +32,10 @@ A norm may ride on the products around it (optional, one flag per role):
         prepared form; it hands `x` to the kernel library's products untouched.
 The block joins a producer and a consumer this way only when all three offer it, and runs the norm
 as a step of its own otherwise.
+A mixer with a "state" cache need updates its rows of `cache.state` in place while it runs.  The cache keeps
+what the step's sequences held before the step and puts it back if the step fails, so a mixer needs no
+second bank; and the engine runs a part's forward exactly once per step, whether the step is launched kernel
+by kernel or replayed from a capture, so a state advances once per token.
 A part may declare `graph_safe = True`: its forward uses only the device tensors of the step
 context (never the host_* lists, never a host-side decision that changes from step to step).
 Decode steps of a model whose parts all say so are captured and replayed as HIP graphs.

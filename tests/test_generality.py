@@ -49,6 +49,44 @@ def test_state_is_zero_when_a_slot_is_used_again(tmp_path):
     assert torch.equal(torch.from_numpy(first), torch.from_numpy(again))
 
 
+def test_a_failed_step_puts_the_state_back(tmp_path):
+    """A step that fails after the state mixer has advanced its state leaves the sequence as it was: the
+    retry gives bit for bit what a cache that never saw the failure gives (the rule of the key/value pages,
+    crates/beholdd-model/src/qwen3moe/forward.rs:2937-2998, kept for state of fixed size)."""
+    import numpy as np
+    import schedules
+    from beholdd.engine import StepEntry
+
+    folder = beholdd.write_random_model(str(tmp_path), toy_parts.config_dict("ToyHybridForCausalLM"), seed=3,
+                                        dtype="float32")
+    tokens = schedules.random_requests(101, [30], seed=2)[0]
+    for cut, rest in ((20, tokens[20:]), (29, tokens[29:])):      # a step of several tokens, and a step of one
+        engine = cpu_engine(folder)
+        slot, other = engine.alloc_slot(), engine.alloc_slot()
+        engine.step([StepEntry(slot, tokens[:cut], []), StepEntry(other, tokens[:5], [])])
+        state = [g for g in engine.cache.groups if g.need.kind == "state"][0].state
+        before = state.clone()
+        real, calls = engine.kernels.swiglu, {"n": 0}
+
+        def failing(*a, **k):
+            calls["n"] += 1
+            if calls["n"] == 4:          # the last layer's feed-forward: both state layers have run
+                raise RuntimeError("injected failure")
+            return real(*a, **k)
+
+        engine.kernels.swiglu = failing
+        with pytest.raises(RuntimeError, match="injected"):
+            engine.step([StepEntry(slot, rest, [len(rest) - 1])])
+        engine.kernels.swiglu = real
+        assert torch.equal(state, before) and engine.cache.length(slot) == cut
+        retried = engine.step([StepEntry(slot, rest, [len(rest) - 1])]).numpy()
+        assert not torch.equal(state[:, slot], before[:, slot]) and torch.equal(state[:, other], before[:, other])
+        fresh = cpu_engine(folder)          # the same steps, none of which fails
+        s2, o2 = fresh.alloc_slot(), fresh.alloc_slot()
+        fresh.step([StepEntry(s2, tokens[:cut], []), StepEntry(o2, tokens[:5], [])])
+        assert np.array_equal(retried, fresh.step([StepEntry(s2, rest, [len(rest) - 1])]).numpy())
+
+
 def test_registering_twice_is_refused():
     with pytest.raises(ValueError, match="already registered"):
         beholdd.register_architecture("Qwen3ForCausalLM", beholdd.Qwen3Config, lambda c: None)

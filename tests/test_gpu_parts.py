@@ -49,9 +49,9 @@ def make_ctx(K, dtype, entry_needs, entries, vocab=1000, max_tokens=1024, cache=
     built = []
     for tokens in entries:
         built.append(StepEntry(cache.alloc_slot(), list(tokens), []))
-    ctx, _, requests = build_step(K, dtype, DEVICE, cache, built, vocab)
+    requests = [(entry.slot, len(entry.tokens)) for entry in built]
     cache.reserve(requests)
-    tables = cache.page_tables([slot for slot, _ in requests])
+    ctx, _, tables = build_step(K, dtype, DEVICE, cache, built)
     return ctx, cache, tables, requests
 
 
@@ -190,9 +190,9 @@ def test_attention_part_in_two_steps(K, dtype, n_heads, kv_heads, head_dim, eps,
             lo, hi = (0, p) if phase == 0 else (p, p + n)
             entries.append(StepEntry(slots[s], [0] * (hi - lo), []))
             inputs.append(x[s][lo:hi])
-        ctx, _, requests = build_step(K, dtype, DEVICE, cache, entries, 10)
+        requests = [(entry.slot, len(entry.tokens)) for entry in entries]
         cache.reserve(requests)
-        tables = cache.page_tables(slots)
+        ctx, _, tables = build_step(K, dtype, DEVICE, cache, entries)
         residual = torch.zeros(ctx.n_rows, hidden_size, device=DEVICE)
         part.forward(ctx, torch.cat(inputs).to(DEVICE), residual, cache.layer_cache(0, True, tables))
         cache.commit(requests)

@@ -20,7 +20,11 @@ DECAY = 0.75
 
 class ToyRunningMeanMixer:
     """state <- DECAY * state + x_t for every token in order; output = W state.
-    Keeps one float32 vector per sequence: a cache need of kind "state"."""
+    Keeps one float32 vector per sequence: a cache need of kind "state".  A step of one token per sequence
+    uses the step's device tensors only, so decode steps of a model with this mixer may be captured and
+    replayed; steps of several tokens are never captured and scan on the host."""
+
+    graph_safe = True
 
     def __init__(self, hidden: int, prefix: str):
         self.hidden, self.name = hidden, prefix + "toy_mix.weight"
@@ -36,6 +40,12 @@ class ToyRunningMeanMixer:
         return CacheNeed(kind="state", state_shape=(self.hidden,), state_dtype=torch.float32)
 
     def forward(self, ctx, x, hidden, cache):
+        if ctx.is_decode:
+            slots = ctx.seq_slot.long()
+            state = cache.state.index_select(0, slots) * DECAY + x.float()
+            cache.state.index_copy_(0, slots, state)
+            ctx.kernels.gemm(state, self.weight, hidden, accumulate=True)
+            return
         for b in range(ctx.n_seqs):
             lo, hi = ctx.host_seq_start[b], ctx.host_seq_start[b + 1]
             state = cache.state[ctx.host_seq_slot[b]]
