@@ -10,14 +10,14 @@ The folder's name is not a Python identifier; import it with
 """
 
 from . import config, weights, parts, cache, kernels, sampling, registry, models, engine, cli   # noqa: F401
-from .config import ConfigError, Qwen3Config
-from .engine import Engine, GenerationResult, StepEntry, load_model
+from .config import ConfigError, ConfigReader, LayerKinds, Qwen3Config
+from .engine import Engine, GenerationResult, MemoryBudgetError, StepEntry, load_model
 from .registry import register_architecture, registered_architectures, resolve_architecture
 from .sampling import SamplingParams
 from .weights import WeightError, write_random_model
 
 __version__ = "0.1.0"
 
-__all__ = ["ConfigError", "Qwen3Config", "Engine", "GenerationResult", "StepEntry", "load_model",
+__all__ = ["ConfigError", "ConfigReader", "LayerKinds", "MemoryBudgetError", "Qwen3Config", "Engine", "GenerationResult", "StepEntry", "load_model",
            "register_architecture", "registered_architectures", "resolve_architecture", "SamplingParams",
            "WeightError", "write_random_model"]

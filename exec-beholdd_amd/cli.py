@@ -22,6 +22,7 @@ USAGE = """usage:
                    [--seed N] [--stop-token-ids a,b] [--max-tokens N] [--slots N] [--batch-size N]
                    [--logits-out PATH] [--step-timing-out PATH] [--memory-budget-bytes N] [--plan-only]
   beholdd random-model --config FILE --out DIR [--seed N] [--dtype bfloat16|float32]
+  beholdd compare REFERENCE CANDIDATE [--tolerance X]
   beholdd architectures"""
 
 
@@ -99,7 +100,9 @@ def _generate(args: list, out) -> int:
     top_p = _number(flags, "--top-p", 1.0, float)
     seed = _number(flags, "--seed", 0)
     stops = _ids(flags["--stop-token-ids"], "--stop-token-ids") if "--stop-token-ids" in flags else None
-    page = 64
+    from .kernels.build import source_page_size
+
+    page = source_page_size()
     default_tokens = sum(-(-(len(p) + max_new) // page) * page for p in prompts)
     max_tokens = _number(flags, "--max-tokens", default_tokens)
     slots = _number(flags, "--slots", None)
@@ -118,23 +121,22 @@ def _generate(args: list, out) -> int:
     dtype = flags.get("--dtype", "bfloat16")
 
     if "--plan-only" in flags:
-        import torch
         from .cache import SequenceCache
-        from .engine import parse_dtype
+        from .engine import open_model, parse_dtype
 
-        model = entry.build(config)
-        size = 4 if parse_dtype(dtype) == torch.float32 else 2
-        weight_bytes = 0
-        for spec in model.tensor_specs():
-            count = 1
-            for axis in spec.shape:
-                count *= axis
-            weight_bytes += count * size
+        model, weights = open_model(flags["--model"], dtype, "cpu")      # the header only: no tensor is read
+        try:
+            weight_bytes = weights.planned_bytes(model.tensor_specs())
+        finally:
+            weights.reader.close()
         cache = SequenceCache(model.entry_needs, max_tokens, parse_dtype(dtype), "cpu", page, max_slots=slots,
-                              max_position=config.max_position)
+                              max_position=model.max_position)
+        total = weight_bytes + cache.plan().total_bytes
         print(f"weights: {weight_bytes} bytes", file=out)
         print(cache.plan().describe(), file=out)
-        return 0
+        print(f"total: {total} bytes" + (f" (budget {budget}: {'fits' if total <= budget else 'does not fit'})"
+                                         if budget is not None else ""), file=out)
+        return 0 if budget is None or total <= budget else 1
 
     from .engine import Engine
     from .engine.artifact import write_logits_artifact
@@ -206,6 +208,34 @@ def _random_model(args: list, out) -> int:
     return 0
 
 
+def _compare(args: list, out) -> int:
+    """Two logits captures: equal descriptors, then
+    equal bytes, or with --tolerance X logits within X of the largest logit.  In the manner of the reference's
+    tools/compare_logits.py:291-316: FAIL with the reason, or the shape, the SHA-256 and PASS."""
+    paths = [a for a in args[:2] if not a.startswith("--")]
+    if len(paths) != 2:
+        raise UsageError("compare needs two captures")
+    flags = _parse_flags(args[2:], valued={"--tolerance"}, switches=set())
+    tolerance = _number(flags, "--tolerance", 0.0, float)
+    if not tolerance >= 0.0:
+        raise UsageError("--tolerance is not negative")
+    from .engine.artifact import ArtifactError
+    from .engine.compare import CompareError, compare
+    try:
+        report = compare(paths[0], paths[1], tolerance)
+    except (CompareError, ArtifactError, OSError) as error:
+        print(f"FAIL: {error}", file=out)
+        return 1
+    print(f"  shape: requests={report['requests']}, rows={report['rows']}, vocab={report['vocab']}", file=out)
+    if tolerance == 0.0:
+        print(f"  SHA-256: {report['sha256']}", file=out)
+        print("  Exact logit comparison: PASS", file=out)
+    else:
+        print(f"  largest difference: {report['error']:.3e} of the largest logit ({report['worst']})", file=out)
+        print(f"  Logit comparison within {tolerance:g}: PASS", file=out)
+    return 0
+
+
 def main(argv=None, out=None) -> int:
     argv = list(sys.argv[1:] if argv is None else argv)
     out = out or sys.stdout
@@ -218,6 +248,8 @@ def main(argv=None, out=None) -> int:
             return _generate(rest, out)
         if command == "random-model":
             return _random_model(rest, out)
+        if command == "compare":
+            return _compare(rest, out)
         if command == "architectures":
             from .registry import registered_architectures
             print("\n".join(registered_architectures()), file=out)

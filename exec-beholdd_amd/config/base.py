@@ -10,10 +10,28 @@ from __future__ import annotations
 import json
 import math
 import os
+from dataclasses import dataclass
 
 
 class ConfigError(ValueError):
     """config.json is missing, malformed, or asks for something that is not implemented."""
+
+
+@dataclass(frozen=True)
+class LayerKinds:
+    """Which parts one layer is made of; the model builder looks each name up in the part registries.
+
+    Any configuration class can describe a decoder to `models.build_decoder` with
+        layer_kinds() -> list[LayerKinds]      one per layer
+        schedule()    -> list[(layer index, cache entry index)]
+        vocab, hidden, max_position            the sizes the generic builder reads itself
+        tie_word_embeddings                    optional, false when absent
+    Everything else (head counts, widths, constants) is read only by the builders registered for the part
+    names it uses, so a configuration with other field names registers builders of its own."""
+    mixer: str
+    feed_forward: str
+    norm: str
+    block: str
 
 
 _MISSING = object()

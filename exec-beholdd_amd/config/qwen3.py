@@ -10,16 +10,7 @@ from __future__ import annotations
 
 from dataclasses import dataclass, field
 
-from .base import ConfigError, ConfigReader
-
-
-@dataclass(frozen=True)
-class LayerKinds:
-    """Which parts one layer is made of; the model builder looks each name up in the part registries."""
-    mixer: str
-    feed_forward: str
-    norm: str
-    block: str
+from .base import ConfigError, ConfigReader, LayerKinds
 
 
 @dataclass(frozen=True)

@@ -35,8 +35,15 @@ def parse_dtype(name) -> torch.dtype:
         raise ValueError(f"engine dtype must be bfloat16 or float32, got {name!r}") from None
 
 
+class MemoryBudgetError(RuntimeError):
+    """Weights and cache together would take more device memory than the caller allows; nothing was loaded."""
+
+
 class Engine:
-    """`Engine(model_dir, dtype, max_tokens)`; then `step(...)` or `generate(...)`."""
+    """`Engine(model_dir, dtype, max_tokens)`; then `step(...)` or `generate(...)`.  `memory_limit_bytes`
+    bounds weights and cache together and is checked from the checkpoint's header and the cache's sizes
+    before a tensor is read or the cache allocated (the reference enforces its limits before any I/O,
+    crates/beholdd-model/src/qwen3moe/recorded_attention.rs:344-365)."""
 
     def __init__(self, model_dir: str | None = None, dtype="bfloat16", max_tokens: int = 4096,
                  max_slots: int | None = None, device="cuda:0", kernels=None, model=None,
@@ -47,17 +54,37 @@ class Engine:
             from ..kernels import HipKernels   # fails loudly without a GPU or the library
             kernels = HipKernels(self.device)
         self.kernels = kernels
+
+        def make_cache(built):
+            return SequenceCache(built.entry_needs, max_tokens, self.dtype, self.device, kernels.page_size,
+                                 max_slots=max_slots, max_position=built.max_position)
+
+        def within_budget(weight_bytes, cache):
+            total = weight_bytes + cache.plan().total_bytes
+            if memory_limit_bytes is not None and total > memory_limit_bytes:
+                raise MemoryBudgetError(f"weights ({weight_bytes} bytes) and cache ({cache.plan().total_bytes} bytes) "
+                                        f"need {total} bytes, the limit is {memory_limit_bytes}")
+
         if model is None:
             if model_dir is None:
                 raise ValueError("give a model folder or a built model")
-            model = load_model(model_dir, self.dtype, self.device)
+            model, weights = open_model(model_dir, self.dtype, self.device)
+            try:
+                self.weight_bytes = weights.planned_bytes(model.tensor_specs())
+                self.cache = make_cache(model)
+                within_budget(self.weight_bytes, self.cache)
+                model.load(weights, self.device)
+            finally:
+                weights.reader.close()
+        else:
+            self.weight_bytes = sum(t.numel() * t.element_size() for t in _model_tensors(model))
+            self.cache = make_cache(model)
+            within_budget(self.weight_bytes, self.cache)
         self.model = model
         self.config = model.config
         if hasattr(model, "prepare"):
             model.prepare(kernels)
-        self.cache = SequenceCache(model.entry_needs, max_tokens, self.dtype, self.device, kernels.page_size,
-                                   max_slots=max_slots, max_position=model.max_position)
-        self.cache_plan = self.cache.allocate(limit_bytes=memory_limit_bytes)
+        self.cache_plan = self.cache.allocate()
         self.sampler = Sampler(kernels, self.device, capacity=self.cache.max_slots)
         self._last_selection = None
         self.graphs = DecodeGraphs(self) if use_graphs and self.device.type == "cuda" else None
@@ -149,8 +176,7 @@ class Engine:
                                    batch_size, control, on_logits)
 
     def memory_plan(self) -> str:
-        weights = sum(t.numel() * t.element_size() for t in _model_tensors(self.model))
-        return f"weights: {weights} bytes\n{self.cache_plan.describe()}"
+        return f"weights: {self.weight_bytes} bytes\n{self.cache_plan.describe()}"
 
 
 def _model_tensors(model):
@@ -173,14 +199,20 @@ def _model_tensors(model):
     return out
 
 
-def load_model(model_dir: str, dtype, device):
-    """config.json -> architecture -> model; model.safetensors -> its tensors, bound by name."""
+def open_model(model_dir: str, dtype, device):
+    """config.json -> architecture -> model (no tensors yet), and the checkpoint's tensors bound to it by name
+    with nothing read yet.  The caller loads (`model.load(weights, device)`) and closes `weights.reader`."""
     dtype = parse_dtype(dtype)
     data, path = read_config_json(model_dir)
     entry = resolve_architecture(data, path)
     config = entry.config_class.from_dict(data, path)
     model = entry.build(config)
-    weights = bind(model.tensor_specs(), model_dir, dtype, device)
+    return model, bind(model.tensor_specs(), model_dir, dtype, device)
+
+
+def load_model(model_dir: str, dtype, device):
+    """config.json -> architecture -> model; model.safetensors -> its tensors, bound by name."""
+    model, weights = open_model(model_dir, dtype, device)
     try:
         model.load(weights, device)
     finally:

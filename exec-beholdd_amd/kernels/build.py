@@ -32,6 +32,17 @@ class BuildError(RuntimeError):
     pass
 
 
+def source_page_size() -> int:
+    """Tokens in one page of the key/value cache: `BH_PAGE` of csrc/common.h, the one place that says so.
+    (The built library reports the same number as `bh_page_size()`; this reads it where no library is loaded.)"""
+    with open(os.path.join(CSRC, "common.h"), "r", encoding="utf-8") as handle:
+        for line in handle:
+            words = line.split()
+            if len(words) >= 3 and words[0] == "#define" and words[1] == "BH_PAGE":
+                return int(words[2])
+    raise BuildError("csrc/common.h does not define BH_PAGE")
+
+
 def _hipcc() -> str:
     for candidate in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
         if candidate and os.path.exists(candidate):

@@ -78,6 +78,9 @@ class HipKernels:
         self.library_path = path
         self._declare()
         self.page_size = int(self.lib.bh_page_size())
+        if self.page_size != _build.source_page_size():
+            raise KernelError(f"{path} was built for pages of {self.page_size} tokens, the sources say "
+                              f"{_build.source_page_size()}: build the library again")
 
     # ---- ctypes declarations ----
     def _declare(self):

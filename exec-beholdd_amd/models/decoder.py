@@ -89,20 +89,32 @@ class DecoderModel:
         return self.head.forward(ctx, self.final_norm.forward(ctx, hidden, rows=want_rows))
 
 
-def build_decoder(config, position_encoding: str = "rope", layer_prefix: str = "model.layers.{}.",
+def build_decoder(config, position_encoding="rope", layer_prefix: str = "model.layers.{}.",
                   embedding_name: str = "model.embed_tokens.weight", final_norm_name: str = "model.norm.weight",
-                  head_name: str = "lm_head.weight", final_norm_kind: str = "rmsnorm") -> DecoderModel:
-    """Put a decoder together from the registered parts that `config` names."""
+                  head_name: str = "lm_head.weight", final_norm_kind: str = "rmsnorm",
+                  make_embedding=None, make_head=None) -> DecoderModel:
+    """Put a decoder together from the registered parts that `config` names.
+
+    `position_encoding` is the registered name of the one encoding that all layers share, or a dictionary
+    label -> registered name when layers differ: part builders find them in `shared["position_encodings"][label]`
+    (and the one labelled "default", or the first, in `shared["position_encoding"]`).  `make_embedding(config)` and
+    `make_head(config, embedding)` replace the plain embedding and head (a scaled embedding, a head that caps
+    its logits); each returns a part with the interface of `parts.embedding`'s."""
     shared = {}
-    shared["position_encoding"] = POSITION_ENCODINGS.get(position_encoding)(config, shared)
-    embedding = Embedding(config.vocab, config.hidden, embedding_name)
+    labelled = position_encoding if isinstance(position_encoding, dict) else {"default": position_encoding}
+    encodings = {label: POSITION_ENCODINGS.get(name)(config, shared) for label, name in labelled.items()}
+    shared["position_encodings"] = encodings
+    shared["position_encoding"] = encodings.get("default", next(iter(encodings.values())))
+    embedding = make_embedding(config) if make_embedding else Embedding(config.vocab, config.hidden, embedding_name)
     blocks = []
     for index, kinds in enumerate(config.layer_kinds()):
         blocks.append(BLOCKS.get(kinds.block)(config, index, layer_prefix.format(index), kinds, shared))
     final_norm = NORMS.get(final_norm_kind)(config, config.hidden, final_norm_name, shared)
-    if getattr(config, "tie_word_embeddings", False):
+    if make_head:
+        head = make_head(config, embedding)
+    elif getattr(config, "tie_word_embeddings", False):
         head = LMHead(config.vocab, config.hidden, None, tied_to=embedding)
     else:
         head = LMHead(config.vocab, config.hidden, head_name)
     return DecoderModel(config, embedding, blocks, config.schedule(), final_norm, head,
-                        shared_parts=[shared["position_encoding"]])
+                        shared_parts=list(encodings.values()))

@@ -91,6 +91,19 @@ class BoundWeights:
         self.engine_dtype = engine_dtype
         self.device = device
 
+    def planned_bytes(self, specs: list) -> int:
+        """Device bytes that the tensors of `specs` will take under the storage rule, from the file's
+        header alone (no payload is read)."""
+        total = 0
+        for spec in specs:
+            entry = self.reader.entries[spec.name]
+            count = 1
+            for axis in entry.shape:
+                count *= int(axis)
+            kept = stored_dtype(entry.torch_dtype, self.engine_dtype)
+            total += count * torch.empty((), dtype=kept).element_size()
+        return total
+
     def __call__(self, name: str) -> torch.Tensor:
         source = self.reader.tensor(name)
         target = stored_dtype(source.dtype, self.engine_dtype)

@@ -107,6 +107,37 @@ def portions(engine, requests, sizes=(2, 62, 1, 64, 2, 63, 1, 1, 65, 3, 61), res
     return [np.concatenate(r, axis=0) for r in rows]
 
 
+class TraceRecorder:
+    """Stands where an engine stands in the functions above and writes down what they do, as the steps of a
+    trace for bin/trace_run: requests are named r0, r1, ... in the order in which they get their slots."""
+
+    def __init__(self):
+        self.steps, self.name_of, self.started = [], {}, 0
+
+    def alloc_slot(self):
+        slot = self.started
+        self.name_of[slot] = f"r{self.started}"
+        self.started += 1
+        return slot
+
+    def free_slot(self, slot):
+        self.steps[-1]["end"].append(self.name_of.pop(slot))
+
+    def step(self, entries):
+        import torch
+        self.steps.append({"step": len(self.steps), "end": [],
+                           "entries": [{"id": self.name_of[e.slot], "tokens": [int(t) for t in e.tokens],
+                                        "want": [int(w) for w in e.want]} for e in entries]})
+        return torch.zeros(sum(len(e.want) for e in entries), 1)
+
+
+def trace_of(schedule, requests, **options):
+    """The steps that `schedule(engine, requests, **options)` would run, as trace records."""
+    recorder = TraceRecorder()
+    schedule(recorder, requests, **options)
+    return recorder.steps
+
+
 def relative_error(got, want):
     """max |got - want| / max |want|: the measure the acceptance tolerance is stated in."""
     return float(np.abs(got.astype(np.float64) - want.astype(np.float64)).max() / np.abs(want).max())

@@ -64,6 +64,17 @@ def test_plan_only_accounts_for_bytes_without_a_gpu(model_dirs):
     assert f"{3 * 2 * 4 * 2 * 64 * 32 * 2} bytes" in text
 
 
+def test_plan_only_holds_weights_and_cache_against_the_budget(model_dirs):
+    common = ["generate", "--model", model_dirs("B", "float32"), "--prompt-ids", "1,2,3", "--max-new-tokens", "10",
+              "--dtype", "bfloat16", "--plan-only", "--memory-budget-bytes"]
+    # stored in 32-bit: stays so in a bfloat16 engine; one page of cache for 3 layers
+    total = 397_152 * 4 + 3 * 2 * 1 * 2 * 64 * 32 * 2
+    code, text = run(common + [str(total)])
+    assert code == 0 and f"total: {total} bytes (budget {total}: fits)" in text
+    code, text = run(common + [str(total - 1)])
+    assert code == 1 and "does not fit" in text
+
+
 def test_random_model_command_writes_a_loadable_folder(tmp_path, tiny_configs):
     config = tmp_path / "c.json"
     config.write_text(json.dumps(tiny_configs["A"]))
@@ -96,7 +107,7 @@ def test_trace_replay_on_the_kernel_double(model_dirs, tmp_path):
     folder = model_dirs("A", "float32")
     cfg, weights = plain.load_plain(folder)
     engine = Engine(folder, dtype="float32", max_tokens=128, device="cpu", kernels=TorchKernels())
-    player = replay.Replayer(engine, str(tmp_path / "out"))
+    player = replay.Replayer(engine, str(tmp_path / "out"), str(tmp_path / "capture.bhdlogit"))
     a, b = [5, 17, 3, 9], [7, 8]
     player.run_step({"step": 0, "entries": [{"id": "a", "tokens": a[:3], "want": [0, 2]}, {"id": "b", "tokens": b[:1], "want": []}], "end": []})
     player.run_step({"step": 1, "entries": [{"id": "a", "tokens": a[3:], "want": [0]}, {"id": "b", "tokens": b[1:], "want": [0]}], "end": ["b"]})
@@ -112,3 +123,105 @@ def test_trace_replay_on_the_kernel_double(model_dirs, tmp_path):
     with pytest.raises(Exception):
         player.run_step({"step": 4, "entries": [{"id": "c", "tokens": [999], "want": [0]}], "end": []})
     assert engine.cache.live_slots() == [] and "c" not in player.slot_of      # a refused start leaves no slot behind
+    # step numbers: integers that are not negative, each once; nothing is written for a refused one
+    for bad, message in (("../../x", "non-negative integer"), (-1, "non-negative integer"), (1.5, "non-negative integer"),
+                         (True, "non-negative integer"), (1, "occurs twice")):
+        with pytest.raises(replay.TraceError, match=message):
+            player.run_step({"step": bad, "entries": [{"id": "d", "tokens": [1], "want": [0]}], "end": ["d"]})
+    assert engine.cache.live_slots() == []
+    # an id that is used again after its request ended is another request in the capture
+    player.run_step({"step": 5, "entries": [{"id": "a", "tokens": b, "want": [1]}], "end": ["a"]})
+    player.close()
+    assert sorted(os.listdir(tmp_path / "out")) == ["0.f32", "1.f32", "5.f32"]
+    from beholdd.engine.artifact import read_position_capture
+    capture = read_position_capture(str(tmp_path / "capture.bhdlogit"))
+    assert capture.requests == {"a": a, "b": b, "a#1": b}
+    assert capture.rows == [("a", 0, 0), ("a", 2, 0), ("a", 3, 1), ("b", 1, 1), ("a#1", 1, 5)]
+    assert np.array_equal(capture.logits[:2], got0) and np.array_equal(capture.logits[2:4], got1)
+    assert np.allclose(capture.logits[4], wb[1], atol=1e-4) and capture.notes == {}
+    # without a capture path the replay writes the bare rows only
+    bare = replay.Replayer(engine, str(tmp_path / "bare"))
+    bare.run_step({"step": 0, "entries": [{"id": "a", "tokens": a, "want": [3]}], "end": ["a"]})
+    bare.close()
+    assert os.listdir(tmp_path / "bare") == ["0.f32"] and engine.cache.live_slots() == []
+
+
+def test_position_capture_round_trip_and_refusals(tmp_path):
+    import numpy as np
+    from beholdd.engine.artifact import ArtifactError, PositionCaptureWriter, read_position_capture
+
+    path = str(tmp_path / "c.bin")
+    rows = np.arange(15, dtype=np.float32).reshape(3, 5)
+    writer = PositionCaptureWriter(path, 5, {"dtype": "float32"})
+    assert writer.feed("long name é", [1, 2]) == 0 and writer.feed("long name é", [3]) == 2
+    writer.feed("x", [4])
+    writer.add(0, [("long name é", 1), ("x", 0)], rows[:2])
+    with pytest.raises(ArtifactError, match="no position 3"):
+        writer.add(1, [("long name é", 3)], rows[2:])
+    with pytest.raises(ArtifactError, match="not finite"):
+        writer.add(1, [("long name é", 2)], np.full((1, 5), np.inf, np.float32))
+    writer.add(7, [("long name é", 2)], rows[2:])
+    assert not os.path.exists(path)             # nothing under the final name until the capture is complete
+    writer.close()
+    capture = read_position_capture(path)
+    assert capture.requests == {"long name é": [1, 2, 3], "x": [4]} and capture.notes == {"dtype": "float32"}
+    assert capture.rows == [("long name é", 1, 0), ("x", 0, 0), ("long name é", 2, 7)]
+    assert np.array_equal(capture.logits, rows)
+    with pytest.raises(ArtifactError, match="never overwritten"):
+        PositionCaptureWriter(path, 5)
+    data = open(path, "rb").read()
+    for broken, message in ((data[:-1], "bad footer"), (data[:40] + b"\x09" + data[41:], "do not agree|not a version"),
+                            (data[:64] + b"\x00\x00\x80\x7f" + data[68:], "not finite"),
+                            (data[:8] + b"\x01" + data[9:], "not a version-2")):
+        bad = tmp_path / "bad.bin"
+        bad.write_bytes(broken)
+        with pytest.raises(ArtifactError, match=message):
+            read_position_capture(str(bad))
+
+
+def test_compare_command(tmp_path, capsys):
+    import numpy as np
+    from beholdd.engine.artifact import PositionCaptureWriter, write_logits_artifact
+
+    rng = np.random.default_rng(0)
+    base = {("a", i): rng.normal(size=9).astype(np.float32) for i in range(4)}
+    base.update({("b", i): rng.normal(size=9).astype(np.float32) for i in range(2)})
+
+    def make(name, order, noise=0.0, tokens_b=(6, 0)):
+        writer = PositionCaptureWriter(str(tmp_path / name), 9)
+        writer.feed("a", [1, 2, 3, 4])
+        writer.feed("b", list(tokens_b))
+        for step, places in enumerate(order):
+            writer.add(step, places, np.stack([base[p] + np.float32(noise) for p in places]))
+        writer.close()
+        return str(tmp_path / name)
+
+    whole = make("whole", [[("a", 0), ("a", 3)], [("b", 1)]])
+    again = make("again", [[("a", 0), ("a", 3)], [("b", 1)]])
+    batched = make("batched", [[("b", 1), ("a", 3)], [("a", 0)]], noise=1e-6)
+    fewer = make("fewer", [[("a", 0), ("a", 3)]])
+    other = make("other", [[("a", 0), ("a", 3)], [("b", 1)]], tokens_b=(6, 1))
+    code, text = run(["compare", whole, again])
+    assert code == 0 and "Exact logit comparison: PASS" in text and "SHA-256" in text
+    code, text = run(["compare", whole, batched, "--tolerance", "1e-5"])
+    assert code == 0 and "within 1e-05: PASS" in text
+    for candidate, tolerance, message in ((batched, "0", "same schedule"), (batched, "1e-9", "logits differ by"),
+                                          (fewer, "1e-3", "different positions"), (other, "1e-3", "tokens of request 'b'"),
+                                          (str(tmp_path / "missing"), "0", "No such file")):
+        code, text = run(["compare", whole, candidate, "--tolerance", tolerance])
+        assert code == 1 and text.startswith("FAIL:") and message in text, text
+    # equal descriptors and rows, one differing byte: the offset and both sums are reported
+    data = bytearray(open(whole, "rb").read())
+    data[70] ^= 1
+    (tmp_path / "flipped").write_bytes(bytes(data))
+    code, text = run(["compare", whole, str(tmp_path / "flipped")])
+    assert code == 1 and "differ at offset 70" in text and text.count("SHA-256") == 2
+    # captures of one request's generated steps compare the same way
+    logits = rng.normal(size=(2, 9)).astype(np.float32)
+    tokens = [int(row.argmax()) for row in logits]
+    for name in ("g1", "g2"):
+        write_logits_artifact(str(tmp_path / name), [1, 2], tokens, logits)
+    assert run(["compare", str(tmp_path / "g1"), str(tmp_path / "g2")])[0] == 0
+    assert run(["compare", str(tmp_path / "g1"), whole])[0] == 1
+    assert run(["compare", whole])[0] == 2
+

@@ -113,6 +113,24 @@ def test_a_reused_slot_gives_the_same_logits_as_a_fresh_cache(model_dirs):
     assert not np.array_equal(first[:75], second)
 
 
+def test_memory_limit_covers_weights_and_cache_and_is_checked_before_anything_is_read(model_dirs, monkeypatch):
+    from beholdd.engine import MemoryBudgetError
+    from beholdd.weights import binder
+
+    folder = model_dirs("A", "bfloat16")
+    weights = 90_496 * 2                                  # tiny A in bfloat16 (tied head: the embedding once)
+    cache = 2 * 2 * 2 * 2 * 64 * 16 * 2                   # 2 layers, keys and values, 2 pages, 2 heads, 64 x 16
+    reads = []
+    real = binder.BoundWeights.__call__
+    monkeypatch.setattr(binder.BoundWeights, "__call__", lambda self, name: reads.append(name) or real(self, name))
+    with pytest.raises(MemoryBudgetError, match=f"need {weights + cache} bytes"):
+        make_engine(folder, dtype="bfloat16", max_tokens=128, memory_limit_bytes=weights + cache - 1)
+    assert reads == []
+    engine = make_engine(folder, dtype="bfloat16", max_tokens=128, memory_limit_bytes=weights + cache)
+    assert len(reads) == 24 and engine.weight_bytes == weights and engine.cache.allocated_bytes() == cache
+    assert f"weights: {weights} bytes" in engine.memory_plan()
+
+
 def test_unknown_architecture_names_the_registered_ones(tmp_path, tiny_configs):
     config = dict(tiny_configs["A"], architectures=["Qwen9ForCausalLM"])
     with pytest.raises(beholdd.ConfigError, match="Qwen3ForCausalLM"):

@@ -22,7 +22,8 @@ def cpu_engine(folder):
     return Engine(folder, dtype="float32", max_tokens=1024, device="cpu", kernels=TorchKernels())
 
 
-@pytest.mark.parametrize("architecture", ["ToyHybridForCausalLM", "ToyTwiceForCausalLM", "ToySharedCacheForCausalLM"])
+@pytest.mark.parametrize("architecture", ["ToyHybridForCausalLM", "ToyTwiceForCausalLM", "ToySharedCacheForCausalLM",
+                                          "ToyOwnForCausalLM"])
 def test_toy_architectures_step_like_their_plain_forms(tmp_path, architecture):
     folder = beholdd.write_random_model(str(tmp_path), toy_parts.config_dict(architecture), seed=3, dtype="float32")
     engine = toy_parts.check_architecture(architecture, folder, cpu_engine, 1e-4)
@@ -34,6 +35,25 @@ def test_toy_architectures_step_like_their_plain_forms(tmp_path, architecture):
         assert state.shape == (2, engine.cache.max_slots, 48)
     elif architecture == "ToyTwiceForCausalLM":
         assert sorted(needs) == [0, 1, 2, 3, 4] and engine.model.run_writes == [True] * 5
+    elif architecture == "ToyOwnForCausalLM":
+        # a configuration class of its own, tensors under names of its own, a routed feed-forward whose
+        # experts are all in use, a rotation of part of each head
+        assert not isinstance(engine.config, beholdd.Qwen3Config)
+        names = {spec.name for spec in engine.model.tensor_specs()}
+        assert "symbols.weight" in names and "blocks.0.routed.experts.2.down_proj.weight" in names
+        assert not any(name.startswith("model.") for name in names)
+        import schedules
+        from beholdd.engine import StepEntry
+        tokens = schedules.random_requests(90, [120], seed=4)[0]
+        slot = engine.alloc_slot()
+        engine.step([StepEntry(slot, tokens, [])])
+        engine.free_slot(slot)
+        _, weights = toy_parts.load_plain_weights(folder)
+        _, routing = toy_parts.plain_own_logits(toy_parts.OWN, weights, tokens)
+        routed = [block.feed_forward for block in engine.model.blocks[::2]]
+        for part, want in zip(routed, routing):
+            assert part.last_routing.tolist() == want.tolist()
+        assert sorted(set(routing[0].tolist())) == [0, 1, 2]
     else:
         assert sorted(needs) == [0, 2] and engine.model.run_writes == [True, False, True, False]
 

@@ -414,8 +414,8 @@ def test_trace_replay_program(model_dirs, tmp_path, dtype):
     trace = "\n".join(json.dumps(s) for s in steps) + "\n"
     # live tokens, each request rounded up to 64: a 64 + b 128 + c 64 = 256 at most
     run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
-                          "--out", str(out_dir), "--max-tokens", "256"], input=trace, capture_output=True, text=True,
-                         timeout=600)
+                          "--out", str(out_dir), "--max-tokens", "256", "--capture", str(tmp_path / "capture")],
+                         input=trace, capture_output=True, text=True, timeout=600)
     assert run.returncode == 0, run.stderr[-2000:]
     assert [line for line in run.stdout.splitlines() if line.startswith("done")] == [f"done {s['step']}" for s in steps]
     assert sorted(os.listdir(out_dir)) == sorted(f"{n}.f32" for n in expect)
@@ -423,6 +423,60 @@ def test_trace_replay_program(model_dirs, tmp_path, dtype):
         got = np.fromfile(out_dir / f"{number}.f32", dtype="<f4").reshape(-1, cfg.vocab)
         assert got.shape == rows.shape
         assert schedules.relative_error(got, rows) < TOLERANCE[dtype], number
+    from beholdd.engine.artifact import read_position_capture
+    capture = read_position_capture(str(tmp_path / "capture"))
+    assert capture.requests == requests and len(capture.rows) == sum(len(rows) for rows in expect.values())
+    assert np.array_equal(capture.logits[:len(expect[0])], np.fromfile(out_dir / "0.f32", dtype="<f4").reshape(-1, cfg.vocab))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replays_of_different_cuts_compare_through_the_tool(model_dirs, tmp_path, dtype):
+    """Capture, then compare: the same requests replayed whole, in batches of unequal lengths and in portions;
+    every replay leaves a capture that says which request and position each row belongs to, and `beholdd compare`
+    holds any two of them, and the plain implementation's logits written as such a capture, to the tolerance;
+    the same schedule replayed twice compares equal byte for byte."""
+    import io
+    from beholdd import cli
+    from beholdd.engine import replay
+    from beholdd.engine.artifact import PositionCaptureWriter
+
+    folder = model_dirs("B", "bfloat16")
+    cfg, weights = plain.load_plain(folder)
+    requests = schedules.random_requests(cfg.vocab, [40, 70, 9, 64, 130], seed=12)
+    traces = {"whole": schedules.trace_of(schedules.whole, requests),
+              "batches": schedules.trace_of(schedules.batches, requests, batch_size=3),
+              "again": schedules.trace_of(schedules.batches, requests, batch_size=3),
+              "portions": schedules.trace_of(schedules.portions, requests)}
+    for name, steps in traces.items():
+        lines = io.StringIO("".join(json.dumps(step) + "\n" for step in steps))
+        said = io.StringIO()
+        code = replay.main(["--model", folder, "--dtype", dtype, "--out", str(tmp_path / f"{name}.out"), "--max-tokens", "512",
+                            "--capture", str(tmp_path / name)], stdin=lines, stdout=said)
+        assert code == 0 and said.getvalue().splitlines() == [f"done {step['step']}" for step in steps]
+    writer = PositionCaptureWriter(str(tmp_path / "plain.bhdlogit"), cfg.vocab, {"tool": "plain implementation"})
+    for index, tokens in enumerate(requests):
+        writer.feed(f"r{index}", tokens)
+        writer.add(index, [(f"r{index}", position) for position in range(len(tokens))], plain.forward_logits(cfg, weights, tokens))
+    writer.close()
+
+    def compare(a, b, tolerance):
+        out = io.StringIO()
+        code = cli.main(["compare", str(tmp_path / a), str(tmp_path / b), "--tolerance", str(tolerance)], out=out)
+        return code, out.getvalue()
+
+    between_cuts = 5e-5 if dtype == "float32" else 1e-2
+    for name in ("batches", "portions"):
+        code, text = compare("whole", name, between_cuts)
+        assert code == 0 and "PASS" in text, text
+    for name in ("whole", "batches", "portions"):
+        code, text = compare("plain.bhdlogit", name, TOLERANCE[dtype])
+        assert code == 0 and "PASS" in text, text
+    code, text = compare("batches", "again", 0)
+    assert code == 0 and "Exact logit comparison: PASS" in text, text
+    code, text = compare("whole", "batches", 0)
+    assert code == 1 and "same schedule" in text
+    code, text = compare("whole", "batches", 1e-12)
+    assert code == 1 and "logits differ by" in text
 
 
 def test_command_line_generate(model_dirs, tmp_path):

@@ -10,9 +10,12 @@ import torch
 
 import beholdd
 import plain_qwen3 as plain
-from beholdd.config import LayerKinds, Qwen3Config
+from dataclasses import dataclass
+
+from beholdd.config import ConfigReader, LayerKinds, Qwen3Config
 from beholdd.models import build_decoder
-from beholdd.parts import MIXERS, CacheNeed
+from beholdd.parts import (FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, CacheNeed, GQAAttention, Linear, RMSNorm,
+                           RotaryEncoding, SwiGLU)
 from beholdd.weights import TensorSpec
 
 DECAY = 0.75
@@ -85,18 +88,144 @@ class ToySharedCacheConfig(Qwen3Config):
         return [(i, i - (i % 2)) for i in range(self.n_layers)]
 
 
+# ---- an architecture with a configuration of its own ----------------------------------------------------
+# Its config.json has other keys, its configuration class inherits nothing from Qwen3's, its tensors have
+# other names, and it brings a feed-forward with routing and a position encoding of its own; the builders
+# below adapt its fields to the parts' constructor parameters.
+
+class ToyRoutedFeedForward:
+    """Top-1 routing over a few small SwiGLU experts: router logits and their softmax in float32; each row goes
+    to its most likely expert (ties to the lowest index), whose output is scaled by that probability.
+    Keeps the last step's routing for inspection."""
+
+    def __init__(self, hidden: int, width: int, n_experts: int, prefix: str):
+        self.hidden, self.width, self.n_experts = hidden, width, n_experts
+        self.router = Linear(hidden, n_experts, prefix + "router.weight")
+        self.experts = [SwiGLU(hidden, width, f"{prefix}experts.{e}.") for e in range(n_experts)]
+        self.last_routing = None
+
+    def tensor_specs(self):
+        return self.router.tensor_specs() + [spec for expert in self.experts for spec in expert.tensor_specs()]
+
+    def load(self, get):
+        self.router.load(get)
+        for expert in self.experts:
+            expert.load(get)
+
+    def forward(self, ctx, x, hidden):
+        logits = self.router.forward(ctx, x, out_dtype=torch.float32)
+        probabilities = torch.softmax(logits, dim=-1)
+        chosen = probabilities.argmax(dim=-1)
+        self.last_routing = chosen
+        for index, expert in enumerate(self.experts):
+            rows = torch.nonzero(chosen == index).flatten()
+            if rows.numel() == 0:
+                continue
+            out = torch.zeros((rows.numel(), self.hidden), dtype=torch.float32, device=hidden.device)
+            expert.forward(ctx, x.index_select(0, rows).contiguous(), out)
+            hidden.index_add_(0, rows, out * probabilities[rows, index].unsqueeze(1))
+
+
+class ToyStretchedRotary(RotaryEncoding):
+    """Rotates only the first `rotary_dim` dimensions of a head, at position / stretch."""
+
+    def __init__(self, rotary_dim, theta, max_position, stretch):
+        super().__init__(rotary_dim, theta, max_position)
+        self.stretch = float(stretch)
+
+    def build_tables(self, device):
+        half = self.rotary_dim // 2
+        freqs = np.array([1.0 / (self.theta ** ((2 * i) / self.rotary_dim)) for i in range(half)], dtype=np.float64)
+        angles = (np.arange(self.max_position, dtype=np.float64) / self.stretch)[:, None] * freqs[None, :]
+        self._tables = (torch.from_numpy(np.cos(angles).astype(np.float32)).to(device).contiguous(),
+                        torch.from_numpy(np.sin(angles).astype(np.float32)).to(device).contiguous())
+
+
+@dataclass(frozen=True)
+class ToyOwnConfig:
+    depth: int
+    width: int
+    readers: int            # query heads
+    stores: int             # key/value heads
+    head_size: int
+    turned: int             # dimensions of a head that the position encoding rotates
+    stretch: float
+    base: float
+    inner: int              # feed-forward width
+    experts: int
+    symbols: int
+    floor: float            # the norms' epsilon
+    longest: int
+
+    @classmethod
+    def from_dict(cls, data, origin="config.json"):
+        r = ConfigReader(data, origin)
+        return cls(depth=r.integer("toy_depth", minimum=1), width=r.integer("toy_width", minimum=1),
+                   readers=r.integer("toy_readers", minimum=1), stores=r.integer("toy_stores", minimum=1),
+                   head_size=r.integer("toy_head_size", minimum=2), turned=r.integer("toy_turned", minimum=2),
+                   stretch=r.number("toy_stretch"), base=r.number("toy_base"), inner=r.integer("toy_inner", minimum=1),
+                   experts=r.integer("toy_experts", minimum=1), symbols=r.integer("toy_symbols", minimum=1),
+                   floor=r.number("toy_floor"), longest=r.integer("toy_longest", minimum=1))
+
+    # what the generic builder reads
+    vocab = property(lambda self: self.symbols)
+    hidden = property(lambda self: self.width)
+    max_position = property(lambda self: self.longest)
+    tie_word_embeddings = False
+
+    def layer_kinds(self):
+        """Attention and a routed feed-forward in even layers, the state mixer and a dense one in odd layers."""
+        return [LayerKinds(mixer="toy_own_attention" if i % 2 == 0 else "toy_own_running_mean",
+                           feed_forward="toy_routed" if i % 2 == 0 else "toy_own_swiglu",
+                           norm="toy_own_rmsnorm", block="pre_norm") for i in range(self.depth)]
+
+    def schedule(self):
+        return [(i, i) for i in range(self.depth)]
+
+
+def build_toy_own(config):
+    return build_decoder(config, position_encoding={"early": "toy_stretched_rotary", "late": "none"}, layer_prefix="blocks.{}.",
+                         embedding_name="symbols.weight", final_norm_name="last_norm.weight",
+                         head_name="readout.weight", final_norm_kind="toy_own_rmsnorm")
+
+
+OWN_PARTS = (
+    (MIXERS, "toy_own_attention", lambda c, index, prefix, shared: GQAAttention(
+        c.width, c.readers, c.stores, c.head_size, prefix + "look.", qk_norm_eps=c.floor,
+        position_encoding=shared["position_encodings"]["early" if index < c.depth // 2 else "late"])),
+    (MIXERS, "toy_own_running_mean", lambda c, index, prefix, shared: ToyRunningMeanMixer(c.width, prefix)),
+    (FEED_FORWARDS, "toy_routed", lambda c, index, prefix, shared: ToyRoutedFeedForward(c.width, c.inner, c.experts, prefix + "routed.")),
+    (FEED_FORWARDS, "toy_own_swiglu", lambda c, index, prefix, shared: SwiGLU(c.width, c.inner, prefix + "dense.")),
+    (NORMS, "toy_own_rmsnorm", lambda c, width, name, shared: RMSNorm(width, c.floor, name)),
+    (POSITION_ENCODINGS, "toy_stretched_rotary", lambda c, shared: ToyStretchedRotary(c.turned, c.base, c.longest, c.stretch)),
+)
+
+OWN = {
+    "architectures": ["ToyOwnForCausalLM"], "toy_depth": 4, "toy_width": 40, "toy_readers": 4, "toy_stores": 2,
+    "toy_head_size": 24, "toy_turned": 16, "toy_stretch": 2.5, "toy_base": 500.0, "toy_inner": 56, "toy_experts": 3,
+    "toy_symbols": 90, "toy_floor": 1e-5, "toy_longest": 512,
+}
+
+
 def register():
     if "toy_running_mean" not in MIXERS:
         MIXERS.register("toy_running_mean", lambda config, index, prefix, shared: ToyRunningMeanMixer(config.hidden, prefix))
-    for name, cls in (("ToyHybridForCausalLM", ToyHybridConfig), ("ToyTwiceForCausalLM", ToyTwiceConfig),
-                      ("ToySharedCacheForCausalLM", ToySharedCacheConfig)):
+    for registry, name, builder in OWN_PARTS:
+        if name not in registry:
+            registry.register(name, builder)
+    for name, cls, build in (("ToyHybridForCausalLM", ToyHybridConfig, build_decoder),
+                             ("ToyTwiceForCausalLM", ToyTwiceConfig, build_decoder),
+                             ("ToySharedCacheForCausalLM", ToySharedCacheConfig, build_decoder),
+                             ("ToyOwnForCausalLM", ToyOwnConfig, build_toy_own)):
         if name not in beholdd.registered_architectures():
-            beholdd.register_architecture(name, cls, build_decoder)
+            beholdd.register_architecture(name, cls, build)
 
 
 def unregister():
     MIXERS.unregister("toy_running_mean")
-    for name in ("ToyHybridForCausalLM", "ToyTwiceForCausalLM", "ToySharedCacheForCausalLM"):
+    for registry, name, _ in OWN_PARTS:
+        registry.unregister(name)
+    for name in ("ToyHybridForCausalLM", "ToyTwiceForCausalLM", "ToySharedCacheForCausalLM", "ToyOwnForCausalLM"):
         beholdd.registry.unregister_architecture(name)
 
 
@@ -108,6 +237,8 @@ BASE = {
 
 
 def config_dict(architecture):
+    if architecture == "ToyOwnForCausalLM":
+        return dict(OWN)
     return dict(BASE, architectures=[architecture])
 
 
@@ -129,7 +260,61 @@ def _attention_parts(cfg, w, prefix, hidden):
     return q.reshape(t_len, -1), k.reshape(t_len, -1), v
 
 
+def plain_own_logits(config, w, tokens):
+    """The plain form of ToyOwnForCausalLM from the plain implementation's part functions."""
+    c = ToyOwnConfig.from_dict(config)
+    hidden = plain.embed(tokens, w["symbols.weight"])
+    t_len, hd = hidden.shape[0], c.head_size
+    freqs = plain.rope_frequencies(c.base, c.turned)
+    scale = np.float32(1) / np.sqrt(np.float32(hd))
+    routing = []
+    for i in range(c.depth):
+        p = f"blocks.{i}."
+        xn = plain.rmsnorm(hidden, w[p + "input_layernorm.weight"], c.floor)
+        if i % 2 == 0:
+            q = plain.rmsnorm(plain.linear(xn, w[p + "look.q_proj.weight"]).reshape(t_len, c.readers, hd), w[p + "look.q_norm.weight"], c.floor)
+            k = plain.rmsnorm(plain.linear(xn, w[p + "look.k_proj.weight"]).reshape(t_len, c.stores, hd), w[p + "look.k_norm.weight"], c.floor)
+            v = plain.linear(xn, w[p + "look.v_proj.weight"])
+            for t in range(t_len if i < c.depth // 2 else 0):      # the later layers' attention has no position encoding
+                cs = plain.rope_cos_sin(freqs, t / c.stretch)
+                q[t, :, :c.turned] = plain.rope_split_half(q[t, :, :c.turned], *cs)
+                k[t, :, :c.turned] = plain.rope_split_half(k[t, :, :c.turned], *cs)
+            attended = plain.causal_attention(q.reshape(t_len, -1), k.reshape(t_len, -1), v, c.readers, c.stores, hd, scale)
+            hidden = (hidden + plain.linear(attended, w[p + "look.o_proj.weight"])).astype(np.float32)
+        else:
+            hidden = (hidden + plain_toy_mixer(xn, w[p + "toy_mix.weight"])).astype(np.float32)
+        xf = plain.rmsnorm(hidden, w[p + "post_attention_layernorm.weight"], c.floor)
+        if i % 2 == 0:
+            probabilities = plain.softmax(plain.linear(xf, w[p + "routed.router.weight"]))
+            chosen = probabilities.argmax(axis=-1)
+            routing.append(chosen)
+            out = np.zeros_like(hidden)
+            for t in range(t_len):
+                e = f"{p}routed.experts.{chosen[t]}."
+                a = plain.swiglu(plain.linear(xf[t], w[e + "gate_proj.weight"]), plain.linear(xf[t], w[e + "up_proj.weight"]))
+                out[t] = plain.linear(a, w[e + "down_proj.weight"]) * probabilities[t, chosen[t]]
+            hidden = (hidden + out).astype(np.float32)
+        else:
+            a = plain.swiglu(plain.linear(xf, w[p + "dense.gate_proj.weight"]), plain.linear(xf, w[p + "dense.up_proj.weight"]))
+            hidden = (hidden + plain.linear(a, w[p + "dense.down_proj.weight"])).astype(np.float32)
+    return plain.linear(plain.rmsnorm(hidden, w["last_norm.weight"], c.floor), w["readout.weight"]), routing
+
+
+def load_plain_weights(folder):
+    """(config.json as a dictionary, tensors as float32 arrays) of any model folder."""
+    import json
+    import os
+    from safetensors import safe_open
+
+    with open(os.path.join(folder, "config.json")) as handle:
+        config = json.load(handle)
+    with safe_open(os.path.join(folder, "model.safetensors"), framework="pt") as handle:
+        return config, {name: handle.get_tensor(name).to(torch.float32).numpy() for name in handle.keys()}
+
+
 def plain_logits(architecture, cfg, w, tokens):
+    if architecture == "ToyOwnForCausalLM":
+        return plain_own_logits(cfg, w, tokens)[0]
     hidden = plain.embed(tokens, w["model.embed_tokens.weight"])
     scale = np.float32(1) / np.sqrt(np.float32(cfg.head_dim))
     if architecture == "ToyHybridForCausalLM":
@@ -163,13 +348,19 @@ def check_architecture(architecture, folder, make_engine, tolerance):
     """Whole, one by one and in batches: all equal to the plain form."""
     import schedules
 
-    cfg, weights = plain.load_plain(folder)
-    requests = schedules.random_requests(cfg.vocab, [3, 70, 21, 40], seed=13)
+    if architecture == "ToyOwnForCausalLM":
+        cfg, weights = load_plain_weights(folder)
+        vocab = cfg["toy_symbols"]
+    else:
+        cfg, weights = plain.load_plain(folder)
+        vocab = cfg.vocab
+    requests = schedules.random_requests(vocab, [3, 70, 21, 40], seed=13)
     want = [plain_logits(architecture, cfg, weights, r) for r in requests]
     engine = make_engine(folder)
     for label, got in (("whole", schedules.whole(engine, requests)),
                        ("one by one", schedules.tail_one_by_one(engine, requests, tail=32)),
-                       ("batches", schedules.batches(engine, requests, batch_size=3))):
+                       ("batches", schedules.batches(engine, requests, batch_size=3)),
+                       ("portions", schedules.portions(engine, requests))):
         for index, (g, e) in enumerate(zip(got, want)):
             error = schedules.relative_error(g, e)
             assert error < tolerance, (architecture, label, index, error)
