@@ -45,7 +45,16 @@ TINY_D = {
     "rms_norm_eps": 1e-6, "max_position_embeddings": 2048, "tie_word_embeddings": True,
     "hidden_act": "silu", "attention_bias": False,
 }
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
+# Seventeen query heads to a kv head: beyond what the decode attention that starts from the projection rows takes,
+# so decode steps run the norm-rotate-write kernel and the attention kernel one after the other.
+TINY_E = {
+    "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3",
+    "num_hidden_layers": 1, "hidden_size": 72, "num_attention_heads": 34, "num_key_value_heads": 2,
+    "head_dim": 64, "intermediate_size": 100, "vocab_size": 211, "rope_theta": 10000.0,
+    "rms_norm_eps": 1e-6, "max_position_embeddings": 512, "tie_word_embeddings": False,
+    "hidden_act": "silu", "attention_bias": False,
+}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
 
 
 @pytest.fixture()

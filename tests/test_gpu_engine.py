@@ -24,7 +24,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 TOLERANCE = {"float32": 1e-4, "bfloat16": 2e-2}
 
 LENGTHS = {"A": [5, 11, 17, 70, 33, 128], "B": [1, 7, 23, 40, 90, 200, 64], "C": [3, 65, 130, 400, 31],
-           "D": [2, 50, 129, 300]}
+           "D": [2, 50, 129, 300], "E": [4, 66, 150]}
 
 
 def engine_for(folder, dtype, max_tokens=4096):
@@ -60,7 +60,7 @@ def check(label, got, want, tolerance):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_every_cut_matches_the_plain_implementation(expected, name, dtype):
     folder, requests, want = expected(name)
     engine = engine_for(folder, dtype)
@@ -161,6 +161,54 @@ def test_prompts_of_many_rows(large_expected):
     together = schedules.batches(engine, requests, batch_size=3, prompt_fraction=1.0)
     check("one step of 2,200 rows", together, want, TOLERANCE["bfloat16"])
     check("together against alone", together, alone, TOLERANCE["bfloat16"] / 2)
+
+
+def _prompt_then_one_by_one(engine, tokens, tail, keep):
+    """The first len - tail tokens in one step (the logits of its last `keep` rows wanted), the rest one by one."""
+    from beholdd.engine import StepEntry
+    cut = len(tokens) - tail
+    slot = engine.alloc_slot()
+    rows = [engine.step([StepEntry(slot, tokens[:cut], list(range(cut - keep, cut)))]).float().cpu().numpy()]
+    for token in tokens[cut:]:
+        rows.append(engine.step([StepEntry(slot, [token], [0])]).float().cpu().numpy())
+    engine.free_slot(slot)
+    return np.concatenate(rows)
+
+
+def test_the_benchmark_context_at_the_large_layer_sizes(large_expected):
+    """Where the benchmark runs: the Qwen3-8B layer sizes (two layers, a small vocabulary) at a context of
+    8,100 tokens, the prompt whole and the last 32 tokens one by one through the captured graphs (127 pages, the
+    keys split over workgroups); and eight requests of 256 to 1,024 tokens decoding 64 tokens together.  bfloat16
+    against the float32 engine, which test_layers_of_the_large_models_sizes holds to the plain implementation at
+    these sizes, and which is held to itself here: whole against one by one."""
+    from beholdd.engine import StepEntry
+    folder = large_expected("8b")[0]
+    long_one = schedules.random_requests(1000, [8100], seed=31)[0]
+    lengths = [256, 1024, 700, 333, 512, 961, 640, 449]
+    batch = schedules.random_requests(1000, [n + 64 for n in lengths], seed=32)
+    got = {}
+    for dtype in ("float32", "bfloat16"):
+        engine = engine_for(folder, dtype, max_tokens=8192)
+        long_rows = _prompt_then_one_by_one(engine, long_one, tail=32, keep=4)
+        if dtype == "float32":
+            slot = engine.alloc_slot()
+            whole = engine.step([StepEntry(slot, long_one, list(range(8100 - 36, 8100)))]).float().cpu().numpy()
+            engine.free_slot(slot)
+            check("float32 whole against one by one", [long_rows], [whole], TOLERANCE["float32"] / 2)
+        slots = [engine.alloc_slot() for _ in batch]
+        rows = [engine.step([StepEntry(s, r[:n], [n - 1]) for s, r, n in zip(slots, batch, lengths)]).float().cpu().numpy()]
+        for step in range(64):
+            rows.append(engine.step([StepEntry(s, [r[n + step]], [0]) for s, r, n in zip(slots, batch, lengths)])
+                        .float().cpu().numpy())
+        for slot in slots:
+            engine.free_slot(slot)
+        if dtype == "bfloat16":
+            assert engine.graphs is not None and len(engine.graphs.graphs) >= 2
+        engine.cache.check_invariants()
+        got[dtype] = (long_rows, np.stack(rows, axis=1))       # [request, step, vocab]
+        del engine
+    check("8,100 tokens", [got["bfloat16"][0]], [got["float32"][0]], TOLERANCE["bfloat16"])
+    check("batch of 8", list(got["bfloat16"][1]), list(got["float32"][1]), TOLERANCE["bfloat16"])
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

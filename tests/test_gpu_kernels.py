@@ -458,6 +458,7 @@ class Layout:
 
 ATTN_SHAPES = [  # heads, kv heads, head size
     (4, 2, 16), (6, 2, 48), (8, 8, 64), (5, 1, 80), (8, 2, 128), (3, 3, 256), (12, 4, 96), (14, 2, 128),
+    (32, 1, 64), (40, 2, 32),          # 32 and 20 query heads to a kv head: more than one tile of columns shares a head
 ]
 
 
