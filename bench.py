@@ -74,7 +74,7 @@ def randomise_cache(engine, torch):
 
 def decode_run(engine, batch, context, steps, warmup, torch):
     """Time `steps` decode steps of `batch` sequences that end at `context` tokens."""
-    from beholdd.engine import StepEntry
+    from beholdd.engine import StepEntry, decode_ahead
     from beholdd.sampling import SamplingParams
 
     start = context - steps - warmup - 1
@@ -83,16 +83,15 @@ def decode_run(engine, batch, context, steps, warmup, torch):
     greedy = [SamplingParams()] * batch
     tokens = [(7 * i + 3) % engine.model.vocab for i in range(batch)]
 
-    # The generation loop's own way of stepping (engine/generation.py): the next step is started with the
-    # tokens still on the device, then the host reads the tokens chosen before it.
+    # The generation loop's own way of stepping (engine/generation.py: decode_ahead): the next step is started
+    # with the tokens still on the device, then the host reads the tokens chosen before it.
     requests = list(range(batch))
     logits = engine.step([StepEntry(slot, [token], [0]) for slot, token in zip(slots, tokens)])
     chosen = engine.select_async(logits, greedy, requests, [0] * batch)
 
     def one(step):
         nonlocal chosen
-        logits = engine.step([StepEntry(slot, [0], [0], fed_row=row) for slot, row in zip(slots, chosen.device_rows)])
-        ahead = engine.select_async(logits, greedy, requests, [step + 1] * batch)
+        ahead = decode_ahead(engine, slots, chosen, greedy, requests, [step + 1] * batch)
         chosen.result()
         chosen = ahead
 
@@ -141,7 +140,7 @@ def workload_run(engine, shape, torch):
     rng = random.Random(0)
     lengths = [rng.randint(shortest, longest) for _ in range(count)]
     prompts = [[rng.randrange(engine.model.vocab) for _ in range(n)] for n in lengths]
-    engine.generate([prompts[0][:64]], max_new_tokens=4)          # warms up: graphs are captured per batch size as they come
+    engine.generate(prompts, max_new_tokens=4)          # warms up: the graph of this batch size and page-table width is captured
     torch.cuda.synchronize()
     begin = time.perf_counter()
     results = engine.generate(prompts, max_new_tokens=new_tokens, temperature=temperature, seed=1)
@@ -220,12 +219,20 @@ def main():
     t = args.prefill_tokens
     prefill_flops = (2.0 * cfg.n_layers * layer_params * t + cfg.n_layers * cfg.n_heads * 2.0 * t * t * cfg.head_dim
                      + 2.0 * cfg.vocab * cfg.hidden)
-    points = {}
+    # Other batch sizes and contexts: tokens a second, and beside each the fraction of the HBM peak that the
+    # bytes of its step (all weights once, the live requests' caches) amount to.
+    points, fractions = {}, {}
     if not args.no_points:
-        for batch in (1, 64):
+        for batch, context, name in ((1, args.context, "decode_b1"), (64, args.context, "decode_b64"),
+                                     (1, 512, "decode_b1_ctx512"), (1, 2048, "decode_b1_ctx2048"),
+                                     (8, 640, "decode_b8_ctx640"), (64, 640, "decode_b64_ctx640")):
             steps = max(4, args.steps // 2)
-            s, _ = decode_run(engine, batch, args.context, steps, 2, torch)
-            points[f"decode_b{batch}"] = round(batch / s, 2)
+            s, length = decode_run(engine, batch, context, steps, 2, torch)
+            points[name] = round(batch / s, 2)
+            fractions[name] = round((weight_bytes + batch * length * kv_bytes_per_token) / s / 1e9 / PEAK_HBM_GBS, 4)
+    generated = None
+    if not args.no_points and args.shape == "8b":
+        generated = workload_run(engine, args.shape, torch)     # the same batch through Engine.generate
 
     line = {
         "metric": f"decode tok/s @ batch {args.batch} ({shape_name}, context {args.context})", "value": round(value, 2), "unit": "tok/s",
@@ -244,7 +251,10 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},
         "points": points,
+        "points_hbm_frac": fractions,
     }
+    if generated is not None:
+        line["generate"] = generated
     print(json.dumps(line))
     return 0
 

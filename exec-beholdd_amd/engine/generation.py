@@ -158,6 +158,14 @@ def _run_batch(stepper, batch, prompts, max_new, params, stops, on_token, contro
             stepper.free_slot(slot)
 
 
+def decode_ahead(stepper, slots: list, chosen, params: list, requests: list, steps: list):
+    """One decode step of the sequences in `slots`, started before the host knows their tokens: `chosen` is the
+    selection (not waited for) that holds them, one element per slot, and the step reads them on the device.
+    Returns the selection of this step's tokens, not waited for either."""
+    logits = stepper.step([StepEntry(slot, [0], [0], fed_row=row) for slot, row in zip(slots, chosen.device_rows)])
+    return stepper.select_async(logits, params, requests, steps)
+
+
 def _run_batch_ahead(stepper, batch, prompts, max_new, params, stops, on_token, control, results):
     """`_run_batch` one step ahead of the host (see the module's text)."""
     slots = {}
@@ -177,10 +185,9 @@ def _run_batch_ahead(stepper, batch, prompts, max_new, params, stops, on_token, 
             if ahead:
                 if control is not None:
                     control()
-                logits = stepper.step([StepEntry(slots[live[at]], [0], [0], fed_row=chosen.device_rows[at])
-                                       for at in ahead])
-                chosen_ahead = stepper.select_async(logits, [params[live[at]] for at in ahead],
-                                                    [live[at] for at in ahead], [step + 1] * len(ahead))
+                chosen_ahead = decode_ahead(stepper, [slots[live[at]] for at in ahead], chosen.take(ahead),
+                                            [params[live[at]] for at in ahead], [live[at] for at in ahead],
+                                            [step + 1] * len(ahead))
             tokens = chosen.result()
             going = set()
             for index, token in zip(live, tokens):
