@@ -153,19 +153,29 @@ def workload_run(engine, shape, torch):
 
 
 def hbm_ceiling(torch):
-    """What library kernels that only stream memory reach here: a sum over 8 GB (read) and a copy of 8 GB
-    (read + write).  Not part of the product path; a yardstick for the roofline fractions."""
+    """What kernels that only stream memory reach here: torch's sum over 8 GB (read) and copy of 8 GB (read +
+    write), and the library's own yardstick kernel, which reads 8 GB the way its weight and cache streams do
+    (256 and 512 workgroups, with and without the streaming hint).  Not part of the product path; a yardstick
+    for the roofline fractions."""
+    from beholdd.kernels import HipKernels
+
     x = torch.empty(2 << 30, dtype=torch.float32, device="cuda:0").normal_()
     y = torch.empty_like(x)
+    kernels = HipKernels("cuda:0")
     out = {}
-    for name, run, moved in (("read", lambda: x.sum(), x.numel() * 4), ("copy", lambda: y.copy_(x), 2 * x.numel() * 4)):
+    runs = [("hbm_read_GBs", lambda: x.sum(), x.numel() * 4), ("hbm_copy_GBs", lambda: y.copy_(x), 2 * x.numel() * 4)]
+    for workgroups in (256, 512):
+        for hint in (True, False):
+            name = f"stream_read_{workgroups}wg_{'streaming' if hint else 'plain'}_GBs"
+            runs.append((name, lambda w=workgroups, h=hint: kernels.stream_read(x, w, h), x.numel() * 4))
+    for name, run, moved in runs:
         run()
         torch.cuda.synchronize()
         begin = time.perf_counter()
         for _ in range(10):
             run()
         torch.cuda.synchronize()
-        out[f"hbm_{name}_GBs"] = round(moved * 10 / (time.perf_counter() - begin) / 1e9, 1)
+        out[name] = round(moved * 10 / (time.perf_counter() - begin) / 1e9, 1)
     return out
 
 
@@ -234,6 +244,16 @@ def main():
     if not args.no_points and args.shape == "8b":
         generated = workload_run(engine, args.shape, torch)     # the same batch through Engine.generate
 
+    # what a kernel that does nothing but read reaches on this GPU (the library's yardstick kernel over 4 GB of the cache)
+    cache_tensor = engine.cache.groups[0].k
+    span = cache_tensor.view(-1)[: min(cache_tensor.numel(), 2 << 30)]
+    engine.kernels.stream_read(span)
+    torch.cuda.synchronize()
+    begin = time.perf_counter()
+    read = sum(engine.kernels.stream_read(span) for _ in range(4))
+    torch.cuda.synchronize()
+    yardstick = read / (time.perf_counter() - begin) / 1e9
+
     line = {
         "metric": f"decode tok/s @ batch {args.batch} ({shape_name}, context {args.context})", "value": round(value, 2), "unit": "tok/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(seconds * 1e3, 4),
@@ -249,7 +269,7 @@ def main():
         "prefill": {"value": round(t / prefill_seconds, 1), "tokens": t, "ms": round(prefill_seconds * 1e3, 3),
                     "frac": round(prefill_flops / prefill_seconds / PEAK_FLOPS[dtype_tag], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+                     "frac": round(achieved / PEAK_HBM_GBS, 4), "plain_read_GBs": round(yardstick, 1)},
         "points": points,
         "points_hbm_frac": fractions,
     }

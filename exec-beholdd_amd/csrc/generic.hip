@@ -642,3 +642,42 @@ extern "C" int bh_swiglu(const void* gu, void* out, int dtype, int n_rows, int F
     return bh_fail("swiglu: unknown dtype %d", dtype);
   return bh_check_launch("swiglu");
 }
+
+// ---- a yardstick for the memory system ----------------------------------------------------------
+// Not a product kernel: reads `bytes` of device memory once, the way the streaming kernels of this library
+// read weights and cache pages (16 bytes a lane, sixteen loads of 1 KB in flight per wave, four waves a
+// workgroup, every workgroup a contiguous share), with or without the hint that nobody reads the bytes again
+// soon.  Its rate is what a kernel that does nothing but read can reach on this GPU; bench.py --hbm-ceiling
+// prints it beside the library routines' rates.
+typedef uint32_t bh_u32x4_t __attribute__((ext_vector_type(4)));
+
+template <bool STREAM>
+__global__ __launch_bounds__(256) void stream_read_kernel(const uint8_t* __restrict__ data, long per_workgroup,
+                                                          uint32_t* __restrict__ sink) {
+  const int wave = threadIdx.x / BH_WAVE, lane = threadIdx.x % BH_WAVE;
+  const uint8_t* mine = data + (size_t)blockIdx.x * per_workgroup + lane * 16;
+  bh_u32x4_t seen = {0u, 0u, 0u, 0u};
+  for (long at = (long)wave * 16384; at + 16384 <= per_workgroup; at += 4 * 16384) {
+    bh_u32x4_t piece[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const bh_u32x4_t* p = reinterpret_cast<const bh_u32x4_t*>(mine + at + u * 1024);
+      piece[u] = STREAM ? __builtin_nontemporal_load(p) : *p;
+    }
+#pragma unroll
+    for (int u = 0; u < 16; ++u) seen ^= piece[u];
+  }
+  if ((seen[0] ^ seen[1] ^ seen[2] ^ seen[3]) == 0x9e3779b9u) sink[0] = 1;   // keeps the loads alive
+}
+
+// Reads the first workgroups * (bytes / workgroups rounded down to 64 KB) bytes; returns that count through `read`.
+extern "C" int bh_stream_read(const void* data, long bytes, int workgroups, int nontemporal, void* sink, long* read,
+                              hipStream_t stream) {
+  BH_REQUIRE(data != nullptr && sink != nullptr && read != nullptr, "stream_read: data, sink and count are required");
+  BH_REQUIRE(workgroups > 0 && bytes >= (long)workgroups * 65536, "stream_read: at least 64 KB per workgroup");
+  const long per_workgroup = bytes / workgroups / 65536 * 65536;
+  *read = per_workgroup * workgroups;
+  if (nontemporal) stream_read_kernel<true><<<dim3(workgroups), dim3(256), 0, stream>>>((const uint8_t*)data, per_workgroup, (uint32_t*)sink);
+  else stream_read_kernel<false><<<dim3(workgroups), dim3(256), 0, stream>>>((const uint8_t*)data, per_workgroup, (uint32_t*)sink);
+  return bh_check_launch("stream_read");
+}

@@ -33,14 +33,14 @@ class BuildError(RuntimeError):
 
 
 def source_page_size() -> int:
-    """Tokens in one page of the key/value cache: `BH_PAGE` of csrc/common.h, the one place that says so.
+    """Tokens in one page of the key/value cache: `BH_PAGE` of csrc/layout.h, the one place that says so.
     (The built library reports the same number as `bh_page_size()`; this reads it where no library is loaded.)"""
-    with open(os.path.join(CSRC, "common.h"), "r", encoding="utf-8") as handle:
+    with open(os.path.join(CSRC, "layout.h"), "r", encoding="utf-8") as handle:
         for line in handle:
             words = line.split()
             if len(words) >= 3 and words[0] == "#define" and words[1] == "BH_PAGE":
                 return int(words[2])
-    raise BuildError("csrc/common.h does not define BH_PAGE")
+    raise BuildError("csrc/layout.h does not define BH_PAGE")
 
 
 def _hipcc() -> str:
@@ -151,6 +151,28 @@ def build(verbose: bool = True, jobs: int | None = None) -> str:
     with open(target + ".stamp", "w", encoding="utf-8") as handle:
         handle.write(source_hash() + "\n")
     say(f"linked {target} ({time.time() - started:.0f} s)")
+    return target
+
+
+def build_plain_twins(out_dir: str, selftest: bool = False) -> str:
+    """Compile csrc/plain_twins.cpp with the host compiler: a shared library of the kernels' plain twins, or with
+    `selftest` a program of its own, built with the address and undefined-behaviour sanitizers, that checks the
+    twins against the reference's test vectors.  Returns the path of what was built."""
+    compiler = os.environ.get("CXX") or shutil.which("g++") or shutil.which("c++")
+    if not compiler:
+        raise BuildError("no host C++ compiler (g++) was found")
+    source = os.path.join(CSRC, "plain_twins.cpp")
+    os.makedirs(out_dir, exist_ok=True)
+    if selftest:
+        target = os.path.join(out_dir, "plain_twins_selftest")
+        command = [compiler, "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
+                   "-DBH_TWINS_SELFTEST", "-I", CSRC, source, "-o", target]
+    else:
+        target = os.path.join(out_dir, "libbeholdd_plain.so")
+        command = [compiler, "-std=c++17", "-O2", "-shared", "-fPIC", "-I", CSRC, source, "-o", target]
+    done = subprocess.run(command, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if done.returncode != 0:
+        raise BuildError(f"{' '.join(command)} failed:\n{done.stdout}")
     return target
 
 

@@ -106,6 +106,7 @@ class HipKernels:
             "bh_attention_decode_fused": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, f, i, i, i, p, p, i, f, p, p, i, i,
                                           i, p],
             "bh_kv_order": [i, i],
+            "bh_stream_read": [p, ctypes.c_long, i, i, p, p, p],
         }
         for name, argtypes in table.items():
             function = getattr(lib, name)
@@ -448,6 +449,15 @@ class HipKernels:
             self._ptr(cos, "cos", (torch.float32,), True), self._ptr(sin, "sin", (torch.float32,), True),
             cos.shape[0] if cos is not None else 0, rot, int(bool(write_kv)), self._stream()))
         return True
+
+    def stream_read(self, data, workgroups=256, nontemporal=True) -> int:
+        """A yardstick, not a product path: read `data` (any contiguous tensor) once the way the streaming kernels
+        read; returns the number of bytes read (whole 64 KB per workgroup)."""
+        sink = torch.zeros(1, dtype=torch.int32, device=self.device)
+        count = ctypes.c_long(0)
+        self._check(self.lib.bh_stream_read(self._ptr(data, "data"), data.numel() * data.element_size(), int(workgroups),
+                                            int(bool(nontemporal)), self._ptr(sink, "sink"), ctypes.byref(count), self._stream()))
+        return int(count.value)
 
     def swiglu(self, gate_up, out):
         """out[r, i] = silu(gate_up[r, i]) * gate_up[r, F + i]."""

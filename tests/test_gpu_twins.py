@@ -1,0 +1,142 @@
+"""Every kernel beside its plain C++ twin (exec-beholdd_amd/csrc/plain_twins.cpp): the same arguments, the same
+cache pages element for element, in float32 and in bfloat16."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import twins as twins_module
+from twins import BF16, F32
+
+pytestmark = pytest.mark.gpu
+DEVICE = "cuda:0"
+RNG = np.random.default_rng(5)
+
+
+@pytest.fixture(scope="module")
+def K():
+    from beholdd.kernels import HipKernels
+    return HipKernels(DEVICE)
+
+
+@pytest.fixture(scope="module")
+def twins(tmp_path_factory):
+    return twins_module.Twins(tmp_path_factory.mktemp("twins"))
+
+
+def dev(array, dtype=None):
+    tensor = torch.from_numpy(np.ascontiguousarray(array)).to(DEVICE)
+    return tensor.to(dtype) if dtype is not None else tensor
+
+
+def host(tensor):
+    return tensor.float().cpu().numpy()
+
+
+def rel(got, want):
+    return float(np.abs(got.astype(np.float64) - want).max() / max(np.abs(want).max(), 1e-30))
+
+
+def test_embed_rmsnorm_swiglu_argmax_and_their_twins(K, twins):
+    table = RNG.normal(size=(331, 96)).astype(np.float32)
+    tokens = RNG.integers(0, 331, size=37).astype(np.int32)
+    out = torch.empty(37, 96, device=DEVICE)
+    K.embed(dev(tokens), dev(table, torch.bfloat16), out)
+    assert np.array_equal(host(out), twins.embed(tokens, table, BF16)[1])
+    x = RNG.normal(size=(33, 1000)).astype(np.float32) * 2
+    w = (1 + 0.3 * RNG.normal(size=1000)).astype(np.float32)
+    for out_dtype, code, bound in ((torch.float32, F32, 2e-6), (torch.bfloat16, BF16, 8e-3)):
+        got = torch.empty(33, 1000, device=DEVICE, dtype=out_dtype)
+        K.rmsnorm(dev(x), dev(w), 1e-5, got)
+        assert rel(host(got), twins.rmsnorm(x, w, 1e-5, out_code=code)) < bound
+    gate_up = RNG.normal(size=(7, 400)).astype(np.float32) * 3
+    for dtype, code, bound in ((torch.float32, F32, 2e-6), (torch.bfloat16, BF16, 8e-3)):
+        got = torch.empty(7, 200, device=DEVICE, dtype=dtype)
+        K.swiglu(dev(gate_up, dtype), got)
+        assert rel(host(got), twins.swiglu(gate_up, code)) < bound
+    logits = RNG.normal(size=(5, 10000)).astype(np.float32)
+    logits[1, 77] = logits[1, 9000] = 50.0
+    logits[3, 5] = np.inf
+    tokens_out = torch.empty(5, dtype=torch.int32, device=DEVICE)
+    bad = torch.empty(5, dtype=torch.int32, device=DEVICE)
+    K.sample(dev(logits), tokens_out, bad)
+    want_tokens, want_bad = twins.argmax(logits)
+    assert tokens_out.cpu().tolist() == want_tokens.tolist() and bad.cpu().tolist() == want_bad.tolist()
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 96, 128), (8, 331, 192), (40, 130, 320), (200, 64, 448)])
+def test_products_and_their_twin(K, twins, m, n, k):
+    a, w = RNG.normal(size=(m, k)).astype(np.float32), RNG.normal(size=(n, k)).astype(np.float32) * 0.1
+    got32 = torch.zeros(m, n, device=DEVICE)
+    K.gemm(dev(a), dev(w), got32)
+    assert rel(host(got32), twins.gemm(a, w)) < 5e-6
+    got16 = torch.ones(m, n, device=DEVICE)          # bfloat16 operands (the matrix cores), added into a float32 residual
+    K.gemm(dev(a, torch.bfloat16), K.pack_weight(dev(w, torch.bfloat16)), got16, accumulate=True)
+    assert rel(host(got16), twins.gemm(a, w, BF16, c=np.ones((m, n), np.float32))) < 5e-6
+
+
+class Layout:
+    def __init__(self, seq_start, n_seqs, max_rows_per_seq, max_position):
+        self.seq_start, self.n_seqs, self.max_rows_per_seq, self.max_position = seq_start, n_seqs, max_rows_per_seq, max_position
+
+
+@pytest.mark.parametrize("dtype,code,head_dim,rot,window", [(torch.float32, F32, 48, 48, 0), (torch.float32, F32, 80, 32, 70),
+                                                            (torch.bfloat16, BF16, 64, 64, 0), (torch.bfloat16, BF16, 128, 128, 100),
+                                                            (torch.bfloat16, BF16, 48, 0, 0)])
+def test_cache_write_and_attention_and_their_twins(K, twins, dtype, code, head_dim, rot, window):
+    """Sequences with pasts of 0, 70 and 5 tokens get 9, 1 and 130 more rows in one step: the writing kernel fills
+    the same places of the same pages as its twin, and the attention kernel (the generic one, or the matrix-core
+    ones for bfloat16 heads in steps of 32) gives what the twin gives over those pages."""
+    n_heads, kv_heads, eps = 6, 2, 1e-5
+    lengths = [(0, 9), (70, 1), (5, 130)]
+    n_pages = 8
+    order = K.kv_order(dtype, head_dim)
+    assert order == (1 if dtype == torch.bfloat16 and head_dim % 32 == 0 else 0)
+    pages = RNG.permutation(n_pages).tolist()
+    table = np.zeros((3, 3), np.int32)
+    for s, (past, new) in enumerate(lengths):
+        for j in range(-(-(past + new) // 64)):
+            table[s, j] = pages.pop()
+    fused = (n_heads + 2 * kv_heads) * head_dim
+    qw = (1 + 0.3 * RNG.normal(size=head_dim)).astype(np.float32)
+    kw = (1 + 0.3 * RNG.normal(size=head_dim)).astype(np.float32)
+    top = max(past + new for past, new in lengths)
+    angles = np.arange(top)[:, None] * (1.0 / 10000.0 ** (2 * np.arange(max(rot, 2) // 2) / max(rot, 2)))[None, :]
+    cos, sin = (np.cos(angles).astype(np.float32), np.sin(angles).astype(np.float32)) if rot else (None, None)
+    kind = torch.float32 if code == F32 else torch.bfloat16
+    k_dev = torch.zeros(n_pages, kv_heads, 64, head_dim, device=DEVICE, dtype=kind)
+    v_dev = torch.zeros(n_pages, kv_heads, head_dim, 64, device=DEVICE, dtype=kind)
+    k_twin = v_twin = None
+    for phase in (0, 1):
+        rows, positions, row_seq, starts = [], [], [], [0]
+        for s, (past, new) in enumerate(lengths):
+            lo, hi = (0, past) if phase == 0 else (past, past + new)
+            rows.append(RNG.normal(size=(hi - lo, fused)).astype(np.float32))
+            positions.extend(range(lo, hi))
+            row_seq.extend([s] * (hi - lo))
+            starts.append(len(positions))
+        qkv = np.concatenate(rows)
+        q_twin, k_twin, v_twin = twins.qk_norm_rope_cache(qkv, qw, kw, eps, cos, sin, positions, row_seq, table, n_pages, n_heads,
+                                                          kv_heads, head_dim, order, code, k_pages=k_twin, v_pages=v_twin)
+        q_dev = torch.empty(len(positions), n_heads * head_dim, device=DEVICE, dtype=kind)
+        K.qk_norm_rope_cache(dev(qkv, kind), q_dev, dev(qw), dev(kw), eps, None if cos is None else dev(cos),
+                             None if sin is None else dev(sin), dev(np.asarray(positions, np.int32)),
+                             dev(np.asarray(row_seq, np.int32)), k_dev, v_dev, dev(table), n_heads, kv_heads, head_dim, True,
+                             max(positions))
+    bound = 2e-6 if code == F32 else 8e-3
+    assert rel(host(q_dev), q_twin) < bound
+    # the pages, element for element in the library's own order: the values are copies, the keys are within rounding
+    k_got, v_got = host(k_dev.reshape(n_pages, kv_heads, -1)), host(v_dev.reshape(n_pages, kv_heads, -1))
+    k_want = k_twin if code == F32 else twins_module.from_bf16_bits(k_twin)
+    v_want = v_twin if code == F32 else twins_module.from_bf16_bits(v_twin)
+    assert np.array_equal(v_got, v_want)
+    assert rel(k_got, k_want) < bound
+    scale = 1 / math.sqrt(head_dim)
+    out = torch.empty_like(q_dev)
+    layout = Layout(dev(np.asarray(starts, np.int32)), 3, max(new for _, new in lengths), max(positions))
+    K.attention(q_dev, out, k_dev, v_dev, dev(table), dev(np.asarray(row_seq, np.int32)), dev(np.asarray(positions, np.int32)),
+                n_heads, kv_heads, head_dim, scale, window, layout=layout)
+    want = twins.attention(host(q_dev), k_twin, v_twin, table, row_seq, positions, n_heads, kv_heads, head_dim, scale, window, order, code)
+    assert rel(host(out), want) < (1e-5 if code == F32 else 1.2e-2)

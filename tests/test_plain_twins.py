@@ -1,0 +1,101 @@
+"""The kernels' plain C++ twins: their self-test under the host sanitizers, and the twins against the plain
+implementation's functions of the same formulas on random data."""
+
+import subprocess
+
+import numpy as np
+import pytest
+
+import plain_qwen3 as plain
+import twins as twins_module
+from beholdd.kernels import build
+
+RNG = np.random.default_rng(77)
+
+
+@pytest.fixture(scope="module")
+def twins(tmp_path_factory):
+    return twins_module.Twins(tmp_path_factory.mktemp("twins"))
+
+
+def test_self_test_under_the_address_and_undefined_behaviour_sanitizers(tmp_path):
+    program = build.build_plain_twins(str(tmp_path), selftest=True)
+    run = subprocess.run([program], capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0 and "self-test ok" in run.stdout, run.stdout + run.stderr
+
+
+def test_elementwise_twins_are_the_plain_functions(twins):
+    x = RNG.normal(size=(5, 200)).astype(np.float32) * 3
+    w = (1 + 0.3 * RNG.normal(size=200)).astype(np.float32)
+    assert np.allclose(twins.rmsnorm(x, w, 1e-5), plain.rmsnorm(x, w, 1e-5), rtol=1e-6, atol=1e-7)
+    assert np.allclose(twins.rmsnorm(x, w, 1e-5, rows=[4, 0]), plain.rmsnorm(x[[4, 0]], w, 1e-5), rtol=1e-6, atol=1e-7)
+    gate_up = RNG.normal(size=(3, 2 * 37)).astype(np.float32) * 4
+    assert np.allclose(twins.swiglu(gate_up), plain.swiglu(gate_up[:, :37], gate_up[:, 37:]), rtol=1e-6, atol=1e-7)
+    a, m = RNG.normal(size=(4, 120)).astype(np.float32), RNG.normal(size=(7, 120)).astype(np.float32)
+    assert np.allclose(twins.gemm(a, m), plain.linear(a, m), rtol=1e-6, atol=1e-6)
+    assert np.allclose(twins.gemm(a, m, c=np.ones((4, 7), np.float32)), plain.linear(a, m) + 1, rtol=1e-6, atol=1e-6)
+    table = RNG.normal(size=(11, 6)).astype(np.float32)
+    status, rows = twins.embed([3, 10, 0], table)
+    assert status == 0 and np.array_equal(rows, plain.embed([3, 10, 0], table))
+    logits = RNG.normal(size=(3, 50)).astype(np.float32)
+    logits[1, 7] = logits[1, 40] = 9.0
+    logits[2, 3] = np.nan
+    tokens, bad = twins.argmax(logits)
+    assert tokens.tolist() == [plain.greedy_token(logits[0]), 7, -1] and bad.tolist() == [0, 0, 1]
+    # bfloat16 storage: the twin rounds what it stores and computes on the rounded values
+    rounded = twins_module.from_bf16_bits(twins_module.to_bf16_bits(gate_up))
+    assert np.allclose(twins.swiglu(gate_up, twins_module.BF16), plain.swiglu(rounded[:, :37], rounded[:, 37:]), rtol=8e-3)
+
+
+@pytest.mark.parametrize("order,head_dim,rot", [(0, 24, 24), (0, 32, 16), (1, 32, 32), (1, 64, 0)])
+def test_cache_write_and_attention_twins_are_the_plain_functions(twins, order, head_dim, rot):
+    """Three sequences with pasts of 0, 70 and 5 tokens get 9, 3 and 130 more: norm, rotation, cache write through
+    shuffled pages, then attention over the pages, against the plain functions on whole sequences."""
+    n_heads, kv_heads, eps, theta, window = 6, 2, 1e-5, 10000.0, 0
+    lengths = [(0, 9), (70, 3), (5, 130)]
+    n_pages = 9
+    pages = RNG.permutation(n_pages).tolist()
+    table = np.zeros((3, 3), np.int32)
+    for s, (past, new) in enumerate(lengths):
+        for j in range(-(-(past + new) // 64)):
+            table[s, j] = pages.pop()
+    fused = (n_heads + 2 * kv_heads) * head_dim
+    whole = [RNG.normal(size=(past + new, fused)).astype(np.float32) for past, new in lengths]
+    qw, kw = (1 + 0.3 * RNG.normal(size=head_dim)).astype(np.float32), (1 + 0.3 * RNG.normal(size=head_dim)).astype(np.float32)
+    freqs = plain.rope_frequencies(theta, rot) if rot else None
+    top = max(past + new for past, new in lengths)
+    cos = np.stack([plain.rope_cos_sin(freqs, p)[0] for p in range(top)]) if rot else None
+    sin = np.stack([plain.rope_cos_sin(freqs, p)[1] for p in range(top)]) if rot else None
+    k_pages = v_pages = None
+    q_new = []
+    for phase in (0, 1):       # the pasts first, then the new rows: two steps onto the same pages
+        rows, positions, row_seq = [], [], []
+        for s, (past, new) in enumerate(lengths):
+            lo, hi = (0, past) if phase == 0 else (past, past + new)
+            rows.append(whole[s][lo:hi])
+            positions.extend(range(lo, hi))
+            row_seq.extend([s] * (hi - lo))
+        q_out, k_pages, v_pages = twins.qk_norm_rope_cache(np.concatenate(rows), qw, kw, eps, cos, sin, positions, row_seq, table,
+                                                           n_pages, n_heads, kv_heads, head_dim, order, k_pages=k_pages, v_pages=v_pages)
+        if phase == 1:
+            q_new, new_positions, new_row_seq = q_out, positions, row_seq
+    scale = 1 / np.sqrt(head_dim)
+    got = twins.attention(q_new, k_pages, v_pages, table, new_row_seq, new_positions, n_heads, kv_heads, head_dim, scale, window, order)
+    at = 0
+    for s, (past, new) in enumerate(lengths):
+        total = past + new
+        q = plain.rmsnorm(whole[s][:, :n_heads * head_dim].reshape(total, n_heads, head_dim), qw, eps)
+        k = plain.rmsnorm(whole[s][:, n_heads * head_dim:(n_heads + kv_heads) * head_dim].reshape(total, kv_heads, head_dim), kw, eps)
+        v = whole[s][:, (n_heads + kv_heads) * head_dim:]
+        for t in range(total if rot else 0):
+            cs = plain.rope_cos_sin(freqs, t)
+            q[t, :, :rot], k[t, :, :rot] = plain.rope_split_half(q[t, :, :rot], *cs), plain.rope_split_half(k[t, :, :rot], *cs)
+        # the cache holds the rotated keys and the raw values where the page table says
+        for t in (0, total - 1, min(64, total - 1)):
+            page = table[s, t // 64]
+            assert np.allclose(twins.key(k_pages, order, page, 1, t % 64, head_dim), k[t, 1], rtol=1e-5, atol=1e-6)
+            assert np.allclose(twins.value(v_pages, order, page, 0, t % 64, head_dim), v[t, :head_dim], rtol=1e-6, atol=1e-7)
+        want = plain.causal_attention(q[past:].reshape(new, -1), k.reshape(total, -1), v, n_heads, kv_heads, head_dim, scale,
+                                      query_start=past)
+        assert np.allclose(got[at:at + new], want, rtol=2e-5, atol=2e-6), s
+        at += new
