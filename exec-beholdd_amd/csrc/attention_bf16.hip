@@ -134,8 +134,12 @@ __device__ inline void pack_head(u32x4_t (&out)[NS], const float (&x)[NS][8]) {
 // NS = head_dim / 32.
 // STREAM = one workgroup per (sequence, kv head, split): each cache byte is read once, past the caches.
 // FUSED = the step is a decode step and `fused.qkv` is given.
-template <int NS, bool STREAM, bool FUSED>
-__global__ __launch_bounds__(256) void attention_mfma_kernel(
+// LEAN (with FUSED) = the queries are normed and rotated before the first page is asked for, and the new key's
+// numbers are asked for after the last page: nothing of that overlaps with the pages any more, but what it needs
+// in registers is gone while the pages stream, so that two workgroups fit a compute unit.  For launches of more
+// workgroups than compute units, where the second workgroup is worth more than the overlap.
+template <int NS, bool STREAM, bool FUSED, bool LEAN = false>
+__global__ __launch_bounds__(256, (LEAN ? 2 : 1)) void attention_mfma_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages,
     const int32_t* __restrict__ page_table, int table_stride, const int32_t* __restrict__ positions,
@@ -171,18 +175,21 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
   HeadPrep<NS> q_prep, k_prep;
   bool q_ready = !FUSED;
   const bool takes_new_key = FUSED && fused.write_kv && split == n_splits - 1 && wave == 0;
+  auto ask_new_key = [&]() {   // one row per sequence: every lane's row is this row
+    const uint16_t* qkv_row = fused.qkv + (size_t)row * (H + 2 * KVH) * HD;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) k_raw[s] = load16(qkv_row + (size_t)(H + kvh) * HD + 32 * s + 8 * g);
+#pragma unroll
+    for (int dt = 0; dt < 2 * NS; ++dt) new_value[dt] = qkv_row[(size_t)(H + KVH + kvh) * HD + 16 * dt + j];
+    // the rotation's numbers are q's, or (LEAN: q's are gone by then) asked for again
+    k_prep.ask(fused.k_weight, fused.weight_f32, LEAN ? fused.cos_table : nullptr, LEAN ? fused.sin_table : nullptr, pos_row, g);
+  };
   if (FUSED) {
     const uint16_t* qkv_row = fused.qkv + (size_t)row * (H + 2 * KVH) * HD;
 #pragma unroll
     for (int s = 0; s < NS; ++s) q_raw[s] = load16(qkv_row + (size_t)head * HD + 32 * s + 8 * g);
     q_prep.ask(fused.q_weight, fused.weight_f32, fused.cos_table, fused.sin_table, pos_row, g);
-    if (takes_new_key) {   // one row per sequence: every lane's row is this row
-#pragma unroll
-      for (int s = 0; s < NS; ++s) k_raw[s] = load16(qkv_row + (size_t)(H + kvh) * HD + 32 * s + 8 * g);
-#pragma unroll
-      for (int dt = 0; dt < 2 * NS; ++dt) new_value[dt] = qkv_row[(size_t)(H + KVH + kvh) * HD + 16 * dt + j];
-      k_prep.ask(fused.k_weight, fused.weight_f32, nullptr, nullptr, pos_row, g);   // the rotation's numbers are q's
-    }
+    if (takes_new_key && !LEAN) ask_new_key();
   } else {
     const uint16_t* qp = q + ((size_t)row * H + head) * HD + 8 * g;
 #pragma unroll
@@ -198,6 +205,7 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
     for (int s = 0; s < NS; ++s) q_vec[s] = as_bf16x8(packed[s]);
     q_ready = true;
   };
+  if (FUSED && LEAN) finish_q();
   const int pos_max = wave_max_int(pos), pos_min = wave_min_int(pos);
   const int lo_min = wave_min_int(lo), lo_max = wave_max_int(lo);
 
@@ -312,15 +320,18 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
     // The new key and value of this (sequence, kv head): normed and rotated here, attended to as a page in
     // which only their own slot is visible, and written into the cache.
     if (!q_ready) finish_q();
+    if (LEAN) ask_new_key();
     float x[NS][8];
     widen_head<NS>(x, k_raw);
+    if (!LEAN) {
 #pragma unroll
-    for (int s = 0; s < HeadPrep<NS>::HS; ++s)
+      for (int s = 0; s < HeadPrep<NS>::HS; ++s)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        k_prep.cos_v[s][e] = q_prep.cos_v[s][e];
-        k_prep.sin_v[s][e] = q_prep.sin_v[s][e];
-      }
+        for (int e = 0; e < 8; ++e) {
+          k_prep.cos_v[s][e] = q_prep.cos_v[s][e];
+          k_prep.sin_v[s][e] = q_prep.sin_v[s][e];
+        }
+    }
     k_prep.apply(x, fused.k_weight != nullptr, fused.weight_f32, fused.eps, fused.cos_table != nullptr);
     u32x4_t new_key[NS];
     pack_head<NS>(new_key, x);
@@ -476,15 +487,17 @@ static int attention_bf16_run(const void* q, void* out, void* part_o, void* part
     return bh_check_launch("attention_prefill_bf16");
   }
   const int tile_groups = tiles, z_count = n_seqs * n_splits;
+  const bool lean = (long)tiles * KVH * z_count > 256;   // more workgroups than compute units: two of them per unit
   dim3 grid(tile_groups * KVH * z_count), block(256);
-#define BH_ATT_ONE(NS, STREAM, FUSED)                                                                           \
-  attention_mfma_kernel<NS, STREAM, FUSED><<<grid, block, 0, stream>>>(                                         \
+#define BH_ATT_ONE(NS, STREAM, FUSED, ...)                                                                      \
+  attention_mfma_kernel<NS, STREAM, FUSED, ##__VA_ARGS__><<<grid, block, 0, stream>>>(                          \
       (const uint16_t*)q, (uint16_t*)out, (float*)part_o, (float*)part_ml, (const uint16_t*)k_pages,            \
       (const uint16_t*)v_pages, page_table, table_stride, positions, seq_start, H, KVH, scale_log2, window,     \
       n_splits, per, tile_groups, fused)
 #define BH_ATT(NS)                                      \
   do {                                                  \
-    if (is_fused) BH_ATT_ONE(NS, true, true);           \
+    if (is_fused && lean && NS <= 4) BH_ATT_ONE(NS, true, true, (NS <= 4));   \
+    else if (is_fused) BH_ATT_ONE(NS, true, true);      \
     else if (tile_groups == 1) BH_ATT_ONE(NS, true, false);  \
     else BH_ATT_ONE(NS, false, false);                  \
   } while (0)

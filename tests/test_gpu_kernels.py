@@ -640,6 +640,48 @@ def test_decode_attention_from_the_projection_rows(K, n_heads, kv_heads, head_di
         assert torch.equal(k_one.cpu(), stored(K, kp, vp)[0].cpu())
 
 
+def test_decode_attention_from_the_projection_rows_of_many_sequences(K):
+    """Forty sequences on eight kv heads: more workgroups than compute units, no split keys; the one launch runs in
+    the form that norms the queries before the first page and takes the new key's numbers after the last."""
+    dtype, n_heads, kv_heads, head_dim = torch.bfloat16, 32, 8, 128
+    lengths = [1 + (37 * i) % 300 for i in range(40)]
+    n = len(lengths)
+    kp, vp, table, keys, values = make_cache(n, lengths, kv_heads, head_dim, dtype, seed=9)
+    gen = torch.Generator().manual_seed(6)
+    qkv = torch.randn(n, (n_heads + 2 * kv_heads) * head_dim, generator=gen).to(dtype)
+    qw = dev((1 + 0.2 * torch.randn(head_dim, generator=gen)).to(dtype))
+    kw = dev((1 + 0.2 * torch.randn(head_dim, generator=gen)).to(dtype))
+    freqs = 1.0 / 1e6 ** (torch.arange(0, head_dim, 2, dtype=torch.float64) / head_dim)
+    angles = torch.arange(512, dtype=torch.float64)[:, None] * freqs
+    cos, sin = dev(angles.cos().float()), dev(angles.sin().float())
+    positions = dev(torch.tensor([length - 1 for length in lengths], dtype=torch.int32))
+    row_seq = dev(torch.arange(n, dtype=torch.int32))
+    layout = Layout(True, dev(torch.arange(n + 1, dtype=torch.int32)), n, 1, max(lengths) - 1)
+    assert K.lib.bh_attention_bf16_splits(n, 1, n_heads, kv_heads, max(lengths) - 1) == 1
+    scale, eps = 1 / math.sqrt(head_dim), 1e-6
+    k_two, v_two = stored(K, kp, vp)
+    q = torch.empty(n, n_heads * head_dim, dtype=dtype, device="cuda:0")
+    out_two = torch.empty_like(q)
+    K.qk_norm_rope_cache(dev(qkv), q, qw, kw, eps, cos, sin, positions, row_seq, k_two, v_two, dev(table), n_heads,
+                         kv_heads, head_dim, True, max(lengths) - 1)
+    K.attention(q, out_two, k_two, v_two, dev(table), row_seq, positions, n_heads, kv_heads, head_dim, scale, 0, layout=layout)
+    k_one, v_one = stored(K, kp, vp)
+    out_one = torch.empty_like(q)
+    assert K.attention_decode_fused(dev(qkv), out_one, qw, kw, eps, cos, sin, positions, k_one, v_one, dev(table), n_heads,
+                                    kv_heads, head_dim, scale, 0, True, layout) is True
+    assert rel(out_one, out_two.double()) < 8e-3
+    assert torch.equal(v_one.cpu(), v_two.cpu()) and rel(k_one, k_two.double()) < 8e-3
+    # and against the plain attention over the dense keys and values, with the new key and value in place
+    k_rows, v_rows = as_rows(K, k_one, v_one)
+    for s in (0, 7, 39):
+        pos = lengths[s] - 1
+        page = int(table[s, pos // PAGE])
+        keys[s][pos] = k_rows[page, :, pos % PAGE].float().to(dtype)
+        values[s][pos] = v_rows[page, :, :, pos % PAGE].float().to(dtype)
+        want = attention_reference(q[s].cpu().reshape(n_heads, head_dim), keys[s], values[s], pos, n_heads, kv_heads, head_dim, scale, 0)
+        assert rel(out_one[s].reshape(n_heads, head_dim), want) < 1.2e-2, s
+
+
 def test_decode_attention_from_the_projection_rows_says_when_it_cannot(K):
     dtype = torch.bfloat16
     kp, vp, table, _, _ = make_cache(1, [10], 2, 48, dtype, seed=1)
