@@ -47,7 +47,8 @@ __device__ inline u32x4_t keep_first(u32x4_t v, int n_valid) {
 }
 
 // Many columns per sequence (prefill): see attention_prefill_bf16.hip.  The caller has checked the sizes.
+// out_blocked: the output [rows][H * hd] goes out in blocks of 16 rows x 32 columns (bh_blocked_index).
 void bh_attention_prefill_launch(const void* q, void* out, const void* k_pages, const void* v_pages,
                                  const int32_t* page_table, int table_stride, const int32_t* positions,
                                  const int32_t* seq_start, int n_seqs, int tiles, int H, int KVH, int hd,
-                                 float scale_log2, int window, hipStream_t stream);
+                                 float scale_log2, int window, int out_blocked, hipStream_t stream);

@@ -462,11 +462,21 @@ extern "C" int bh_attention_bf16_splits(int n_seqs, int max_rows_per_seq, int H,
   return (pages + per - 1) / per;
 }
 
+#define PREFILL_FROM_TILES 1024   // column tiles x kv heads x sequences from which the prefill kernel runs a step
+// Whether a step of these sizes can write its output in blocks of 16 rows x 32 columns (bh_blocked_index) for
+// the product that reads it: the steps of the prefill kernel.
+extern "C" int bh_attention_bf16_writes_blocked(int n_seqs, int max_rows_per_seq, int H, int KVH, int max_position) {
+  if (n_seqs <= 0 || max_rows_per_seq <= 0 || H <= 0 || KVH <= 0 || H % KVH) return 0;
+  const long tiles = (long)((max_rows_per_seq * (H / KVH) + 15) / 16) * KVH * n_seqs;
+  return bh_attention_bf16_splits(n_seqs, max_rows_per_seq, H, KVH, max_position) == 1 && tiles >= PREFILL_FROM_TILES ? 1 : 0;
+}
+
 static int attention_bf16_run(const void* q, void* out, void* part_o, void* part_ml, const void* k_pages,
                               const void* v_pages, const int32_t* page_table, int table_stride,
                               const int32_t* positions, const int32_t* seq_start, int n_seqs, int n_rows,
                               int max_rows_per_seq, int H, int KVH, int hd, float scale, int window,
-                              int max_position, int n_splits, const FusedQkv& fused, hipStream_t stream) {
+                              int max_position, int n_splits, const FusedQkv& fused, int out_blocked,
+                              hipStream_t stream) {
   BH_REQUIRE(n_seqs > 0 && n_rows > 0 && max_rows_per_seq > 0, "attention_bf16: empty batch");
   BH_REQUIRE(H > 0 && KVH > 0 && H % KVH == 0, "attention_bf16: %d query heads do not group evenly into %d kv heads", H, KVH);
   BH_REQUIRE(hd % 32 == 0 && hd >= 32 && hd <= 256, "attention_bf16: head size %d is not a multiple of 32 up to 256", hd);
@@ -481,11 +491,12 @@ static int attention_bf16_run(const void* q, void* out, void* part_o, void* part
   const bool is_fused = fused.qkv != nullptr;
   BH_REQUIRE(!is_fused || (tiles == 1 && max_rows_per_seq == 1 && n_rows == n_seqs),
              "attention_bf16: the fused projection rows are taken in decode steps of at most 16 heads per kv head only");
-  if (!is_fused && n_splits == 1 && (long)tiles * KVH * n_seqs >= 1024) {   // many columns: the prefill kernel
+  if (!is_fused && n_splits == 1 && (long)tiles * KVH * n_seqs >= PREFILL_FROM_TILES) {   // many columns: the prefill kernel
     bh_attention_prefill_launch(q, out, k_pages, v_pages, page_table, table_stride, positions, seq_start, n_seqs,
-                                tiles, H, KVH, hd, scale_log2, window, stream);
+                                tiles, H, KVH, hd, scale_log2, window, out_blocked, stream);
     return bh_check_launch("attention_prefill_bf16");
   }
+  BH_REQUIRE(!out_blocked, "attention_bf16: this step's output cannot go out in blocks (bh_attention_bf16_writes_blocked)");
   const int tile_groups = tiles, z_count = n_seqs * n_splits;
   const bool lean = (long)tiles * KVH * z_count > 256;   // more workgroups than compute units: two of them per unit
   dim3 grid(tile_groups * KVH * z_count), block(256);
@@ -526,11 +537,11 @@ extern "C" int bh_attention_bf16(const void* q, void* out, void* part_o, void* p
                                  const void* v_pages, const int32_t* page_table, int table_stride,
                                  const int32_t* positions, const int32_t* seq_start, int n_seqs, int n_rows,
                                  int max_rows_per_seq, int H, int KVH, int hd, float scale, int window,
-                                 int max_position, int n_splits, hipStream_t stream) {
+                                 int max_position, int n_splits, int out_blocked, hipStream_t stream) {
   const FusedQkv none = {nullptr, nullptr, nullptr, 0, 0.f, nullptr, nullptr, 0, nullptr, nullptr};
   return attention_bf16_run(q, out, part_o, part_ml, k_pages, v_pages, page_table, table_stride, positions,
                             seq_start, n_seqs, n_rows, max_rows_per_seq, H, KVH, hd, scale, window, max_position,
-                            n_splits, none, stream);
+                            n_splits, none, out_blocked, stream);
 }
 
 // A decode step (one row per sequence) straight from the fused projection rows [q heads | k heads | v heads]:
@@ -556,5 +567,5 @@ extern "C" int bh_attention_decode_fused(const void* qkv, void* out, void* part_
                           write_kv, (uint16_t*)k_pages, (uint16_t*)v_pages};
   return attention_bf16_run(nullptr, out, part_o, part_ml, k_pages, v_pages, page_table, table_stride, positions,
                             seq_start, n_seqs, n_seqs, 1, H, KVH, hd, scale, window, max_position, n_splits, fused,
-                            stream);
+                            0, stream);
 }

@@ -25,7 +25,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
     const uint16_t* __restrict__ q, uint16_t* __restrict__ out, const uint16_t* __restrict__ k_pages,
     const uint16_t* __restrict__ v_pages, const int32_t* __restrict__ page_table, int table_stride,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_start, int H, int KVH,
-    float scale_log2, int window, int tile_groups, int n_seqs) {
+    float scale_log2, int window, int tile_groups, int n_seqs, int out_blocked) {
   constexpr int HD = 32 * NS;
   constexpr int PIECES = BH_PAGE * HD / 8;        // 16-byte pieces of one head's keys (or values) in a page
   constexpr int STAGE = 2 * PIECES / 256;         // pieces of a page (keys, then values) one thread copies
@@ -238,13 +238,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
     total += __shfl_xor(total, 32, 64);
     if (cc >= n_cols) continue;
     const float inv = 1.0f / total;
-    uint16_t* op = out + ((size_t)(row0 + cc / G) * H + kvh * G + cc % G) * HD + 4 * g;
+    const int out_row = row0 + cc / G, out_column = (kvh * G + cc % G) * HD + 4 * g;
 #pragma unroll
     for (int dt = 0; dt < 2 * NS; ++dt) {
       uint2 packed;
       packed.x = pack_bf16(o[ct][dt][0] * inv, o[ct][dt][1] * inv);
       packed.y = pack_bf16(o[ct][dt][2] * inv, o[ct][dt][3] * inv);
-      *reinterpret_cast<uint2*>(op + 16 * dt) = packed;
+      const size_t at = out_blocked ? (size_t)bh_blocked_index(out_row, out_column + 16 * dt, H * HD)
+                                    : (size_t)out_row * (H * HD) + out_column + 16 * dt;
+      *reinterpret_cast<uint2*>(out + at) = packed;
     }
   }
 }
@@ -252,13 +254,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
 void bh_attention_prefill_launch(const void* q, void* out, const void* k_pages, const void* v_pages,
                                  const int32_t* page_table, int table_stride, const int32_t* positions,
                                  const int32_t* seq_start, int n_seqs, int tiles, int H, int KVH, int hd,
-                                 float scale_log2, int window, hipStream_t stream) {
+                                 float scale_log2, int window, int out_blocked, hipStream_t stream) {
 #define BH_PREFILL(NS, CTW)                                                                                  \
   do {                                                                                                       \
     const int tile_groups = (tiles + 4 * CTW - 1) / (4 * CTW);                                               \
     attention_prefill_kernel<NS, CTW><<<dim3(tile_groups * KVH * n_seqs), dim3(256), 0, stream>>>(           \
         (const uint16_t*)q, (uint16_t*)out, (const uint16_t*)k_pages, (const uint16_t*)v_pages, page_table,  \
-        table_stride, positions, seq_start, H, KVH, scale_log2, window, tile_groups, n_seqs);                \
+        table_stride, positions, seq_start, H, KVH, scale_log2, window, tile_groups, n_seqs, out_blocked);   \
   } while (0)
   // Two column tiles per wave while the accumulators leave room for two workgroups per compute unit; one
   // where that gives fewer than two workgroups per compute unit (a page costs a workgroup nearly the same

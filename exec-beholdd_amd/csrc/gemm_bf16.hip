@@ -358,54 +358,103 @@ __global__ __launch_bounds__(256) void gemm_parts_finish_kernel(const float* __r
 // ---- tiled -----------------------------------------------------------------------------------
 
 // The same for a product that completes the float32 residual right before an RMSNorm reads it, with many rows
-// (the parts come from the kernel whose wave groups take turns): a block owns a whole row, so it can finish the
-// norm itself and the norm needs no launch and no second pass over the residual.  Thread t has the groups of
-// four columns t, t + 256, ...; the parts are added in their order, then the residual's old values, as the kernel
-// above does; the row's sum of squares is added up as rmsnorm does it for this width.
-#define FINISH_NORM_GROUPS 8   // groups of four columns per thread: rows of up to 8,192
-__global__ __launch_bounds__(256) void gemm_parts_finish_norm_kernel(const float* __restrict__ sums, float* __restrict__ c,
-                                                                     int M, int N, int parts, const void* __restrict__ weight,
-                                                                     int weight_f32, float eps, uint16_t* __restrict__ normed) {
-  __shared__ float scratch[4];
-  const int row = blockIdx.x, fours = N / 4;
-  f32x4_t* residual = reinterpret_cast<f32x4_t*>(c + (size_t)row * N);
-  f32x4_t value[FINISH_NORM_GROUPS];
+// (the parts come from the kernel whose wave groups take turns): a block owns eight whole rows, so it can finish
+// the norm itself and the norm needs no launch and no second pass over the residual.  Lane l of wave w has row
+// l % 8 of the block's rows and the pieces of eight columns 8 w + l / 8, + 128, ...: a wave reads 256 contiguous
+// bytes of each of its rows and writes 128 contiguous bytes of the norm's output per row, or, with
+// normed_blocked (the output in blocks of 16 rows x 32 columns, bh_blocked_index, for a product that reads it
+// that way), the 128 bytes that eight rows' pieces of the same columns fill there.  The parts are added in their
+// order, then the residual's old values, as the kernel above does; a row's sum of squares is added up in an
+// order that depends on the width only.
+#define FINISH_NORM_PIECES 8   // pieces of eight columns per thread: rows of up to 8,192
+typedef uint32_t finish_u32x4_t __attribute__((ext_vector_type(4)));
+template <int PARTS, int ROWS>   // PARTS: at least `parts`, what the loop over them is unrolled to; ROWS per block, 128 threads each
+__global__ __launch_bounds__(128 * ROWS) void gemm_parts_finish_norm_kernel(const float* __restrict__ sums, float* __restrict__ c,
+                                                                      int M, int N, int parts, const void* __restrict__ weight,
+                                                                      int weight_f32, float eps, uint16_t* __restrict__ normed,
+                                                                      int normed_blocked) {
+  constexpr int WAVES = 2 * ROWS, WAVE_PIECES = 64 / ROWS;   // a step over the row is 128 pieces wide
+  __shared__ float partial[WAVES][ROWS];
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const int r = lane % ROWS, row = blockIdx.x * ROWS + r, pieces = N / 8;
+  const bool row_there = row < M;
+  const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+  constexpr bool KEEP = PARTS <= 4;   // with more parts the registers do not hold the new values too: they are read again
+  f32x4_t value[KEEP ? FINISH_NORM_PIECES : 1][2];
   float ss = 0.f;
 #pragma unroll
-  for (int j = 0; j < FINISH_NORM_GROUPS; ++j) {
-    const int i = threadIdx.x + j * 256;
-    value[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    if (i >= fours) continue;
-    f32x4_t part[MAX_TURNS_PARTS];
-    const f32x4_t old = residual[i];
+  for (int j = 0; j < FINISH_NORM_PIECES; ++j) {
+    const int piece = WAVE_PIECES * wave + lane / ROWS + 128 * j;
+    const bool there = row_there && piece < pieces;
+    if (KEEP) value[j][0] = value[j][1] = zero;
+    if (!there) continue;
+    f32x4_t* residual = reinterpret_cast<f32x4_t*>(c + (size_t)row * N + 8 * piece);
+    constexpr int GROUP = PARTS < 4 ? PARTS : 4;   // parts whose loads are on their way together
+    const f32x4_t old[2] = {residual[0], residual[1]};
+    f32x4_t sum[2] = {zero, zero};
 #pragma unroll
-    for (int p = 0; p < MAX_TURNS_PARTS; ++p)
-      part[p] = p < parts ? reinterpret_cast<const f32x4_t*>(sums + ((size_t)p * M + row) * N)[i] : f32x4_t{0.f, 0.f, 0.f, 0.f};
-    f32x4_t sum = part[0];
+    for (int p0 = 0; p0 < PARTS; p0 += GROUP) {
+      f32x4_t part[GROUP][2];
 #pragma unroll
-    for (int p = 1; p < MAX_TURNS_PARTS; ++p) sum += part[p];
-    value[j] = sum + old;
-    residual[i] = value[j];
-    ss += value[j][0] * value[j][0] + value[j][1] * value[j][1] + value[j][2] * value[j][2] + value[j][3] * value[j][3];
-  }
-  ss = block_sum(ss, scratch);
-  const float inv = 1.0f / sqrtf(ss / (float)N + eps);
+      for (int u = 0; u < GROUP; ++u) {
+        const int p = p0 + u;
+        const f32x4_t* from = reinterpret_cast<const f32x4_t*>(sums + ((size_t)(p < parts ? p : 0) * M + row) * N + 8 * piece);
+        part[u][0] = p < parts ? from[0] : zero;
+        part[u][1] = p < parts ? from[1] : zero;
+      }
 #pragma unroll
-  for (int j = 0; j < FINISH_NORM_GROUPS; ++j) {
-    const int i = threadIdx.x + j * 256;
-    if (i >= fours) continue;
-    f32x4_t g;
-    if (weight_f32) {
-      g = reinterpret_cast<const f32x4_t*>(weight)[i];
-    } else {
-      const u16x4_t raw = reinterpret_cast<const u16x4_t*>(weight)[i];
+      for (int half = 0; half < 2; ++half)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) g[e] = bf16_bits_to_f32(raw[e]);
+        for (int u = 0; u < GROUP; ++u) sum[half] = p0 + u == 0 ? part[u][half] : sum[half] + part[u][half];
     }
-    u16x4_t bits;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) bits[e] = f32_to_bf16_bits(value[j][e] * inv * g[e]);
-    reinterpret_cast<u16x4_t*>(normed + (size_t)row * N)[i] = bits;
+    for (int half = 0; half < 2; ++half) {
+      const f32x4_t v = sum[half] + old[half];
+      if (KEEP) value[j][half] = v;
+      residual[half] = v;
+      ss += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+    }
+  }
+#pragma unroll
+  for (int step = ROWS; step < 64; step *= 2) ss += __shfl_xor(ss, step, 64);
+  if (lane < ROWS) partial[wave][lane] = ss;
+  __syncthreads();
+  float total = 0.f;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) total += partial[w][r];
+  const float inv = 1.0f / sqrtf(total / (float)N + eps);
+#pragma unroll
+  for (int j = 0; j < FINISH_NORM_PIECES; ++j) {
+    const int piece = WAVE_PIECES * wave + lane / ROWS + 128 * j;
+    if (!row_there || piece >= pieces) continue;
+    f32x4_t g[2];
+    if (weight_f32) {
+      g[0] = reinterpret_cast<const f32x4_t*>(weight)[2 * piece];
+      g[1] = reinterpret_cast<const f32x4_t*>(weight)[2 * piece + 1];
+    } else {
+      const finish_u32x4_t raw = reinterpret_cast<const finish_u32x4_t*>(weight)[piece];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        g[e / 2][2 * (e % 2)] = bf16_bits_to_f32((uint16_t)(raw[e] & 0xffffu));
+        g[e / 2][2 * (e % 2) + 1] = bf16_bits_to_f32((uint16_t)(raw[e] >> 16));
+      }
+    }
+    f32x4_t v[2];
+    if (KEEP) {
+      v[0] = value[j][0], v[1] = value[j][1];
+    } else {
+      const f32x4_t* residual = reinterpret_cast<const f32x4_t*>(c + (size_t)row * N + 8 * piece);
+      v[0] = residual[0], v[1] = residual[1];
+    }
+    finish_u32x4_t bits;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int half = e / 2, i = 2 * (e % 2);
+      bits[e] = (uint32_t)f32_to_bf16_bits(v[half][i] * inv * g[half][i]) |
+                ((uint32_t)f32_to_bf16_bits(v[half][i + 1] * inv * g[half][i + 1]) << 16);
+    }
+    const size_t at = normed_blocked ? (size_t)bh_blocked_index(row, 8 * piece, N) : (size_t)row * N + 8 * piece;
+    *reinterpret_cast<finish_u32x4_t*>(normed + at) = bits;
   }
 }
 
@@ -958,6 +1007,13 @@ extern "C" int bh_gemm_bf16_takes_norm(int M, int N, int K, int layout, int acti
   return tiled_whole(M, N, K, layout, rows, columns) ? 1 : 0;
 }
 
+// Whether a product of these sizes reads its activations faster from blocks of 16 rows x 32 columns
+// (bh_blocked_index, layout.h) and takes them that way: those of the kernel whose wave groups take turns.
+extern "C" int bh_gemm_bf16_reads_blocked(int M, int N, int K, int layout, int activation) {
+  if (M <= 0 || N <= 0 || K <= 0 || K % 32 != 0) return 0;
+  return gemm_turns_blocks(M, N, K, layout, activation) || gemm_turns_parts(M, N, K, layout, activation) > 1 ? 1 : 0;
+}
+
 // layout: 0 = rows, 1 = tiles.  activation: 0 = none; 1 = SwiGLU (W has 2 * N rows: gate rows then up rows).
 // Bytes of scratch memory that bh_gemm_bf16 wants for this product (0: none).
 extern "C" long bh_gemm_bf16_scratch(int M, int N, int K, int layout, int activation) {
@@ -976,7 +1032,7 @@ extern "C" long bh_gemm_bf16_scratch(int M, int N, int K, int layout, int activa
 extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, int accumulate, int M, int N, int K,
                             int layout, int activation, const float* ahead_ss, int ahead_blocks, float ahead_eps,
                             const void* behind_weight, int behind_weight_dtype, void* behind_rows,
-                            float* behind_ss, void* scratch, hipStream_t stream) {
+                            float* behind_ss, void* scratch, int a_blocked, int c_blocked, hipStream_t stream) {
   BH_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_bf16: sizes M=%d N=%d K=%d must be positive", M, N, K);
   BH_REQUIRE(K % 8 == 0, "gemm_bf16: K=%d must be a multiple of 8", K);
   BH_REQUIRE(c_dtype == BH_F32 || c_dtype == BH_BF16, "gemm_bf16: unknown output dtype %d", c_dtype);
@@ -998,9 +1054,13 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
   const RidingNorm norm = {ahead_ss, ahead_blocks, ahead_eps, behind_weight, behind_weight_dtype == BH_F32,
                            (uint16_t*)behind_rows, behind_ss};
   const bool f32 = c_dtype == BH_F32;
+  BH_REQUIRE((!a_blocked && !c_blocked) || (!ahead_ss && !behind_weight && (f32 || !accumulate) &&
+                                            bh_gemm_bf16_reads_blocked(M, N, K, layout, activation)),
+             "gemm_bf16: a product of M=%d N=%d K=%d does not take rows in blocks (bh_gemm_bf16_reads_blocked)", M, N, K);
+  BH_REQUIRE(!c_blocked || gemm_turns_blocks(M, N, K, layout, activation), "gemm_bf16: this product writes no blocks");
   if (!ahead_ss && !behind_weight && (f32 || !accumulate)) {   // many rows: the kernel whose wave groups take turns
     if (const int blocks = gemm_turns_blocks(M, N, K, layout, activation))
-      return gemm_turns_launch(a, w, c, c_dtype, accumulate, M, N, K, activation, blocks, stream);
+      return gemm_turns_launch(a, w, c, c_dtype, accumulate, M, N, K, activation, blocks, a_blocked, c_blocked, stream);
   }
 #define BH_PICK(FN, TILES, EXTRA, ...)                                             \
   do {                                                                              \
@@ -1008,6 +1068,8 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
     else FN<TILES, EXTRA, bf16_t>(__VA_ARGS__);                                     \
   } while (0)
   const bool in_parts = scratch != nullptr && bh_gemm_bf16_scratch(M, N, K, layout, activation) > 0;
+  BH_REQUIRE(!a_blocked || (in_parts && gemm_turns_parts(M, N, K, layout, activation) > 1),
+             "gemm_bf16: a product of M=%d N=%d K=%d that reads rows in blocks needs its scratch memory", M, N, K);
   BH_REQUIRE(in_parts || !behind_weight || bh_gemm_bf16_scratch(M, N, K, layout, activation) == 0,
              "gemm_bf16: a product of M=%d N=%d K=%d carries a norm through its finishing kernel and needs scratch memory", M, N, K);
   if (in_parts) {   // K in parts, then the finishing kernel
@@ -1016,7 +1078,7 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
     int parts, each;
     if (const int turns_parts = gemm_turns_parts(M, N, K, layout, activation); turns_parts > 1) {
       parts = turns_parts;
-      if (int status = gemm_turns_launch_parts(a, w, (float*)scratch, M, N, K, parts, stream)) return status;
+      if (int status = gemm_turns_launch_parts(a, w, (float*)scratch, M, N, K, parts, a_blocked, stream)) return status;
     } else {
       tiled_parts(M, N, K, layout, activation != 0, &parts, &each);
       const RidingNorm none = {};
@@ -1061,13 +1123,13 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
 // many rows whose K the turns kernel multiplies in parts (bh_gemm_bf16_finishes_norm says which), whose finishing
 // kernel streams the residual anyway.  `scratch`: bh_gemm_bf16_scratch() bytes.
 extern "C" int bh_gemm_bf16_finishes_norm(int M, int N, int K, int layout) {
-  if (M <= 0 || N <= 0 || K <= 0 || N % 4 != 0 || N > 4 * 256 * FINISH_NORM_GROUPS) return 0;
+  if (M <= 0 || N <= 0 || K <= 0 || N % 8 != 0 || N > 8 * 128 * FINISH_NORM_PIECES) return 0;
   const int parts = gemm_turns_parts(M, N, K, layout, 0);
   return parts > 1 && parts <= MAX_TURNS_PARTS ? 1 : 0;
 }
 extern "C" int bh_gemm_bf16_then_norm(const void* a, const void* w, float* residual, int M, int N, int K, int layout,
                                       const void* norm_weight, int norm_weight_dtype, float eps, void* normed,
-                                      void* scratch, hipStream_t stream) {
+                                      void* scratch, int a_blocked, int normed_blocked, hipStream_t stream) {
   BH_REQUIRE(bh_gemm_bf16_finishes_norm(M, N, K, layout),
              "gemm_bf16_then_norm: a product of M=%d N=%d K=%d does not finish a norm (bh_gemm_bf16_finishes_norm)", M, N, K);
   BH_REQUIRE(a && w && residual && norm_weight && normed && scratch, "gemm_bf16_then_norm: every operand is needed");
@@ -1075,9 +1137,26 @@ extern "C" int bh_gemm_bf16_then_norm(const void* a, const void* w, float* resid
   BH_REQUIRE(eps >= 0.f, "gemm_bf16_then_norm: eps must not be negative");
   BH_REQUIRE(((uintptr_t)a | (uintptr_t)w | (uintptr_t)residual | (uintptr_t)normed | (uintptr_t)scratch | (uintptr_t)norm_weight) % 16 == 0,
              "gemm_bf16_then_norm: operands must be 16-byte aligned");
+  BH_REQUIRE(!normed_blocked || N % 32 == 0, "gemm_bf16_then_norm: rows in blocks need N=%d to be a multiple of 32", N);
   const int parts = gemm_turns_parts(M, N, K, layout, 0);
-  if (int status = gemm_turns_launch_parts(a, w, (float*)scratch, M, N, K, parts, stream)) return status;
-  gemm_parts_finish_norm_kernel<<<M, 256, 0, stream>>>((const float*)scratch, residual, M, N, parts, norm_weight,
-                                                       norm_weight_dtype == BH_F32, eps, (uint16_t*)normed);
+  if (int status = gemm_turns_launch_parts(a, w, (float*)scratch, M, N, K, parts, a_blocked, stream)) return status;
+#define BH_FINISH_NORM_ROWS(PARTS, ROWS)                                                                              \
+  gemm_parts_finish_norm_kernel<PARTS, ROWS><<<(M + ROWS - 1) / ROWS, 128 * ROWS, 0, stream>>>(                        \
+      (const float*)scratch, residual, M, N, parts, norm_weight, norm_weight_dtype == BH_F32, eps, (uint16_t*)normed, \
+      normed_blocked)
+  // Rows per block: at 1,024 rows two ran 4 % faster than eight (more and smaller blocks), from 2,048 rows on all ran
+  // alike; full 128-byte lines of the blocked output take eight.
+  const int rows_per_block = M >= 4096 ? 8 : M >= 2048 ? 4 : 2;
+#define BH_FINISH_NORM(PARTS)                          \
+  do {                                                 \
+    if (rows_per_block == 8) BH_FINISH_NORM_ROWS(PARTS, 8); \
+    else if (rows_per_block == 4) BH_FINISH_NORM_ROWS(PARTS, 4); \
+    else BH_FINISH_NORM_ROWS(PARTS, 2); \
+  } while (0)
+  if (parts <= 2) BH_FINISH_NORM(2);
+  else if (parts <= 4) BH_FINISH_NORM(4);
+  else BH_FINISH_NORM(MAX_TURNS_PARTS);
+#undef BH_FINISH_NORM_ROWS
+#undef BH_FINISH_NORM
   return bh_check_launch("gemm_parts_finish_norm");
 }

@@ -73,9 +73,13 @@ __device__ inline void tile_of_workgroup(int n_tiles, int m_tiles, int* tile_n, 
 // (N outputs; W has 2 N rows, gate rows then up rows; a wave's weight rows are the gate and the up rows of
 // the same outputs).  YB: blocks of 16 weight rows per wave.
 // A tile that would stick out of the matrix is moved back inside and stores only what it owns.
+// a_blocked: A lies in blocks of 16 rows x 32 k in operand order (bh_blocked_index), so that a wave's load of an
+// operand is 1 KB of contiguous memory; its buffer holds whole tiles of 256 rows, and a tile that sticks out
+// below stays where it is and stores only the rows that exist.  c_blocked (MODE 2): the output likewise.
 template <int MODE, int YB>
 __global__ __launch_bounds__(512) void gemm_turns_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ w,
-                                                      void* __restrict__ c, int M, int N, int K, int accumulate) {
+                                                      void* __restrict__ c, int M, int N, int K, int accumulate,
+                                                      int a_blocked, int c_blocked) {
   constexpr int OUTS = MODE == 2 ? 16 * YB : 32 * YB;
   constexpr int CHUNKS = 16 + 2 * YB;
   constexpr int WL = YB / 2;   // W chunks per loading wave
@@ -87,7 +91,7 @@ __global__ __launch_bounds__(512) void gemm_turns_kernel(const uint16_t* __restr
   int tile_n, tile_m;
   tile_of_workgroup((N + OUTS - 1) / OUTS, (M + 255) / 256, &tile_n, &tile_m);
   const int m_own = tile_m * 256, n_own = tile_n * OUTS;
-  const int m0 = min(m_own, M - 256), n0 = min(n_own, N - OUTS);
+  const int m0 = a_blocked ? m_own : min(m_own, M - 256), n0 = min(n_own, N - OUTS);
   // K in parts (blockIdx.y, MODE 1 only): part p multiplies its share of k and leaves the bare sums at
   // c + p * M * N for the finishing kernel of gemm_bf16.hip; one part is the whole product.
   const int k_part = K / gridDim.y, k_first = blockIdx.y * k_part;
@@ -97,7 +101,9 @@ __global__ __launch_bounds__(512) void gemm_turns_kernel(const uint16_t* __restr
   // A step takes 32 consecutive k: lane (row r = lane % 16, group q = lane / 16) holds k 8 q .. 8 q + 7 of them,
   // so four lanes bring 64 consecutive bytes of a row.  In W's tiles layout those are the 16-byte pieces
   // 4 v + q of the row (v: first or second step of the slice), piece p at half p % 2, lane 16 (p / 2) + r.
-  const uint16_t* a_src = a + (size_t)(m0 + 64 * i4 + lane % 16) * K + k_first + 8 * (lane / 16);
+  const uint16_t* a_src = a_blocked ? a + ((size_t)((m0 + 64 * i4) / 16) * (K / 32) + k_first / 32) * 512 + lane * 8
+                                    : a + (size_t)(m0 + 64 * i4 + lane % 16) * K + k_first + 8 * (lane / 16);
+  const size_t a_block = a_blocked ? (size_t)(K / 32) * 512 : (size_t)16 * K;   // from 16 rows to the next
   const int w_lane = ((lane / 16) % 2) * 512 + (16 * (lane / 32) + lane % 16) * 8;   // + 256 elements for the second step
   const uint16_t* w_src[WL];
 #pragma unroll
@@ -110,7 +116,7 @@ __global__ __launch_bounds__(512) void gemm_turns_kernel(const uint16_t* __restr
     const int s = j >> 1, u = j & 1;
 #pragma unroll
     for (int b = 0; b < 4; ++b)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_src + (size_t)b * 16 * K + s * 64 + u * 32),
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_src + b * a_block + (a_blocked ? j * 512 : s * 64 + u * 32)),
                                        (__attribute__((address_space(3))) void*)&lds[(region * CHUNKS + 4 * i4 + b) * 64], 16, 0, 0);
   };
   auto fetch_w = [&](int j, int region) {
@@ -194,7 +200,7 @@ __global__ __launch_bounds__(512) void gemm_turns_kernel(const uint16_t* __restr
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
       const int row = m + 16 * x;
-      if (row < m_own) continue;
+      if (row < m_own || row >= M) continue;
 #pragma unroll
       for (int y = 0; y < YB / 2; ++y) {
         const int n = n0 + 8 * YB * g + 16 * y + 4 * (lane / 16);
@@ -202,14 +208,14 @@ __global__ __launch_bounds__(512) void gemm_turns_kernel(const uint16_t* __restr
         u32x2_t packed;
         packed[0] = f32_to_bf16_bits(silu_mul(acc[x][y][0], acc[x][y + YB / 2][0])) | ((uint32_t)f32_to_bf16_bits(silu_mul(acc[x][y][1], acc[x][y + YB / 2][1])) << 16);
         packed[1] = f32_to_bf16_bits(silu_mul(acc[x][y][2], acc[x][y + YB / 2][2])) | ((uint32_t)f32_to_bf16_bits(silu_mul(acc[x][y][3], acc[x][y + YB / 2][3])) << 16);
-        *reinterpret_cast<u32x2_t*>(out + (size_t)row * N + n) = packed;
+        *reinterpret_cast<u32x2_t*>(out + (c_blocked ? (size_t)bh_blocked_index(row, n, N) : (size_t)row * N + n)) = packed;
       }
     }
   } else {
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
       const int row = m + 16 * x;
-      if (row < m_own) continue;
+      if (row < m_own || row >= M) continue;
 #pragma unroll
       for (int y = 0; y < YB; ++y) {
         const int n = n0 + 16 * YB * g + 16 * y + 4 * (lane / 16);
@@ -236,12 +242,12 @@ __global__ __launch_bounds__(512) void gemm_turns_kernel(const uint16_t* __restr
 #undef TICK
 
 template <int MODE>
-void launch(const void* a, const void* w, void* c, int blocks, int M, int N, int K, int accumulate, hipStream_t stream,
-            int parts = 1) {
+void launch(const void* a, const void* w, void* c, int blocks, int M, int N, int K, int accumulate, int a_blocked,
+            int c_blocked, hipStream_t stream, int parts = 1) {
   const int outs = (MODE == 2 ? 16 : 32) * blocks;
   dim3 grid(((N + outs - 1) / outs) * ((M + 255) / 256), parts);
 #define BH_TURNS(YB) \
-  gemm_turns_kernel<MODE, YB><<<grid, 512, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, c, M, N, K, accumulate)
+  gemm_turns_kernel<MODE, YB><<<grid, 512, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, c, M, N, K, accumulate, a_blocked, c_blocked)
   if (blocks == 8) BH_TURNS(8);
   else if (blocks == 6) BH_TURNS(6);
   else BH_TURNS(4);
@@ -310,16 +316,17 @@ int gemm_turns_parts(int M, int N, int K, int layout, int activation) {
   return turns_plan(M, N, K, layout, activation).parts;
 }
 
-int gemm_turns_launch_parts(const void* a, const void* w, float* sums, int M, int N, int K, int parts, hipStream_t stream) {
+int gemm_turns_launch_parts(const void* a, const void* w, float* sums, int M, int N, int K, int parts, int a_blocked,
+                            hipStream_t stream) {
   BH_REQUIRE(parts >= 1 && K % (128 * parts) == 0 && gemm_turns_can(M, N, K / parts, 1, 0, 8),
              "gemm_turns: M=%d N=%d K=%d cannot be multiplied in %d parts of K", M, N, K, parts);
   BH_REQUIRE(((uintptr_t)a | (uintptr_t)w | (uintptr_t)sums) % 16 == 0, "gemm_turns: operands must be 16-byte aligned");
-  launch<1>(a, w, sums, 8, M, N, K, 0, stream, parts);
+  launch<1>(a, w, sums, 8, M, N, K, 0, a_blocked, 0, stream, parts);
   return bh_check_launch("gemm_turns");
 }
 
 int gemm_turns_launch(const void* a, const void* w, void* c, int c_dtype, int accumulate, int M, int N, int K,
-                      int activation, int blocks, hipStream_t stream) {
+                      int activation, int blocks, int a_blocked, int c_blocked, hipStream_t stream) {
   BH_REQUIRE(gemm_turns_can(M, N, K, 1, activation, blocks),
              "gemm_turns: a product of M=%d N=%d K=%d with %d blocks per wave is not one this kernel takes "
              "(M >= 256, K a multiple of 128, N a multiple of 16 and at least a tile)", M, N, K, blocks);
@@ -328,16 +335,17 @@ int gemm_turns_launch(const void* a, const void* w, void* c, int c_dtype, int ac
   BH_REQUIRE(!activation || c_dtype == BH_BF16, "gemm_turns: SwiGLU writes bfloat16");
   BH_REQUIRE(((uintptr_t)a | (uintptr_t)w | (uintptr_t)c) % 16 == 0 && (c_dtype == BH_F32 || N % 4 == 0),
              "gemm_turns: operands and output must be 16-byte aligned");
-  if (activation) launch<2>(a, w, c, blocks, M, N, K, 0, stream);
-  else if (c_dtype == BH_F32) launch<1>(a, w, c, blocks, M, N, K, accumulate, stream);
-  else launch<0>(a, w, c, blocks, M, N, K, 0, stream);
+  BH_REQUIRE(!c_blocked || (activation && N % 32 == 0), "gemm_turns: only SwiGLU writes its output in blocks, and N=%d must be a multiple of 32", N);
+  if (activation) launch<2>(a, w, c, blocks, M, N, K, 0, a_blocked, c_blocked, stream);
+  else if (c_dtype == BH_F32) launch<1>(a, w, c, blocks, M, N, K, accumulate, a_blocked, 0, stream);
+  else launch<0>(a, w, c, blocks, M, N, K, 0, a_blocked, 0, stream);
   return bh_check_launch("gemm_turns");
 }
 
 // For tests and measurements: the kernel at a given tile width, whatever gemm_turns_blocks would choose.
 extern "C" int bh_gemm_bf16_turns(const void* a, const void* w, void* c, int c_dtype, int accumulate, int M, int N,
-                                  int K, int activation, int blocks, hipStream_t stream) {
-  return gemm_turns_launch(a, w, c, c_dtype, accumulate, M, N, K, activation, blocks, stream);
+                                  int K, int activation, int blocks, int a_blocked, int c_blocked, hipStream_t stream) {
+  return gemm_turns_launch(a, w, c, c_dtype, accumulate, M, N, K, activation, blocks, a_blocked, c_blocked, stream);
 }
 extern "C" int bh_gemm_bf16_turns_blocks(int M, int N, int K, int layout, int activation) {
   return gemm_turns_blocks(M, N, K, layout, activation);

@@ -643,6 +643,41 @@ extern "C" int bh_swiglu(const void* gu, void* out, int dtype, int n_rows, int F
   return bh_check_launch("swiglu");
 }
 
+// ---- activation rows in blocks ---------------------------------------------------------------------
+// A bfloat16 matrix [rows][width] into the blocks of 16 rows x 32 columns that products of many rows read
+// fastest (bh_blocked_index in layout.h), and back.  One thread moves one piece of 16 bytes (8 columns of a
+// row).  Producers that know their reader write the blocks themselves; this is for the ones that do not.
+// Rows of the last block that the matrix does not have are filled with zeros.
+typedef uint32_t blocked_u32x4_t __attribute__((ext_vector_type(4)));
+template <bool TO_BLOCKS>
+__global__ __launch_bounds__(256) void rows_blocked_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst,
+                                                           int n_rows, int width, long pieces) {
+  const long piece = (long)blockIdx.x * 256 + threadIdx.x;   // in the order of the blocked matrix
+  if (piece >= pieces) return;
+  const int r = piece % 16, q = (piece / 16) % 4;
+  const long block = piece / 64;
+  const int column = (int)(block % (width / 32)) * 32 + 8 * q, row = (int)(block / (width / 32)) * 16 + r;
+  const blocked_u32x4_t zero = {0u, 0u, 0u, 0u};
+  if (TO_BLOCKS) {
+    reinterpret_cast<blocked_u32x4_t*>(dst)[piece] =
+        row < n_rows ? *reinterpret_cast<const blocked_u32x4_t*>(src + (size_t)row * width + column) : zero;
+  } else if (row < n_rows) {
+    *reinterpret_cast<blocked_u32x4_t*>(dst + (size_t)row * width + column) = reinterpret_cast<const blocked_u32x4_t*>(src)[piece];
+  }
+}
+
+extern "C" int bh_rows_blocked(const void* src, void* dst, int n_rows, int width, int to_blocks, hipStream_t stream) {
+  BH_REQUIRE(src != nullptr && dst != nullptr && n_rows > 0 && width > 0, "rows_blocked: a matrix with rows and a width");
+  BH_REQUIRE(width % 32 == 0, "rows_blocked: the width %d must be a multiple of 32", width);
+  BH_REQUIRE(((uintptr_t)src | (uintptr_t)dst) % 16 == 0, "rows_blocked: buffers must be 16-byte aligned");
+  const long pieces = (long)((n_rows + 15) / 16) * (width / 32) * 64;
+  BH_REQUIRE((pieces + 255) / 256 < (1L << 31), "rows_blocked: too many blocks");
+  dim3 grid((unsigned)((pieces + 255) / 256)), block(256);
+  if (to_blocks) rows_blocked_kernel<true><<<grid, block, 0, stream>>>((const uint16_t*)src, (uint16_t*)dst, n_rows, width, pieces);
+  else rows_blocked_kernel<false><<<grid, block, 0, stream>>>((const uint16_t*)src, (uint16_t*)dst, n_rows, width, pieces);
+  return bh_check_launch("rows_blocked");
+}
+
 // ---- a yardstick for the memory system ----------------------------------------------------------
 // Not a product kernel: reads `bytes` of device memory once, the way the streaming kernels of this library
 // read weights and cache pages (16 bytes a lane, sixteen loads of 1 KB in flight per wave, four waves a

@@ -41,6 +41,18 @@ BH_BOTH inline int bh_value_index(int order, int token, int dim, int hd) {
   return (((dt * 2 + u) * 64) + 16 * g + j) * 8 + token % 8;
 }
 
+// ---- activation rows in blocks ---------------------------------------------------------------
+// A bfloat16 matrix [rows][width] that a product of many rows reads as its activations may be kept in
+// blocks of 16 rows x 32 columns, each 1 KB in the order in which one matrix-core operand lies in a
+// wave's lanes: lane 16 q + r holds row r of the block, columns 8 q .. 8 q + 7.  The blocks of 16 rows
+// follow each other along the width, then down the rows.  A wave then takes an operand with one load of
+// contiguous memory instead of 64 bytes from each of 16 rows.  Needs width to be a multiple of 32; the
+// buffer holds whole blocks (rows rounded up; readers round them up to BH_BLOCKED_ROWS_PAD).
+#define BH_BLOCKED_ROWS_PAD 256
+BH_BOTH inline long bh_blocked_index(int row, int column, int width) {
+  return ((long)(row / 16) * (width / 32) + column / 32) * 512 + (((column % 32) / 8) * 16 + row % 16) * 8 + column % 8;
+}
+
 // bfloat16 kept as its 16 bits; widening is a shift, narrowing rounds to nearest even.
 struct bf16_t {
   uint16_t bits;

@@ -54,7 +54,24 @@ class NormedRows:
         return 2
 
 
-def _code(tensor: torch.Tensor, what: str) -> int:
+class BlockedRows:
+    """A bfloat16 activation matrix [rows, width] kept in blocks of 16 rows x 32 columns, each block 1 KB in the
+    order in which a matrix-core operand lies in a wave's lanes (`bh_blocked_index` in csrc/layout.h): what the
+    products of many rows read fastest.  `HipKernels.new_rows` hands one out where the product named as the
+    matrix's reader takes it; the kernels that produce activations (`rmsnorm`, `gemm_swiglu`, `attention`, a
+    `gemm` that finishes a norm) write into it, and `gemm` / `gemm_swiglu` read it.  `data` holds whole tiles of
+    256 rows; rows the matrix does not have hold nothing.  `shape` and `dtype` are those of the matrix."""
+
+    ROWS_PAD = 256
+
+    def __init__(self, data: torch.Tensor, rows: int, width: int):
+        self.data, self.shape, self.dtype, self.device = data, (rows, width), data.dtype, data.device
+
+    def dim(self):
+        return 2
+
+
+def _code(tensor, what: str) -> int:
     code = _CODES.get(tensor.dtype)
     if code is None:
         raise KernelError(f"{what}: dtype {tensor.dtype} is not supported (float32 or bfloat16)")
@@ -97,12 +114,14 @@ class HipKernels:
             "bh_swiglu": [p, p, i, i, i, p],
             "bh_sample": [p, p, p, p, p, p, p, p, i, i, p],
             "bh_sample_scratch": [i, i],
-            "bh_gemm_bf16": [p, p, p, i, i, i, i, i, i, i, p, i, f, p, i, p, p, p, p],
-            "bh_gemm_bf16_turns": [p, p, p, i, i, i, i, i, i, i, p],
-            "bh_gemm_bf16_then_norm": [p, p, p, i, i, i, i, p, i, f, p, p, p],
+            "bh_gemm_bf16": [p, p, p, i, i, i, i, i, i, i, p, i, f, p, i, p, p, p, i, i, p],
+            "bh_gemm_bf16_turns": [p, p, p, i, i, i, i, i, i, i, i, i, p],
+            "bh_gemm_bf16_then_norm": [p, p, p, i, i, i, i, p, i, f, p, p, i, i, p],
+            "bh_rows_blocked": [p, p, i, i, i, p],
             "bh_gemm_bf16_finishes_norm": [i, i, i, i],
-            "bh_attention_bf16": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, i, i, f, i, i, i, p],
+            "bh_attention_bf16": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, i, i, f, i, i, i, i, p],
             "bh_attention_bf16_splits": [i, i, i, i, i],
+            "bh_attention_bf16_writes_blocked": [i, i, i, i, i],
             "bh_attention_decode_fused": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, f, i, i, i, p, p, i, f, p, p, i, i,
                                           i, p],
             "bh_kv_order": [i, i],
@@ -114,7 +133,8 @@ class HipKernels:
             function.restype = i
         lib.bh_gemm_bf16_scratch.argtypes = [i, i, i, i, i]
         lib.bh_gemm_bf16_scratch.restype = ctypes.c_long
-        for query in (lib.bh_gemm_bf16_norm_blocks, lib.bh_gemm_bf16_takes_norm, lib.bh_gemm_bf16_turns_blocks):
+        for query in (lib.bh_gemm_bf16_norm_blocks, lib.bh_gemm_bf16_takes_norm, lib.bh_gemm_bf16_turns_blocks,
+                      lib.bh_gemm_bf16_reads_blocked):
             query.argtypes, query.restype = [i, i, i, i, i], ctypes.c_int
     # ---- helpers ----
     def _stream(self):
@@ -129,6 +149,8 @@ class HipKernels:
             if optional:
                 return None
             raise KernelError(f"{what}: tensor is required")
+        if isinstance(tensor, BlockedRows):
+            tensor = tensor.data
         if not isinstance(tensor, torch.Tensor) or tensor.device != self.device:
             raise KernelError(f"{what}: expected a tensor on {self.device}, got "
                               f"{getattr(tensor, 'device', type(tensor))}")
@@ -157,6 +179,11 @@ class HipKernels:
 
     def rmsnorm(self, x, weight, eps, out, rows=None):
         """out[r] = x[rows[r] if rows is given else r] * inv_rms * weight; x f32 [*, D], out [n, D]."""
+        if isinstance(out, BlockedRows):      # this kernel writes rows: regroup them afterwards
+            rows_out = torch.empty(out.shape, dtype=out.dtype, device=self.device)
+            self.rmsnorm(x, weight, eps, rows_out, rows=rows)
+            self.to_blocked(rows_out, out)
+            return
         n_rows, width = out.shape
         if x.dim() != 2 or x.shape[1] != width or (weight is not None and weight.shape != (width,)):
             raise KernelError(f"rmsnorm: shapes x {tuple(x.shape)}, out {tuple(out.shape)} do not fit")
@@ -169,6 +196,36 @@ class HipKernels:
             self._ptr(x, "rmsnorm x", (torch.float32,)), self._ptr(rows, "rmsnorm rows", (torch.int32,), True),
             self._ptr(weight, "rmsnorm weight", None, True), _code(weight, "rmsnorm weight") if weight is not None else F32,
             self._ptr(out, "rmsnorm out"), _code(out, "rmsnorm out"), n_rows, width, float(eps), self._stream()))
+
+    def new_rows(self, rows, width, dtype, reader_outputs=None, reader_swiglu=False):
+        """An empty activation matrix [rows, width] for a kernel of this library to fill.  With `reader_outputs`,
+        the product that reads it next has that many outputs (`reader_swiglu`: through the gate, so twice as
+        many weight rows): where that product takes `BlockedRows` and reads them faster, the matrix is one."""
+        if (reader_outputs is not None and dtype == torch.bfloat16 and width % 64 == 0
+                and self.lib.bh_gemm_bf16_reads_blocked(int(rows), int(reader_outputs), int(width), 1, int(bool(reader_swiglu)))):
+            padded = -(-int(rows) // BlockedRows.ROWS_PAD) * BlockedRows.ROWS_PAD
+            return BlockedRows(torch.empty(padded * int(width), dtype=dtype, device=self.device), int(rows), int(width))
+        return torch.empty((int(rows), int(width)), dtype=dtype, device=self.device)
+
+    def to_blocked(self, x, out=None):
+        """The bfloat16 matrix `x` as `BlockedRows` (into `out` if given)."""
+        rows, width = x.shape
+        if x.dtype != torch.bfloat16 or width % 32:
+            raise KernelError(f"to_blocked: a bfloat16 matrix whose width is a multiple of 32, not {x.dtype} {tuple(x.shape)}")
+        if out is None:
+            padded = -(-rows // BlockedRows.ROWS_PAD) * BlockedRows.ROWS_PAD
+            out = BlockedRows(torch.empty(padded * width, dtype=x.dtype, device=self.device), rows, width)
+        elif not isinstance(out, BlockedRows) or tuple(out.shape) != (rows, width):
+            raise KernelError(f"to_blocked: the output stands for {tuple(out.shape)}, the matrix is {tuple(x.shape)}")
+        self._check(self.lib.bh_rows_blocked(self._ptr(x, "rows"), self._ptr(out, "blocks"), rows, width, 1, self._stream()))
+        return out
+
+    def from_blocked(self, blocked):
+        """The matrix that `blocked` stands for, row after row."""
+        rows, width = blocked.shape
+        out = torch.empty((rows, width), dtype=blocked.dtype, device=self.device)
+        self._check(self.lib.bh_rows_blocked(self._ptr(blocked, "blocks"), self._ptr(out, "rows"), rows, width, 0, self._stream()))
+        return out
 
     def pack_weight(self, w):
         """The form of a weight matrix that the matrix products read fastest: a `PackedWeight` for a
@@ -189,6 +246,7 @@ class HipKernels:
         fast = self.lib.bh_gemm_bf16
         packed = isinstance(w, PackedWeight)
         ahead = a if isinstance(a, NormedRows) else None
+        a_blocked, c_blocked = isinstance(a, BlockedRows), isinstance(out, BlockedRows)
         if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or a.shape[1] % 8:
             if packed:
                 raise KernelError("gemm: a packed weight needs bfloat16 activations")
@@ -198,6 +256,8 @@ class HipKernels:
         m, k = a.shape
         n = out.shape[1]
         sizes = (m, n, k, int(packed), int(activation))
+        if (a_blocked or c_blocked) and not self.lib.bh_gemm_bf16_reads_blocked(*sizes):
+            raise KernelError(f"gemm: a product of {m} x {n} x {k} neither reads nor writes rows in blocks")
         if ahead is not None and (ahead.ss.shape[0] != m or ahead.ss.dtype != torch.float32
                                   or not self.lib.bh_gemm_bf16_takes_norm(*sizes)):
             raise KernelError(f"gemm: a product of {m} x {n} x {k} does not take these prepared norm rows")
@@ -205,12 +265,14 @@ class HipKernels:
                 and not activation and then_norm.weight.shape == (n,) and then_norm.weight.dtype in _CODES
                 and self.lib.bh_gemm_bf16_finishes_norm(m, n, k, 1)):
             # many rows, K in parts: the finishing kernel owns whole rows and finishes the norm itself
-            normed = torch.empty((m, n), dtype=torch.bfloat16, device=self.device)
+            reader = getattr(then_norm, "reader", None)
+            normed = self.new_rows(m, n, torch.bfloat16, *((reader.outputs, reader.swiglu) if reader is not None else ()))
             scratch = torch.empty(int(self.lib.bh_gemm_bf16_scratch(*sizes)) // 4, dtype=torch.float32, device=self.device)
             self._check(self.lib.bh_gemm_bf16_then_norm(
                 self._ptr(a, "gemm a"), self._ptr(w.data, "gemm w"), self._ptr(out, "gemm out", (torch.float32,)), m, n, k, 1,
                 self._ptr(then_norm.weight, "norm weight"), _code(then_norm.weight, "norm weight"), float(then_norm.eps),
-                self._ptr(normed, "norm rows"), self._ptr(scratch, "gemm scratch"), self._stream()))
+                self._ptr(normed, "norm rows"), self._ptr(scratch, "gemm scratch"), int(a_blocked),
+                int(isinstance(normed, BlockedRows)), self._stream()))
             return True, normed
         behind = None
         if (then_norm is not None and out.dtype == torch.float32 and not activation
@@ -234,7 +296,7 @@ class HipKernels:
             _code(then_norm.weight, "norm weight") if behind is not None else 0,
             self._ptr(behind.rows, "norm rows") if behind is not None else None,
             self._ptr(behind.ss, "norm sums") if behind is not None else None,
-            self._ptr(scratch, "gemm scratch", None, True), self._stream()))
+            self._ptr(scratch, "gemm scratch", None, True), int(a_blocked), int(c_blocked), self._stream()))
         return True, behind
 
     def gemm(self, a, w, out, accumulate=False, then_norm=None):
@@ -247,13 +309,15 @@ class HipKernels:
             raise KernelError("gemm: operands must be matrices")
         m, k = a.shape
         n = w.shape[0]
-        if w.shape[1] != k or out.shape != (m, n):
+        if w.shape[1] != k or tuple(out.shape) != (m, n):
             raise KernelError(f"gemm: shapes a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
         if isinstance(a, NormedRows) and not self._takes_norm(a, w, n, 0):
             a = self._run_norm(a)
         done, prepared = self._gemm_fast(a, w, out, accumulate, 0, then_norm)
         if done:
             return prepared
+        if isinstance(a, BlockedRows):
+            raise KernelError("gemm: only the matrix-core product of many rows reads rows in blocks")
         self._check(self.lib.bh_gemm_generic(
             self._ptr(a, "gemm a"), _code(a, "gemm a"), self._ptr(w, "gemm w"), _code(w, "gemm w"),
             self._ptr(out, "gemm out"), _code(out, "gemm out"), int(bool(accumulate)), m, n, k, self._stream()))
@@ -264,14 +328,15 @@ class HipKernels:
         weight rows per wave: 8, 6 or 4), whatever `gemm` would choose for these sizes: out[M, N] (+)= a @ w^T,
         or with `swiglu` out[M, F] = silu(a @ w[:F]^T) * (a @ w[F:]^T).  `w` is a PackedWeight."""
         if not isinstance(w, PackedWeight) or a.dim() != 2 or out.dim() != 2 or a.dtype != torch.bfloat16:
-            raise KernelError("gemm_turns: bfloat16 activations [M, K] and a packed weight")
+            raise KernelError("gemm_turns: bfloat16 activations [M, K] (rows or `BlockedRows`) and a packed weight")
         m, k = a.shape
         n = out.shape[1]
         if w.shape[1] != k or w.shape[0] != (2 * n if swiglu else n) or out.shape[0] != m:
             raise KernelError(f"gemm_turns: shapes a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
         self._check(self.lib.bh_gemm_bf16_turns(
             self._ptr(a, "gemm a"), self._ptr(w.data, "gemm w"), self._ptr(out, "gemm out"), _code(out, "gemm out"),
-            int(bool(accumulate)), m, n, k, int(bool(swiglu)), int(blocks), self._stream()))
+            int(bool(accumulate)), m, n, k, int(bool(swiglu)), int(blocks), int(isinstance(a, BlockedRows)),
+            int(isinstance(out, BlockedRows)), self._stream()))
 
     def gemm_turns_blocks(self, m, n, k, swiglu=False):
         """The tile width `gemm` uses for a packed product of these sizes (0: another kernel runs it)."""
@@ -296,13 +361,21 @@ class HipKernels:
             raise KernelError("gemm_swiglu: operands must be matrices")
         m, k = a.shape
         width = out.shape[1]
-        if w.shape != (2 * width, k) or out.shape[0] != m or out.dtype != a.dtype:
+        if tuple(w.shape) != (2 * width, k) or out.shape[0] != m or out.dtype != a.dtype:
             raise KernelError(f"gemm_swiglu: shapes a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} "
                               "do not fit")
         if isinstance(a, NormedRows) and width % 16 == 0 and not self._takes_norm(a, w, width, 1):
             a = self._run_norm(a)
+        if isinstance(out, BlockedRows) and not (isinstance(w, PackedWeight) and a.dtype == torch.bfloat16 and
+                                                 self.lib.bh_gemm_bf16_turns_blocks(m, width, k, 1, 1)):
+            rows_out = torch.empty((m, width), dtype=out.dtype, device=self.device)   # this product writes rows
+            self.gemm_swiglu(a, w, rows_out)
+            self.to_blocked(rows_out, out)
+            return
         if self._gemm_fast(a, w, out, False, 1)[0]:
             return
+        if isinstance(a, BlockedRows) or isinstance(out, BlockedRows):
+            raise KernelError("gemm_swiglu: only the matrix-core product of many rows reads or writes rows in blocks")
         both = torch.empty((m, 2 * width), dtype=a.dtype, device=self.device)
         self.gemm(a, w, both)
         self.swiglu(both, out)
@@ -369,8 +442,17 @@ class HipKernels:
         max_rows_per_seq, max_position), which the matrix-core kernel needs; rows of one sequence
         are consecutive and in position order."""
         n_rows = q.shape[0]
-        if q.shape != (n_rows, n_heads * head_dim) or out.shape != q.shape or out.dtype != q.dtype:
+        if q.shape != (n_rows, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape) or out.dtype != q.dtype:
             raise KernelError(f"attention: shapes q {tuple(q.shape)}, out {tuple(out.shape)} do not fit")
+        if isinstance(out, BlockedRows) and not (
+                q.dtype == torch.bfloat16 and layout is not None and head_dim % 32 == 0 and head_dim <= 256
+                and self.lib.bh_attention_bf16_writes_blocked(int(layout.n_seqs), int(layout.max_rows_per_seq), n_heads,
+                                                              n_kv_heads, int(layout.max_position))):
+            rows_out = torch.empty(tuple(q.shape), dtype=q.dtype, device=self.device)   # this step's kernel writes rows
+            self.attention(q, rows_out, k_pages, v_pages, page_table, row_seq, positions, n_heads, n_kv_heads, head_dim,
+                           scale, window, layout)
+            self.to_blocked(rows_out, out)
+            return
         if n_heads % n_kv_heads != 0:
             raise KernelError(f"attention: {n_heads} query heads do not group evenly into {n_kv_heads} kv heads")
         if positions.shape != (n_rows,) or row_seq.shape != (n_rows,):
@@ -396,7 +478,7 @@ class HipKernels:
                              page_table.shape[1], self._ptr(positions, "positions", (torch.int32,)),
                              self._ptr(layout.seq_start, "seq_start", (torch.int32,)), n_seqs, n_rows, max_rows,
                              n_heads, n_kv_heads, head_dim, float(scale), int(window), int(layout.max_position),
-                             n_splits, self._stream()))
+                             n_splits, int(isinstance(out, BlockedRows)), self._stream()))
             return
         self._check(self.lib.bh_attention_generic(
             *common, _code(q, "q"), self._ptr(k_pages, "k_pages"), self._ptr(v_pages, "v_pages"),

@@ -32,6 +32,12 @@ A norm may ride on the products around it (optional, one flag per role):
         prepared form; it hands `x` to the kernel library's products untouched.
 The block joins a producer and a consumer this way only when all three offer it, and runs the norm
 as a step of its own otherwise.
+A matrix that one product alone reads may be kept the way that product reads it fastest (optional):
+    consumer with `input_reader` (a ProductReader: the product its `x` goes to, and nowhere else): its `x` may
+        then be in the kernel library's own form for that product; it hands `x` to that product untouched.
+    norm with `serves_reader = True`: forward(..., reader=) and request(reader) take that ProductReader.
+    Inside a part, `ctx.new_activations(rows, width, reader=linear.reader())` asks for such a matrix between two
+    of its own kernel calls.  Parts that say nothing get and give plain matrices.
 A mixer with a "state" cache need updates its rows of `cache.state` in place while it runs.  The cache keeps
 what the step's sequences held before the step and puts it back if the step fails, so a mixer needs no
 second bank; and the engine runs a part's forward exactly once per step, whether the step is launched kernel
@@ -109,7 +115,12 @@ class StepContext:
     fed_tokens: torch.Tensor | None = None # int32: tokens chosen on the device that the host has not read yet
     extras: dict = field(default_factory=dict)
 
-    def new_activations(self, *shape) -> torch.Tensor:
+    def new_activations(self, *shape, reader=None):
+        """An empty matrix of the activation type.  `reader` (a ProductReader) names the product that reads it
+        next and nothing else does: the kernel library may then hand out the matrix in the form that product
+        reads fastest, which only its own kernels fill and read."""
+        if reader is not None and len(shape) == 2 and hasattr(self.kernels, "new_rows"):
+            return self.kernels.new_rows(shape[0], shape[1], self.act_dtype, reader.outputs, reader.swiglu)
         return torch.empty(shape, dtype=self.act_dtype, device=self.device)
 
     def new_f32(self, *shape) -> torch.Tensor:
@@ -117,10 +128,20 @@ class StepContext:
 
 
 @dataclass
+class ProductReader:
+    """The matrix product that reads an activation matrix next: `outputs` columns of result, through the
+    gated activation or not (then its weight has twice as many rows)."""
+    outputs: int
+    swiglu: bool = False
+
+
+@dataclass
 class NormRequest:
-    """An RMSNorm (weight [width], eps) offered to the product that completes its input."""
+    """An RMSNorm (weight [width], eps) offered to the product that completes its input; `reader`: the
+    product that reads the norm's output, if it is the only one that does."""
     weight: torch.Tensor
     eps: float
+    reader: ProductReader | None = None
 
 
 @dataclass

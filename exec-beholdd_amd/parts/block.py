@@ -42,8 +42,19 @@ class PreNormBlock:
         """The request to hand `producer` so that its last product prepares `norm` for `consumer`, or None."""
         if (getattr(producer, "prepares_next_norm", False) and getattr(consumer, "takes_prepared_input", False)
                 and hasattr(norm, "request")):
-            return norm.request()
+            reader = PreNormBlock._reader(norm, consumer)
+            return norm.request(reader) if reader is not None else norm.request()
         return None
+
+    @staticmethod
+    def _reader(norm, consumer):
+        """The product of `consumer` that alone reads what `norm` writes, if both parts say so."""
+        return getattr(consumer, "input_reader", None) if getattr(norm, "serves_reader", False) else None
+
+    @staticmethod
+    def _normed(ctx, norm, consumer, hidden):
+        reader = PreNormBlock._reader(norm, consumer)
+        return norm.forward(ctx, hidden, reader=reader) if reader is not None else norm.forward(ctx, hidden)
 
     def entry_request(self, producer):
         """What the part that runs before this block (`producer`) may prepare of this block's first norm."""
@@ -53,7 +64,7 @@ class PreNormBlock:
         """One layer.  `prepared`: the mixer's input if the block before has prepared it already;
         `next_block`: the block that runs after this one, whose first norm this block's feed-forward
         may prepare.  Returns that prepared input, or None."""
-        x = prepared if prepared is not None else self.mixer_norm.forward(ctx, hidden)
+        x = prepared if prepared is not None else self._normed(ctx, self.mixer_norm, self.mixer, hidden)
         request = self._joined(self.mixer, self.feed_forward_norm, self.feed_forward)
         if request is not None:
             x = self.mixer.forward(ctx, x, hidden, cache, then_norm=request)
@@ -61,7 +72,7 @@ class PreNormBlock:
             self.mixer.forward(ctx, x, hidden, cache)
             x = None
         if x is None:
-            x = self.feed_forward_norm.forward(ctx, hidden)
+            x = self._normed(ctx, self.feed_forward_norm, self.feed_forward, hidden)
         request = next_block.entry_request(self.feed_forward) if hasattr(next_block, "entry_request") else None
         if request is not None:
             return self.feed_forward.forward(ctx, x, hidden, then_norm=request)

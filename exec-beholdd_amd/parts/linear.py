@@ -11,6 +11,7 @@ from __future__ import annotations
 import torch
 
 from ..weights.binder import TensorSpec
+from .base import ProductReader
 
 
 class Linear:
@@ -46,6 +47,10 @@ class Linear:
                              f"{(self.out_features, self.in_features)}")
         self.weight = weight
         self.shared = True
+
+    def reader(self, swiglu: bool = False) -> ProductReader:
+        """This map as the only reader of an activation matrix (`swiglu`: its rows are gate rows, then up rows)."""
+        return ProductReader(self.out_features // 2 if swiglu else self.out_features, swiglu)
 
     def prepare(self, kernels):
         """Let the kernel library regroup the matrix into the layout it reads fastest."""

@@ -20,6 +20,7 @@ class SwiGLU:
         self.gate_up = Linear(hidden, [intermediate, intermediate],
                               [prefix + "gate_proj.weight", prefix + "up_proj.weight"])
         self.down = Linear(intermediate, hidden, prefix + "down_proj.weight")
+        self.input_reader = self.gate_up.reader(swiglu=True)    # x goes to that product and nowhere else
 
     def tensor_specs(self):
         return self.gate_up.tensor_specs() + self.down.tensor_specs()
@@ -33,7 +34,7 @@ class SwiGLU:
         self.down.prepare(kernels)
 
     def forward(self, ctx, x, hidden, then_norm=None):
-        activated = ctx.new_activations(x.shape[0], self.intermediate)
+        activated = ctx.new_activations(x.shape[0], self.intermediate, reader=self.down.reader())
         ctx.kernels.gemm_swiglu(x, self.gate_up.weight, activated)     # both products and the gate in one pass
         return self.down.add_into(ctx, activated, hidden, then_norm)
 

@@ -27,15 +27,17 @@ class RMSNorm:
     def load(self, get):
         self.weight = get(self.name)
 
-    def forward(self, ctx, hidden, rows=None):
+    serves_reader = True   # forward and request take the product that reads the output
+
+    def forward(self, ctx, hidden, rows=None, reader=None):
         n = hidden.shape[0] if rows is None else rows.shape[0]
-        out = ctx.new_activations(n, self.width)
+        out = ctx.new_activations(n, self.width, reader=reader)
         ctx.kernels.rmsnorm(hidden, self.weight, self.eps, out, rows=rows)
         return out
 
-    def request(self):
+    def request(self, reader=None):
         """This norm as the product that completes its input may prepare it."""
-        return NormRequest(self.weight, self.eps)
+        return NormRequest(self.weight, self.eps, reader)
 
 
 @NORMS.register("rmsnorm")

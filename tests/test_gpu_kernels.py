@@ -226,7 +226,8 @@ def test_norm_rides_on_wide_products(K, m, n, k, n2, g_dtype):
 
 
 @pytest.mark.parametrize("g_dtype", DTYPES)
-@pytest.mark.parametrize("m,n,k", [(2048, 4096, 4096), (1000, 4096, 2048 * 4), (1800, 5120 - 1024, 2048)])
+@pytest.mark.parametrize("m,n,k", [(2048, 4096, 4096), (1000, 4096, 2048 * 4), (1800, 5120 - 1024, 2048),
+                                   (601, 4096, 12288), (2047, 4080, 4096)])   # eight parts; rows and pieces that fill no block
 def test_product_in_parts_of_many_rows_finishes_the_norm(K, g_dtype, m, n, k):
     """Beyond 256 rows, where K goes through the turns kernel in parts, the finishing kernel owns whole rows and
     writes the norm's output itself: `gemm(..., then_norm=)` returns it as a plain bfloat16 matrix."""
@@ -291,6 +292,96 @@ def test_gemm_whose_wave_groups_take_turns(K, blocks, m, n, k):
         act = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda:0")
         K.gemm_turns(dev(a), both, act, blocks, swiglu=True)
         assert rel(act, want_act) < 6e-3, rel(act, want_act)
+
+
+def blocked_reference(x):
+    """x [rows, width] in blocks of 16 rows x 32 columns, each block as [4 groups of 8 columns][16 rows][8], the
+    blocks of 16 rows one after the other along the width; rows that x lacks are zero."""
+    rows, width = x.shape
+    padded = -(-rows // 16) * 16
+    full = torch.zeros(padded, width, dtype=x.dtype)
+    full[:rows] = x
+    return full.view(padded // 16, 16, width // 32, 4, 8).permute(0, 2, 3, 1, 4).reshape(-1)
+
+
+@pytest.mark.parametrize("rows,width", [(1, 32), (16, 64), (300, 96), (257, 4096), (1000, 160)])
+def test_rows_into_blocks_and_back(K, rows, width):
+    x = torch.randn(rows, width, generator=torch.Generator().manual_seed(rows)).to(torch.bfloat16)
+    blocked = K.to_blocked(dev(x))
+    assert tuple(blocked.shape) == (rows, width) and blocked.data.numel() % (256 * width) == 0
+    want = blocked_reference(x)
+    assert torch.equal(blocked.data[:want.numel()].cpu(), want)
+    assert torch.equal(K.from_blocked(blocked).cpu(), x)
+    from beholdd.kernels import KernelError
+    with pytest.raises(KernelError, match="multiple of 32"):
+        K.to_blocked(dev(torch.zeros(4, 48, dtype=torch.bfloat16)))
+
+
+@pytest.mark.parametrize("blocks", [8, 6, 4])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (300, 416, 384), (527, 1056, 256), (257, 288, 1152), (1024, 768, 2048)])
+def test_gemm_with_turns_reads_and_writes_rows_in_blocks(K, blocks, m, n, k):
+    """The same product from activations in blocks of 16 x 32 gives the same bits as from rows (the sums run
+    in the same order), also where the last tile of rows sticks out of the matrix and the buffer's rows beyond
+    the matrix hold NaN; the gated product writes blocks that hold what it writes as rows."""
+    g = torch.Generator().manual_seed(m + n + blocks)
+    a = dev(torch.randn(m, k, generator=g).to(torch.bfloat16))
+    w = (torch.randn(2 * n, k, generator=g) * 0.05).to(torch.bfloat16)
+    plain, both = K.pack_weight(dev(w[:n].contiguous())), K.pack_weight(dev(w))
+    from beholdd.kernels.library import BlockedRows
+    in_blocks = BlockedRows(torch.full((-(-m // 256) * 256 * k,), float("nan"), dtype=torch.bfloat16, device="cuda:0"), m, k)
+    K.to_blocked(a, in_blocks)
+    if m % 16:
+        assert bool(torch.isnan(in_blocks.data.float()).any())      # the rows of the last tile that do not exist
+    for dtype, accumulate in ((torch.float32, False), (torch.float32, True), (torch.bfloat16, False)):
+        base = torch.randn(m, n, generator=g).to(dtype)
+        from_rows, from_blocks = dev(base.clone()), dev(base.clone())
+        K.gemm_turns(a, plain, from_rows, blocks, accumulate=accumulate)
+        K.gemm_turns(in_blocks, plain, from_blocks, blocks, accumulate=accumulate)
+        assert torch.equal(from_rows, from_blocks)
+    if n >= 16 * blocks and n % 32 == 0:
+        rows_out = torch.empty(m, n, dtype=torch.bfloat16, device="cuda:0")
+        K.gemm_turns(a, both, rows_out, blocks, swiglu=True)
+        for source in (a, in_blocks):
+            out = BlockedRows(torch.full((-(-m // 256) * 256 * n,), float("nan"), dtype=torch.bfloat16, device="cuda:0"), m, n)
+            K.gemm_turns(source, both, out, blocks, swiglu=True)
+            assert torch.equal(K.from_blocked(out), rows_out)
+
+
+@pytest.mark.parametrize("m", [300, 1000, 2048])
+def test_products_of_many_rows_hand_each_other_blocks(K, m):
+    """`new_rows` names the reader: norm -> gated product -> down product with the next norm finished, all through
+    rows in blocks, give what the same chain gives through plain matrices."""
+    from beholdd.kernels.library import BlockedRows
+    from beholdd.parts.base import NormRequest, ProductReader
+    hidden, inter = 2048, 8192
+    g = torch.Generator().manual_seed(m)
+    residual = torch.randn(m, hidden, generator=g)
+    gate_up = K.pack_weight(dev((torch.randn(2 * inter, hidden, generator=g) * 0.05).to(torch.bfloat16)))
+    down = K.pack_weight(dev((torch.randn(hidden, inter, generator=g) * 0.05).to(torch.bfloat16)))
+    g1, g2 = dev(1 + 0.3 * torch.randn(hidden, generator=g)), dev(1 + 0.3 * torch.randn(hidden, generator=g))
+
+    def chain(blocks):
+        h = dev(residual.clone())
+        reader = lambda outputs, swiglu=False: (outputs, swiglu) if blocks else ()
+        x = K.new_rows(m, hidden, torch.bfloat16, *reader(inter, True))
+        K.rmsnorm(h, g1, 1e-5, x)
+        act = K.new_rows(m, inter, torch.bfloat16, *reader(hidden))
+        K.gemm_swiglu(x, gate_up, act)
+        normed = K.gemm(act, down, h, accumulate=True,
+                        then_norm=NormRequest(g2, 1e-5, ProductReader(inter, True) if blocks else None))
+        kinds = [type(x), type(act), type(normed)]
+        if normed is None:
+            normed = torch.empty(m, hidden, dtype=torch.bfloat16, device="cuda:0")
+            K.rmsnorm(h, g2, 1e-5, normed)
+        return h, K.from_blocked(normed) if isinstance(normed, BlockedRows) else normed, kinds
+
+    h_rows, normed_rows, kinds_rows = chain(False)
+    h_blocks, normed_blocks, kinds_blocks = chain(True)
+    assert BlockedRows not in kinds_rows
+    if m >= 1000:       # these sizes go to the kernel that reads blocks, and the down product finishes the norm
+        assert kinds_blocks == [BlockedRows, BlockedRows, BlockedRows]
+    assert torch.equal(h_rows, h_blocks) and torch.equal(normed_rows, normed_blocks)
+    assert bool(torch.isfinite(h_blocks).all())
 
 
 def test_gemm_with_turns_refuses_what_it_cannot_do(K):
@@ -589,6 +680,12 @@ def test_attention_prefill_many_columns(K, n_heads, kv_heads, head_dim, window, 
         want = attention_reference_rows(q[rows], keys[s], values[s], positions[rows].long(), n_heads, kv_heads,
                                         head_dim, scale, window)
         assert rel(out[rows], want) < 1.2e-2, (s, rel(out[rows], want))
+    from beholdd.kernels.library import BlockedRows     # the same output in blocks of 16 rows x 32 columns
+    width = n_heads * head_dim
+    blocked = BlockedRows(torch.full((-(-n_rows // 256) * 256 * width,), float("nan"), dtype=dtype, device="cuda:0"), n_rows, width)
+    K.attention(dev(q), blocked, *stored(K, kp, vp), dev(table), dev(row_seq), dev(positions), n_heads, kv_heads,
+                head_dim, scale, window, layout=Layout(False, dev(starts), len(lengths), max(news), max(lengths) - 1))
+    assert torch.equal(K.from_blocked(blocked), out)
 
 
 @pytest.mark.parametrize("window", [0, 70])
