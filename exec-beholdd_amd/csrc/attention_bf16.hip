@@ -144,7 +144,7 @@ __global__ __launch_bounds__(256, (LEAN ? 2 : 1)) void attention_mfma_kernel(
     float* __restrict__ part_ml, const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages,
     const int32_t* __restrict__ page_table, int table_stride, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ seq_start, int H, int KVH, float scale_log2, int window, int n_splits,
-    int pages_per_split, int tile_groups, FusedQkv fused) {
+    int pages_per_split, int tile_groups, FusedQkv fused, int out_block_rows) {
   constexpr int HD = 32 * NS;
   __shared__ float sm_m[4][16];
   __shared__ float sm_l[4][16];
@@ -394,8 +394,8 @@ __global__ __launch_bounds__(256, (LEAN ? 2 : 1)) void attention_mfma_kernel(
         value += sm_o[v][col][d] * f;
       }
       const size_t column = (size_t)(row0 + cc / G) * H + kvh * G + cc % G;
-      if (n_splits == 1) {
-        out[column * HD + d] = f32_to_bf16_bits(value / sum);
+      if (n_splits == 1) {   // out_block_rows: the output [rows][H * HD] lies in blocks of that many rows (bh_rows_index)
+        out[bh_rows_index(out_block_rows, row0 + cc / G, (kvh * G + cc % G) * HD + d, H * HD)] = f32_to_bf16_bits(value / sum);
       } else {
         part_o[(column * n_splits + split) * HD + d] = value;
         if (d == 0) {
@@ -411,7 +411,7 @@ __global__ __launch_bounds__(256, (LEAN ? 2 : 1)) void attention_mfma_kernel(
 // one's: with 32 splits that is 32 trips to the L2 in a row.  So the lanes of a wave fetch the splits'
 // (maximum, sum) pairs side by side, and the partial outputs are fetched eight splits at a time.
 __global__ void attention_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                         uint16_t* __restrict__ out, int n_splits, int HD) {
+                                         uint16_t* __restrict__ out, int n_splits, int HD, int H, int out_block_rows) {
   const size_t column = blockIdx.x;
   const float* ml = part_ml + column * n_splits * 2;
   const int lane = threadIdx.x % BH_WAVE;
@@ -437,7 +437,7 @@ __global__ void attention_combine_kernel(const float* __restrict__ part_o, const
 #pragma unroll
       for (int u = 0; u < 8; ++u) value += part[u] * exp2f(weight[u] - top);
     }
-    out[column * HD + d] = f32_to_bf16_bits(value * inv);
+    out[bh_rows_index(out_block_rows, (int)(column / H), (int)(column % H) * HD + d, H * HD)] = f32_to_bf16_bits(value * inv);
   }
 }
 
@@ -463,8 +463,8 @@ extern "C" int bh_attention_bf16_splits(int n_seqs, int max_rows_per_seq, int H,
 }
 
 #define PREFILL_FROM_TILES 1024   // column tiles x kv heads x sequences from which the prefill kernel runs a step
-// Whether a step of these sizes can write its output in blocks of 16 rows x 32 columns (bh_blocked_index) for
-// the product that reads it: the steps of the prefill kernel.
+// Whether a step of these sizes goes to the kernel for many columns per sequence, which writes its output in rows
+// or in blocks of 16 rows x 32 columns (bh_blocked_index); the other steps' kernels write blocks of 8 or 16 rows.
 extern "C" int bh_attention_bf16_writes_blocked(int n_seqs, int max_rows_per_seq, int H, int KVH, int max_position) {
   if (n_seqs <= 0 || max_rows_per_seq <= 0 || H <= 0 || KVH <= 0 || H % KVH) return 0;
   const long tiles = (long)((max_rows_per_seq * (H / KVH) + 15) / 16) * KVH * n_seqs;
@@ -492,11 +492,13 @@ static int attention_bf16_run(const void* q, void* out, void* part_o, void* part
   BH_REQUIRE(!is_fused || (tiles == 1 && max_rows_per_seq == 1 && n_rows == n_seqs),
              "attention_bf16: the fused projection rows are taken in decode steps of at most 16 heads per kv head only");
   if (!is_fused && n_splits == 1 && (long)tiles * KVH * n_seqs >= PREFILL_FROM_TILES) {   // many columns: the prefill kernel
+    BH_REQUIRE(out_blocked == 0 || out_blocked == 16, "attention_bf16: a step of many columns writes rows or blocks of 16 rows, not of %d", out_blocked);
     bh_attention_prefill_launch(q, out, k_pages, v_pages, page_table, table_stride, positions, seq_start, n_seqs,
-                                tiles, H, KVH, hd, scale_log2, window, out_blocked, stream);
+                                tiles, H, KVH, hd, scale_log2, window, out_blocked == 16, stream);
     return bh_check_launch("attention_prefill_bf16");
   }
-  BH_REQUIRE(!out_blocked, "attention_bf16: this step's output cannot go out in blocks (bh_attention_bf16_writes_blocked)");
+  BH_REQUIRE(out_blocked == 0 || ((out_blocked == 8 || out_blocked == 16) && (H * hd) % 32 == 0),
+             "attention_bf16: the output's rows lie in blocks of 8 or 16, or one after the other (0), not %d", out_blocked);
   const int tile_groups = tiles, z_count = n_seqs * n_splits;
   const bool lean = (long)tiles * KVH * z_count > 256;   // more workgroups than compute units: two of them per unit
   dim3 grid(tile_groups * KVH * z_count), block(256);
@@ -504,7 +506,7 @@ static int attention_bf16_run(const void* q, void* out, void* part_o, void* part
   attention_mfma_kernel<NS, STREAM, FUSED, ##__VA_ARGS__><<<grid, block, 0, stream>>>(                          \
       (const uint16_t*)q, (uint16_t*)out, (float*)part_o, (float*)part_ml, (const uint16_t*)k_pages,            \
       (const uint16_t*)v_pages, page_table, table_stride, positions, seq_start, H, KVH, scale_log2, window,     \
-      n_splits, per, tile_groups, fused)
+      n_splits, per, tile_groups, fused, out_blocked)
 #define BH_ATT(NS)                                      \
   do {                                                  \
     if (is_fused && lean && NS <= 4) BH_ATT_ONE(NS, true, true, (NS <= 4));   \
@@ -527,7 +529,7 @@ static int attention_bf16_run(const void* q, void* out, void* part_o, void* part
   if (int status = bh_check_launch("attention_mfma")) return status;
   if (n_splits > 1) {
     attention_combine_kernel<<<dim3(n_rows * H), dim3(hd >= 128 ? 128 : 64), 0, stream>>>(
-        (const float*)part_o, (const float*)part_ml, (uint16_t*)out, n_splits, hd);
+        (const float*)part_o, (const float*)part_ml, (uint16_t*)out, n_splits, hd, H, out_blocked);
     return bh_check_launch("attention_combine");
   }
   return 0;
@@ -554,7 +556,7 @@ extern "C" int bh_attention_decode_fused(const void* qkv, void* out, void* part_
                                          int KVH, int hd, float scale, int window, int max_position, int n_splits,
                                          const void* q_weight, const void* k_weight, int w_dtype, float eps,
                                          const float* cos_table, const float* sin_table, int table_positions,
-                                         int rot, int write_kv, hipStream_t stream) {
+                                         int rot, int write_kv, int out_block_rows, hipStream_t stream) {
   BH_REQUIRE(qkv != nullptr, "attention_decode_fused: the projection rows are required");
   BH_REQUIRE((q_weight == nullptr) == (k_weight == nullptr), "attention_decode_fused: give both norm weights or neither");
   BH_REQUIRE(q_weight == nullptr || w_dtype == BH_F32 || w_dtype == BH_BF16, "attention_decode_fused: unknown weight dtype %d", w_dtype);
@@ -567,5 +569,5 @@ extern "C" int bh_attention_decode_fused(const void* qkv, void* out, void* part_
                           write_kv, (uint16_t*)k_pages, (uint16_t*)v_pages};
   return attention_bf16_run(nullptr, out, part_o, part_ml, k_pages, v_pages, page_table, table_stride, positions,
                             seq_start, n_seqs, n_seqs, 1, H, KVH, hd, scale, window, max_position, n_splits, fused,
-                            0, stream);
+                            out_block_rows, stream);
 }

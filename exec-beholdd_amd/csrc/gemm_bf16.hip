@@ -84,12 +84,29 @@ struct RidingNorm {
   float* behind_ss;           // [M][bh_gemm_bf16_norm_blocks()] out
 };
 
-template <int MB, int WAVES, bool TILES, int RT, typename TC>
+// Rows in blocks (bh_rows_index in layout.h; 0: rows one after the other) for the skinny kernel's bfloat16
+// matrices: its activations, its output (SwiGLU's, which the next product reads) and the rows it prepares for a
+// norm behind it.  A lane's two loads of a 64-wide chunk of activations then are the pieces 2 g and 2 g + 1 of the
+// chunk's two 32-wide steps: 16 lanes read 256 contiguous bytes (128 with blocks of 8 rows, where the lanes of
+// rows 8 to 15 read what the first eight read) instead of 64 bytes from each of 16 rows, which weighs as much as
+// the weights' loads do: the eight waves of every workgroup read all of the activations.
+// Measured (Qwen3-8B sizes, us per product, qkv / o / gate+up / down): 8 rows 12.7 / 9.2 / 34.1 / 21.0 -> 11.4 /
+// 8.6 / 33.7 / 19.9; 16 rows 15.3 / 10.4 / 35.9 / 24.2 -> 12.4 / 8.9 / 33.1 / 20.4; 32 rows (tiles with K in
+// parts before) 16.2 / 12.6 / 49.4 / 26.4 -> 14.9 / 10.0 / 40.5 / 23.1; 48 rows 18.2 / 14.3 / 50.1 / 28.7 -> 18.6 /
+// 11.8 / 46.0 / 28.4; at 64 rows the tiles are as fast, and a single row is read fastest as it lies.  (Each product
+// alone; inside a decode step 48 rows did not gain, see SKINNY_UP_TO_ROWS.)
+struct RowBlocks {
+  int a, c, behind;
+};
+
+// XB: the rows per block of the activations (RowBlocks::a), known when the kernel is compiled: as a number that
+// only the launch knows it cost the kernel for rows 2 % of a decode step.
+template <int MB, int WAVES, bool TILES, int RT, typename TC, int XB = 0>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t* __restrict__ a,
                                                                  const uint16_t* __restrict__ w,
                                                                  TC* __restrict__ c, int M, int N, int K,
                                                                  int accumulate, int pair_blocks,
-                                                                 RidingNorm norm) {
+                                                                 RidingNorm norm, RowBlocks blocks) {
   __shared__ float partial[WAVES][RT][MB][256];
   __shared__ float row_factor[MB * 16];
   // The norm ahead: 32 threads per row, each with every 32nd partial sum.  The first 256 of a row are asked
@@ -128,10 +145,17 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
     }
   }
   const uint16_t* xp[MB];
+  // from a chunk's first piece of this lane to its second, and to the next chunk
+  constexpr int x_half = XB ? XB * 8 : 8, x_chunk = XB ? 64 * XB : 64;
 #pragma unroll
   for (int b = 0; b < MB; ++b) {
-    const int row = (b * 16 + i < M) ? b * 16 + i : M - 1;
-    xp[b] = a + (size_t)row * K + g * 16;
+    if (XB) {   // piece p = 2 g + u of a chunk is lane group p % 4 of its step p / 4
+      constexpr int step = 32 * (XB ? XB : 1);
+      xp[b] = a + (size_t)(b * 16 / (XB ? XB : 1)) * (K / 32) * step + (g / 2) * step + ((2 * g) % 4 * XB + i % (XB ? XB : 1)) * 8;
+    } else {
+      const int row = (b * 16 + i < M) ? b * 16 + i : M - 1;
+      xp[b] = a + (size_t)row * K + g * 16;
+    }
   }
   f32x4_t acc[RT][MB];
 #pragma unroll
@@ -141,7 +165,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
 
   int chunk = wave;
   // U chunks per trip, all their loads issued before the first multiply, to keep bytes in flight
-  constexpr int U = (MB * RT <= 2) ? 4 : (MB * RT <= 4 ? 2 : 1);
+  constexpr int U = (MB * RT <= 2) ? 4 : (MB * RT <= 4 ? (MB == 4 ? 4 : 2) : 2);
   for (; chunk + (U - 1) * WAVES < full; chunk += U * WAVES) {
     u32x4_t wv[U][RT][2], xv[U][MB][2];
 #pragma unroll
@@ -155,8 +179,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
       }
 #pragma unroll
       for (int b = 0; b < MB; ++b) {
-        xv[u][b][0] = load16(xp[b] + at * 64);
-        xv[u][b][1] = load16(xp[b] + at * 64 + 8);
+        xv[u][b][0] = load16(xp[b] + at * x_chunk);
+        xv[u][b][1] = load16(xp[b] + at * x_chunk + x_half);
       }
     }
 #pragma unroll
@@ -176,7 +200,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
       const u32x4_t w0 = load16(p), w1 = load16(p + half_offset);
 #pragma unroll
       for (int b = 0; b < MB; ++b) {
-        const u32x4_t x0 = load16(xp[b] + chunk * 64), x1 = load16(xp[b] + chunk * 64 + 8);
+        const u32x4_t x0 = load16(xp[b] + chunk * x_chunk), x1 = load16(xp[b] + chunk * x_chunk + x_half);
         acc[t][b] = MFMA16(w0, x0, acc[t][b]);
         acc[t][b] = MFMA16(w1, x1, acc[t][b]);
       }
@@ -232,7 +256,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
     float value = 0.f;   // what the residual holds afterwards (norm.behind_weight: float32 output, RT == 1)
     if (valid) {
       if (RT == 2) {
-        store_out<TC>(c, (size_t)m * N + n, silu_mul(sum[0], sum[RT - 1]), false);
+        store_out<TC>(c, (size_t)bh_rows_index(blocks.c, m, n, N), silu_mul(sum[0], sum[RT - 1]), false);
       } else if (norm.behind_weight) {
         float* cf = reinterpret_cast<float*>(c);
         value = accumulate ? cf[(size_t)m * N + n] + sum[0] : sum[0];
@@ -250,7 +274,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
       if (valid) {
         const float g = norm.behind_weight_f32 ? reinterpret_cast<const float*>(norm.behind_weight)[n]
                                                : bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(norm.behind_weight)[n]);
-        norm.behind_rows[(size_t)m * N + n] = f32_to_bf16_bits(value * g);
+        norm.behind_rows[bh_rows_index(blocks.behind, m, n, N)] = f32_to_bf16_bits(value * g);
         if (e % 16 == 0) norm.behind_ss[(size_t)m * gridDim.x + blockIdx.x] = sq;
       }
     }
@@ -868,17 +892,30 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_whole_kernel(const ui
 
 template <bool TILES, int RT, typename TC>
 static void launch_skinny(const void* a, const void* w, void* c, int M, int N, int K, int accumulate,
-                          int pair_blocks, const RidingNorm& norm, hipStream_t stream) {
+                          int pair_blocks, const RidingNorm& norm, const RowBlocks& blocks, hipStream_t stream) {
   constexpr int WAVES = 8;
   dim3 grid((N + 15) / 16), block(WAVES * 64);
-#define BH_SKINNY(MB)                                                                                     \
-  gemm_skinny_kernel<MB, WAVES, TILES, RT, TC><<<grid, block, 0, stream>>>(                               \
-      (const uint16_t*)a, (const uint16_t*)w, (TC*)c, M, N, K, accumulate, pair_blocks, norm)
+#define BH_SKINNY(MB, XB)                                                                                 \
+  gemm_skinny_kernel<MB, WAVES, TILES, RT, TC, XB><<<grid, block, 0, stream>>>(                           \
+      (const uint16_t*)a, (const uint16_t*)w, (TC*)c, M, N, K, accumulate, pair_blocks, norm, blocks)
+  if constexpr (TILES) {   // activations in blocks come with packed weights only, up to SKINNY_UP_TO_ROWS rows
+    if (blocks.a == 8) {
+      BH_SKINNY(1, 8);
+      return;
+    }
+    if (blocks.a == 16) {
+      switch ((M + 15) / 16) {
+        case 1: BH_SKINNY(1, 16); break;
+        default: BH_SKINNY(2, 16); break;
+      }
+      return;
+    }
+  }
   switch ((M + 15) / 16) {
-    case 1: BH_SKINNY(1); break;
-    case 2: BH_SKINNY(2); break;
-    case 3: BH_SKINNY(3); break;
-    default: BH_SKINNY(4); break;
+    case 1: BH_SKINNY(1, 0); break;
+    case 2: BH_SKINNY(2, 0); break;
+    case 3: BH_SKINNY(3, 0); break;
+    default: BH_SKINNY(4, 0); break;
   }
 #undef BH_SKINNY
 }
@@ -911,10 +948,18 @@ static TiledConfig tiled_config(int M, int N, bool swiglu, int* rows, int* colum
   *columns = (big ? 256 : 128) / (swiglu ? 2 : 1);
   return big ? TILED_256 : tiles_128 > 512 && tiles_128 <= 1024 ? TILED_128_ONE_BUFFER : TILED_128;
 }
+// Up to how many rows the skinny kernel takes a product of packed weights (it reads its activations in blocks
+// from three rows on, see struct RowBlocks); without packed weights, or where the tiles do not fit, up to 64.
+// Decode steps of the Qwen3-8B sizes at context 8,192, against tiles with K in parts from 17 rows on: 16
+// sequences 6.88 -> 6.64 ms, 32 sequences 10.38 -> 9.93 ms, 48 sequences 14.24 -> 14.43 ms (so not those).
+#define SKINNY_UP_TO_ROWS 32
+static bool skinny_first(int M, int N, int K, int layout) {
+  return layout == 1 && K % TK == 0 && N % 16 == 0 && M <= SKINNY_UP_TO_ROWS;
+}
 // Whether the product runs as whole tiles (gemm_tiled_whole_kernel): the way that cuts K into parts and
-// the only tiled way a norm rides on.  Up to 16 rows belong to the skinny kernel.
+// the only tiled way a norm rides on.
 static bool tiled_whole(int M, int N, int K, int layout, int rows, int columns) {
-  return layout == 1 && K % TK == 0 && N % 16 == 0 && M > 16 && (M >= rows || rows <= 64) && N >= columns &&
+  return layout == 1 && K % TK == 0 && N % 16 == 0 && M > SKINNY_UP_TO_ROWS && (M >= rows || rows <= 64) && N >= columns &&
          (long)rows * K < (1L << 31);
 }
 
@@ -1007,11 +1052,25 @@ extern "C" int bh_gemm_bf16_takes_norm(int M, int N, int K, int layout, int acti
   return tiled_whole(M, N, K, layout, rows, columns) ? 1 : 0;
 }
 
-// Whether a product of these sizes reads its activations faster from blocks of 16 rows x 32 columns
-// (bh_blocked_index, layout.h) and takes them that way: those of the kernel whose wave groups take turns.
+// The rows per block (16 or 8) if a product of these sizes reads its activations faster from blocks of that
+// many rows x 32 columns (bh_rows_index, layout.h) and takes them that way, else 0: the products of the kernel
+// whose wave groups take turns (16), and those of 3 to 32 rows of the skinny kernel (8 up to 8 rows, else 16).
 extern "C" int bh_gemm_bf16_reads_blocked(int M, int N, int K, int layout, int activation) {
   if (M <= 0 || N <= 0 || K <= 0 || K % 32 != 0) return 0;
-  return gemm_turns_blocks(M, N, K, layout, activation) || gemm_turns_parts(M, N, K, layout, activation) > 1 ? 1 : 0;
+  if (gemm_turns_blocks(M, N, K, layout, activation) || gemm_turns_parts(M, N, K, layout, activation) > 1) return 16;
+  if (M >= 3 && skinny_first(M, N, K, layout)) return M <= 8 ? 8 : 16;
+  return 0;
+}
+
+// In what form a product of these sizes can write the bfloat16 rows it produces for the next product (a SwiGLU's
+// output, the rows prepared for a norm behind it): 2 = rows or blocks of 8 or 16 rows (the skinny kernel),
+// 1 = rows or, for SwiGLU, blocks of 16 (the kernel whose wave groups take turns), 0 = rows only.
+extern "C" int bh_gemm_bf16_writes_blocked(int M, int N, int K, int layout, int activation) {
+  if (M <= 0 || N <= 0 || K <= 0 || N % 32 != 0) return 0;
+  if (gemm_turns_blocks(M, N, K, layout, activation)) return activation ? 1 : 0;
+  int rows, columns;
+  tiled_config(M, N, activation != 0, &rows, &columns);
+  return M <= 64 && !tiled_whole(M, N, K, layout, rows, columns) ? 2 : 0;
 }
 
 // layout: 0 = rows, 1 = tiles.  activation: 0 = none; 1 = SwiGLU (W has 2 * N rows: gate rows then up rows).
@@ -1029,10 +1088,15 @@ extern "C" long bh_gemm_bf16_scratch(int M, int N, int K, int layout, int activa
 // The `ahead_*` and `behind_*` arguments (null when unused) let an RMSNorm ride on the products before and
 // after it (struct RidingNorm) where bh_gemm_bf16_takes_norm / bh_gemm_bf16_norm_blocks say so.  `scratch`: bh_gemm_bf16_scratch() bytes, or
 // null (then K is not cut into parts where that would be faster).
+// a_block_rows: the activations (for a norm ahead: its unscaled rows) lie in blocks of that many rows, as
+// bh_gemm_bf16_reads_blocked says this product reads them, or in rows (0).  c_block_rows: a SwiGLU's output goes out
+// that way (16 in the kernel for many rows; 0, 8 or 16 in the skinny one); behind_block_rows: so do the rows
+// prepared for a norm behind (the skinny kernel's).
 extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, int accumulate, int M, int N, int K,
                             int layout, int activation, const float* ahead_ss, int ahead_blocks, float ahead_eps,
                             const void* behind_weight, int behind_weight_dtype, void* behind_rows,
-                            float* behind_ss, void* scratch, int a_blocked, int c_blocked, hipStream_t stream) {
+                            float* behind_ss, void* scratch, int a_block_rows, int c_block_rows, int behind_block_rows,
+                            hipStream_t stream) {
   BH_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_bf16: sizes M=%d N=%d K=%d must be positive", M, N, K);
   BH_REQUIRE(K % 8 == 0, "gemm_bf16: K=%d must be a multiple of 8", K);
   BH_REQUIRE(c_dtype == BH_F32 || c_dtype == BH_BF16, "gemm_bf16: unknown output dtype %d", c_dtype);
@@ -1054,10 +1118,21 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
   const RidingNorm norm = {ahead_ss, ahead_blocks, ahead_eps, behind_weight, behind_weight_dtype == BH_F32,
                            (uint16_t*)behind_rows, behind_ss};
   const bool f32 = c_dtype == BH_F32;
-  BH_REQUIRE((!a_blocked && !c_blocked) || (!ahead_ss && !behind_weight && (f32 || !accumulate) &&
-                                            bh_gemm_bf16_reads_blocked(M, N, K, layout, activation)),
-             "gemm_bf16: a product of M=%d N=%d K=%d does not take rows in blocks (bh_gemm_bf16_reads_blocked)", M, N, K);
-  BH_REQUIRE(!c_blocked || gemm_turns_blocks(M, N, K, layout, activation), "gemm_bf16: this product writes no blocks");
+  const auto block_rows_ok = [](int rows) { return rows == 0 || rows == 8 || rows == 16; };
+  BH_REQUIRE(block_rows_ok(a_block_rows) && block_rows_ok(c_block_rows) && block_rows_ok(behind_block_rows),
+             "gemm_bf16: rows lie in blocks of 8 or 16, or one after the other (0)");
+  BH_REQUIRE(a_block_rows == 0 || a_block_rows == bh_gemm_bf16_reads_blocked(M, N, K, layout, activation),
+             "gemm_bf16: a product of M=%d N=%d K=%d does not read rows in blocks of %d (bh_gemm_bf16_reads_blocked)", M, N, K, a_block_rows);
+  BH_REQUIRE(c_block_rows == 0 || (activation && N % 32 == 0), "gemm_bf16: only SwiGLU's output goes out in blocks, N=%d a multiple of 32", N);
+  BH_REQUIRE(behind_block_rows == 0 || (behind_weight && N % 32 == 0), "gemm_bf16: rows in blocks for a norm behind need that norm, N=%d a multiple of 32", N);
+  const bool skinny = [&] {
+    int rows, columns;
+    tiled_config(M, N, activation != 0, &rows, &columns);
+    return M <= 64 && !tiled_whole(M, N, K, layout, rows, columns);
+  }();
+  BH_REQUIRE(skinny || (c_block_rows != 8 && behind_block_rows == 0 && (c_block_rows == 0 || gemm_turns_blocks(M, N, K, layout, activation))),
+             "gemm_bf16: a product of M=%d N=%d K=%d does not write these blocks", M, N, K);
+  const int a_blocked = a_block_rows == 16 && !skinny, c_blocked = c_block_rows == 16 && !skinny;
   if (!ahead_ss && !behind_weight && (f32 || !accumulate)) {   // many rows: the kernel whose wave groups take turns
     if (const int blocks = gemm_turns_blocks(M, N, K, layout, activation))
       return gemm_turns_launch(a, w, c, c_dtype, accumulate, M, N, K, activation, blocks, a_blocked, c_blocked, stream);
@@ -1095,16 +1170,15 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
 #undef BH_FINISH
     return bh_check_launch("gemm_parts_finish");
   }
-  int tile_rows, tile_columns;
-  tiled_config(M, N, activation != 0, &tile_rows, &tile_columns);
-  if (M <= 64 && !tiled_whole(M, N, K, layout, tile_rows, tile_columns)) {
+  if (skinny) {
     const int pair_blocks = N / 16;
+    const RowBlocks blocks = {a_block_rows, c_block_rows, behind_block_rows};
     if (activation) {
-      if (layout) BH_PICK(launch_skinny, true, 2, a, w, c, M, N, K, 0, pair_blocks, norm, stream);
-      else BH_PICK(launch_skinny, false, 2, a, w, c, M, N, K, 0, pair_blocks, norm, stream);
+      if (layout) BH_PICK(launch_skinny, true, 2, a, w, c, M, N, K, 0, pair_blocks, norm, blocks, stream);
+      else BH_PICK(launch_skinny, false, 2, a, w, c, M, N, K, 0, pair_blocks, norm, blocks, stream);
     } else {
-      if (layout) BH_PICK(launch_skinny, true, 1, a, w, c, M, N, K, accumulate, 0, norm, stream);
-      else BH_PICK(launch_skinny, false, 1, a, w, c, M, N, K, accumulate, 0, norm, stream);
+      if (layout) BH_PICK(launch_skinny, true, 1, a, w, c, M, N, K, accumulate, 0, norm, blocks, stream);
+      else BH_PICK(launch_skinny, false, 1, a, w, c, M, N, K, accumulate, 0, norm, blocks, stream);
     }
     return bh_check_launch("gemm_skinny");
   }

@@ -10,17 +10,25 @@
 //
 // Global memory goes to LDS directly (16-byte loads that write LDS at the wave's base + 16 * lane): 1 KB per
 // load, which is one operand of 16 rows x 32 k in lane order, so that reading it back is one conflict-free
-// 16-byte read per lane.  Four lanes bring 64 consecutive bytes of a row of A, or 256 bytes of a block of W.
+// 16-byte read per lane.  Four lanes bring 256 bytes of a block of W; of A they bring 64 consecutive bytes of a
+// row when A lies in rows, so that a quarter of a wave touches 16 cache lines, each for a quarter of its bytes,
+// and every line is asked for again by the next step.  A in blocks of 16 rows x 32 k in operand order
+// (bh_blocked_index in layout.h; the kernels that produce activations write it that way for this reader) makes
+// an operand 1 KB of contiguous memory like W's: gate/up at 2,048 rows 333 -> 293 us (1.41 PFLOP/s), qkv 100 -> 85,
+// down with 128-wide tiles 247 -> 181, with 256-wide tiles at 4,096 rows 348 -> 284 (1.45).  The vendor library's
+// product (torch.matmul, bfloat16) takes 287 us for the gate/up shape without the gate (1.44 PFLOP/s), 81 us for qkv,
+// and reaches 1.51 to 1.55 at its best shapes (4,096 and 8,192 rows): that, not 2.5, is what these matrix cores
+// give with operands from memory.
 // LDS holds four steps (4 x (16 + 2 YB) KB); a step's region is loaded again as soon as both groups have read
 // it, which is five to six turns before it is read next.
 //
-// Measured at the Qwen3-8B shapes, 2,048 rows, each product alone: gate/up with SwiGLU 404 -> 330 us
+// Measured at the Qwen3-8B shapes, 2,048 rows, activations in rows, each product alone: gate/up with SwiGLU 404 -> 330 us
 // (1.25 PFLOP/s), qkv 132 -> 104 us with tiles of 192 weight rows (256 of them, one per compute unit), o 102 ->
 // 84 us with 128; in the whole model 381 -> 338, 115 -> 101 and 87 -> 94 us (which is why the o and down
 // projections there go through K in parts of the widest tile instead, see turns_plan: 77 us for o, finishing
 // kernel included).
-// What bounds it: the loads alone (no multiplies) take 0.9 of the whole kernel's time, the multiplies alone
-// 0.6.  It is not the loads' latency (five or six steps in LDS instead of four changed nothing; touching the
+// What bounds it (activations in rows): the loads alone (no multiplies) take 0.9 of the whole kernel's time, the
+// multiplies alone 0.6, the multiplies with their operand reads from LDS 0.8 (1.46 to 1.58 PFLOP/s).  It is not the loads' latency (five or six steps in LDS instead of four changed nothing; touching the
 // lines three slices ahead with 4-byte loads made it slower, 0.9 PFLOP/s for gate/up: loads retire in order, so
 // the loads for LDS waited behind the touches), not LDS (a compute unit reads 256 bytes per clock from it and
 // needs a third of that) and not memory beyond L2 (87 % of the L2 requests hit; 0.3 to 0.6 GB come from beyond
@@ -264,7 +272,8 @@ bool gemm_turns_can(int M, int N, int K, int layout, int activation, int blocks)
 }
 
 // Which way, if any.  A tile of YB blocks per wave costs a compute unit YB x cost(YB) units of time, where cost
-// is what the narrower tiles lose (measured 1.25, 1.11 and 0.90 PFLOP/s for 8, 6 and 4 with the chip full), and
+// is what the narrower tiles lose (measured 1.43, 1.16 and 1.07 PFLOP/s for 8, 6 and 4 with the chip full and the
+// activations in blocks; 1.25, 1.11 and 0.90 with activations in rows), and
 // the chip works in rounds of 256 tiles; a tile of its own is taken if that estimate beats what the other tiled
 // kernels reach at their best (about 0.8 PFLOP/s).  Products with so few of the widest tiles that much of the
 // chip would idle can instead cut K into parts over as many times the workgroups, each leaving its bare sums in
@@ -287,8 +296,8 @@ TurnsPlan turns_plan(int M, int N, int K, int layout, int activation) {
     const int outs = (activation ? 16 : 32) * blocks;
     const long tiles = (long)((N + outs - 1) / outs) * ((M + 255) / 256);
     const long rounds = (tiles + 255) / 256;
-    const double cost = blocks == 8 ? 1.0 : blocks == 6 ? 1.12 : 1.39;
-    const double rate = 1250.0 * work / ((double)rounds * 256 * 256 * (activation ? 2 : 1) * outs * cost);
+    const double cost = blocks == 8 ? 1.0 : blocks == 6 ? 1.23 : 1.34;
+    const double rate = 1430.0 * work / ((double)rounds * 256 * 256 * (activation ? 2 : 1) * outs * cost);
     if (rate >= best_rate) best_rate = direct_rate = rate, plan.blocks = blocks;
   }
   if (!activation && M >= 512 && gemm_turns_can(M, N, K, layout, 0, 8)) {
@@ -301,7 +310,7 @@ TurnsPlan turns_plan(int M, int N, int K, int layout, int activation) {
     int parts = 8;
     while (parts > 1 && (tiles * parts > 256 || K / parts < 1024 || K % (128 * parts) != 0)) parts /= 2;
     if (parts > 1 && tiles * parts >= 160) {
-      const double rate = 0.85 * 1250.0 * work / (256.0 * 256 * 256 / parts);
+      const double rate = 0.85 * 1430.0 * work / (256.0 * 256 * 256 / parts);
       if (rate > direct_rate) plan.blocks = 0, plan.parts = parts;
     }
   }

@@ -73,12 +73,13 @@ extern "C" int bh_embed(const int32_t* tokens, const int32_t* token_src, const i
 // where latency is all there is).  PER == 0: any width, in loops.
 template <typename TW, typename TO, int PER>
 __global__ void rmsnorm_kernel(const float* __restrict__ x, const int32_t* __restrict__ rows,
-                               const TW* __restrict__ w, TO* __restrict__ out, int width, float eps) {
+                               const TW* __restrict__ w, TO* __restrict__ out, int width, float eps, int block_rows) {
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const int src = rows ? rows[r] : r;
   const float* xr = x + (size_t)src * width;
-  TO* o = out + (size_t)r * width;
+  // block_rows: the output's rows lie in blocks of that many (bh_rows_index), or one after the other (0)
+  auto at = [&](int i) { return out + bh_rows_index(block_rows, r, i, width); };
   if (PER > 0) {
     float xv[PER > 0 ? PER : 1], wv[PER > 0 ? PER : 1];
     float ss = 0.f;
@@ -95,7 +96,7 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const int32_t* __res
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
       const int i = threadIdx.x + j * blockDim.x;
-      if (i < width) o[i] = from_f32<TO>(xv[j] * inv * wv[j]);
+      if (i < width) *at(i) = from_f32<TO>(xv[j] * inv * wv[j]);
     }
     return;
   }
@@ -109,7 +110,7 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const int32_t* __res
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     float y = xr[i] * inv;
     if (w) y *= to_f32(w[i]);
-    o[i] = from_f32<TO>(y);
+    *at(i) = from_f32<TO>(y);
   }
 }
 
@@ -121,7 +122,8 @@ typedef float norm_f32x4_t __attribute__((ext_vector_type(4)));
 typedef uint16_t norm_u16x4_t __attribute__((ext_vector_type(4)));
 template <typename TW, typename TO, int NV>
 __global__ void rmsnorm_wide_kernel(const float* __restrict__ x, const int32_t* __restrict__ rows,
-                                    const TW* __restrict__ w, TO* __restrict__ out, int width, float eps) {
+                                    const TW* __restrict__ w, TO* __restrict__ out, int width, float eps,
+                                    int block_rows) {
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const int src = rows ? rows[r] : r;
@@ -154,12 +156,12 @@ __global__ void rmsnorm_wide_kernel(const float* __restrict__ x, const int32_t* 
     const int i = threadIdx.x + j * blockDim.x;
     if (i >= fours) continue;
     if constexpr (sizeof(TO) == 4) {
-      reinterpret_cast<norm_f32x4_t*>(out + (size_t)r * width)[i] = xv[j] * inv * wv[j];
+      *reinterpret_cast<norm_f32x4_t*>(out + bh_rows_index(block_rows, r, 4 * i, width)) = xv[j] * inv * wv[j];
     } else {
       norm_u16x4_t bits;
 #pragma unroll
       for (int e = 0; e < 4; ++e) bits[e] = f32_to_bf16_bits(xv[j][e] * inv * wv[j][e]);
-      reinterpret_cast<norm_u16x4_t*>(out + (size_t)r * width)[i] = bits;
+      *reinterpret_cast<norm_u16x4_t*>(out + bh_rows_index(block_rows, r, 4 * i, width)) = bits;
     }
   }
 }
@@ -167,7 +169,7 @@ __global__ void rmsnorm_wide_kernel(const float* __restrict__ x, const int32_t* 
 #define NORM_WIDE_FROM_ROWS 64   // fewer rows are latency, not bytes: the kernel above with its scalar loads was measured for them
 template <typename TW, typename TO>
 static void launch_rmsnorm(const float* x, const int32_t* rows, const void* w, void* out, int n_rows, int width,
-                           float eps, hipStream_t stream) {
+                           float eps, int block_rows, hipStream_t stream) {
   if (n_rows >= NORM_WIDE_FROM_ROWS && width % 4 == 0 && width <= 4 * 4 * 1024 &&
       ((uintptr_t)x | (uintptr_t)w | (uintptr_t)out) % 16 == 0) {
     const int fours = width / 4;
@@ -175,7 +177,7 @@ static void launch_rmsnorm(const float* x, const int32_t* rows, const void* w, v
     const int each = (fours + wide_threads - 1) / wide_threads;
     dim3 grid(n_rows), block(wide_threads);
 #define BH_NORM_WIDE(NV) \
-  rmsnorm_wide_kernel<TW, TO, NV><<<grid, block, 0, stream>>>(x, rows, (const TW*)w, (TO*)out, width, eps)
+  rmsnorm_wide_kernel<TW, TO, NV><<<grid, block, 0, stream>>>(x, rows, (const TW*)w, (TO*)out, width, eps, block_rows)
     if (each == 1) BH_NORM_WIDE(1);
     else if (each == 2) BH_NORM_WIDE(2);
     else BH_NORM_WIDE(4);
@@ -186,21 +188,26 @@ static void launch_rmsnorm(const float* x, const int32_t* rows, const void* w, v
   const int per = (width + threads - 1) / threads;
   dim3 grid(n_rows), block(threads);
 #define BH_NORM(PER) \
-  rmsnorm_kernel<TW, TO, PER><<<grid, block, 0, stream>>>(x, rows, (const TW*)w, (TO*)out, width, eps)
+  rmsnorm_kernel<TW, TO, PER><<<grid, block, 0, stream>>>(x, rows, (const TW*)w, (TO*)out, width, eps, block_rows)
   if (per <= 4) BH_NORM(4);
   else if (per <= 8) BH_NORM(8);
   else BH_NORM(0);
 #undef BH_NORM
 }
 
+// out_block_rows: the output's rows lie in blocks of 8 or 16 rows x 32 columns (bh_rows_index; bfloat16, width a
+// multiple of 32), or one after the other (0).
 extern "C" int bh_rmsnorm(const float* x, const int32_t* rows, const void* w, int w_dtype, void* out,
-                          int out_dtype, int n_rows, int width, float eps, hipStream_t stream) {
+                          int out_dtype, int n_rows, int width, float eps, int out_block_rows, hipStream_t stream) {
   BH_REQUIRE(n_rows > 0 && width > 0, "rmsnorm: rows %d and width %d must be positive", n_rows, width);
   BH_REQUIRE(eps >= 0.f, "rmsnorm: eps must not be negative");
-  if (w_dtype == BH_F32 && out_dtype == BH_F32) launch_rmsnorm<float, float>(x, rows, w, out, n_rows, width, eps, stream);
-  else if (w_dtype == BH_F32 && out_dtype == BH_BF16) launch_rmsnorm<float, bf16_t>(x, rows, w, out, n_rows, width, eps, stream);
-  else if (w_dtype == BH_BF16 && out_dtype == BH_F32) launch_rmsnorm<bf16_t, float>(x, rows, w, out, n_rows, width, eps, stream);
-  else if (w_dtype == BH_BF16 && out_dtype == BH_BF16) launch_rmsnorm<bf16_t, bf16_t>(x, rows, w, out, n_rows, width, eps, stream);
+  BH_REQUIRE(out_block_rows == 0 || ((out_block_rows == 8 || out_block_rows == 16) && out_dtype == BH_BF16 && width % 32 == 0),
+             "rmsnorm: rows in blocks of %d need bfloat16 and a width that is a multiple of 32 (got %d)", out_block_rows, width);
+  const int b = out_block_rows;
+  if (w_dtype == BH_F32 && out_dtype == BH_F32) launch_rmsnorm<float, float>(x, rows, w, out, n_rows, width, eps, b, stream);
+  else if (w_dtype == BH_F32 && out_dtype == BH_BF16) launch_rmsnorm<float, bf16_t>(x, rows, w, out, n_rows, width, eps, b, stream);
+  else if (w_dtype == BH_BF16 && out_dtype == BH_F32) launch_rmsnorm<bf16_t, float>(x, rows, w, out, n_rows, width, eps, b, stream);
+  else if (w_dtype == BH_BF16 && out_dtype == BH_BF16) launch_rmsnorm<bf16_t, bf16_t>(x, rows, w, out, n_rows, width, eps, b, stream);
   else return bh_fail("rmsnorm: unknown dtypes %d/%d", w_dtype, out_dtype);
   return bh_check_launch("rmsnorm");
 }
@@ -651,12 +658,12 @@ extern "C" int bh_swiglu(const void* gu, void* out, int dtype, int n_rows, int F
 typedef uint32_t blocked_u32x4_t __attribute__((ext_vector_type(4)));
 template <bool TO_BLOCKS>
 __global__ __launch_bounds__(256) void rows_blocked_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst,
-                                                           int n_rows, int width, long pieces) {
+                                                           int n_rows, int width, long pieces, int block_rows) {
   const long piece = (long)blockIdx.x * 256 + threadIdx.x;   // in the order of the blocked matrix
   if (piece >= pieces) return;
-  const int r = piece % 16, q = (piece / 16) % 4;
-  const long block = piece / 64;
-  const int column = (int)(block % (width / 32)) * 32 + 8 * q, row = (int)(block / (width / 32)) * 16 + r;
+  const int r = piece % block_rows, q = (piece / block_rows) % 4;
+  const long block = piece / (4 * block_rows);
+  const int column = (int)(block % (width / 32)) * 32 + 8 * q, row = (int)(block / (width / 32)) * block_rows + r;
   const blocked_u32x4_t zero = {0u, 0u, 0u, 0u};
   if (TO_BLOCKS) {
     reinterpret_cast<blocked_u32x4_t*>(dst)[piece] =
@@ -666,15 +673,17 @@ __global__ __launch_bounds__(256) void rows_blocked_kernel(const uint16_t* __res
   }
 }
 
-extern "C" int bh_rows_blocked(const void* src, void* dst, int n_rows, int width, int to_blocks, hipStream_t stream) {
+extern "C" int bh_rows_blocked(const void* src, void* dst, int n_rows, int width, int to_blocks, int block_rows,
+                               hipStream_t stream) {
   BH_REQUIRE(src != nullptr && dst != nullptr && n_rows > 0 && width > 0, "rows_blocked: a matrix with rows and a width");
   BH_REQUIRE(width % 32 == 0, "rows_blocked: the width %d must be a multiple of 32", width);
+  BH_REQUIRE(block_rows == 8 || block_rows == 16, "rows_blocked: blocks of 8 or 16 rows, not %d", block_rows);
   BH_REQUIRE(((uintptr_t)src | (uintptr_t)dst) % 16 == 0, "rows_blocked: buffers must be 16-byte aligned");
-  const long pieces = (long)((n_rows + 15) / 16) * (width / 32) * 64;
+  const long pieces = (long)((n_rows + block_rows - 1) / block_rows) * (width / 32) * 4 * block_rows;
   BH_REQUIRE((pieces + 255) / 256 < (1L << 31), "rows_blocked: too many blocks");
   dim3 grid((unsigned)((pieces + 255) / 256)), block(256);
-  if (to_blocks) rows_blocked_kernel<true><<<grid, block, 0, stream>>>((const uint16_t*)src, (uint16_t*)dst, n_rows, width, pieces);
-  else rows_blocked_kernel<false><<<grid, block, 0, stream>>>((const uint16_t*)src, (uint16_t*)dst, n_rows, width, pieces);
+  if (to_blocks) rows_blocked_kernel<true><<<grid, block, 0, stream>>>((const uint16_t*)src, (uint16_t*)dst, n_rows, width, pieces, block_rows);
+  else rows_blocked_kernel<false><<<grid, block, 0, stream>>>((const uint16_t*)src, (uint16_t*)dst, n_rows, width, pieces, block_rows);
   return bh_check_launch("rows_blocked");
 }
 

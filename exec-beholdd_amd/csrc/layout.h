@@ -47,10 +47,19 @@ BH_BOTH inline int bh_value_index(int order, int token, int dim, int hd) {
 // wave's lanes: lane 16 q + r holds row r of the block, columns 8 q .. 8 q + 7.  The blocks of 16 rows
 // follow each other along the width, then down the rows.  A wave then takes an operand with one load of
 // contiguous memory instead of 64 bytes from each of 16 rows.  Needs width to be a multiple of 32; the
-// buffer holds whole blocks (rows rounded up; readers round them up to BH_BLOCKED_ROWS_PAD).
+// buffer holds whole blocks (rows rounded up; the products of many rows read whole tiles of
+// BH_BLOCKED_ROWS_PAD rows).  Steps of at most 8 rows use blocks of 8 rows instead (the same order with 8 in
+// the place of 16: 512 bytes, of which the product of few rows reads each 16-byte piece into two lanes).
 #define BH_BLOCKED_ROWS_PAD 256
-BH_BOTH inline long bh_blocked_index(int row, int column, int width) {
-  return ((long)(row / 16) * (width / 32) + column / 32) * 512 + (((column % 32) / 8) * 16 + row % 16) * 8 + column % 8;
+BH_BOTH inline long bh_blocked_index_of(int block_rows, int row, int column, int width) {
+  return ((long)(row / block_rows) * (width / 32) + column / 32) * (32 * block_rows) +
+         (((column % 32) / 8) * block_rows + row % block_rows) * 8 + column % 8;
+}
+BH_BOTH inline long bh_blocked_index(int row, int column, int width) { return bh_blocked_index_of(16, row, column, width); }
+// Where element (row, column) of a matrix lies whose rows are in blocks of `block_rows` (8 or 16), or one after
+// the other (0).
+BH_BOTH inline long bh_rows_index(int block_rows, int row, int column, int width) {
+  return block_rows ? bh_blocked_index_of(block_rows, row, column, width) : (long)row * width + column;
 }
 
 // bfloat16 kept as its 16 bits; widening is a shift, narrowing rounds to nearest even.

@@ -55,20 +55,33 @@ class NormedRows:
 
 
 class BlockedRows:
-    """A bfloat16 activation matrix [rows, width] kept in blocks of 16 rows x 32 columns, each block 1 KB in the
-    order in which a matrix-core operand lies in a wave's lanes (`bh_blocked_index` in csrc/layout.h): what the
-    products of many rows read fastest.  `HipKernels.new_rows` hands one out where the product named as the
-    matrix's reader takes it; the kernels that produce activations (`rmsnorm`, `gemm_swiglu`, `attention`, a
-    `gemm` that finishes a norm) write into it, and `gemm` / `gemm_swiglu` read it.  `data` holds whole tiles of
-    256 rows; rows the matrix does not have hold nothing.  `shape` and `dtype` are those of the matrix."""
+    """A bfloat16 activation matrix [rows, width] kept in blocks of `block_rows` (16 or 8) rows x 32 columns, each
+    block in the order in which a matrix-core operand lies in a wave's lanes (`bh_rows_index` in csrc/layout.h):
+    what the products of many rows and those of 3 to 32 rows read fastest.  `HipKernels.new_rows` hands one out
+    where the product named as the matrix's reader takes it; the kernels that produce activations (`rmsnorm`,
+    `gemm_swiglu`, `attention`, a `gemm` that prepares or finishes a norm) write into it, and `gemm` /
+    `gemm_swiglu` read it.  `data` holds whole blocks (for more than 32 rows whole tiles of 256 rows); rows the
+    matrix does not have hold nothing.  `shape` and `dtype` are those of the matrix."""
 
     ROWS_PAD = 256
 
-    def __init__(self, data: torch.Tensor, rows: int, width: int):
+    def __init__(self, data: torch.Tensor, rows: int, width: int, block_rows: int = 16):
         self.data, self.shape, self.dtype, self.device = data, (rows, width), data.dtype, data.device
+        self.block_rows = int(block_rows)
 
     def dim(self):
         return 2
+
+    @staticmethod
+    def padded_rows(rows: int, block_rows: int) -> int:
+        """Rows that the buffer of a matrix of `rows` rows holds."""
+        unit = BlockedRows.ROWS_PAD if rows > 32 else block_rows
+        return -(-rows // unit) * unit
+
+
+def _block_rows(x) -> int:
+    """In blocks of how many rows a matrix lies (0: row after row)."""
+    return x.block_rows if isinstance(x, BlockedRows) else 0
 
 
 def _code(tensor, what: str) -> int:
@@ -107,23 +120,23 @@ class HipKernels:
         lib.bh_page_size.restype = i
         table = {
             "bh_embed": [p, p, p, p, i, p, i, i, i, p],
-            "bh_rmsnorm": [p, p, p, i, p, i, i, i, f, p],
+            "bh_rmsnorm": [p, p, p, i, p, i, i, i, f, i, p],
             "bh_gemm_generic": [p, i, p, i, p, i, i, i, i, i, p],
             "bh_qk_norm_rope_cache": [p, i, p, p, p, i, f, p, p, i, i, p, p, p, p, p, i, i, i, i, i, i, i, i, p],
             "bh_attention_generic": [p, p, i, p, p, p, i, p, p, i, i, i, i, f, i, i, p],
             "bh_swiglu": [p, p, i, i, i, p],
             "bh_sample": [p, p, p, p, p, p, p, p, i, i, p],
             "bh_sample_scratch": [i, i],
-            "bh_gemm_bf16": [p, p, p, i, i, i, i, i, i, i, p, i, f, p, i, p, p, p, i, i, p],
+            "bh_gemm_bf16": [p, p, p, i, i, i, i, i, i, i, p, i, f, p, i, p, p, p, i, i, i, p],
             "bh_gemm_bf16_turns": [p, p, p, i, i, i, i, i, i, i, i, i, p],
             "bh_gemm_bf16_then_norm": [p, p, p, i, i, i, i, p, i, f, p, p, i, i, p],
-            "bh_rows_blocked": [p, p, i, i, i, p],
+            "bh_rows_blocked": [p, p, i, i, i, i, p],
             "bh_gemm_bf16_finishes_norm": [i, i, i, i],
             "bh_attention_bf16": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, i, i, f, i, i, i, i, p],
             "bh_attention_bf16_splits": [i, i, i, i, i],
             "bh_attention_bf16_writes_blocked": [i, i, i, i, i],
             "bh_attention_decode_fused": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, f, i, i, i, p, p, i, f, p, p, i, i,
-                                          i, p],
+                                          i, i, p],
             "bh_kv_order": [i, i],
             "bh_stream_read": [p, ctypes.c_long, i, i, p, p, p],
         }
@@ -134,7 +147,7 @@ class HipKernels:
         lib.bh_gemm_bf16_scratch.argtypes = [i, i, i, i, i]
         lib.bh_gemm_bf16_scratch.restype = ctypes.c_long
         for query in (lib.bh_gemm_bf16_norm_blocks, lib.bh_gemm_bf16_takes_norm, lib.bh_gemm_bf16_turns_blocks,
-                      lib.bh_gemm_bf16_reads_blocked):
+                      lib.bh_gemm_bf16_reads_blocked, lib.bh_gemm_bf16_writes_blocked):
             query.argtypes, query.restype = [i, i, i, i, i], ctypes.c_int
     # ---- helpers ----
     def _stream(self):
@@ -179,11 +192,6 @@ class HipKernels:
 
     def rmsnorm(self, x, weight, eps, out, rows=None):
         """out[r] = x[rows[r] if rows is given else r] * inv_rms * weight; x f32 [*, D], out [n, D]."""
-        if isinstance(out, BlockedRows):      # this kernel writes rows: regroup them afterwards
-            rows_out = torch.empty(out.shape, dtype=out.dtype, device=self.device)
-            self.rmsnorm(x, weight, eps, rows_out, rows=rows)
-            self.to_blocked(rows_out, out)
-            return
         n_rows, width = out.shape
         if x.dim() != 2 or x.shape[1] != width or (weight is not None and weight.shape != (width,)):
             raise KernelError(f"rmsnorm: shapes x {tuple(x.shape)}, out {tuple(out.shape)} do not fit")
@@ -195,37 +203,51 @@ class HipKernels:
         self._check(self.lib.bh_rmsnorm(
             self._ptr(x, "rmsnorm x", (torch.float32,)), self._ptr(rows, "rmsnorm rows", (torch.int32,), True),
             self._ptr(weight, "rmsnorm weight", None, True), _code(weight, "rmsnorm weight") if weight is not None else F32,
-            self._ptr(out, "rmsnorm out"), _code(out, "rmsnorm out"), n_rows, width, float(eps), self._stream()))
+            self._ptr(out, "rmsnorm out"), _code(out, "rmsnorm out"), n_rows, width, float(eps), _block_rows(out),
+            self._stream()))
 
     def new_rows(self, rows, width, dtype, reader_outputs=None, reader_swiglu=False):
         """An empty activation matrix [rows, width] for a kernel of this library to fill.  With `reader_outputs`,
         the product that reads it next has that many outputs (`reader_swiglu`: through the gate, so twice as
         many weight rows): where that product takes `BlockedRows` and reads them faster, the matrix is one."""
-        if (reader_outputs is not None and dtype == torch.bfloat16 and width % 64 == 0
-                and self.lib.bh_gemm_bf16_reads_blocked(int(rows), int(reader_outputs), int(width), 1, int(bool(reader_swiglu)))):
-            padded = -(-int(rows) // BlockedRows.ROWS_PAD) * BlockedRows.ROWS_PAD
-            return BlockedRows(torch.empty(padded * int(width), dtype=dtype, device=self.device), int(rows), int(width))
-        return torch.empty((int(rows), int(width)), dtype=dtype, device=self.device)
+        rows, width = int(rows), int(width)
+        if reader_outputs is not None and dtype == torch.bfloat16 and width % 64 == 0:
+            block_rows = int(self.lib.bh_gemm_bf16_reads_blocked(rows, int(reader_outputs), width, 1, int(bool(reader_swiglu))))
+            if block_rows:
+                return self._new_blocked(rows, width, block_rows)
+        return torch.empty((rows, width), dtype=dtype, device=self.device)
 
-    def to_blocked(self, x, out=None):
-        """The bfloat16 matrix `x` as `BlockedRows` (into `out` if given)."""
+    def _new_blocked(self, rows, width, block_rows):
+        padded = BlockedRows.padded_rows(rows, block_rows)
+        return BlockedRows(torch.empty(padded * width, dtype=torch.bfloat16, device=self.device), rows, width, block_rows)
+
+    def to_blocked(self, x, out=None, block_rows=16):
+        """The bfloat16 matrix `x` as `BlockedRows` (into `out` if given, in its blocks)."""
         rows, width = x.shape
         if x.dtype != torch.bfloat16 or width % 32:
             raise KernelError(f"to_blocked: a bfloat16 matrix whose width is a multiple of 32, not {x.dtype} {tuple(x.shape)}")
         if out is None:
-            padded = -(-rows // BlockedRows.ROWS_PAD) * BlockedRows.ROWS_PAD
-            out = BlockedRows(torch.empty(padded * width, dtype=x.dtype, device=self.device), rows, width)
+            out = self._new_blocked(rows, width, block_rows)
         elif not isinstance(out, BlockedRows) or tuple(out.shape) != (rows, width):
             raise KernelError(f"to_blocked: the output stands for {tuple(out.shape)}, the matrix is {tuple(x.shape)}")
-        self._check(self.lib.bh_rows_blocked(self._ptr(x, "rows"), self._ptr(out, "blocks"), rows, width, 1, self._stream()))
+        self._check(self.lib.bh_rows_blocked(self._ptr(x, "rows"), self._ptr(out, "blocks"), rows, width, 1, out.block_rows,
+                                             self._stream()))
         return out
 
     def from_blocked(self, blocked):
         """The matrix that `blocked` stands for, row after row."""
         rows, width = blocked.shape
         out = torch.empty((rows, width), dtype=blocked.dtype, device=self.device)
-        self._check(self.lib.bh_rows_blocked(self._ptr(blocked, "blocks"), self._ptr(out, "rows"), rows, width, 0, self._stream()))
+        self._check(self.lib.bh_rows_blocked(self._ptr(blocked, "blocks"), self._ptr(out, "rows"), rows, width, 0,
+                                             blocked.block_rows, self._stream()))
         return out
+
+    def _in_blocks_of(self, x, block_rows):
+        """`x` (rows or `BlockedRows`) in blocks of `block_rows` rows (0: as rows), regrouped if it lies otherwise."""
+        if _block_rows(x) == block_rows:
+            return x
+        rows = self.from_blocked(x) if isinstance(x, BlockedRows) else x
+        return self.to_blocked(rows, block_rows=block_rows) if block_rows else rows
 
     def pack_weight(self, w):
         """The form of a weight matrix that the matrix products read fastest: a `PackedWeight` for a
@@ -246,7 +268,6 @@ class HipKernels:
         fast = self.lib.bh_gemm_bf16
         packed = isinstance(w, PackedWeight)
         ahead = a if isinstance(a, NormedRows) else None
-        a_blocked, c_blocked = isinstance(a, BlockedRows), isinstance(out, BlockedRows)
         if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or a.shape[1] % 8:
             if packed:
                 raise KernelError("gemm: a packed weight needs bfloat16 activations")
@@ -256,8 +277,17 @@ class HipKernels:
         m, k = a.shape
         n = out.shape[1]
         sizes = (m, n, k, int(packed), int(activation))
-        if (a_blocked or c_blocked) and not self.lib.bh_gemm_bf16_reads_blocked(*sizes):
-            raise KernelError(f"gemm: a product of {m} x {n} x {k} neither reads nor writes rows in blocks")
+        # the activations in the form this product reads: whoever produced them for this reader wrote them so
+        a_block_rows = int(self.lib.bh_gemm_bf16_reads_blocked(*sizes))
+        if ahead is not None:
+            if _block_rows(ahead.rows) != a_block_rows:
+                ahead = NormedRows(self._in_blocks_of(ahead.rows, a_block_rows), ahead.ss, ahead.eps, ahead.source, ahead.weight)
+        else:
+            a = self._in_blocks_of(a, a_block_rows)
+        writes = int(self.lib.bh_gemm_bf16_writes_blocked(*sizes))     # 2: any blocks, 1: SwiGLU's in blocks of 16, 0: rows
+        c_block_rows = _block_rows(out)
+        if c_block_rows and not (activation and (writes == 2 or (writes == 1 and c_block_rows == 16))):
+            return False, None      # the caller regroups
         if ahead is not None and (ahead.ss.shape[0] != m or ahead.ss.dtype != torch.float32
                                   or not self.lib.bh_gemm_bf16_takes_norm(*sizes)):
             raise KernelError(f"gemm: a product of {m} x {n} x {k} does not take these prepared norm rows")
@@ -265,13 +295,14 @@ class HipKernels:
                 and not activation and then_norm.weight.shape == (n,) and then_norm.weight.dtype in _CODES
                 and self.lib.bh_gemm_bf16_finishes_norm(m, n, k, 1)):
             # many rows, K in parts: the finishing kernel owns whole rows and finishes the norm itself
-            reader = getattr(then_norm, "reader", None)
-            normed = self.new_rows(m, n, torch.bfloat16, *((reader.outputs, reader.swiglu) if reader is not None else ()))
+            normed = self.new_rows(m, n, torch.bfloat16, *self._reader_of(then_norm))
+            if _block_rows(normed) not in (0, 16):
+                normed = torch.empty((m, n), dtype=torch.bfloat16, device=self.device)
             scratch = torch.empty(int(self.lib.bh_gemm_bf16_scratch(*sizes)) // 4, dtype=torch.float32, device=self.device)
             self._check(self.lib.bh_gemm_bf16_then_norm(
                 self._ptr(a, "gemm a"), self._ptr(w.data, "gemm w"), self._ptr(out, "gemm out", (torch.float32,)), m, n, k, 1,
                 self._ptr(then_norm.weight, "norm weight"), _code(then_norm.weight, "norm weight"), float(then_norm.eps),
-                self._ptr(normed, "norm rows"), self._ptr(scratch, "gemm scratch"), int(a_blocked),
+                self._ptr(normed, "norm rows"), self._ptr(scratch, "gemm scratch"), int(a_block_rows == 16),
                 int(isinstance(normed, BlockedRows)), self._stream()))
             return True, normed
         behind = None
@@ -279,8 +310,9 @@ class HipKernels:
                 and then_norm.weight.shape == (n,) and then_norm.weight.dtype in _CODES):
             blocks = int(self.lib.bh_gemm_bf16_norm_blocks(*sizes))      # 0: this product carries no norm
             if blocks:
-                behind = NormedRows(torch.empty((m, n), dtype=torch.bfloat16, device=self.device),
-                                    torch.empty((m, blocks), dtype=torch.float32, device=self.device), then_norm.eps,
+                rows = self.new_rows(m, n, torch.bfloat16, *self._reader_of(then_norm)) if writes == 2 else \
+                    torch.empty((m, n), dtype=torch.bfloat16, device=self.device)
+                behind = NormedRows(rows, torch.empty((m, blocks), dtype=torch.float32, device=self.device), then_norm.eps,
                                     out, then_norm.weight)
         a_rows = ahead.rows if ahead is not None else a
         scratch = None       # products of few tiles add up parts of K through scratch memory
@@ -296,8 +328,15 @@ class HipKernels:
             _code(then_norm.weight, "norm weight") if behind is not None else 0,
             self._ptr(behind.rows, "norm rows") if behind is not None else None,
             self._ptr(behind.ss, "norm sums") if behind is not None else None,
-            self._ptr(scratch, "gemm scratch", None, True), int(a_blocked), int(c_blocked), self._stream()))
+            self._ptr(scratch, "gemm scratch", None, True), a_block_rows, c_block_rows,
+            _block_rows(behind.rows) if behind is not None else 0, self._stream()))
         return True, behind
+
+    @staticmethod
+    def _reader_of(then_norm):
+        """The arguments of `new_rows` that name the product reading a norm's output, if the request names one."""
+        reader = getattr(then_norm, "reader", None)
+        return (reader.outputs, reader.swiglu) if reader is not None else ()
 
     def gemm(self, a, w, out, accumulate=False, then_norm=None):
         """out[M, N] (+)= a[M, K] @ w[N, K]^T with float32 accumulation; `w` may be a PackedWeight and
@@ -317,7 +356,7 @@ class HipKernels:
         if done:
             return prepared
         if isinstance(a, BlockedRows):
-            raise KernelError("gemm: only the matrix-core product of many rows reads rows in blocks")
+            a = self.from_blocked(a)
         self._check(self.lib.bh_gemm_generic(
             self._ptr(a, "gemm a"), _code(a, "gemm a"), self._ptr(w, "gemm w"), _code(w, "gemm w"),
             self._ptr(out, "gemm out"), _code(out, "gemm out"), int(bool(accumulate)), m, n, k, self._stream()))
@@ -327,16 +366,17 @@ class HipKernels:
         """The product for many rows whose wave groups take turns, at a given tile width (`blocks` of 16
         weight rows per wave: 8, 6 or 4), whatever `gemm` would choose for these sizes: out[M, N] (+)= a @ w^T,
         or with `swiglu` out[M, F] = silu(a @ w[:F]^T) * (a @ w[F:]^T).  `w` is a PackedWeight."""
-        if not isinstance(w, PackedWeight) or a.dim() != 2 or out.dim() != 2 or a.dtype != torch.bfloat16:
-            raise KernelError("gemm_turns: bfloat16 activations [M, K] (rows or `BlockedRows`) and a packed weight")
+        if (not isinstance(w, PackedWeight) or a.dim() != 2 or out.dim() != 2 or a.dtype != torch.bfloat16
+                or _block_rows(a) not in (0, 16) or _block_rows(out) not in (0, 16)):
+            raise KernelError("gemm_turns: bfloat16 activations [M, K] (rows or `BlockedRows` of 16) and a packed weight")
         m, k = a.shape
         n = out.shape[1]
         if w.shape[1] != k or w.shape[0] != (2 * n if swiglu else n) or out.shape[0] != m:
             raise KernelError(f"gemm_turns: shapes a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
         self._check(self.lib.bh_gemm_bf16_turns(
             self._ptr(a, "gemm a"), self._ptr(w.data, "gemm w"), self._ptr(out, "gemm out"), _code(out, "gemm out"),
-            int(bool(accumulate)), m, n, k, int(bool(swiglu)), int(blocks), int(isinstance(a, BlockedRows)),
-            int(isinstance(out, BlockedRows)), self._stream()))
+            int(bool(accumulate)), m, n, k, int(bool(swiglu)), int(blocks), int(_block_rows(a) == 16),
+            int(_block_rows(out) == 16), self._stream()))
 
     def gemm_turns_blocks(self, m, n, k, swiglu=False):
         """The tile width `gemm` uses for a packed product of these sizes (0: another kernel runs it)."""
@@ -366,16 +406,15 @@ class HipKernels:
                               "do not fit")
         if isinstance(a, NormedRows) and width % 16 == 0 and not self._takes_norm(a, w, width, 1):
             a = self._run_norm(a)
-        if isinstance(out, BlockedRows) and not (isinstance(w, PackedWeight) and a.dtype == torch.bfloat16 and
-                                                 self.lib.bh_gemm_bf16_turns_blocks(m, width, k, 1, 1)):
-            rows_out = torch.empty((m, width), dtype=out.dtype, device=self.device)   # this product writes rows
+        if self._gemm_fast(a, w, out, False, 1)[0]:
+            return
+        if isinstance(out, BlockedRows):      # this product writes rows, or not these blocks: regroup them afterwards
+            rows_out = torch.empty((m, width), dtype=out.dtype, device=self.device)
             self.gemm_swiglu(a, w, rows_out)
             self.to_blocked(rows_out, out)
             return
-        if self._gemm_fast(a, w, out, False, 1)[0]:
-            return
-        if isinstance(a, BlockedRows) or isinstance(out, BlockedRows):
-            raise KernelError("gemm_swiglu: only the matrix-core product of many rows reads or writes rows in blocks")
+        if isinstance(a, BlockedRows):
+            a = self.from_blocked(a)
         both = torch.empty((m, 2 * width), dtype=a.dtype, device=self.device)
         self.gemm(a, w, both)
         self.swiglu(both, out)
@@ -444,10 +483,11 @@ class HipKernels:
         n_rows = q.shape[0]
         if q.shape != (n_rows, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape) or out.dtype != q.dtype:
             raise KernelError(f"attention: shapes q {tuple(q.shape)}, out {tuple(out.shape)} do not fit")
+        # the matrix-core kernels write blocks themselves: of 16 rows in steps of many columns, of 8 or 16 otherwise
         if isinstance(out, BlockedRows) and not (
                 q.dtype == torch.bfloat16 and layout is not None and head_dim % 32 == 0 and head_dim <= 256
-                and self.lib.bh_attention_bf16_writes_blocked(int(layout.n_seqs), int(layout.max_rows_per_seq), n_heads,
-                                                              n_kv_heads, int(layout.max_position))):
+                and (out.block_rows == 16 or not self.lib.bh_attention_bf16_writes_blocked(
+                    int(layout.n_seqs), int(layout.max_rows_per_seq), n_heads, n_kv_heads, int(layout.max_position)))):
             rows_out = torch.empty(tuple(q.shape), dtype=q.dtype, device=self.device)   # this step's kernel writes rows
             self.attention(q, rows_out, k_pages, v_pages, page_table, row_seq, positions, n_heads, n_kv_heads, head_dim,
                            scale, window, layout)
@@ -478,7 +518,7 @@ class HipKernels:
                              page_table.shape[1], self._ptr(positions, "positions", (torch.int32,)),
                              self._ptr(layout.seq_start, "seq_start", (torch.int32,)), n_seqs, n_rows, max_rows,
                              n_heads, n_kv_heads, head_dim, float(scale), int(window), int(layout.max_position),
-                             n_splits, int(isinstance(out, BlockedRows)), self._stream()))
+                             n_splits, _block_rows(out), self._stream()))
             return
         self._check(self.lib.bh_attention_generic(
             *common, _code(q, "q"), self._ptr(k_pages, "k_pages"), self._ptr(v_pages, "v_pages"),
@@ -490,8 +530,9 @@ class HipKernels:
     def attention_decode_fused(self, qkv, out, q_weight, k_weight, eps, cos, sin, positions, k_pages, v_pages,
                                page_table, n_heads, n_kv_heads, head_dim, scale, window, write_kv, layout):
         """`qk_norm_rope_cache` and `attention` in one launch for a step of one row per sequence, from
-        the fused projection rows `qkv` [n, (heads + 2 kv_heads) * head_dim].  Returns False, having done
-        nothing, where the one kernel that does it does not take the operands (then call the two)."""
+        the fused projection rows `qkv` [n, (heads + 2 kv_heads) * head_dim]; `out` may be `BlockedRows`.
+        Returns False, having done nothing, where the one kernel that does it does not take the operands
+        (then call the two)."""
         n_rows = qkv.shape[0]
         rot = 2 * cos.shape[1] if cos is not None else 0
         if (qkv.dtype != torch.bfloat16 or k_pages.dtype != torch.bfloat16 or layout is None
@@ -500,7 +541,7 @@ class HipKernels:
                 or (cos is not None and (rot != head_dim or head_dim % 64))
                 or self.kv_order(k_pages.dtype, head_dim) != 1):
             return False
-        if qkv.shape != (n_rows, (n_heads + 2 * n_kv_heads) * head_dim) or out.shape != (n_rows, n_heads * head_dim) \
+        if qkv.shape != (n_rows, (n_heads + 2 * n_kv_heads) * head_dim) or tuple(out.shape) != (n_rows, n_heads * head_dim) \
                 or out.dtype != qkv.dtype:
             raise KernelError(f"attention_decode_fused: shapes qkv {tuple(qkv.shape)}, out {tuple(out.shape)} do not fit "
                               f"{n_heads}+2x{n_kv_heads} heads of {head_dim}")
@@ -529,7 +570,7 @@ class HipKernels:
             n_rows, n_heads, n_kv_heads, head_dim, float(scale), int(window), int(layout.max_position), n_splits,
             self._ptr(q_weight, "q_norm", None, True), self._ptr(k_weight, "k_norm", None, True), w_code, float(eps),
             self._ptr(cos, "cos", (torch.float32,), True), self._ptr(sin, "sin", (torch.float32,), True),
-            cos.shape[0] if cos is not None else 0, rot, int(bool(write_kv)), self._stream()))
+            cos.shape[0] if cos is not None else 0, rot, int(bool(write_kv)), _block_rows(out), self._stream()))
         return True
 
     def stream_read(self, data, workgroups=256, nontemporal=True) -> int:

@@ -86,7 +86,10 @@ class DecoderModel:
             prepared = self.blocks[layer].forward(ctx, hidden, cache_for_run(run), prepared, following)
         if want_rows is None or want_rows.numel() == 0:
             return None
-        return self.head.forward(ctx, self.final_norm.forward(ctx, hidden, rows=want_rows))
+        reader = getattr(self.head, "input_reader", None) if getattr(self.final_norm, "serves_reader", False) else None
+        normed = (self.final_norm.forward(ctx, hidden, rows=want_rows, reader=reader) if reader is not None
+                  else self.final_norm.forward(ctx, hidden, rows=want_rows))
+        return self.head.forward(ctx, normed)
 
 
 def build_decoder(config, position_encoding="rope", layer_prefix: str = "model.layers.{}.",

@@ -73,15 +73,14 @@ class GQAAttention:
         k = ctx.kernels
         qkv = self.qkv.forward(ctx, x)
         cos, sin = self.position_encoding.tables() if self.position_encoding is not None else (None, None)
+        attended = ctx.new_activations(ctx.n_rows, self.n_heads * self.head_dim, reader=self.out.reader())
         # a decode step: norm, rotation, cache write and attention in one launch where the kernels offer it
         one_launch = getattr(k, "attention_decode_fused", None)
-        if ctx.is_decode and one_launch is not None:
-            attended = ctx.new_activations(ctx.n_rows, self.n_heads * self.head_dim)
-            if one_launch(qkv, attended, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0, cos, sin, ctx.positions,
-                          cache.k_pages, cache.v_pages, cache.page_table, self.n_heads, self.n_kv_heads, self.head_dim,
-                          self.scale, self.window, cache.writes, ctx):
-                return self.out.add_into(ctx, attended, hidden, then_norm)
-        attended = ctx.new_activations(ctx.n_rows, self.n_heads * self.head_dim, reader=self.out.reader())
+        if ctx.is_decode and one_launch is not None and one_launch(
+                qkv, attended, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0, cos, sin, ctx.positions,
+                cache.k_pages, cache.v_pages, cache.page_table, self.n_heads, self.n_kv_heads, self.head_dim,
+                self.scale, self.window, cache.writes, ctx):
+            return self.out.add_into(ctx, attended, hidden, then_norm)
         q = ctx.new_activations(ctx.n_rows, self.n_heads * self.head_dim)
         k.qk_norm_rope_cache(qkv, q, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0, cos, sin,
                              ctx.positions, ctx.row_seq, cache.k_pages, cache.v_pages, cache.page_table,

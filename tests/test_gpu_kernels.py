@@ -294,22 +294,24 @@ def test_gemm_whose_wave_groups_take_turns(K, blocks, m, n, k):
         assert rel(act, want_act) < 6e-3, rel(act, want_act)
 
 
-def blocked_reference(x):
-    """x [rows, width] in blocks of 16 rows x 32 columns, each block as [4 groups of 8 columns][16 rows][8], the
-    blocks of 16 rows one after the other along the width; rows that x lacks are zero."""
+def blocked_reference(x, block_rows=16):
+    """x [rows, width] in blocks of 16 (or 8) rows x 32 columns, each block as [4 groups of 8 columns][rows][8],
+    the blocks of a group of rows one after the other along the width; rows that x lacks are zero."""
     rows, width = x.shape
-    padded = -(-rows // 16) * 16
+    padded = -(-rows // block_rows) * block_rows
     full = torch.zeros(padded, width, dtype=x.dtype)
     full[:rows] = x
-    return full.view(padded // 16, 16, width // 32, 4, 8).permute(0, 2, 3, 1, 4).reshape(-1)
+    return full.view(padded // block_rows, block_rows, width // 32, 4, 8).permute(0, 2, 3, 1, 4).reshape(-1)
 
 
-@pytest.mark.parametrize("rows,width", [(1, 32), (16, 64), (300, 96), (257, 4096), (1000, 160)])
-def test_rows_into_blocks_and_back(K, rows, width):
+@pytest.mark.parametrize("block_rows", [16, 8])
+@pytest.mark.parametrize("rows,width", [(1, 32), (16, 64), (300, 96), (257, 4096), (1000, 160), (5, 4096), (40, 128)])
+def test_rows_into_blocks_and_back(K, rows, width, block_rows):
     x = torch.randn(rows, width, generator=torch.Generator().manual_seed(rows)).to(torch.bfloat16)
-    blocked = K.to_blocked(dev(x))
-    assert tuple(blocked.shape) == (rows, width) and blocked.data.numel() % (256 * width) == 0
-    want = blocked_reference(x)
+    blocked = K.to_blocked(dev(x), block_rows=block_rows)
+    assert tuple(blocked.shape) == (rows, width) and blocked.block_rows == block_rows
+    assert blocked.data.numel() == (-(-rows // 256) * 256 if rows > 32 else -(-rows // block_rows) * block_rows) * width
+    want = blocked_reference(x, block_rows)
     assert torch.equal(blocked.data[:want.numel()].cpu(), want)
     assert torch.equal(K.from_blocked(blocked).cpu(), x)
     from beholdd.kernels import KernelError
@@ -345,6 +347,57 @@ def test_gemm_with_turns_reads_and_writes_rows_in_blocks(K, blocks, m, n, k):
             out = BlockedRows(torch.full((-(-m // 256) * 256 * n,), float("nan"), dtype=torch.bfloat16, device="cuda:0"), m, n)
             K.gemm_turns(source, both, out, blocks, swiglu=True)
             assert torch.equal(K.from_blocked(out), rows_out)
+
+
+@pytest.mark.parametrize("g_dtype", DTYPES)
+@pytest.mark.parametrize("m", [1, 2, 3, 8, 9, 16, 17, 32, 33, 48, 64])
+def test_products_of_few_rows_hand_each_other_blocks(K, m, g_dtype):
+    """A layer's feed-forward and the norms around it as a decode step of m sequences runs them: the norm writes
+    its rows for the gated product, that one its output for the down product, which adds into the residual and
+    prepares the next norm for the product after it.  From 3 to 32 rows every matrix on the way lies in blocks (of
+    8 rows up to 8, of 16 beyond), as `new_rows` hands them out for their readers; the numbers are those of float64
+    within bfloat16's rounding, and matrices handed over as plain rows give the same bits (they are regrouped)."""
+    from beholdd.kernels.library import BlockedRows, NormedRows
+    from beholdd.parts.base import NormRequest, ProductReader
+    hidden, inter = 1024, 1536
+    g = torch.Generator().manual_seed(m)
+    residual = torch.randn(m, hidden, generator=g)
+    w_gate_up = (torch.randn(2 * inter, hidden, generator=g) * 0.05).to(torch.bfloat16)
+    w_down = (torch.randn(hidden, inter, generator=g) * 0.05).to(torch.bfloat16)
+    g1 = (1 + 0.3 * torch.randn(hidden, generator=g)).to(g_dtype)
+    g2 = (1 + 0.3 * torch.randn(hidden, generator=g)).to(g_dtype)
+    gate_up, down = K.pack_weight(dev(w_gate_up)), K.pack_weight(dev(w_down))
+    eps = 1e-5
+
+    def chain(readers):
+        h = dev(residual.clone())
+        reader = lambda outputs, swiglu=False: (outputs, swiglu) if readers else ()
+        x = K.new_rows(m, hidden, torch.bfloat16, *reader(inter, True))
+        K.rmsnorm(h, dev(g1), eps, x)
+        act = K.new_rows(m, inter, torch.bfloat16, *reader(hidden))
+        K.gemm_swiglu(x, gate_up, act)
+        prepared = K.gemm(act, down, h, accumulate=True,
+                          then_norm=NormRequest(dev(g2), eps, ProductReader(inter, True) if readers else None))
+        assert isinstance(prepared, NormedRows)          # up to 256 rows the norm rides on the products around it
+        again = torch.empty(m, inter, dtype=torch.bfloat16, device="cuda:0")
+        K.gemm_swiglu(prepared, gate_up, again)
+        return h, again, [x, act, prepared.rows]
+
+    h_rows, again_rows, kinds_rows = chain(False)
+    h_blocks, again_blocks, kinds_blocks = chain(True)
+    assert not any(isinstance(t, BlockedRows) for t in kinds_rows)
+    want_blocks = 0 if m <= 2 or m > 32 else 8 if m <= 8 else 16
+    assert [t.block_rows if isinstance(t, BlockedRows) else 0 for t in kinds_blocks] == [want_blocks] * 3
+    assert torch.equal(h_rows, h_blocks) and torch.equal(again_rows, again_blocks)
+    on = lambda t: t.double().to("cuda:0")
+    norm = lambda t, w: t / torch.sqrt((t ** 2).mean(-1, keepdim=True) + eps) * on(w)
+    x64 = norm(on(residual), g1).to(torch.bfloat16).double()
+    both = x64 @ on(w_gate_up).t()
+    act64 = (both[:, :inter] / (1 + torch.exp(-both[:, :inter])) * both[:, inter:]).to(torch.bfloat16).double()
+    h64 = on(residual) + act64 @ on(w_down).t()
+    assert rel(h_blocks, h64.cpu()) < 3e-3
+    both = norm(h64, g2) @ on(w_gate_up).t()
+    assert rel(again_blocks, (both[:, :inter] / (1 + torch.exp(-both[:, :inter])) * both[:, inter:]).cpu()) < 2e-2
 
 
 @pytest.mark.parametrize("m", [300, 1000, 2048])
@@ -735,6 +788,18 @@ def test_decode_attention_from_the_projection_rows(K, n_heads, kv_heads, head_di
     assert (k_one.cpu() != k_two.cpu()).float().mean() < 1e-3
     if not write_kv:
         assert torch.equal(k_one.cpu(), stored(K, kp, vp)[0].cpu())
+    from beholdd.kernels.library import BlockedRows      # the same output in blocks of 8 and of 16 rows
+    width = n_heads * head_dim
+    for block_rows in (8, 16):
+        k_b, v_b = stored(K, kp, vp)
+        blocked = BlockedRows(torch.full((16 * width,), float("nan"), dtype=dtype, device="cuda:0"), n, width, block_rows)
+        assert K.attention_decode_fused(dev(qkv), blocked, qw, kw, eps, cos, sin, positions, k_b, v_b, dev(table),
+                                        n_heads, kv_heads, head_dim, scale, window, write_kv, layout) is True
+        assert torch.equal(K.from_blocked(blocked), out_one)
+        # and from finished queries, by the kernels for few columns (a step of seven rows here)
+        K.attention(q, blocked, k_two, v_two, dev(table), row_seq, positions, n_heads, kv_heads, head_dim, scale, window,
+                    layout=layout)
+        assert torch.equal(K.from_blocked(blocked), out_two)
 
 
 def test_decode_attention_from_the_projection_rows_of_many_sequences(K):
