@@ -60,6 +60,15 @@ __device__ inline void store_out<bf16_t>(bf16_t* c, size_t at, float v, bool acc
 
 __device__ inline float silu_mul(float gate, float up) { return gate / (1.0f + expf(-gate)) * up; }
 
+// every lane's value of the lane eight further on in its group of 16 (lanes 8 to 15: nothing that matters)
+__device__ inline u32x4_t from_lane_plus_8(u32x4_t v) {
+  u32x4_t out;
+#pragma unroll
+  for (int word = 0; word < 4; ++word)
+    out[word] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v[word], 0x108 /* row_shl:8 */, 0xf, 0xf, true);
+  return out;
+}
+
 #define MFMA16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(b), c, 0, 0, 0)
 
 // ---- skinny --------------------------------------------------------------------------------
@@ -151,7 +160,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
   for (int b = 0; b < MB; ++b) {
     if (XB) {   // piece p = 2 g + u of a chunk is lane group p % 4 of its step p / 4
       constexpr int step = 32 * (XB ? XB : 1);
-      xp[b] = a + (size_t)(b * 16 / (XB ? XB : 1)) * (K / 32) * step + (g / 2) * step + ((2 * g) % 4 * XB + i % (XB ? XB : 1)) * 8;
+      // (blocks of 8 rows: lanes 8 to 15 of a group take the second piece of rows 0 to 7, which lies right behind
+      // the first pieces, so that one load brings both and a lane move hands the second to the lane of its row)
+      xp[b] = a + (size_t)(b * 16 / (XB ? XB : 1)) * (K / 32) * step + (g / 2) * step + ((2 * g) % 4 * XB + (XB == 8 ? i : i % (XB ? XB : 1))) * 8;
     } else {
       const int row = (b * 16 + i < M) ? b * 16 + i : M - 1;
       xp[b] = a + (size_t)row * K + g * 16;
@@ -180,7 +191,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
 #pragma unroll
       for (int b = 0; b < MB; ++b) {
         xv[u][b][0] = load16(xp[b] + at * x_chunk);
-        xv[u][b][1] = load16(xp[b] + at * x_chunk + x_half);
+        if (XB != 8) xv[u][b][1] = load16(xp[b] + at * x_chunk + x_half);
       }
     }
 #pragma unroll
@@ -189,6 +200,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
       for (int t = 0; t < RT; ++t)
 #pragma unroll
         for (int b = 0; b < MB; ++b) {
+          if (XB == 8 && t == 0) xv[u][b][1] = from_lane_plus_8(xv[u][b][0]);
           acc[t][b] = MFMA16(wv[u][t][0], xv[u][b][0], acc[t][b]);
           acc[t][b] = MFMA16(wv[u][t][1], xv[u][b][1], acc[t][b]);
         }
@@ -200,7 +212,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
       const u32x4_t w0 = load16(p), w1 = load16(p + half_offset);
 #pragma unroll
       for (int b = 0; b < MB; ++b) {
-        const u32x4_t x0 = load16(xp[b] + chunk * x_chunk), x1 = load16(xp[b] + chunk * x_chunk + x_half);
+        const u32x4_t x0 = load16(xp[b] + chunk * x_chunk);
+        const u32x4_t x1 = XB == 8 ? from_lane_plus_8(x0) : load16(xp[b] + chunk * x_chunk + x_half);
         acc[t][b] = MFMA16(w0, x0, acc[t][b]);
         acc[t][b] = MFMA16(w1, x1, acc[t][b]);
       }
