@@ -208,6 +208,7 @@ int bhp_argmax(const float* logits, int32_t* tokens, int32_t* bad, int n_rows, i
 int bhp_page_size() { return BH_PAGE; }
 int bhp_key_index(int order, int token, int dim, int hd) { return bh_key_index(order, token, dim, hd); }
 int bhp_value_index(int order, int token, int dim, int hd) { return bh_value_index(order, token, dim, hd); }
+long bhp_rows_index(int block_rows, int row, int column, int width) { return bh_rows_index(block_rows, row, column, width); }
 
 }  // extern "C"
 
@@ -238,6 +239,20 @@ int main() {
           seen_v[v]++;
         }
       for (int i = 0; i < BH_PAGE * hd; ++i) EXPECT(seen_k[i] == 1 && seen_v[i] == 1);
+    }
+  // every element of a matrix whose rows lie in blocks of 8 or 16 has a place of its own within the whole blocks
+  for (int block_rows = 8; block_rows <= 16; block_rows += 8)
+    for (int rows = 1; rows <= 40; rows += 13) {
+      const int width = 96, padded = (rows + block_rows - 1) / block_rows * block_rows;
+      std::vector<int> seen(padded * width, 0);
+      for (int row = 0; row < rows; ++row)
+        for (int column = 0; column < width; ++column) {
+          const long at = bh_rows_index(block_rows, row, column, width);
+          EXPECT(at >= 0 && at < (long)padded * width);
+          seen[at]++;
+          EXPECT(bh_rows_index(0, row, column, width) == (long)row * width + column);
+        }
+      for (int i = 0; i < padded * width; ++i) EXPECT(seen[i] <= 1);
     }
   // bfloat16: widening is exact, narrowing rounds to nearest even (crates/beholdd-core/src/quant.rs:486-502)
   EXPECT(bf16_bits_to_f32(0x3F80) == 1.0f && bf16_bits_to_f32(0xC000) == -2.0f);

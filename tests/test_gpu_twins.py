@@ -39,6 +39,24 @@ def rel(got, want):
     return float(np.abs(got.astype(np.float64) - want).max() / max(np.abs(want).max(), 1e-30))
 
 
+@pytest.mark.parametrize("block_rows,rows", [(8, 5), (8, 8), (16, 16), (16, 21), (16, 300)])
+def test_rows_in_blocks_lie_where_the_twin_says(K, twins, block_rows, rows):
+    """The regrouping kernel and the norm that writes blocks itself put every element where the index function
+    that host and device code share says."""
+    width = 96
+    x = RNG.normal(size=(rows, width)).astype(np.float32)
+    index = twins.rows_index(block_rows, rows, width)
+    blocked = K.to_blocked(dev(x, torch.bfloat16), block_rows=block_rows)
+    assert np.array_equal(host(blocked.data)[index], host(dev(x, torch.bfloat16)))
+    from beholdd.kernels.library import BlockedRows
+    normed = BlockedRows(torch.zeros_like(blocked.data), rows, width, block_rows)
+    weight = RNG.normal(size=width).astype(np.float32)
+    K.rmsnorm(dev(x), dev(weight), 1e-5, normed)
+    as_rows = torch.empty(rows, width, dtype=torch.bfloat16, device=DEVICE)
+    K.rmsnorm(dev(x), dev(weight), 1e-5, as_rows)
+    assert np.array_equal(host(normed.data)[index], host(as_rows))
+
+
 def test_embed_rmsnorm_swiglu_argmax_and_their_twins(K, twins):
     table = RNG.normal(size=(331, 96)).astype(np.float32)
     tokens = RNG.integers(0, 331, size=37).astype(np.int32)

@@ -99,3 +99,20 @@ def test_cache_write_and_attention_twins_are_the_plain_functions(twins, order, h
                                       query_start=past)
         assert np.allclose(got[at:at + new], want, rtol=2e-5, atol=2e-6), s
         at += new
+
+
+@pytest.mark.parametrize("block_rows", [8, 16])
+def test_rows_in_blocks_are_a_permutation_in_operand_order(twins, block_rows):
+    """Every element of a matrix whose rows lie in blocks has a place of its own within the whole blocks; a block is
+    32 columns of `block_rows` rows, and inside it eight columns of a row lie together, the rows of those eight
+    columns one after the other, then the next eight columns: what one matrix-core operand load takes."""
+    rows, width = 2 * block_rows + 3, 96
+    index = twins.rows_index(block_rows, rows, width)
+    padded = -(-rows // block_rows) * block_rows
+    assert len(set(index.ravel().tolist())) == rows * width and index.min() == 0 and index.max() < padded * width
+    assert np.array_equal(twins.rows_index(0, rows, width), np.arange(rows * width).reshape(rows, width))
+    for r in (0, 1, block_rows - 1, block_rows, rows - 1):
+        for c in (0, 7, 8, 31, 32, 95):
+            block = (r // block_rows) * (width // 32) + c // 32
+            want = block * 32 * block_rows + (((c % 32) // 8) * block_rows + r % block_rows) * 8 + c % 8
+            assert index[r, c] == want

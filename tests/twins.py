@@ -116,6 +116,11 @@ class Twins:
         assert self.lib.bhp_argmax(self._p(logits), self._p(tokens), self._p(bad), logits.shape[0], logits.shape[1]) == 0
         return tokens, bad
 
+    def rows_index(self, block_rows, rows, width):
+        """Where each element of a [rows, width] matrix lies when its rows are in blocks of `block_rows`."""
+        self.lib.bhp_rows_index.restype = ctypes.c_long
+        return np.array([[self.lib.bhp_rows_index(block_rows, r, c, width) for c in range(width)] for r in range(rows)])
+
     def key(self, k_pages, order, page, kv_head, token, head_dim, code=F32):
         """The key vector [head_dim] that lies at (page, kv_head, token)."""
         index = [self.lib.bhp_key_index(order, token, d, head_dim) for d in range(head_dim)]
