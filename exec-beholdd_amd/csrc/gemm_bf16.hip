@@ -102,8 +102,9 @@ struct RidingNorm {
 // Measured (Qwen3-8B sizes, us per product, qkv / o / gate+up / down): 8 rows 12.7 / 9.2 / 34.1 / 21.0 -> 11.4 /
 // 8.6 / 33.7 / 19.9; 16 rows 15.3 / 10.4 / 35.9 / 24.2 -> 12.4 / 8.9 / 33.1 / 20.4; 32 rows (tiles with K in
 // parts before) 16.2 / 12.6 / 49.4 / 26.4 -> 14.9 / 10.0 / 40.5 / 23.1; 48 rows 18.2 / 14.3 / 50.1 / 28.7 -> 18.6 /
-// 11.8 / 46.0 / 28.4; at 64 rows the tiles are as fast, and a single row is read fastest as it lies.  (Each product
-// alone; inside a decode step 48 rows did not gain, see SKINNY_UP_TO_ROWS.)
+// 11.8 / 46.0 / 28.4; at 64 rows the tiles are as fast.  (Each product alone; inside a decode step 48 rows did not
+// gain, see SKINNY_UP_TO_ROWS, and a single row, which alone is read as fast as it lies (10.9 / 8.4 / 33.7 / 19.6
+// against 11.2 / 8.6 / 33.8 / 19.9), did: the step of one sequence 3.61 -> 3.55 ms, of two 3.79 -> 3.71.)
 struct RowBlocks {
   int a, c, behind;
 };
@@ -961,8 +962,8 @@ static TiledConfig tiled_config(int M, int N, bool swiglu, int* rows, int* colum
   *columns = (big ? 256 : 128) / (swiglu ? 2 : 1);
   return big ? TILED_256 : tiles_128 > 512 && tiles_128 <= 1024 ? TILED_128_ONE_BUFFER : TILED_128;
 }
-// Up to how many rows the skinny kernel takes a product of packed weights (it reads its activations in blocks
-// from three rows on, see struct RowBlocks); without packed weights, or where the tiles do not fit, up to 64.
+// Up to how many rows the skinny kernel takes a product of packed weights (it reads its activations in blocks,
+// see struct RowBlocks); without packed weights, or where the tiles do not fit, up to 64.
 // Decode steps of the Qwen3-8B sizes at context 8,192, against tiles with K in parts from 17 rows on: 16
 // sequences 6.88 -> 6.64 ms, 32 sequences 10.38 -> 9.93 ms, 48 sequences 14.24 -> 14.43 ms (so not those).
 #define SKINNY_UP_TO_ROWS 32
@@ -1067,11 +1068,11 @@ extern "C" int bh_gemm_bf16_takes_norm(int M, int N, int K, int layout, int acti
 
 // The rows per block (16 or 8) if a product of these sizes reads its activations faster from blocks of that
 // many rows x 32 columns (bh_rows_index, layout.h) and takes them that way, else 0: the products of the kernel
-// whose wave groups take turns (16), and those of 3 to 32 rows of the skinny kernel (8 up to 8 rows, else 16).
+// whose wave groups take turns (16), and those of up to 32 rows of the skinny kernel (8 up to 8 rows, else 16).
 extern "C" int bh_gemm_bf16_reads_blocked(int M, int N, int K, int layout, int activation) {
   if (M <= 0 || N <= 0 || K <= 0 || K % 32 != 0) return 0;
   if (gemm_turns_blocks(M, N, K, layout, activation) || gemm_turns_parts(M, N, K, layout, activation) > 1) return 16;
-  if (M >= 3 && skinny_first(M, N, K, layout)) return M <= 8 ? 8 : 16;
+  if (skinny_first(M, N, K, layout)) return M <= 8 ? 8 : 16;
   return 0;
 }
 

@@ -57,7 +57,7 @@ class NormedRows:
 class BlockedRows:
     """A bfloat16 activation matrix [rows, width] kept in blocks of `block_rows` (16 or 8) rows x 32 columns, each
     block in the order in which a matrix-core operand lies in a wave's lanes (`bh_rows_index` in csrc/layout.h):
-    what the products of many rows and those of 3 to 32 rows read fastest.  `HipKernels.new_rows` hands one out
+    what the products of many rows and those of up to 32 rows read fastest.  `HipKernels.new_rows` hands one out
     where the product named as the matrix's reader takes it; the kernels that produce activations (`rmsnorm`,
     `gemm_swiglu`, `attention`, a `gemm` that prepares or finishes a norm) write into it, and `gemm` /
     `gemm_swiglu` read it.  `data` holds whole blocks (for more than 32 rows whole tiles of 256 rows); rows the

@@ -354,7 +354,7 @@ def test_gemm_with_turns_reads_and_writes_rows_in_blocks(K, blocks, m, n, k):
 def test_products_of_few_rows_hand_each_other_blocks(K, m, g_dtype):
     """A layer's feed-forward and the norms around it as a decode step of m sequences runs them: the norm writes
     its rows for the gated product, that one its output for the down product, which adds into the residual and
-    prepares the next norm for the product after it.  From 3 to 32 rows every matrix on the way lies in blocks (of
+    prepares the next norm for the product after it.  Up to 32 rows every matrix on the way lies in blocks (of
     8 rows up to 8, of 16 beyond), as `new_rows` hands them out for their readers; the numbers are those of float64
     within bfloat16's rounding, and matrices handed over as plain rows give the same bits (they are regrouped)."""
     from beholdd.kernels.library import BlockedRows, NormedRows
@@ -386,7 +386,7 @@ def test_products_of_few_rows_hand_each_other_blocks(K, m, g_dtype):
     h_rows, again_rows, kinds_rows = chain(False)
     h_blocks, again_blocks, kinds_blocks = chain(True)
     assert not any(isinstance(t, BlockedRows) for t in kinds_rows)
-    want_blocks = 0 if m <= 2 or m > 32 else 8 if m <= 8 else 16
+    want_blocks = 0 if m > 32 else 8 if m <= 8 else 16
     assert [t.block_rows if isinstance(t, BlockedRows) else 0 for t in kinds_blocks] == [want_blocks] * 3
     assert torch.equal(h_rows, h_blocks) and torch.equal(again_rows, again_blocks)
     on = lambda t: t.double().to("cuda:0")
