@@ -206,12 +206,13 @@ class HipKernels:
             self._ptr(out, "rmsnorm out"), _code(out, "rmsnorm out"), n_rows, width, float(eps), _block_rows(out),
             self._stream()))
 
-    def new_rows(self, rows, width, dtype, reader_outputs=None, reader_swiglu=False):
+    def new_rows(self, rows, width, dtype, reader_outputs=None, reader_swiglu=False, reader_packed=True):
         """An empty activation matrix [rows, width] for a kernel of this library to fill.  With `reader_outputs`,
         the product that reads it next has that many outputs (`reader_swiglu`: through the gate, so twice as
-        many weight rows): where that product takes `BlockedRows` and reads them faster, the matrix is one."""
+        many weight rows; `reader_packed`: its weight is a `PackedWeight`): where that product takes `BlockedRows`
+        and reads them faster, the matrix is one."""
         rows, width = int(rows), int(width)
-        if reader_outputs is not None and dtype == torch.bfloat16 and width % 64 == 0:
+        if reader_outputs is not None and reader_packed and dtype == torch.bfloat16 and width % 64 == 0:
             block_rows = int(self.lib.bh_gemm_bf16_reads_blocked(rows, int(reader_outputs), width, 1, int(bool(reader_swiglu))))
             if block_rows:
                 return self._new_blocked(rows, width, block_rows)
@@ -336,7 +337,7 @@ class HipKernels:
     def _reader_of(then_norm):
         """The arguments of `new_rows` that name the product reading a norm's output, if the request names one."""
         reader = getattr(then_norm, "reader", None)
-        return (reader.outputs, reader.swiglu) if reader is not None else ()
+        return (reader.outputs, reader.swiglu, getattr(reader, "packed", True)) if reader is not None else ()
 
     def gemm(self, a, w, out, accumulate=False, then_norm=None):
         """out[M, N] (+)= a[M, K] @ w[N, K]^T with float32 accumulation; `w` may be a PackedWeight and

@@ -43,8 +43,11 @@ class GQAAttention:
         self.qkv = Linear(hidden, [q_width, kv_width, kv_width],
                           [prefix + "q_proj.weight", prefix + "k_proj.weight", prefix + "v_proj.weight"])
         self.out = Linear(q_width, hidden, prefix + "o_proj.weight")
-        self.input_reader = self.qkv.reader()    # x goes to that product and nowhere else
         self.q_norm = self.k_norm = None
+
+    @property
+    def input_reader(self):
+        return self.qkv.reader()    # x goes to that product and nowhere else
 
     def tensor_specs(self):
         specs = self.qkv.tensor_specs() + self.out.tensor_specs()

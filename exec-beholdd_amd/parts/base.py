@@ -120,7 +120,8 @@ class StepContext:
         next and nothing else does: the kernel library may then hand out the matrix in the form that product
         reads fastest, which only its own kernels fill and read."""
         if reader is not None and len(shape) == 2 and hasattr(self.kernels, "new_rows"):
-            return self.kernels.new_rows(shape[0], shape[1], self.act_dtype, reader.outputs, reader.swiglu)
+            return self.kernels.new_rows(shape[0], shape[1], self.act_dtype, reader.outputs, reader.swiglu,
+                                         getattr(reader, "packed", True))
         return torch.empty(shape, dtype=self.act_dtype, device=self.device)
 
     def new_f32(self, *shape) -> torch.Tensor:
@@ -130,9 +131,11 @@ class StepContext:
 @dataclass
 class ProductReader:
     """The matrix product that reads an activation matrix next: `outputs` columns of result, through the
-    gated activation or not (then its weight has twice as many rows)."""
+    gated activation or not (then its weight has twice as many rows); `packed`: its weight is in the kernel
+    library's own form (`Linear.prepare`), not a plain matrix."""
     outputs: int
     swiglu: bool = False
+    packed: bool = True
 
 
 @dataclass

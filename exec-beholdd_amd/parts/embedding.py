@@ -42,7 +42,6 @@ class LMHead:
             raise ValueError("a head has either its own tensor or an embedding it is tied to")
         self.vocab, self.width, self.tied_to = vocab, width, tied_to
         self.linear = Linear(width, vocab, name or tied_to.name)
-        self.input_reader = self.linear.reader()    # x goes to that product and nowhere else
 
     def tensor_specs(self):
         return [] if self.tied_to is not None else self.linear.tensor_specs()
@@ -55,6 +54,10 @@ class LMHead:
 
     def prepare(self, kernels):
         self.linear.prepare(kernels)        # a tied head keeps the embedding's own matrix
+
+    @property
+    def input_reader(self):
+        return self.linear.reader()    # x goes to that product and nowhere else
 
     def forward(self, ctx, x):
         """x [n, width] -> float32 logits [n, vocab]."""

@@ -50,7 +50,8 @@ class Linear:
 
     def reader(self, swiglu: bool = False) -> ProductReader:
         """This map as the only reader of an activation matrix (`swiglu`: its rows are gate rows, then up rows)."""
-        return ProductReader(self.out_features // 2 if swiglu else self.out_features, swiglu)
+        return ProductReader(self.out_features // 2 if swiglu else self.out_features, swiglu,
+                             packed=self.weight is not None and not isinstance(self.weight, torch.Tensor))
 
     def prepare(self, kernels):
         """Let the kernel library regroup the matrix into the layout it reads fastest."""

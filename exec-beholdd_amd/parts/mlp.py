@@ -20,7 +20,10 @@ class SwiGLU:
         self.gate_up = Linear(hidden, [intermediate, intermediate],
                               [prefix + "gate_proj.weight", prefix + "up_proj.weight"])
         self.down = Linear(intermediate, hidden, prefix + "down_proj.weight")
-        self.input_reader = self.gate_up.reader(swiglu=True)    # x goes to that product and nowhere else
+
+    @property
+    def input_reader(self):
+        return self.gate_up.reader(swiglu=True)    # x goes to that product and nowhere else
 
     def tensor_specs(self):
         return self.gate_up.tensor_specs() + self.down.tensor_specs()
