@@ -163,6 +163,42 @@ def test_prompts_of_many_rows(large_expected):
     check("together against alone", together, alone, TOLERANCE["bfloat16"] / 2)
 
 
+@pytest.mark.parametrize("batch", [1, 8, 24])
+def test_every_product_gets_its_rows_the_way_it_reads_them(large_expected, batch):
+    """At the Qwen3-8B layer sizes the products of a prompt of 1,500 rows and of decode steps of 1, 8 and 24
+    sequences read their activations from blocks.  Every kernel before them knows its reader and writes the blocks
+    itself: the binding's regrouping kernel, which would make up for a part that does not, never runs."""
+    from beholdd.engine import StepEntry
+    folder = large_expected("8b")[0]
+    engine = engine_for(folder, "bfloat16", max_tokens=4096)
+    kernels, calls = engine.kernels, []
+    to_blocked, from_blocked, new_rows = kernels.to_blocked, kernels.from_blocked, kernels.new_rows
+    kinds = set()
+
+    def watched_new_rows(*args, **kwargs):
+        out = new_rows(*args, **kwargs)
+        kinds.add(getattr(out, "block_rows", 0))
+        return out
+
+    kernels.to_blocked = lambda *a, **k: (calls.append("to_blocked"), to_blocked(*a, **k))[1]
+    kernels.from_blocked = lambda *a, **k: (calls.append("from_blocked"), from_blocked(*a, **k))[1]
+    kernels.new_rows = watched_new_rows
+    try:
+        requests = schedules.random_requests(1000, [1500 if i == 0 else 20 + i for i in range(batch)], seed=40)
+        slots = [engine.alloc_slot() for _ in requests]
+        engine.step([StepEntry(s, r[:-2], [len(r) - 3]) for s, r in zip(slots, requests)])
+        assert 16 in kinds                                   # the prompt step's products of many rows
+        kinds.clear()
+        for back in (2, 1):                                  # the first decode step runs as it is, the second is captured
+            engine.step([StepEntry(s, [r[-back]], [0]) for s, r in zip(slots, requests)])
+        assert kinds == {8 if batch <= 8 else 16, 0}         # 0: matrices that no product reads (queries for the attention)
+        assert calls == []
+    finally:
+        kernels.to_blocked, kernels.from_blocked, kernels.new_rows = to_blocked, from_blocked, new_rows
+        for slot in slots:
+            engine.free_slot(slot)
+
+
 def _prompt_then_one_by_one(engine, tokens, tail, keep):
     """The first len - tail tokens in one step (the logits of its last `keep` rows wanted), the rest one by one."""
     from beholdd.engine import StepEntry
