@@ -163,6 +163,13 @@ class HipKernels:
                 return None
             raise KernelError(f"{what}: tensor is required")
         if isinstance(tensor, BlockedRows):
+            rows, width = tensor.shape
+            if (tensor.block_rows not in (8, 16) or width % 32 or tensor.data.dtype != torch.bfloat16
+                    or tensor.data.numel() < BlockedRows.padded_rows(rows, tensor.block_rows) * width):
+                raise KernelError(f"{what}: a matrix of {rows} x {width} in blocks of {tensor.block_rows} rows needs a bfloat16 "
+                                  f"buffer of {BlockedRows.padded_rows(rows, tensor.block_rows) * width} elements (whole "
+                                  f"blocks; whole tiles of {BlockedRows.ROWS_PAD} rows beyond 32 rows), a width that is a "
+                                  f"multiple of 32 and blocks of 8 or 16 rows; it has {tensor.data.numel()} elements")
             tensor = tensor.data
         if not isinstance(tensor, torch.Tensor) or tensor.device != self.device:
             raise KernelError(f"{what}: expected a tensor on {self.device}, got "

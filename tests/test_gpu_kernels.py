@@ -317,6 +317,10 @@ def test_rows_into_blocks_and_back(K, rows, width, block_rows):
     from beholdd.kernels import KernelError
     with pytest.raises(KernelError, match="multiple of 32"):
         K.to_blocked(dev(torch.zeros(4, 48, dtype=torch.bfloat16)))
+    from beholdd.kernels.library import BlockedRows
+    short = BlockedRows(torch.zeros(rows * width, dtype=torch.bfloat16, device="cuda:0")[:-1], rows, width, block_rows)
+    with pytest.raises(KernelError, match="whole blocks"):      # a buffer that does not hold what the kernels will read
+        K.from_blocked(short)
 
 
 @pytest.mark.parametrize("blocks", [8, 6, 4])
