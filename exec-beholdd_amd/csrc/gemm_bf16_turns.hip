@@ -268,7 +268,7 @@ bool gemm_turns_can(int M, int N, int K, int layout, int activation, int blocks)
   if (blocks != 8 && blocks != 6 && blocks != 4) return false;
   const int outs = (activation ? 16 : 32) * blocks;
   return layout == 1 && M >= 256 && N >= outs && N % 16 == 0 && K >= 128 && K % 128 == 0 &&
-         (long)M * K < (1L << 31) && (long)((N + outs - 1) / outs) * ((M + 255) / 256) < (1L << 31);
+         (long)((N + outs - 1) / outs) * ((M + 255) / 256) < (1L << 31);   // offsets into A, W and C are 64-bit
 }
 
 // Which way, if any.  A tile of YB blocks per wave costs a compute unit YB x cost(YB) units of time, where cost

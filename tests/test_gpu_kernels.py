@@ -441,6 +441,29 @@ def test_products_of_many_rows_hand_each_other_blocks(K, m):
     assert bool(torch.isfinite(h_blocks).all())
 
 
+def test_product_of_more_than_two_to_the_31_activation_elements(K):
+    """A step of 131,328 rows times 16,384 inputs (batches of long prompts at the large models' feed-forward widths
+    come near it): offsets beyond 32 bits into the activations, in rows and in blocks; the first and the last
+    rows against float64."""
+    m, n, k = 131072 + 256, 256, 16384
+    g = torch.Generator(device="cuda:0").manual_seed(3)
+    a = torch.empty(m, k, dtype=torch.bfloat16, device="cuda:0")
+    for start in range(0, m, 16384):
+        a[start:start + 16384] = torch.randn(min(16384, m - start), k, generator=g, device="cuda:0").to(torch.bfloat16)
+    w = (torch.randn(n, k, generator=g, device="cuda:0") * 0.02).to(torch.bfloat16)
+    packed = K.pack_weight(w)
+    assert K.gemm_turns_blocks(m, n, k) == 8
+    out = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
+    K.gemm(a, packed, out)                    # regrouped into blocks on the way
+    rows = torch.cat([torch.arange(0, 300), torch.arange(m - 300, m)]).to("cuda:0")
+    want = a[rows].double() @ w.double().t()
+    assert rel(out[rows], want.cpu()) < 4 * math.sqrt(k) * 2.0 ** -24
+    assert bool(torch.isfinite(out).all())
+    from_rows = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
+    K.gemm_turns(a, packed, from_rows, 8)
+    assert torch.equal(out, from_rows)
+
+
 def test_gemm_with_turns_refuses_what_it_cannot_do(K):
     from beholdd.kernels import KernelError
     a = dev(torch.zeros(256, 192, dtype=torch.bfloat16))
