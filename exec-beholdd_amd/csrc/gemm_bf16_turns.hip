@@ -293,8 +293,9 @@ bool gemm_turns_can(int M, int N, int K, int layout, int activation, int blocks)
 // Which way, if any.  A tile of YB blocks per wave costs a compute unit YB x cost(YB) units of time, where cost
 // is what the narrower tiles lose (measured 1.43, 1.16 and 1.07 PFLOP/s for 8, 6 and 4 with the chip full and the
 // activations in blocks; 1.25, 1.11 and 0.90 with activations in rows), and
-// the chip works in rounds of 256 tiles; a tile of its own is taken if that estimate beats what the other tiled
-// kernels reach at their best (about 0.8 PFLOP/s).  Products with so few of the widest tiles that much of the
+// the chip works in rounds of 256 tiles; a tile of its own is taken if that estimate reaches 0.6 PFLOP/s, which
+// the other tiled kernels stay below at these sizes (with 0.8 as the bar, prefill steps of 320 to 768 tokens were 2 to
+// 18 % slower at the Qwen3-8B, 14B and 32B widths, and no length was faster).  Products with so few of the widest tiles that much of the
 // chip would idle can instead cut K into parts over as many times the workgroups, each leaving its bare sums in
 // scratch memory ([part][row][weight row], float32) for a finishing kernel of gemm_bf16.hip; that costs about
 // 0.85 of the tile's rate (for the o projection of the Qwen3-8B shape at 2,048 rows the parts and the 128-wide
@@ -307,7 +308,7 @@ struct TurnsPlan {
 TurnsPlan turns_plan(int M, int N, int K, int layout, int activation) {
   TurnsPlan plan = {0, 1};
   if (M <= 256) return plan;   // up to there a norm may ride on the product, which this kernel does not carry
-  double best_rate = 800.0;    // TFLOP/s, roughly: what the other kernels reach at their best
+  double best_rate = 600.0;    // TFLOP/s: what a tile of its own has to reach
   double direct_rate = 0.0;
   const double work = (double)M * (activation ? 2.0 * N : (double)N);   // rows x weight rows
   for (int blocks = 8; blocks >= 4; blocks -= 2) {
@@ -320,14 +321,15 @@ TurnsPlan turns_plan(int M, int N, int K, int layout, int activation) {
     if (rate >= best_rate) best_rate = direct_rate = rate, plan.blocks = blocks;
   }
   if (!activation && M >= 512 && gemm_turns_can(M, N, K, layout, 0, 8)) {
-    // As many parts (8, 4 or 2) as keep the workgroups within one round and every part at least 1,024 long; worth
+    // As many parts (8, 4 or 2) as keep the workgroups within one round and every part at least 512 long; worth
     // it from about five eighths of the chip on.  Measured at the Qwen3-8B widths against the other kernels, us:
-    // 512 rows: down in 8 parts 88 -> 72 (o in 4 parts, half the chip, 41 -> 45: left alone); 768 rows: o 71 -> 53,
+    // 512 rows: down in 8 parts 88 -> 72 (o in 4 parts, half the chip, 41 -> 45; in 8 parts of 512 the prefill step of
+    // 512 tokens is 0.5 % faster than with the older tiles); 768 rows: o 71 -> 53,
     // down 195 -> 102 in 4; 1,024 rows: o 72 -> 57, down 196 -> 111 in 4; 1,536 rows: o 93 -> 77, down 219 -> 173 in 2;
     // 2,048 rows: down 240 -> 199 in 2; 384 rows: slower for qkv and o, so not below 512.
     const long tiles = (long)((N + 255) / 256) * ((M + 255) / 256);
     int parts = 8;
-    while (parts > 1 && (tiles * parts > 256 || K / parts < 1024 || K % (128 * parts) != 0)) parts /= 2;
+    while (parts > 1 && (tiles * parts > 256 || K / parts < 512 || K % (128 * parts) != 0)) parts /= 2;
     if (parts > 1 && tiles * parts >= 160) {
       const double rate = 0.85 * 1430.0 * work / (256.0 * 256 * 256 / parts);
       if (rate > direct_rate) plan.blocks = 0, plan.parts = parts;
