@@ -266,10 +266,12 @@ def test_norm_does_not_ride_on_wide_steps(K):
 
 @pytest.mark.parametrize("blocks", [8, 6, 4])
 @pytest.mark.parametrize("m,n,k", [(256, 256, 128), (300, 400, 384), (520, 1040, 256), (257, 272, 1152),
-                                   (1024, 768, 2048)])
+                                   (1024, 768, 2048), (2400, 1296, 128)])
 def test_gemm_whose_wave_groups_take_turns(K, blocks, m, n, k):
     """The product for many rows at each of its tile widths: whole tiles, tiles moved back inside at both
-    edges, one and many k steps; float32 with and without accumulation, bfloat16, SwiGLU."""
+    edges, one and many k steps; float32 with and without accumulation, bfloat16, SwiGLU.  The last size has
+    more than eight tiles of rows and a number of weight tiles that is no multiple of four: there the order in
+    which the workgroups take the tiles goes in blocks of 8 x 4, with a short block at either edge."""
     g = torch.Generator().manual_seed(m + n + blocks)
     a = torch.randn(m, k, generator=g).to(torch.bfloat16)
     w = (torch.randn(2 * n, k, generator=g) * 0.05).to(torch.bfloat16)
@@ -324,7 +326,8 @@ def test_rows_into_blocks_and_back(K, rows, width, block_rows):
 
 
 @pytest.mark.parametrize("blocks", [8, 6, 4])
-@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (300, 416, 384), (527, 1056, 256), (257, 288, 1152), (1024, 768, 2048)])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (300, 416, 384), (527, 1056, 256), (257, 288, 1152), (1024, 768, 2048),
+                                   (2400, 1312, 128)])
 def test_gemm_with_turns_reads_and_writes_rows_in_blocks(K, blocks, m, n, k):
     """The same product from activations in blocks of 16 x 32 gives the same bits as from rows (the sums run
     in the same order), also where the last tile of rows sticks out of the matrix and the buffer's rows beyond
