@@ -15,10 +15,31 @@
 //     S^T[key, column] = K[key, :] . Q[column, :],   tile t, row i <-> key 32 (t/2) + 4 (t%2) + 8 (i/4) + i%4
 //     online softmax per column in float32, exponent base 2
 //     O^T[d, column] += V^T[d, key] . P^T[key, column]
+// The walk over a page is bound by the vector instructions of the softmax, not by the products (counters: the
+// vector units busy 57 % of the kernel's time, the matrix cores 38 %), so they are kept few: the maximum by
+// v_maximum3_f32 (three numbers an instruction, no quieting of each score first as fmaxf needs), over the four
+// lanes of a column by two row exchanges between registers instead of two shuffles through LDS, the sum of the
+// probabilities by one more row of the value product, and a page's operands asked of LDS in two goes ahead of
+// the arithmetic that hides the wait.  Measured, one sequence at 32 query and 8 kv heads of 128: 2,048 rows
+// 72 -> 63.5 us, 4,096 rows 194 -> 176 us, 8,192 rows 604 -> 540 us.
 // A wave skips pages none of whose keys any of its columns may see.  Values beyond the last position
 // of the workgroup's columns are zeroed in LDS before the last page is used (their probabilities are
 // zero, but what lies there may be anything).
 #include "attention_bf16.h"
+
+// The larger of two numbers, a NaN if either is one (v_maximum3_f32, which takes its operands as they are; fmaxf
+// has to make each of them a quiet number first, one more instruction per score).
+__device__ inline float larger(float a, float b) { return __builtin_elementwise_maximum(a, b); }
+
+// The largest of the values that the lanes j, 16 + j, 32 + j and 48 + j hold, in all four of them, by two
+// exchanges of rows between registers (no trip through LDS as a shuffle takes): the first leaves rows 0 and 2 in
+// one register and rows 1 and 3 in the other, each twice; the second the lower and the upper half.
+__device__ inline float largest_of_column(float x) {
+  const auto rows = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  const float pairs = larger(__uint_as_float(rows[0]), __uint_as_float(rows[1]));
+  const auto halves = __builtin_amdgcn_permlane32_swap(__float_as_uint(pairs), __float_as_uint(pairs), false, false);
+  return larger(__uint_as_float(halves[0]), __uint_as_float(halves[1]));
+}
 
 template <int NS, int CTW>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2 : 1))) void attention_prefill_kernel(
@@ -53,7 +74,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
   const int group_col0 = tile_group * GROUP_TILES * 16;
   if (group_col0 >= n_cols) return;                // the whole workgroup: no barrier is left behind
 
-  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int tid = threadIdx.x, lane = tid % 64;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64);   // the same in all lanes: what depends on it alone stays out of the vector registers
   const int j = lane % 16, g = lane / 16;
 
   // rows of a sequence are consecutive and in position order: the workgroup's first and last row bound its keys
@@ -90,12 +112,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
   lo_min = wave_min_int(lo_min);
   lo_max = wave_max_int(lo_max);
 
-  f32x4_t o[CTW][2 * NS];
-  float run_max[CTW], run_sum[CTW];  // run_sum: this lane's share of the column's sum
+  // The sum of a column's probabilities is one more row of the value product: the probabilities, as they enter
+  // that product (rounded to bfloat16), times a block of ones; every one of a lane's four sums is its column's.
+  f32x4_t o[CTW][2 * NS], run_sum[CTW];
+  float run_max[CTW];
+  const u32x4_t ones = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
 #pragma unroll
   for (int ct = 0; ct < CTW; ++ct) {
     run_max[ct] = -INFINITY;
-    run_sum[ct] = 0.f;
+    run_sum[ct] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int dt = 0; dt < 2 * NS; ++dt) o[ct][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
@@ -107,10 +132,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
     const int page = table[p];
     const uint16_t* kb = k_pages + ((size_t)page * KVH + kvh) * BH_PAGE * HD;
     const uint16_t* vb = v_pages + ((size_t)page * KVH + kvh) * HD * BH_PAGE;
+    static_assert(PIECES % 256 == 0, "the first half of a thread's pieces are keys, the second half values");
 #pragma unroll
     for (int i = 0; i < STAGE; ++i) {
-      const int piece = tid + i * 256;
-      const uint16_t* src = piece < PIECES ? kb + (size_t)piece * 8 : vb + (size_t)(piece - PIECES) * 8;
+      const uint16_t* src = (i < STAGE / 2 ? kb : vb) + (size_t)(tid + (i % (STAGE / 2)) * 256) * 8;
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                        (__attribute__((address_space(3))) void*)&page_lds[buffer][i * 256 + wave * 64],
                                        16, 0, 0);
@@ -141,6 +166,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
     // a page none of whose keys this wave's columns may see changes nothing
     const bool visible = wave_active && p * BH_PAGE <= pos_max && p * BH_PAGE + BH_PAGE - 1 >= lo_min;
     if (visible) {
+      // A page's operands are asked of LDS in two goes, each before the arithmetic that hides the wait: all the
+      // keys' before the first score product, all the values' before the softmax.
+      u32x4_t operand[4 * NS];
+#pragma unroll
+      for (int i = 0; i < 4 * NS; ++i) operand[i] = kl[i * 64 + lane];
+      __builtin_amdgcn_sched_barrier(0);
       f32x4_t st[CTW][4];
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
@@ -148,41 +179,45 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
         for (int ct = 0; ct < CTW; ++ct) st[ct][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
-          const bf16x8_t kf = as_bf16x8(kl[(t * NS + s) * 64 + lane]);
 #pragma unroll
           for (int ct = 0; ct < CTW; ++ct)
-            st[ct][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, q_vec[ct][s], st[ct][t], 0, 0, 0);
+            st[ct][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(operand[t * NS + s]), q_vec[ct][s], st[ct][t], 0, 0, 0);
         }
       }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 4 * NS; ++i) operand[i] = vl[i * 64 + lane];
+      __builtin_amdgcn_sched_barrier(0);
       const int key0 = p * BH_PAGE + 8 * g;  // lane (j, g) holds keys key0 + 32 * (t / 2) + 4 * (t % 2) + r
       const bool mask_needed = (p * BH_PAGE + BH_PAGE - 1 > pos_min) || (p * BH_PAGE < lo_max);
       u32x4_t p_vec[CTW][2];
 #pragma unroll
       for (int ct = 0; ct < CTW; ++ct) {
-        if (mask_needed) {
+        if (mask_needed) {   // key k0 + d of the page is seen if lo <= k0 + d <= pos: two numbers per column, then constants
+          const int d_last = pos[ct] - key0, d_first = lo[ct] - key0;
 #pragma unroll
           for (int t = 0; t < 4; ++t)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-              const int key = key0 + 32 * (t / 2) + 4 * (t % 2) + r;
-              if (key > pos[ct] || key < lo[ct]) st[ct][t][r] = -INFINITY;
+              const int d = 32 * (t / 2) + 4 * (t % 2) + r;
+              if (d > d_last || d < d_first) st[ct][t][r] = -INFINITY;
             }
         }
         // Online softmax with few instructions: the maximum is taken over the raw scores, the scale
         // enters through one fused multiply-add per score, and the exponentials are bare v_exp_f32
         // (arguments <= 0; results below the normal range may flush to zero).
-        float local_max = fmaxf(fmaxf(st[ct][0][0], st[ct][0][1]), fmaxf(st[ct][0][2], st[ct][0][3]));
+        float local_max = larger(larger(st[ct][0][0], st[ct][0][1]), st[ct][0][2]);
+        local_max = larger(larger(local_max, st[ct][0][3]), st[ct][1][0]);
 #pragma unroll
-        for (int t = 1; t < 4; ++t)
-          local_max = fmaxf(local_max, fmaxf(fmaxf(st[ct][t][0], st[ct][t][1]), fmaxf(st[ct][t][2], st[ct][t][3])));
-        local_max = fmaxf(local_max, __shfl_xor(local_max, 16, 64));
-        local_max = fmaxf(local_max, __shfl_xor(local_max, 32, 64));
-        const float new_max = fmaxf(run_max[ct], local_max);              // raw (unscaled) scores
+        for (int t = 1; t < 4; ++t) {
+          local_max = larger(larger(local_max, st[ct][t][1]), st[ct][t][2]);
+          local_max = larger(larger(local_max, st[ct][t][3]), t < 3 ? st[ct][t + 1][0] : run_max[ct]);
+        }
+        const float new_max = largest_of_column(local_max);               // raw (unscaled) scores, the earlier pages' too
         const float shift = (new_max == -INFINITY) ? 0.f : -new_max * scale_log2;
         // exactly 1 while the maximum stands still, 0 when nothing was seen before
         const float alpha =
             (run_max[ct] == new_max) ? 1.0f : __builtin_amdgcn_exp2f((run_max[ct] - new_max) * scale_log2);
-        float page_sum = 0.f;
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -192,21 +227,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
             const float e1 = __builtin_amdgcn_exp2f(fmaf(st[ct][t][1], scale_log2, shift));
             const float e2 = __builtin_amdgcn_exp2f(fmaf(st[ct][t][2], scale_log2, shift));
             const float e3 = __builtin_amdgcn_exp2f(fmaf(st[ct][t][3], scale_log2, shift));
-            page_sum += (e0 + e1) + (e2 + e3);
             p_vec[ct][u][2 * half] = pack_bf16(e0, e1);
             p_vec[ct][u][2 * half + 1] = pack_bf16(e2, e3);
           }
-        run_sum[ct] = run_sum[ct] * alpha + page_sum;
         run_max[ct] = new_max;
         if (__any(alpha != 1.0f)) {   // after the first pages the maximum seldom moves
+          run_sum[ct] = run_sum[ct] * alpha;
 #pragma unroll
           for (int dt = 0; dt < 2 * NS; ++dt) o[ct][dt] = o[ct][dt] * alpha;
         }
       }
 #pragma unroll
+      for (int ct = 0; ct < CTW; ++ct) {
+        run_sum[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(ones), as_bf16x8(p_vec[ct][0]), run_sum[ct], 0, 0, 0);
+        run_sum[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(ones), as_bf16x8(p_vec[ct][1]), run_sum[ct], 0, 0, 0);
+      }
+#pragma unroll
       for (int dt = 0; dt < 2 * NS; ++dt) {
-        const bf16x8_t v0 = as_bf16x8(vl[(dt * 2) * 64 + lane]);
-        const bf16x8_t v1 = as_bf16x8(vl[(dt * 2 + 1) * 64 + lane]);
+        const bf16x8_t v0 = as_bf16x8(operand[dt * 2]);
+        const bf16x8_t v1 = as_bf16x8(operand[dt * 2 + 1]);
 #pragma unroll
         for (int ct = 0; ct < CTW; ++ct) {
           f32x4_t acc = o[ct][dt];
@@ -229,15 +268,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
   clear_tail(last, (last - begin) & 1);
   attend(last, (last - begin) & 1);
 
-  // lane (j, g) holds O^T[16 dt + 4 g + r, column j] and its share of the column's sum
+  // lane (j, g) holds O^T[16 dt + 4 g + r, column j] and the column's sum
 #pragma unroll
   for (int ct = 0; ct < CTW; ++ct) {
     const int cc = (wave_tile0 + ct) * 16 + j;
-    float total = run_sum[ct];
-    total += __shfl_xor(total, 16, 64);
-    total += __shfl_xor(total, 32, 64);
     if (cc >= n_cols) continue;
-    const float inv = 1.0f / total;
+    const float inv = 1.0f / run_sum[ct][0];
     const int out_row = row0 + cc / G, out_column = (kvh * G + cc % G) * HD + 4 * g;
 #pragma unroll
     for (int dt = 0; dt < 2 * NS; ++dt) {
