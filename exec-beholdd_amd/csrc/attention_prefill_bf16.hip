@@ -19,9 +19,10 @@
 // vector units busy 57 % of the kernel's time, the matrix cores 38 %), so they are kept few: the maximum by
 // v_maximum3_f32 (three numbers an instruction, no quieting of each score first as fmaxf needs), over the four
 // lanes of a column by two row exchanges between registers instead of two shuffles through LDS, the sum of the
-// probabilities by one more row of the value product, and a page's operands asked of LDS in two goes ahead of
-// the arithmetic that hides the wait.  Measured, one sequence at 32 query and 8 kv heads of 128: 2,048 rows
-// 72 -> 63.5 us, 4,096 rows 194 -> 176 us, 8,192 rows 604 -> 540 us.
+// probabilities by one more row of the value product, a page's operands asked of LDS in two goes ahead of
+// the arithmetic that hides the wait, and the exponentials' reference moved (and the sums so far scaled) only
+// when the maximum has grown by more than 2^8.  Measured, one sequence at 32 query and 8 kv heads of 128:
+// 2,048 rows 72 -> 60 us, 4,096 rows 194 -> 166 us, 8,192 rows 604 -> 533 us.
 // A wave skips pages none of whose keys any of its columns may see.  Values beyond the last position
 // of the workgroup's columns are zeroed in LDS before the last page is used (their probabilities are
 // zero, but what lies there may be anything).
@@ -51,6 +52,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
   constexpr int PIECES = BH_PAGE * HD / 8;        // 16-byte pieces of one head's keys (or values) in a page
   constexpr int STAGE = 2 * PIECES / 256;         // pieces of a page (keys, then values) one thread copies
   constexpr int GROUP_TILES = 4 * CTW;            // column tiles of a workgroup
+  constexpr float SLACK = 8.0f;
   __shared__ u32x4_t page_lds[2][2 * PIECES];
 
   // Workgroups go to the eight XCDs in turn, each with an L2 of its own: when the number of
@@ -214,10 +216,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
           local_max = larger(larger(local_max, st[ct][t][3]), t < 3 ? st[ct][t + 1][0] : run_max[ct]);
         }
         const float new_max = largest_of_column(local_max);               // raw (unscaled) scores, the earlier pages' too
-        const float shift = (new_max == -INFINITY) ? 0.f : -new_max * scale_log2;
-        // exactly 1 while the maximum stands still, 0 when nothing was seen before
+        // The exponentials' reference moves only when the maximum has grown by more than SLACK powers of two (or
+        // from nothing): until then probabilities may reach 2^SLACK, which float32 sums and bfloat16 operands
+        // hold as well as numbers up to one, and what was summed so far needs no factor.
+        const bool stays = (new_max - run_max[ct]) * scale_log2 <= SLACK;   // false from -inf, and while nothing was seen
+        const float reference = stays ? run_max[ct] : new_max;
+        const float shift = (reference == -INFINITY) ? 0.f : -reference * scale_log2;
+        // exactly 1 while the reference stands still, 0 when nothing was seen before
         const float alpha =
-            (run_max[ct] == new_max) ? 1.0f : __builtin_amdgcn_exp2f((run_max[ct] - new_max) * scale_log2);
+            (run_max[ct] == reference) ? 1.0f : __builtin_amdgcn_exp2f((run_max[ct] - reference) * scale_log2);
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -230,8 +237,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
             p_vec[ct][u][2 * half] = pack_bf16(e0, e1);
             p_vec[ct][u][2 * half + 1] = pack_bf16(e2, e3);
           }
-        run_max[ct] = new_max;
-        if (__any(alpha != 1.0f)) {   // after the first pages the maximum seldom moves
+        run_max[ct] = reference;
+        if (__any(alpha != 1.0f)) {   // after the first pages the reference seldom moves
           run_sum[ct] = run_sum[ct] * alpha;
 #pragma unroll
           for (int dt = 0; dt < 2 * NS; ++dt) o[ct][dt] = o[ct][dt] * alpha;

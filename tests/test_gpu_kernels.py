@@ -771,6 +771,38 @@ def test_attention_prefill_many_columns(K, n_heads, kv_heads, head_dim, window, 
     assert torch.equal(K.from_blocked(blocked), out)
 
 
+@pytest.mark.parametrize("n_heads,kv_heads,head_dim", [(32, 8, 128), (16, 4, 64)])
+def test_attention_prefill_when_the_largest_score_keeps_growing(K, n_heads, kv_heads, head_dim):
+    """One direction is planted in every query and in the keys with a weight that grows along the sequence: by a
+    little from key to key (the largest score so far grows by less than a factor of two a page), then twentyfold
+    from one key on (a jump by more than two hundred powers of two, which no float32 holds).  The kernel that keeps
+    the exponentials' reference while the maximum grows little has to follow both: a reference not moved at the jump
+    gives infinite probabilities, one moved without scaling what was summed before gives wrong rows after it."""
+    dtype = torch.bfloat16
+    n = 1500
+    g = torch.Generator().manual_seed(head_dim)
+    kp, vp, table, keys, values = make_cache(1, [n], kv_heads, head_dim, dtype, seed=7)
+    direction = torch.randn(head_dim, generator=g)
+    direction /= direction.norm()
+    weight = 0.02 * torch.arange(n, dtype=torch.float32)             # scores along the direction grow by 0.02 * |q.d| * scale a key
+    weight[1100:] *= 20.0
+    planted = (keys[0].float() * 0.3 + weight[:, None, None] * direction).to(dtype)
+    keys[0] = planted
+    for t in range(n):
+        kp[int(table[0, t // PAGE]), :, t % PAGE] = planted[t]
+    q = (torch.randn(n, n_heads, head_dim, generator=g) * 0.3 + 4.0 * direction).to(dtype).reshape(n, n_heads * head_dim)
+    positions = torch.arange(n, dtype=torch.int32)
+    starts = torch.tensor([0, n], dtype=torch.int32)
+    scale = 1 / math.sqrt(head_dim)
+    assert -(-n * (n_heads // kv_heads) // 16) * kv_heads >= 1024      # what sends the step to the kernel for many columns
+    out = torch.empty(n, n_heads * head_dim, dtype=dtype, device="cuda:0")
+    K.attention(dev(q), out, *stored(K, kp, vp), dev(table), dev(torch.zeros(n, dtype=torch.int32)), dev(positions),
+                n_heads, kv_heads, head_dim, scale, 0, layout=Layout(False, dev(starts), 1, n, n - 1))
+    want = attention_reference_rows(q, keys[0], values[0], positions.long(), n_heads, kv_heads, head_dim, scale, 0)
+    for rows in (slice(0, 64), slice(64, 1100), slice(1100, 1164), slice(1164, n)):
+        assert rel(out[rows], want[rows]) < 1.2e-2, (rows, rel(out[rows], want[rows]))
+
+
 @pytest.mark.parametrize("window", [0, 70])
 @pytest.mark.parametrize("with_norm,with_rope,write_kv", [(True, True, True), (False, True, True), (True, False, True),
                                                           (True, True, False)])
