@@ -392,24 +392,71 @@ __device__ inline void load_eight(const bf16_t* p, float (&v)[8]) {
 
 // The same for many bfloat16 rows: a lane takes 8 consecutive elements of a head (16 bytes), LPH = head_dim / 8
 // lanes a head, 64 / LPH heads a wave, four waves a block.  The rotation spans the whole head or is absent, so
-// that an element's partner sits LPH / 2 lanes away.  Per head: one 16-byte load, one 16-byte store (values:
-// eight 2-byte stores, as their neighbours in memory are other tokens).
+// that an element's partner sits LPH / 2 lanes away.  Per q or k head: one 16-byte load, one 16-byte store.
+// The values have waves of their own, behind the `main_waves` that take the q and k heads (`n_heads` of them):
+// a value's neighbours in memory are the same dim of other tokens, eight tokens to a 16-byte piece in either
+// cache order, so a wave takes eight rows and (up to) 64 / LPH kv heads, and where the eight tokens of a piece
+// are rows of this step (the same sequence, positions 8 x .. 8 x + 7) the lanes of its first row load all eight
+// rows, turn the 8 x 8 elements and store whole pieces; rows whose piece is not whole in this step (a step's
+// first and last tokens) store their eight elements one by one.  (8,192 rows of 32 query and 8 kv heads of
+// 128: the stores of the values one by one were 35 of the kernel's 57 us.)
 template <typename TW, int LPH>
 __global__ __launch_bounds__(256) void qk_norm_rope_cache_rows_kernel(
     const uint16_t* __restrict__ qkv, uint16_t* __restrict__ q_out, const TW* __restrict__ q_weight,
     const TW* __restrict__ k_weight, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
     uint16_t* __restrict__ k_pages, uint16_t* __restrict__ v_pages, const int32_t* __restrict__ page_table,
-    int table_stride, int H, int KVH, int kv_order, int n_rows, int n_heads) {
+    int table_stride, int H, int KVH, int kv_order, int n_rows, int n_heads, int main_waves) {
   constexpr int HD = 8 * LPH, HPW = BH_WAVE / LPH;
   const int waves_per_row = (n_heads + HPW - 1) / HPW;
-  const int wave = blockIdx.x * 4 + threadIdx.x / BH_WAVE, lane = threadIdx.x % BH_WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * 4 + threadIdx.x / BH_WAVE), lane = threadIdx.x % BH_WAVE;
+  if (wave >= main_waves) {   // the values of eight rows and HPW kv heads
+    const int chunks = (KVH + HPW - 1) / HPW, group = (wave - main_waves) / chunks;
+    const int kv_head = ((wave - main_waves) % chunks) * HPW + lane / LPH, c = lane % LPH;
+    if (kv_head >= KVH) return;
+    const size_t fused = (size_t)(H + 2 * KVH) * HD;
+    const uint16_t* src = qkv + (size_t)(H + KVH + kv_head) * HD + 8 * c;   // + row * fused
+    for (int row = 8 * group; row < 8 * group + 8 && row < n_rows; ++row) {
+      const int pos = positions[row], seq = row_seq[row];
+      const int first = row - pos % 8;   // where the row of the piece's first token would lie
+      const bool whole = first >= 0 && first + 7 < n_rows && row_seq[first] == seq && row_seq[first + 7] == seq &&
+                         positions[first] == pos - pos % 8 && positions[first + 7] == pos - pos % 8 + 7;
+      if (whole && pos % 8 != 0) continue;   // the first row of the piece stores it
+      const int page = page_table[(size_t)seq * table_stride + pos / BH_PAGE];
+      uint16_t* block = v_pages + ((size_t)page * KVH + kv_head) * BH_PAGE * HD;
+      if (!whole) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(src + (size_t)row * fused);
+        const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          block[bh_value_index(kv_order, pos % BH_PAGE, 8 * c + e, HD)] = (uint16_t)(words[e / 2] >> (16 * (e % 2)));
+        continue;
+      }
+      uint4 raw[8];   // token t's dims 8 c .. 8 c + 7
+#pragma unroll
+      for (int t = 0; t < 8; ++t) raw[t] = *reinterpret_cast<const uint4*>(src + (size_t)(row + t) * fused);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {   // dim 8 c + e of the eight tokens: the halves e % 2 of the words e / 2
+        const uint32_t pick = e % 2 ? 0x07060302u : 0x05040100u;
+        uint32_t word[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) word[t] = e / 2 == 0 ? raw[t].x : e / 2 == 1 ? raw[t].y : e / 2 == 2 ? raw[t].z : raw[t].w;
+        uint4 piece;
+        piece.x = __builtin_amdgcn_perm(word[1], word[0], pick);
+        piece.y = __builtin_amdgcn_perm(word[3], word[2], pick);
+        piece.z = __builtin_amdgcn_perm(word[5], word[4], pick);
+        piece.w = __builtin_amdgcn_perm(word[7], word[6], pick);
+        *reinterpret_cast<uint4*>(block + bh_value_index(kv_order, pos % BH_PAGE, 8 * c + e, HD)) = piece;
+      }
+    }
+    return;
+  }
   const int row = wave / waves_per_row;
   if (row >= n_rows) return;   // whole waves leave; nothing below synchronises the block
   const int wanted = (wave % waves_per_row) * HPW + lane / LPH, c = lane % LPH;
   const bool active = wanted < n_heads;
   const int head = active ? wanted : n_heads - 1;   // lanes without a head of their own follow the last one and store nothing
-  const bool is_q = head < H, is_value = head >= H + KVH;
+  const bool is_q = head < H;
   const int pos = positions[row];
   const uint16_t* src = qkv + ((size_t)row * (H + 2 * KVH) + head) * HD + 8 * c;
   const uint4 raw = *reinterpret_cast<const uint4*>(src);
@@ -418,7 +465,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_rows_kernel(
 #pragma unroll
   for (int e = 0; e < 8; ++e) x[e] = bf16_bits_to_f32((uint16_t)(words[e / 2] >> (16 * (e % 2))));
   const TW* weight = is_q ? q_weight : k_weight;
-  if (!is_value) {
+  {
     if (weight != nullptr) {
       float ss = 0.f;
 #pragma unroll
@@ -455,16 +502,9 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_rows_kernel(
     return;
   }
   const int page = page_table[(size_t)row_seq[row] * table_stride + pos / BH_PAGE];
-  const int token = pos % BH_PAGE, kv_head = (head - H) % KVH;
-  if (!is_value) {
-    uint16_t* block = k_pages + ((size_t)page * KVH + kv_head) * BH_PAGE * HD;
-    *reinterpret_cast<uint4*>(block + bh_key_index(kv_order, token, 8 * c, HD)) = packed;   // 8 dims lie together in both orders
-  } else {
-    uint16_t* block = v_pages + ((size_t)page * KVH + kv_head) * BH_PAGE * HD;
-#pragma unroll
-    for (int e = 0; e < 8; ++e)
-      block[bh_value_index(kv_order, token, 8 * c + e, HD)] = (uint16_t)(words[e / 2] >> (16 * (e % 2)));
-  }
+  const int token = pos % BH_PAGE, kv_head = head - H;
+  uint16_t* block = k_pages + ((size_t)page * KVH + kv_head) * BH_PAGE * HD;
+  *reinterpret_cast<uint4*>(block + bh_key_index(kv_order, token, 8 * c, HD)) = packed;   // 8 dims lie together in both orders
 }
 
 extern "C" int bh_qk_norm_rope_cache(const void* qkv, int dtype, void* q_out, const void* q_weight,
@@ -485,14 +525,18 @@ extern "C" int bh_qk_norm_rope_cache(const void* qkv, int dtype, void* q_out, co
   if (cos_table == nullptr) rot = 0;
   const int n_heads = write_kv ? H + 2 * KVH : H;
   if (dtype == BH_BF16 && n_rows >= 64 && (hd == 64 || hd == 128 || hd == 256) && (rot == 0 || rot == hd)) {
-    const int lanes_per_head = hd / 8, waves = n_rows * ((n_heads + 64 / lanes_per_head - 1) / (64 / lanes_per_head));
-    dim3 wide_grid((waves + 3) / 4), wide_block(4 * BH_WAVE);
+    // waves for the q and k heads of every row, then (write_kv) waves for the values of eight rows each
+    const int lanes_per_head = hd / 8, heads_per_wave = 64 / lanes_per_head, main_heads = write_kv ? H + KVH : H;
+    const long main_waves = (long)n_rows * ((main_heads + heads_per_wave - 1) / heads_per_wave);
+    const long value_waves = write_kv ? (long)((n_rows + 7) / 8) * ((KVH + heads_per_wave - 1) / heads_per_wave) : 0;
+    BH_REQUIRE(main_waves + value_waves < (1L << 31), "qk_norm_rope: too many rows");
+    dim3 wide_grid((unsigned)((main_waves + value_waves + 3) / 4)), wide_block(4 * BH_WAVE);
 #define BH_QK_ROWS(TW, LPH)                                                                                       \
   qk_norm_rope_cache_rows_kernel<TW, LPH><<<wide_grid, wide_block, 0, stream>>>(                                   \
       (const uint16_t*)qkv, (uint16_t*)q_out, (const TW*)q_weight, (const TW*)k_weight, eps,                        \
       rot ? cos_table : nullptr, rot ? sin_table : nullptr,                                                          \
       positions, row_seq, (uint16_t*)k_pages, (uint16_t*)v_pages, page_table, table_stride, H, KVH, kv_order,      \
-      n_rows, n_heads)
+      n_rows, main_heads, (int)main_waves)
 #define BH_QK_ROWS_W(LPH)                              \
   do {                                                 \
     if (w_dtype == BH_F32) BH_QK_ROWS(float, LPH);     \
