@@ -406,11 +406,12 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_rows_kernel(
     const TW* __restrict__ k_weight, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
     uint16_t* __restrict__ k_pages, uint16_t* __restrict__ v_pages, const int32_t* __restrict__ page_table,
-    int table_stride, int H, int KVH, int kv_order, int n_rows, int n_heads, int main_waves) {
+    int table_stride, int H, int KVH, int kv_order, int n_rows, int n_heads, int main_waves, int value_waves) {
   constexpr int HD = 8 * LPH, HPW = BH_WAVE / LPH;
   const int waves_per_row = (n_heads + HPW - 1) / HPW;
   const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * 4 + threadIdx.x / BH_WAVE), lane = threadIdx.x % BH_WAVE;
   if (wave >= main_waves) {   // the values of eight rows and HPW kv heads
+    if (wave - main_waves >= value_waves) return;   // the last block's waves beyond the work (none at all without write_kv)
     const int chunks = (KVH + HPW - 1) / HPW, group = (wave - main_waves) / chunks;
     const int kv_head = ((wave - main_waves) % chunks) * HPW + lane / LPH, c = lane % LPH;
     if (kv_head >= KVH) return;
@@ -536,7 +537,7 @@ extern "C" int bh_qk_norm_rope_cache(const void* qkv, int dtype, void* q_out, co
       (const uint16_t*)qkv, (uint16_t*)q_out, (const TW*)q_weight, (const TW*)k_weight, eps,                        \
       rot ? cos_table : nullptr, rot ? sin_table : nullptr,                                                          \
       positions, row_seq, (uint16_t*)k_pages, (uint16_t*)v_pages, page_table, table_stride, H, KVH, kv_order,      \
-      n_rows, main_heads, (int)main_waves)
+      n_rows, main_heads, (int)main_waves, (int)value_waves)
 #define BH_QK_ROWS_W(LPH)                              \
   do {                                                 \
     if (w_dtype == BH_F32) BH_QK_ROWS(float, LPH);     \

@@ -968,13 +968,14 @@ def test_attention_window_edge(K, dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("w_dtype", DTYPES)
-@pytest.mark.parametrize("news", [[3, 5, 1], [70, 5, 1]])        # few rows, and enough for the kernel for many rows
+# few rows; enough for the kernel for many rows; and the same with a sequence whose whole pieces of eight tokens
+# begin at rows 3, 11, ... and steps that begin and end inside a piece
+@pytest.mark.parametrize("news,pasts", [([3, 5, 1], [0, 62, 130]), ([70, 5, 1], [0, 62, 130]), ([3, 70, 2], [5, 16, 7])])
 @pytest.mark.parametrize("n_heads,kv_heads,head_dim,rot", [(4, 2, 16, 16), (6, 2, 48, 48), (5, 1, 80, 32),
                                                            (8, 2, 128, 128), (3, 3, 256, 256), (5, 1, 64, 64),
                                                            (5, 1, 128, 0), (7, 7, 128, 128), (4, 2, 128, 64)])
-def test_qk_norm_rope_cache(K, dtype, w_dtype, n_heads, kv_heads, head_dim, rot, news):
+def test_qk_norm_rope_cache(K, dtype, w_dtype, n_heads, kv_heads, head_dim, rot, news, pasts):
     g = torch.Generator().manual_seed(head_dim)
-    pasts = [0, 62, 130]
     n_rows = sum(news)
     fused = (n_heads + 2 * kv_heads) * head_dim
     qkv = torch.randn(n_rows, fused, generator=g).to(dtype)
