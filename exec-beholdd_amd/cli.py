@@ -20,7 +20,7 @@ USAGE = """usage:
   beholdd generate --model DIR [--dtype bfloat16|float32] --prompt-ids 1,2,3 [--prompt-ids 4,5 ...]
                    [--prompt-ids-file FILE] [--max-new-tokens N] [--temperature X] [--top-k K] [--top-p P]
                    [--seed N] [--stop-token-ids a,b] [--max-tokens N] [--slots N] [--batch-size N]
-                   [--logits-out PATH] [--step-timing-out PATH] [--memory-budget-bytes N] [--plan-only]
+                   [--max-rows-per-step N] [--logits-out PATH] [--step-timing-out PATH] [--memory-budget-bytes N] [--plan-only]
   beholdd random-model --config FILE --out DIR [--seed N] [--dtype bfloat16|float32]
   beholdd compare REFERENCE CANDIDATE [--tolerance X]
   beholdd architectures"""
@@ -82,7 +82,7 @@ def _generate(args: list, out) -> int:
         args,
         valued={"--model", "--dtype", "--prompt-ids", "--prompt-ids-file", "--max-new-tokens", "--temperature",
                 "--top-k", "--top-p", "--seed", "--stop-token-ids", "--max-tokens", "--slots", "--batch-size",
-                "--logits-out", "--step-timing-out", "--memory-budget-bytes"},
+                "--logits-out", "--step-timing-out", "--memory-budget-bytes", "--max-rows-per-step"},
         switches={"--plan-only"}, repeatable={"--prompt-ids"})
     if "--model" not in flags:
         raise UsageError("--model DIR is required")
@@ -108,6 +108,9 @@ def _generate(args: list, out) -> int:
     slots = _number(flags, "--slots", None)
     batch_size = _number(flags, "--batch-size", None)
     budget = _number(flags, "--memory-budget-bytes", None)
+    step_rows = _number(flags, "--max-rows-per-step", None)
+    if step_rows is not None and step_rows <= 0:
+        raise UsageError("--max-rows-per-step is positive")
     for path_flag in ("--logits-out", "--step-timing-out"):
         if path_flag in flags and os.path.lexists(flags[path_flag]):
             raise UsageError(f"{path_flag}: {flags[path_flag]} exists and is never overwritten")
@@ -121,8 +124,13 @@ def _generate(args: list, out) -> int:
     dtype = flags.get("--dtype", "bfloat16")
 
     if "--plan-only" in flags:
+        import torch
+
         from .cache import SequenceCache
         from .engine import open_model, parse_dtype
+        from .engine.engine import GRAPH_LIMIT
+        from .engine.memory import plan_memory
+        from .kernels import KernelSizes
 
         model, weights = open_model(flags["--model"], dtype, "cpu")      # the header only: no tensor is read
         try:
@@ -131,43 +139,56 @@ def _generate(args: list, out) -> int:
             weights.reader.close()
         cache = SequenceCache(model.entry_needs, max_tokens, parse_dtype(dtype), "cpu", page, max_slots=slots,
                               max_position=model.max_position)
-        total = weight_bytes + cache.plan().total_bytes
-        print(f"weights: {weight_bytes} bytes", file=out)
+        capacity = cache.n_pages * cache.page_size
+        # the kernel library's own account of what its calls allocate: host code, no GPU is touched
+        plan = plan_memory(model, weight_bytes, cache.plan(), 2 if parse_dtype(dtype) == torch.bfloat16 else 4,
+                           KernelSizes(), min(step_rows or capacity, capacity), cache.max_slots, cache.max_position,
+                           page, GRAPH_LIMIT)
+        total = plan.total_bytes
+        print(plan.describe() + (f" (budget {budget}: {'fits' if total <= budget else 'does not fit'})"
+                                 if budget is not None else ""), file=out)
         print(cache.plan().describe(), file=out)
-        print(f"total: {total} bytes" + (f" (budget {budget}: {'fits' if total <= budget else 'does not fit'})"
-                                         if budget is not None else ""), file=out)
         return 0 if budget is None or total <= budget else 1
 
     from .engine import Engine
     from .engine.artifact import write_logits_artifact
 
     engine = Engine(flags["--model"], dtype=dtype, max_tokens=max_tokens, max_slots=slots,
-                    memory_limit_bytes=budget)
+                    memory_limit_bytes=budget, max_rows_per_step=step_rows)
     if stops is None:
         stops = list(getattr(config, "eos_token_ids", ()))
-    step_logits = {i: [] for i in range(len(prompts))}
+    # Without a capture the loop runs one step ahead of the host and nothing waits per token; the per-step
+    # report (each token's logit, each step's duration) needs the logits row and a wait per step, so it is
+    # made only where --logits-out or --step-timing-out asks for it.
     keep = "--logits-out" in flags
+    per_step = keep or "--step-timing-out" in flags
+    step_logits = {i: [] for i in range(len(prompts))}
+    stamps = []
 
     def on_logits(index, step, row):
         step_logits[index].append(row.float().cpu().numpy() if keep else float(row.max()))
-
-    stamps = [time.perf_counter()]
 
     def control():
         import torch
         torch.cuda.synchronize()
         stamps.append(time.perf_counter())
 
+    import torch
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    stamps.append(started)
     results = engine.generate(prompts, max_new, temperature=temperature, top_k=top_k, top_p=top_p, seed=seed,
-                              stop_token_ids=stops, batch_size=batch_size, control=control, on_logits=on_logits)
-    control()
-    elapsed = stamps[-1] - stamps[0]
+                              stop_token_ids=stops, batch_size=batch_size, control=control if per_step else None,
+                              on_logits=on_logits if per_step else None)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - started
+    stamps.append(started + elapsed)
     print(flags["--model"], file=out)
     for index, (prompt, result) in enumerate(zip(prompts, results)):
         print(f"  request {index}", file=out)
         print(f"  prompt:    {prompt}", file=out)
         print(f"  generated: {result.token_ids}", file=out)
-        for step, token in enumerate(result.token_ids):
+        for step, token in enumerate(result.token_ids if per_step else ()):
             row = step_logits[index][step]
             value = float(row[token]) if keep else row
             note = "" if keep or temperature == 0.0 else " (largest logit of the step)"
@@ -177,7 +198,8 @@ def _generate(args: list, out) -> int:
     total = sum(r.completion_tokens for r in results)
     print(f"  device:    {engine.device} ({dtype})", file=out)
     if total:
-        print(f"  decode:     {elapsed:.2f}s ({elapsed / total:.4f}s / generated token)", file=out)
+        print(f"  decode:     {elapsed:.2f}s ({elapsed / total:.4f}s / generated token, {total / elapsed:.1f} generated "
+              f"tokens/s, prompts included)", file=out)
     else:
         print(f"  decode:     {elapsed:.2f}s (no generated tokens)", file=out)
     if keep:

@@ -19,7 +19,8 @@ from ..weights.binder import bind
 from ..weights.random_init import random_tensor_on_device
 from . import generation
 from .graphs import DecodeGraphs
-from .step import StepEntry, build_step, cache_for_runs, check_entries
+from .memory import plan_memory
+from .step import StepEntry, StepError, build_step, cache_for_runs, check_entries
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
 
@@ -39,31 +40,48 @@ class MemoryBudgetError(RuntimeError):
     """Weights and cache together would take more device memory than the caller allows; nothing was loaded."""
 
 
+GRAPH_LIMIT = 48      # captured decode steps an engine keeps (least recently used goes first)
+
+
 class Engine:
-    """`Engine(model_dir, dtype, max_tokens)`; then `step(...)` or `generate(...)`.  `memory_limit_bytes`
-    bounds weights and cache together and is checked from the checkpoint's header and the cache's sizes
-    before a tensor is read or the cache allocated (the reference enforces its limits before any I/O,
+    """`Engine(model_dir, dtype, max_tokens)`; then `step(...)` or `generate(...)`.
+
+    `max_rows_per_step` bounds the tokens one step may bring (default: as many as the cache holds); the
+    generation loop feeds prompts beyond it in portions, and `step` refuses more.  It sizes the step's working
+    memory in the byte plan (`plan`, `memory_plan()`): weights as kept, the transient while they are loaded,
+    the cache, the largest step's temporaries and logits, the sampler and the captured decode steps.
+    `memory_limit_bytes` bounds that plan's total and is checked from the checkpoint's header and the sizes
+    alone, before a tensor is read or the cache allocated (the reference enforces its limits before any I/O,
     crates/beholdd-model/src/qwen3moe/recorded_attention.rs:344-365)."""
 
     def __init__(self, model_dir: str | None = None, dtype="bfloat16", max_tokens: int = 4096,
                  max_slots: int | None = None, device="cuda:0", kernels=None, model=None,
-                 memory_limit_bytes: int | None = None, use_graphs: bool = True):
+                 memory_limit_bytes: int | None = None, use_graphs: bool = True,
+                 max_rows_per_step: int | None = None, graph_limit: int = GRAPH_LIMIT):
         self.dtype = parse_dtype(dtype)
         self.device = torch.device(device)
         if kernels is None:
             from ..kernels import HipKernels   # fails loudly without a GPU or the library
             kernels = HipKernels(self.device)
         self.kernels = kernels
+        if max_rows_per_step is not None and max_rows_per_step <= 0:
+            raise ValueError("max_rows_per_step must be positive")
+        with_graphs = bool(use_graphs and self.device.type == "cuda")
 
         def make_cache(built):
             return SequenceCache(built.entry_needs, max_tokens, self.dtype, self.device, kernels.page_size,
                                  max_slots=max_slots, max_position=built.max_position)
 
         def within_budget(weight_bytes, cache):
-            total = weight_bytes + cache.plan().total_bytes
-            if memory_limit_bytes is not None and total > memory_limit_bytes:
-                raise MemoryBudgetError(f"weights ({weight_bytes} bytes) and cache ({cache.plan().total_bytes} bytes) "
-                                        f"need {total} bytes, the limit is {memory_limit_bytes}")
+            capacity = cache.n_pages * cache.page_size
+            # never below one token for every sequence, so that a decode step of a full batch fits
+            self.max_rows_per_step = min(max(int(max_rows_per_step), cache.max_slots), capacity) if max_rows_per_step else capacity
+            self.plan = plan_memory(model, weight_bytes, cache.plan(), 2 if self.dtype == torch.bfloat16 else 4,
+                                    kernels if hasattr(kernels, "gemm_working_bytes") else None, self.max_rows_per_step,
+                                    cache.max_slots, cache.max_position, cache.page_size, graph_limit, with_graphs)
+            if memory_limit_bytes is not None and self.plan.total_bytes > memory_limit_bytes:
+                raise MemoryBudgetError(f"the engine needs {self.plan.total_bytes} bytes, the limit is "
+                                        f"{memory_limit_bytes}:\n{self.plan.describe()}")
 
         if model is None:
             if model_dir is None:
@@ -87,7 +105,7 @@ class Engine:
         self.cache_plan = self.cache.allocate()
         self.sampler = Sampler(kernels, self.device, capacity=self.cache.max_slots)
         self._last_selection = None
-        self.graphs = DecodeGraphs(self) if use_graphs and self.device.type == "cuda" else None
+        self.graphs = DecodeGraphs(self, graph_limit) if with_graphs else None
 
     # ---- what the generation loop needs of a stepper ----
     @property
@@ -126,7 +144,7 @@ class Engine:
         """Run the given tokens of each entry's sequence from the cache; return float32 logits
         [wanted, vocab] in the order of the entries and of their `want` lists (None if nothing is
         wanted).  On an error no sequence's length changes.  The logits of a decode step stand in memory
-        that the next decode step of the same shape writes again: copy what has to outlive it."""
+        that a later decode step may write again: copy what has to outlive the next step."""
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
         if self.graphs is not None and entries and self.graphs.usable(entries):
             return self._graph_step(entries)
@@ -138,6 +156,10 @@ class Engine:
                        else StepEntry(e.slot, [self._last_selection.token_at(e.fed_row)], e.want) for e in entries]
         check_entries(entries, self.cache, self.model.vocab)
         requests = [(e.slot, len(e.tokens)) for e in entries]
+        n_rows = sum(n for _, n in requests)
+        if n_rows > self.max_rows_per_step:
+            raise StepError(f"the step brings {n_rows} tokens, this engine takes {self.max_rows_per_step} a step "
+                            "(max_rows_per_step): feed the prompts in portions")
         self.cache.reserve(requests)
         try:
             ctx, want_rows, tables = build_step(self.kernels, self.dtype, self.device, self.cache, entries)
@@ -176,7 +198,7 @@ class Engine:
                                    batch_size, control, on_logits)
 
     def memory_plan(self) -> str:
-        return f"weights: {self.weight_bytes} bytes\n{self.cache_plan.describe()}"
+        return f"{self.plan.describe()}\n{self.cache_plan.describe()}"
 
 
 def _model_tensors(model):

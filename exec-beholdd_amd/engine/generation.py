@@ -14,6 +14,9 @@ The loop decides on the host and talks to the model only through a *stepper*:
     stepper.alloc_slot() -> slot;  stepper.free_slot(slot)
     stepper.step(entries: list[StepEntry]) -> logits (one row per entry that wants one)
     stepper.select(logits, params, request_indices, steps) -> list[int]
+A stepper may say `stepper.max_rows_per_step`: the most tokens one step takes.  Prompts that together bring more
+are fed in portions, step after step, before the first token is chosen (`prefill`); the step function gives the
+same logits however the tokens are cut.
 A stepper may also offer
     stepper.select_async(logits, params, request_indices, steps) -> selection with `result() -> list[int]`,
         `device_rows` and `take(positions)`
@@ -115,6 +118,51 @@ def generate(stepper, prompts: list, max_new_tokens, sampling=None, stop_token_i
     return results
 
 
+def prefill_portions(prompt_lens: list, max_rows: int | None) -> list:
+    """How the prompts of a batch go through steps of at most `max_rows` tokens: a list of steps, each a list of
+    (index into the batch, first token, tokens).  Prompts are taken in order; a step is filled before the next
+    one starts, so a prompt may be cut where a step is full."""
+    if not max_rows or sum(prompt_lens) <= max_rows:
+        return [[(index, 0, n) for index, n in enumerate(prompt_lens)]]
+    steps, current, room = [], [], max_rows
+    for index, n in enumerate(prompt_lens):
+        fed = 0
+        while fed < n:
+            take = min(n - fed, room)
+            current.append((index, fed, take))
+            fed += take
+            room -= take
+            if room == 0:
+                steps.append(current)
+                current, room = [], max_rows
+    if current:
+        steps.append(current)
+    return steps
+
+
+def prefill(stepper, slots: list, prompts: list, control=None):
+    """Feed every prompt whole, in as many steps as `stepper.max_rows_per_step` asks for; returns the logits of
+    each prompt's last token, one row per prompt in order."""
+    plan = prefill_portions([len(p) for p in prompts], getattr(stepper, "max_rows_per_step", None))
+    if len(plan) == 1:
+        return stepper.step([StepEntry(slot, list(prompt), [len(prompt) - 1]) for slot, prompt in zip(slots, prompts)])
+    import torch
+    rows = [None] * len(prompts)
+    for number, portion in enumerate(plan):
+        if number and control is not None:
+            control()
+        entries, ending = [], []
+        for index, first, count in portion:
+            last = first + count == len(prompts[index])
+            entries.append(StepEntry(slots[index], list(prompts[index][first:first + count]), [count - 1] if last else []))
+            if last:
+                ending.append(index)
+        logits = stepper.step(entries)
+        for row, index in enumerate(ending):
+            rows[index] = logits[row]
+    return torch.stack(rows)
+
+
 def _run_batch(stepper, batch, prompts, max_new, params, stops, on_token, control, results, on_logits):
     if on_logits is None and hasattr(stepper, "select_async"):
         return _run_batch_ahead(stepper, batch, prompts, max_new, params, stops, on_token, control, results)
@@ -125,7 +173,7 @@ def _run_batch(stepper, batch, prompts, max_new, params, stops, on_token, contro
         if control is not None:
             control()
         live = list(batch)
-        logits = stepper.step([StepEntry(slots[i], list(prompts[i]), [len(prompts[i]) - 1]) for i in live])
+        logits = prefill(stepper, [slots[i] for i in live], [prompts[i] for i in live], control)
         step = 0
         while live:
             tokens = stepper.select(logits, [params[i] for i in live], live, [step] * len(live))
@@ -175,7 +223,7 @@ def _run_batch_ahead(stepper, batch, prompts, max_new, params, stops, on_token, 
         if control is not None:
             control()
         live = list(batch)
-        logits = stepper.step([StepEntry(slots[i], list(prompts[i]), [len(prompts[i]) - 1]) for i in live])
+        logits = prefill(stepper, [slots[i] for i in live], [prompts[i] for i in live], control)
         step = 0
         chosen = stepper.select_async(logits, [params[i] for i in live], live, [step] * len(live))
         while live:

@@ -30,7 +30,8 @@ PAGE_BUCKET = 16      # page-table widths are rounded up to a multiple of this m
 
 
 class DecodeGraph:
-    def __init__(self, engine, n_seqs: int, table_width: int):
+    def __init__(self, engine, n_seqs: int, table_width: int, pool=None):
+        self.pool = pool
         # the engine owns its graphs; they point back weakly, so that an engine nobody holds any more is
         # freed at once and not by a later garbage collection
         self.engine, self.n_seqs, self.table_width = _weakly(engine), n_seqs, table_width
@@ -97,7 +98,7 @@ class DecodeGraph:
             collecting = gc.isenabled()
             gc.disable()
             try:
-                with torch.cuda.graph(graph):
+                with torch.cuda.graph(graph, pool=self.pool):
                     self.logits = self._forward()
             finally:
                 if collecting:
@@ -120,8 +121,12 @@ class DecodeGraphs:
     """The graphs of one engine, by (sequences, page-table width)."""
 
     def __init__(self, engine, limit: int = 48):
-        self.engine, self.limit = _weakly(engine), limit
+        self.engine, self.limit = _weakly(engine), max(int(limit), 1)
         self.graphs: dict = {}
+        # One pool of device memory for all captures of the engine: only one of them runs at a time, on one
+        # stream, so the temporaries of one step may stand where another's stood; what a capture returns (its
+        # logits) stays its own for as long as the capture lives.
+        self.pool = torch.cuda.graph_pool_handle()
 
     def usable(self, ctx_entries) -> bool:
         model = self.engine.model
@@ -139,7 +144,7 @@ class DecodeGraphs:
         if graph is None:
             if len(self.graphs) >= self.limit:
                 self.graphs.pop(next(iter(self.graphs)))        # the least recently used
-            graph = DecodeGraph(self.engine, *key)
+            graph = DecodeGraph(self.engine, *key, pool=self.pool)
         self.graphs[key] = graph
         graph.fill(entries, pasts)
         return graph.run()

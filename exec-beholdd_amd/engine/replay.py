@@ -17,7 +17,8 @@ import sys
 import numpy as np
 
 from .engine import Engine
-from .step import StepEntry
+from ..cache.sequence_cache import CacheError
+from .step import StepEntry, StepError
 
 
 class TraceError(ValueError):
@@ -102,6 +103,19 @@ class Replayer:
             raise TraceError(f"'step' must be a non-negative integer, got {step!r}")
         if step in self.steps_seen:
             raise TraceError(f"step {step} occurs twice")
+        if not isinstance(record["entries"], list) or not isinstance(record.get("end", []), list):
+            raise TraceError(f"step {step}: 'entries' and 'end' are lists")
+        seen = set()
+        for index, item in enumerate(record["entries"]):      # refuse a malformed entry before anything is started
+            if not isinstance(item, dict) or "id" not in item or "tokens" not in item:
+                raise TraceError(f"step {step}: entry {index} is an object with 'id' and 'tokens' (and maybe 'want')")
+            if not isinstance(item["id"], (str, int)) or isinstance(item["id"], bool):
+                raise TraceError(f"step {step}: entry {index}: 'id' is a string or an integer, got {item['id']!r}")
+            if not isinstance(item["tokens"], list) or not isinstance(item.get("want", []), list):
+                raise TraceError(f"step {step}: entry {index} (request {item['id']!r}): 'tokens' and 'want' are lists")
+            if item["id"] in seen:
+                raise TraceError(f"step {step}: request {item['id']!r} occurs twice")
+            seen.add(item["id"])
         entries, fresh, places = [], [], []
         for item in record["entries"]:
             name = item["id"]
@@ -164,7 +178,7 @@ def main(argv=None, stdin=None, stdout=None) -> int:
                 return 1
             try:
                 replayer.run_step(record)
-            except TraceError as error:
+            except (TraceError, StepError, CacheError) as error:      # a refused step: its reason, not a traceback
                 print(f"trace_run: {error}", file=sys.stderr)
                 return 1
             print(f"done {record['step']}", file=stdout, flush=True)

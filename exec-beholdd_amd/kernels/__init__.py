@@ -1,6 +1,6 @@
 """The gfx950 kernel library and its Python binding."""
 
-from .library import HipKernels, KernelError, NormedRows, PackedWeight
+from .library import HipKernels, KernelError, KernelSizes, NormedRows, PackedWeight
 from . import build
 
-__all__ = ["HipKernels", "KernelError", "NormedRows", "PackedWeight", "build"]
+__all__ = ["HipKernels", "KernelError", "KernelSizes", "NormedRows", "PackedWeight", "build"]

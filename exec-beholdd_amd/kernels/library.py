@@ -91,15 +91,20 @@ def _code(tensor, what: str) -> int:
     return code
 
 
-class HipKernels:
-    """The kernel set of the product path."""
+ALLOCATION_UNIT = 512     # torch's allocator hands out device memory in multiples of this many bytes
 
-    def __init__(self, device="cuda:0", verbose_build: bool = True):
-        if not torch.cuda.is_available():
-            raise KernelError("no GPU is visible to this process: the HIP kernel library has no CPU fallback")
-        self.device = torch.device(device)
-        if self.device.type != "cuda":
-            raise KernelError(f"the HIP kernel library runs on a GPU, not on {device!r}")
+
+def _rounded(n_bytes: int) -> int:
+    return -(-int(n_bytes) // ALLOCATION_UNIT) * ALLOCATION_UNIT
+
+
+class KernelSizes:
+    """What the kernels allocate beside their inputs and outputs, from sizes alone: the library's own host-side
+    answers (how a product cuts K into parts, how an attention call splits its keys, in what blocks a matrix
+    lies), which need the built library but no GPU.  The engine's byte plan asks here before anything is
+    allocated; `HipKernels` is one of these and launches as well."""
+
+    def __init__(self, verbose_build: bool = True):
         path = _build.ensure_built(verbose=verbose_build)
         try:
             self.lib = ctypes.CDLL(path)
@@ -107,10 +112,6 @@ class HipKernels:
             raise KernelError(f"cannot load the HIP kernel library {path}: {error}") from None
         self.library_path = path
         self._declare()
-        self.page_size = int(self.lib.bh_page_size())
-        if self.page_size != _build.source_page_size():
-            raise KernelError(f"{path} was built for pages of {self.page_size} tokens, the sources say "
-                              f"{_build.source_page_size()}: build the library again")
 
     # ---- ctypes declarations ----
     def _declare(self):
@@ -149,6 +150,75 @@ class HipKernels:
         for query in (lib.bh_gemm_bf16_norm_blocks, lib.bh_gemm_bf16_takes_norm, lib.bh_gemm_bf16_turns_blocks,
                       lib.bh_gemm_bf16_reads_blocked, lib.bh_gemm_bf16_writes_blocked):
             query.argtypes, query.restype = [i, i, i, i, i], ctypes.c_int
+
+    def rows_bytes(self, rows, width, act_size, reader_outputs=None, reader_swiglu=False, reader_packed=True) -> int:
+        """Bytes of the matrix that `new_rows` hands out for these arguments."""
+        rows, width = int(rows), int(width)
+        if reader_outputs is not None and reader_packed and act_size == 2 and width % 64 == 0:
+            block_rows = int(self.lib.bh_gemm_bf16_reads_blocked(rows, int(reader_outputs), width, 1, int(bool(reader_swiglu))))
+            if block_rows:
+                return _rounded(BlockedRows.padded_rows(rows, block_rows) * width * 2)
+        return _rounded(rows * width * act_size)
+
+    def gemm_working_bytes(self, m, n, k, act_size, packed=True, swiglu=False, then_norm=False) -> int:
+        """Bytes that `gemm` (or `gemm_swiglu`) of these sizes allocates for the length of the call or returns
+        as a prepared norm: partial sums of K in parts, the rows and sums of a norm behind it, a regrouped copy
+        of activations that came in another form than the product reads, SwiGLU's two halves where the fused
+        epilogue does not apply."""
+        m, n, k = int(m), int(n), int(k)
+        if act_size != 2 or k % 8:
+            return _rounded(m * 2 * n * act_size) if swiglu else 0
+        sizes = (m, n, k, int(bool(packed)), int(bool(swiglu)))
+        total = _rounded(int(self.lib.bh_gemm_bf16_scratch(*sizes)))
+        if k % 32 == 0:
+            total += 2 * _rounded(BlockedRows.padded_rows(m, 16) * k * 2)      # regrouping: out of blocks, into others
+        if then_norm:
+            blocks = max(int(self.lib.bh_gemm_bf16_norm_blocks(*sizes)), 1)
+            total += _rounded(BlockedRows.padded_rows(m, 16) * n * 2) + _rounded(m * blocks * 4)
+        if swiglu and n % 16:
+            total += _rounded(m * 2 * n * act_size)
+        return total
+
+    def attention_working_bytes(self, n_rows, n_seqs, max_rows_per_seq, n_heads, n_kv_heads, head_dim, max_position,
+                                act_size) -> int:
+        """Bytes that an attention call allocates: the partial results of its key splits."""
+        if act_size != 2 or head_dim % 32 or head_dim > 256:
+            return 0
+        n_splits = int(self.lib.bh_attention_bf16_splits(int(n_seqs), int(max_rows_per_seq), int(n_heads), int(n_kv_heads),
+                                                         int(max_position)))
+        if n_splits <= 1:
+            return 0
+        return _rounded(n_rows * n_heads * n_splits * head_dim * 4) + _rounded(n_rows * n_heads * n_splits * 2 * 4)
+
+    def sample_working_bytes(self, n_rows, vocab) -> int:
+        return _rounded(int(self.lib.bh_sample_scratch(int(n_rows), int(vocab))) * 4) + 4 * _rounded(n_rows * 4)
+
+    def packs(self, rows, cols, act_size) -> bool:
+        """Whether `pack_weight` regroups a matrix of this shape and element size."""
+        return act_size == 2 and cols % 64 == 0
+
+    def packed_bytes(self, rows, cols, act_size) -> int:
+        """Device bytes of a weight matrix as `pack_weight` keeps it (rows padded to whole blocks of 16)."""
+        if self.packs(rows, cols, act_size):
+            return _rounded(-(-rows // 16) * 16 * cols * 2)
+        return _rounded(rows * cols * act_size)
+
+
+class HipKernels(KernelSizes):
+    """The kernel set of the product path."""
+
+    def __init__(self, device="cuda:0", verbose_build: bool = True):
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible to this process: the HIP kernel library has no CPU fallback")
+        self.device = torch.device(device)
+        if self.device.type != "cuda":
+            raise KernelError(f"the HIP kernel library runs on a GPU, not on {device!r}")
+        super().__init__(verbose_build)
+        self.page_size = int(self.lib.bh_page_size())
+        if self.page_size != _build.source_page_size():
+            raise KernelError(f"{self.library_path} was built for pages of {self.page_size} tokens, the sources say "
+                              f"{_build.source_page_size()}: build the library again")
+
     # ---- helpers ----
     def _stream(self):
         return ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)

@@ -75,6 +75,26 @@ class DecoderModel:
             if hasattr(part, "prepare"):
                 part.prepare(kernels)
 
+    def working_bytes(self, step) -> int:
+        """Bytes a step of these sizes allocates at its peak: the residual, the widest layer (a layer's
+        temporaries are freed before the next one runs; what a block prepares for the next is counted with
+        the block that made it), the final norm on the wanted rows and the logits."""
+        total = self.embedding.working_bytes(step) if hasattr(self.embedding, "working_bytes") else 0
+        widest = max([block.working_bytes(step) for block in self.blocks if hasattr(block, "working_bytes")], default=0)
+        last = 0
+        if hasattr(self.final_norm, "working_bytes"):
+            last += self.final_norm.working_bytes(step, rows=step.wanted)
+        if hasattr(self.head, "working_bytes"):
+            last += self.head.working_bytes(step)
+        return total + widest + last
+
+    def unaccounted_parts(self) -> list:
+        """Names of parts that do not say what their forward allocates (the byte plan lists them)."""
+        names = [type(part).__name__ for part in (self.embedding, self.final_norm, self.head) if not hasattr(part, "working_bytes")]
+        for block in self.blocks:
+            names += block.unaccounted_parts() if hasattr(block, "unaccounted_parts") else [type(block).__name__]
+        return sorted(set(names))
+
     def forward(self, ctx, cache_for_run, want_rows):
         """Run one step.  `cache_for_run(i)` gives the LayerCache of the i-th scheduled run (or
         None); `want_rows` (int32 device tensor, may be empty) lists the rows whose logits are

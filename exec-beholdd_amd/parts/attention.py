@@ -72,6 +72,16 @@ class GQAAttention:
     def cache_need(self):
         return CacheNeed(kind="kv", kv_heads=self.n_kv_heads, head_dim=self.head_dim, window=self.window)
 
+    def working_bytes(self, step) -> int:
+        q_width = self.n_heads * self.head_dim
+        total = self.qkv.working_bytes(step, step.rows)
+        total += step.matrix(step.rows, q_width, reader=self.out.reader_for_plan(step.act_size))     # attended
+        total += step.matrix(step.rows, q_width)                                                     # normed, rotated queries
+        if step.sizes is not None:
+            total += step.sizes.attention_working_bytes(step.rows, step.seqs, step.max_rows_per_seq, self.n_heads,
+                                                        self.n_kv_heads, self.head_dim, step.max_position, step.act_size)
+        return total + self.out.working_bytes(step, step.rows, accumulate=True, then_norm=True)
+
     def forward(self, ctx, x, hidden, cache, then_norm=None):
         k = ctx.kernels
         qkv = self.qkv.forward(ctx, x)

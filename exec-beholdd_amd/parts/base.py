@@ -42,6 +42,8 @@ A mixer with a "state" cache need updates its rows of `cache.state` in place whi
 what the step's sequences held before the step and puts it back if the step fails, so a mixer needs no
 second bank; and the engine runs a part's forward exactly once per step, whether the step is launched kernel
 by kernel or replayed from a capture, so a state advances once per token.
+Every part may say what its forward allocates: working_bytes(step: StepSize) -> int, from sizes alone; the
+engine's byte plan adds them up before anything is allocated and names the parts that do not say.
 A part may declare `graph_safe = True`: its forward uses only the device tensors of the step
 context (never the host_* lists, never a host-side decision that changes from step to step).
 Decode steps of a model whose parts all say so are captured and replayed as HIP graphs.
@@ -126,6 +128,35 @@ class StepContext:
 
     def new_f32(self, *shape) -> torch.Tensor:
         return torch.empty(shape, dtype=torch.float32, device=self.device)
+
+
+@dataclass
+class StepSize:
+    """The sizes of a step, for the byte plan: a part's optional `working_bytes(step)` answers from them how many
+    bytes its `forward` allocates in such a step (its output included), before anything is allocated.  `sizes`
+    is the kernel library's own account of what its calls allocate (`kernels.KernelSizes`), or None for a
+    stepper without one."""
+    rows: int
+    seqs: int
+    wanted: int
+    act_size: int
+    max_position: int
+    max_rows_per_seq: int
+    sizes: object | None = None
+
+    def matrix(self, rows: int, width: int, element_size: int | None = None, reader=None) -> int:
+        """Bytes of a matrix as `StepContext.new_activations` / `new_f32` hand it out."""
+        size = self.act_size if element_size is None else element_size
+        if reader is not None and self.sizes is not None and size == self.act_size:
+            return self.sizes.rows_bytes(rows, width, size, reader.outputs, reader.swiglu, getattr(reader, "packed", True))
+        return -(-int(rows) * int(width) * size // 512) * 512
+
+    def product(self, rows: int, outputs: int, inputs: int, packed: bool = True, swiglu: bool = False,
+                then_norm: bool = False) -> int:
+        """Bytes that a matrix product of the kernel library allocates beside its output."""
+        if self.sizes is None:
+            return 0
+        return self.sizes.gemm_working_bytes(rows, outputs, inputs, self.act_size, packed, swiglu, then_norm)
 
 
 @dataclass

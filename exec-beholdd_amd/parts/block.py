@@ -34,6 +34,19 @@ class PreNormBlock:
             if hasattr(part, "prepare"):
                 part.prepare(kernels)
 
+    def working_bytes(self, step) -> int:
+        """Everything the four parts allocate, as if nothing were freed before the layer ends."""
+        total = 0
+        for norm, consumer in ((self.mixer_norm, self.mixer), (self.feed_forward_norm, self.feed_forward)):
+            if hasattr(norm, "working_bytes"):
+                total += norm.working_bytes(step)
+            if hasattr(consumer, "working_bytes"):
+                total += consumer.working_bytes(step)
+        return total
+
+    def unaccounted_parts(self) -> list:
+        return [type(part).__name__ for part in self.parts() if not hasattr(part, "working_bytes")]
+
     def cache_need(self):
         return self.mixer.cache_need()
 

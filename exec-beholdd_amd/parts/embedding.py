@@ -26,6 +26,9 @@ class Embedding:
     def load(self, get):
         self.weight = get(self.name)
 
+    def working_bytes(self, step) -> int:
+        return step.matrix(step.rows, self.width, 4)      # the float32 residual, which lives as long as the step
+
     def forward(self, ctx):
         hidden = ctx.new_f32(ctx.n_rows, self.width)
         if ctx.token_src is not None:
@@ -58,6 +61,9 @@ class LMHead:
     @property
     def input_reader(self):
         return self.linear.reader()    # x goes to that product and nowhere else
+
+    def working_bytes(self, step) -> int:
+        return self.linear.working_bytes(step, step.wanted, out_size=4)
 
     def forward(self, ctx, x):
         """x [n, width] -> float32 logits [n, vocab]."""

@@ -53,6 +53,22 @@ class Linear:
         return ProductReader(self.out_features // 2 if swiglu else self.out_features, swiglu,
                              packed=self.weight is not None and not isinstance(self.weight, torch.Tensor))
 
+    def packs(self, act_size: int) -> bool:
+        """Whether `prepare` regroups this matrix in an engine of that element size."""
+        return not self.shared and act_size == 2 and self.in_features % 64 == 0
+
+    def reader_for_plan(self, act_size: int, swiglu: bool = False) -> ProductReader:
+        """`reader()` as it will be once the weights are loaded and prepared."""
+        return ProductReader(self.out_features // 2 if swiglu else self.out_features, swiglu, packed=self.packs(act_size))
+
+    def working_bytes(self, step, rows: int, out_size: int | None = None, accumulate: bool = False,
+                      then_norm: bool = False, swiglu: bool = False) -> int:
+        """Bytes one product of `rows` rows allocates: its output unless it adds into one, and what the
+        kernel library allocates on the way."""
+        outputs = self.out_features // 2 if swiglu else self.out_features
+        total = 0 if accumulate else step.matrix(rows, outputs, out_size)
+        return total + step.product(rows, outputs, self.in_features, self.packs(step.act_size), swiglu, then_norm)
+
     def prepare(self, kernels):
         """Let the kernel library regroup the matrix into the layout it reads fastest."""
         if not self.shared and hasattr(kernels, "pack_weight"):

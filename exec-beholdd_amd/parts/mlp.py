@@ -36,6 +36,11 @@ class SwiGLU:
         self.gate_up.prepare(kernels)
         self.down.prepare(kernels)
 
+    def working_bytes(self, step) -> int:
+        activated = step.matrix(step.rows, self.intermediate, reader=self.down.reader_for_plan(step.act_size))
+        return (activated + self.gate_up.working_bytes(step, step.rows, accumulate=True, swiglu=True)
+                + self.down.working_bytes(step, step.rows, accumulate=True, then_norm=True))
+
     def forward(self, ctx, x, hidden, then_norm=None):
         activated = ctx.new_activations(x.shape[0], self.intermediate, reader=self.down.reader())
         ctx.kernels.gemm_swiglu(x, self.gate_up.weight, activated)     # both products and the gate in one pass

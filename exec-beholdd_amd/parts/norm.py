@@ -35,6 +35,9 @@ class RMSNorm:
         ctx.kernels.rmsnorm(hidden, self.weight, self.eps, out, rows=rows)
         return out
 
+    def working_bytes(self, step, rows: int | None = None, reader=None) -> int:
+        return step.matrix(step.rows if rows is None else rows, self.width, reader=reader)
+
     def request(self, reader=None):
         """This norm as the product that completes its input may prepare it."""
         return NormRequest(self.weight, self.eps, reader)

@@ -101,10 +101,15 @@ class Sampler:
         self._allocate(int(capacity))
 
     def _allocate(self, capacity):
+        # row 0: tokens, row 1: the not-finite flags.  Captured graphs read row 0; the engine sizes the sampler
+        # for its largest batch, so this buffer is replaced only when a caller selects for more rows than the
+        # engine has slots.  The new buffer then takes over what the old one held (a selection whose tokens
+        # the next step reads on the device stays good), and captures that read the old one are made again.
+        before = getattr(self, "out", None)
         self.capacity = capacity
-        # row 0: tokens, row 1: the not-finite flags.  Captured graphs read row 0, so the engine sizes the
-        # sampler once for its largest batch and this buffer is never replaced under it.
         self.out = torch.zeros((2, capacity), dtype=torch.int32, device=self.device)
+        if before is not None:
+            self.out[:, :before.shape[1]].copy_(before)
         pin = self.device.type == "cuda"
         self._hosts = [torch.zeros((2, capacity), dtype=torch.int32, pin_memory=pin) for _ in range(self.RING)]
         self._turn = 0

@@ -151,15 +151,21 @@ def causal_attention(q, k, v, n_heads, n_kv_heads, head_dim, scale, query_start=
     kh = k.reshape(tk, n_kv_heads, head_dim)
     vh = v.reshape(tk, n_kv_heads, head_dim)
     out = np.zeros((tq, n_heads, head_dim), dtype=F32)
-    for t in range(tq):
-        visible = query_start + t + 1
-        assert visible <= tk, "a query may not stand beyond the keys"
-        for h in range(n_heads):
-            kvh = h // group
-            dots = kh[:visible, kvh, :].astype(F64) @ qh[t, h, :].astype(F64)
+    assert query_start + tq <= tk, "a query may not stand beyond the keys"
+    some = 256        # queries taken together (the arithmetic of each is the same as if it stood alone)
+    for h in range(n_heads):
+        kvh = h // group
+        keys, values = kh[:, kvh, :].astype(F64), vh[:, kvh, :].astype(F64)
+        for t in range(0, tq, some):
+            last = min(t + some, tq)
+            visible = query_start + last                       # keys that the last of these queries sees
+            dots = qh[t:last, h, :].astype(F64) @ keys[:visible].T
             scores = (dots * F64(F32(scale))).astype(F32)
+            # the reference's mask is the loop bound: a key beyond a query's position takes no part
+            beyond = np.arange(visible)[None, :] > (query_start + np.arange(t, last))[:, None]
+            scores[beyond] = -np.inf
             p = softmax(scores)
-            out[t, h, :] = (p.astype(F64) @ vh[:visible, kvh, :].astype(F64)).astype(F32)
+            out[t:last, h, :] = (p.astype(F64) @ values[:visible]).astype(F32)
     return out.reshape(tq, n_heads * head_dim)
 
 
@@ -274,26 +280,28 @@ def layer(cfg, w, index, hidden, first_position=0):
     return mlp_block(cfg, w, prefix, hidden)
 
 
-def head(cfg, w, hidden):
+def head(cfg, w, hidden, rows=None):
     """Final RMSNorm then the LM head (the embedding itself when tied).
 
     crates/beholdd-model/src/qwen3moe/forward.rs:1416-1455 (there for the last row only;
-    here for every row) and crates/beholdd-model/src/qwen3moe.rs:948-955 (tied head).
+    here for every row, or for the rows asked for) and crates/beholdd-model/src/qwen3moe.rs:948-955 (tied head).
     """
+    if rows is not None:
+        hidden = hidden[np.asarray(rows, dtype=np.int64)]
     xl = rmsnorm(hidden, w["model.norm.weight"], cfg.eps)
     out = w["model.embed_tokens.weight"] if cfg.tied else w["lm_head.weight"]
     return linear(xl, out)
 
 
-def forward_logits(cfg, w, tokens, first_position=0):
-    """Logits [T, vocab] of every position of one whole sequence.
+def forward_logits(cfg, w, tokens, first_position=0, rows=None):
+    """Logits [T, vocab] of every position of one whole sequence (or of the positions `rows`).
 
     crates/beholdd-model/src/qwen3moe/forward.rs:412-436 (the non-cached forward).
     """
     hidden = embed(tokens, w["model.embed_tokens.weight"])
     for index in range(cfg.n_layers):
         hidden = layer(cfg, w, index, hidden, first_position)
-    return head(cfg, w, hidden)
+    return head(cfg, w, hidden, rows)
 
 
 def greedy_generate(cfg, w, prompt, max_new_tokens, stop_tokens=()):

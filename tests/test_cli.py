@@ -68,11 +68,22 @@ def test_plan_only_holds_weights_and_cache_against_the_budget(model_dirs):
     common = ["generate", "--model", model_dirs("B", "float32"), "--prompt-ids", "1,2,3", "--max-new-tokens", "10",
               "--dtype", "bfloat16", "--plan-only", "--memory-budget-bytes"]
     # stored in 32-bit: stays so in a bfloat16 engine; one page of cache for 3 layers
-    total = 397_152 * 4 + 3 * 2 * 1 * 2 * 64 * 32 * 2
+    code, text = run(common + [str(10 ** 9)])
+    import re
+    items = {m.group(1): int(m.group(2)) for m in (re.match(r"^(\S[^:]*): (\d+) bytes", line) for line in text.splitlines()) if m}
+    assert items["weights"] == 397_152 * 4 and items["cache"] == 3 * 2 * 1 * 2 * 64 * 32 * 2
+    # the plan goes beyond weights and cache: the largest step's working memory, the captured decode steps, the sampler
+    assert any(label.startswith("working memory of a step of 64 rows") and value > 0 for label, value in items.items())
+    assert any(label.startswith("captured decode steps") and value > 0 for label, value in items.items())
+    total = items.pop("total")
+    assert total == sum(items.values()) and total > items["weights"] + items["cache"]
     code, text = run(common + [str(total)])
     assert code == 0 and f"total: {total} bytes (budget {total}: fits)" in text
     code, text = run(common + [str(total - 1)])
     assert code == 1 and "does not fit" in text
+    # fewer rows a step, less working memory
+    code, less = run(common + [str(total), "--max-rows-per-step", "16"])
+    assert code == 0 and "working memory of a step of 16 rows" in less
 
 
 def test_random_model_command_writes_a_loadable_folder(tmp_path, tiny_configs):
@@ -129,6 +140,14 @@ def test_trace_replay_on_the_kernel_double(model_dirs, tmp_path):
         with pytest.raises(replay.TraceError, match=message):
             player.run_step({"step": bad, "entries": [{"id": "d", "tokens": [1], "want": [0]}], "end": ["d"]})
     assert engine.cache.live_slots() == []
+    # malformed entries are refused with a reason before any request is started
+    for entries, message in (([{"tokens": [1]}], "'id' and 'tokens'"), ([{"id": "e"}], "'id' and 'tokens'"), (["e"], "'id' and 'tokens'"),
+                             ([{"id": "e", "tokens": 3}], "are lists"), ([{"id": "e", "tokens": [1], "want": 0}], "are lists"),
+                             ([{"id": ["e"], "tokens": [1]}], "a string or an integer"),
+                             ([{"id": "e", "tokens": [1]}, {"id": "e", "tokens": [2]}], "occurs twice"), ("e", "are lists")):
+        with pytest.raises(replay.TraceError, match=message):
+            player.run_step({"step": 6, "entries": entries, "end": []})
+        assert engine.cache.live_slots() == [] and player.slot_of == {}
     # an id that is used again after its request ended is another request in the capture
     player.run_step({"step": 5, "entries": [{"id": "a", "tokens": b, "want": [1]}], "end": ["a"]})
     player.close()

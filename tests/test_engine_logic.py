@@ -123,12 +123,28 @@ def test_memory_limit_covers_weights_and_cache_and_is_checked_before_anything_is
     reads = []
     real = binder.BoundWeights.__call__
     monkeypatch.setattr(binder.BoundWeights, "__call__", lambda self, name: reads.append(name) or real(self, name))
-    with pytest.raises(MemoryBudgetError, match=f"need {weights + cache} bytes"):
-        make_engine(folder, dtype="bfloat16", max_tokens=128, memory_limit_bytes=weights + cache - 1)
+    # the plan holds weights and cache, and beyond them what a step of as many rows as the cache holds allocates
+    # (the kernel double says nothing about its calls, so the parts' own matrices only)
+    with pytest.raises(MemoryBudgetError, match="the engine needs") as refused:
+        make_engine(folder, dtype="bfloat16", max_tokens=128, memory_limit_bytes=weights + cache)
+    assert reads == [] and f"weights: {weights} bytes" in str(refused.value) and f"cache: {cache} bytes" in str(refused.value)
+    total = int(str(refused.value).split("the engine needs ")[1].split()[0])
+    assert total > weights + cache
+    with pytest.raises(MemoryBudgetError):
+        make_engine(folder, dtype="bfloat16", max_tokens=128, memory_limit_bytes=total - 1)
     assert reads == []
-    engine = make_engine(folder, dtype="bfloat16", max_tokens=128, memory_limit_bytes=weights + cache)
+    engine = make_engine(folder, dtype="bfloat16", max_tokens=128, memory_limit_bytes=total)
     assert len(reads) == 24 and engine.weight_bytes == weights and engine.cache.allocated_bytes() == cache
-    assert f"weights: {weights} bytes" in engine.memory_plan()
+    assert f"weights: {weights} bytes" in engine.memory_plan() and engine.plan.total_bytes == total
+    assert engine.max_rows_per_step == 128
+    assert engine.plan.bytes_of("working memory of a step of 128 rows") > 128 * 64 * 4
+    smaller = make_engine(folder, dtype="bfloat16", max_tokens=128, max_rows_per_step=16)
+    assert smaller.plan.bytes_of("working memory of a step of 16 rows") < engine.plan.bytes_of("working memory of a step of 128 rows") / 4
+    slot = smaller.alloc_slot()
+    with pytest.raises(beholdd.engine.step.StepError, match="max_rows_per_step"):
+        smaller.step([beholdd.StepEntry(slot, list(range(17)), [16])])
+    assert smaller.cache.length(slot) == 0
+    smaller.step([beholdd.StepEntry(slot, list(range(16)), [15])])
 
 
 def test_unknown_architecture_names_the_registered_ones(tmp_path, tiny_configs):

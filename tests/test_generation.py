@@ -281,3 +281,60 @@ def test_the_loop_ahead_batches_errors_and_limits():
     looked = []
     generate(s, [[1], [2]], 3, on_logits=lambda i, step, row: looked.append((i, step)))
     assert s.results_read == 0 and looked == [(0, 0), (1, 0), (0, 1), (1, 1), (0, 2), (1, 2)]
+
+
+def test_prompts_beyond_a_step_are_fed_in_portions():
+    from beholdd.engine.generation import prefill_portions
+    assert prefill_portions([5, 11, 17], None) == [[(0, 0, 5), (1, 0, 11), (2, 0, 17)]]
+    assert prefill_portions([5, 11, 17], 33) == [[(0, 0, 5), (1, 0, 11), (2, 0, 17)]]
+    plan = prefill_portions([5, 11, 17], 8)
+    assert plan == [[(0, 0, 5), (1, 0, 3)], [(1, 3, 8)], [(2, 0, 8)], [(2, 8, 8)], [(2, 16, 1)]]
+    for lens, cap in (([1, 1, 1], 1), ([40, 3, 29, 64], 16), ([7], 3)):
+        plan = prefill_portions(lens, cap)
+        assert all(0 < sum(count for _, _, count in step) <= cap for step in plan)
+        for index, n in enumerate(lens):       # every prompt whole, in order, each token once
+            pieces = [(first, count) for step in plan for i, first, count in step if i == index]
+            assert pieces[0][0] == 0 and sum(count for _, count in pieces) == n
+            assert all(a[0] + a[1] == b[0] for a, b in zip(pieces, pieces[1:]))
+
+
+class PortionStepper(ScriptedStepper):
+    """The scripted stepper with a limit on a step's tokens: prompts arrive in portions, and a sequence's next
+    token is asked for only with the portion that ends its prompt."""
+
+    def __init__(self, max_rows_per_step, **kw):
+        super().__init__(**kw)
+        self.max_rows_per_step = max_rows_per_step
+        self.fed = {}
+
+    def step(self, entries):
+        assert sum(len(e.tokens) for e in entries) <= self.max_rows_per_step
+        rows = []
+        for e in entries:
+            started = self.state[e.slot]
+            if started is None or started[2]:       # still in its prompt
+                first = e.tokens[0] if started is None else started[0]
+                length = len(e.tokens) + (0 if started is None else started[1])
+                self.state[e.slot] = (first, length, not e.want)
+            else:
+                first, length, _ = started
+                assert e.tokens == [self.next_token(first, length)] and e.want == [0]
+                self.state[e.slot] = (first, length + 1, False)
+            if e.want:
+                assert e.want == [len(e.tokens) - 1]
+                first, length, _ = self.state[e.slot]
+                row = torch.zeros(self.vocab)
+                row[self.next_token(first, length)] = 5.0
+                rows.append(row)
+        self.steps.append([(e.slot, len(e.tokens)) for e in entries])
+        return torch.stack(rows) if rows else None
+
+
+def test_generation_with_a_limit_on_a_steps_tokens():
+    prompts = [[3] * 5, [9] * 11, [4] * 17, [6]]
+    s = PortionStepper(8)
+    results = generate(s, prompts, [4, 2, 3, 5])
+    for prompt, result, n in zip(prompts, results, [4, 2, 3, 5]):
+        assert result.token_ids == expected_tokens(s, prompt, n)
+    assert s.steps[:6] == [[(0, 5), (1, 3)], [(1, 8)], [(2, 8)], [(2, 8)], [(2, 1), (3, 1)], [(0, 1), (1, 1), (2, 1), (3, 1)]]
+    assert s.state == {}

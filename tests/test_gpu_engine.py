@@ -583,3 +583,32 @@ def test_command_line_generate(model_dirs, tmp_path):
     full = plain.forward_logits(cfg, weights, prompt + want[:-1])
     assert schedules.relative_error(logits, full[len(prompt) - 1:]) < 1e-4
     assert timing.read_text().splitlines()[0] == "step\tduration_ms"
+
+
+def test_command_line_generate_without_captures(model_dirs):
+    """`beholdd generate` in bfloat16 with three prompts and a temperature, no capture flags: the loop that runs a
+    step ahead of the host, no per-step lines; the tokens are those `Engine.generate` draws with the same seed."""
+    import re
+
+    import beholdd
+    folder, cfg, weights, prompts, _, _ = _varied(model_dirs)
+    prompts = prompts[1:]
+    command = [sys.executable, os.path.join(ROOT, "bin", "beholdd"), "generate", "--model", folder, "--dtype", "bfloat16",
+               "--max-new-tokens", "10", "--temperature", "0.7", "--top-k", "30", "--seed", "9", "--max-tokens", "512"]
+    for prompt in prompts:
+        command += ["--prompt-ids", ",".join(str(t) for t in prompt)]
+    run = subprocess.run(command, capture_output=True, text=True, timeout=600)
+    assert run.returncode == 0, run.stderr[-2000:]
+    engine = beholdd.Engine(folder, dtype="bfloat16", max_tokens=512)
+    want = engine.generate(prompts, max_new_tokens=10, temperature=0.7, top_k=30, seed=9)
+    printed = re.findall(r"generated: (\[.*\])", run.stdout)
+    assert [json.loads(text) for text in printed] == [r.token_ids for r in want]
+    assert len({tuple(r.token_ids) for r in want}) == 3 and all(len(r.token_ids) == 10 for r in want)
+    assert "step   0" not in run.stdout and "generated tokens/s" in run.stdout
+    # every drawn token had a chance by the plain implementation's logits
+    for prompt, result in zip(prompts, want):
+        tokens = list(prompt)
+        for token in result.token_ids:
+            logits = plain.forward_logits(cfg, weights, tokens)[-1]
+            assert logits[token] >= np.sort(logits)[-30] - TOLERANCE["bfloat16"] * np.abs(logits).max()
+            tokens.append(token)
