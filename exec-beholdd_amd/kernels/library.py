@@ -214,6 +214,10 @@ class HipKernels(KernelSizes):
         if self.device.type != "cuda":
             raise KernelError(f"the HIP kernel library runs on a GPU, not on {device!r}")
         super().__init__(verbose_build)
+        self._device_index = self.device.index if self.device.index is not None else torch.cuda.current_device()
+        self.device = torch.device("cuda", self._device_index)
+        self._raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+        self._plans: dict = {}      # (m, n, k, packed, activation) -> what the library says of such a product
         self.page_size = int(self.lib.bh_page_size())
         if self.page_size != _build.source_page_size():
             raise KernelError(f"{self.library_path} was built for pages of {self.page_size} tokens, the sources say "
@@ -221,13 +225,20 @@ class HipKernels(KernelSizes):
 
     # ---- helpers ----
     def _stream(self):
-        return ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+        """The current HIP stream of the device as a raw handle (asked of torch without building a stream object:
+        a step makes a few hundred launches)."""
+        if self._raw_stream is not None:
+            return self._raw_stream(self._device_index)
+        return torch.cuda.current_stream(self.device).cuda_stream
 
     def _check(self, status: int):
         if status != 0:
             raise KernelError(self.lib.bh_last_error().decode("utf-8", "replace"))
 
     def _ptr(self, tensor, what: str, dtypes=None, optional: bool = False):
+        if type(tensor) is torch.Tensor and tensor.device == self.device and tensor.is_contiguous() \
+                and (dtypes is None or tensor.dtype in dtypes):
+            return tensor.data_ptr()
         if tensor is None:
             if optional:
                 return None
@@ -248,7 +259,21 @@ class HipKernels(KernelSizes):
             raise KernelError(f"{what}: tensor must be contiguous")
         if dtypes is not None and tensor.dtype not in dtypes:
             raise KernelError(f"{what}: dtype {tensor.dtype} is not one of {dtypes}")
-        return ctypes.c_void_p(tensor.data_ptr())
+        return tensor.data_ptr()
+
+    def _product(self, m, n, k, packed, activation):
+        """What the library says of a product of these sizes, asked once per shape: (blocks its activations are
+        read in, blocks it writes, whether it takes prepared norm rows, the blocks of a norm behind it, scratch
+        bytes, whether its finishing kernel finishes a norm)."""
+        key = (m, n, k, packed, activation)
+        plan = self._plans.get(key)
+        if plan is None:
+            lib = self.lib
+            plan = self._plans[key] = (
+                int(lib.bh_gemm_bf16_reads_blocked(*key)), int(lib.bh_gemm_bf16_writes_blocked(*key)),
+                bool(lib.bh_gemm_bf16_takes_norm(*key)) if k % 8 == 0 else False, int(lib.bh_gemm_bf16_norm_blocks(*key)),
+                int(lib.bh_gemm_bf16_scratch(*key)), bool(packed and lib.bh_gemm_bf16_finishes_norm(m, n, k, 1)))
+        return plan
 
     # ---- kernels ----
     def embed(self, tokens, table, out, token_src=None, fed_tokens=None):
@@ -290,7 +315,7 @@ class HipKernels(KernelSizes):
         and reads them faster, the matrix is one."""
         rows, width = int(rows), int(width)
         if reader_outputs is not None and reader_packed and dtype == torch.bfloat16 and width % 64 == 0:
-            block_rows = int(self.lib.bh_gemm_bf16_reads_blocked(rows, int(reader_outputs), width, 1, int(bool(reader_swiglu))))
+            block_rows = self._product(rows, int(reader_outputs), width, 1, int(bool(reader_swiglu)))[0]
             if block_rows:
                 return self._new_blocked(rows, width, block_rows)
         return torch.empty((rows, width), dtype=dtype, device=self.device)
@@ -355,28 +380,29 @@ class HipKernels(KernelSizes):
         m, k = a.shape
         n = out.shape[1]
         sizes = (m, n, k, int(packed), int(activation))
+        a_block_rows, writes, takes_norm, norm_blocks, scratch_bytes, finishes_norm = self._product(*sizes)
+        if a_block_rows == 16 and m > 32 and not scratch_bytes and (ahead is not None or (accumulate and out.dtype != torch.float32)):
+            a_block_rows = 0      # the kernel for many rows that reads blocks does not take these operands; the tiles read rows
         # the activations in the form this product reads: whoever produced them for this reader wrote them so
-        a_block_rows = int(self.lib.bh_gemm_bf16_reads_blocked(*sizes))
         if ahead is not None:
             if _block_rows(ahead.rows) != a_block_rows:
                 ahead = NormedRows(self._in_blocks_of(ahead.rows, a_block_rows), ahead.ss, ahead.eps, ahead.source, ahead.weight)
         else:
             a = self._in_blocks_of(a, a_block_rows)
-        writes = int(self.lib.bh_gemm_bf16_writes_blocked(*sizes))     # 2: any blocks, 1: SwiGLU's in blocks of 16, 0: rows
-        c_block_rows = _block_rows(out)
+        c_block_rows = _block_rows(out)       # writes 2: any blocks, 1: SwiGLU's in blocks of 16, 0: rows
         if c_block_rows and not (activation and (writes == 2 or (writes == 1 and c_block_rows == 16))):
             return False, None      # the caller regroups
         if ahead is not None and (ahead.ss.shape[0] != m or ahead.ss.dtype != torch.float32
-                                  or not self.lib.bh_gemm_bf16_takes_norm(*sizes)):
+                                  or not takes_norm):
             raise KernelError(f"gemm: a product of {m} x {n} x {k} does not take these prepared norm rows")
         if (then_norm is not None and ahead is None and accumulate and packed and out.dtype == torch.float32
                 and not activation and then_norm.weight.shape == (n,) and then_norm.weight.dtype in _CODES
-                and self.lib.bh_gemm_bf16_finishes_norm(m, n, k, 1)):
+                and finishes_norm):
             # many rows, K in parts: the finishing kernel owns whole rows and finishes the norm itself
             normed = self.new_rows(m, n, torch.bfloat16, *self._reader_of(then_norm))
             if _block_rows(normed) not in (0, 16):
                 normed = torch.empty((m, n), dtype=torch.bfloat16, device=self.device)
-            scratch = torch.empty(int(self.lib.bh_gemm_bf16_scratch(*sizes)) // 4, dtype=torch.float32, device=self.device)
+            scratch = torch.empty(scratch_bytes // 4, dtype=torch.float32, device=self.device)
             self._check(self.lib.bh_gemm_bf16_then_norm(
                 self._ptr(a, "gemm a"), self._ptr(w.data, "gemm w"), self._ptr(out, "gemm out", (torch.float32,)), m, n, k, 1,
                 self._ptr(then_norm.weight, "norm weight"), _code(then_norm.weight, "norm weight"), float(then_norm.eps),
@@ -386,7 +412,7 @@ class HipKernels(KernelSizes):
         behind = None
         if (then_norm is not None and out.dtype == torch.float32 and not activation
                 and then_norm.weight.shape == (n,) and then_norm.weight.dtype in _CODES):
-            blocks = int(self.lib.bh_gemm_bf16_norm_blocks(*sizes))      # 0: this product carries no norm
+            blocks = norm_blocks      # 0: this product carries no norm
             if blocks:
                 rows = self.new_rows(m, n, torch.bfloat16, *self._reader_of(then_norm)) if writes == 2 else \
                     torch.empty((m, n), dtype=torch.bfloat16, device=self.device)
@@ -394,7 +420,6 @@ class HipKernels(KernelSizes):
                                     out, then_norm.weight)
         a_rows = ahead.rows if ahead is not None else a
         scratch = None       # products of few tiles add up parts of K through scratch memory
-        scratch_bytes = int(self.lib.bh_gemm_bf16_scratch(*sizes))
         if scratch_bytes:
             scratch = torch.empty(scratch_bytes // 4, dtype=torch.float32, device=self.device)
         self._check(fast(
@@ -464,7 +489,7 @@ class HipKernels(KernelSizes):
         """Whether the matrix-core product of these operands applies the row factors of prepared norm rows."""
         m, k = a.shape
         return bool(w.dtype == torch.bfloat16 and k % 8 == 0 and (not activation or n % 16 == 0)
-                    and self.lib.bh_gemm_bf16_takes_norm(m, n, k, int(isinstance(w, PackedWeight)), int(activation)))
+                    and self._product(m, n, k, int(isinstance(w, PackedWeight)), int(activation))[2])
 
     def _run_norm(self, prepared):
         """The norm that `prepared` stands for, as a step of its own."""

@@ -133,6 +133,12 @@ def test_gemm_with_packed_weights(K, m, n, k):
     acc = dev(base.clone())
     K.gemm(dev(a), packed, acc, accumulate=True)
     assert rel(acc, want + base.double()) < f32_bound
+    # adding into a bfloat16 matrix: where the kernel for many rows would read blocks it does not run (it adds
+    # into float32 only), so the product must not be handed blocks
+    base16 = base.to(torch.bfloat16)
+    acc16 = dev(base16.clone())
+    K.gemm(dev(a), packed, acc16, accumulate=True)
+    assert rel(acc16, want + base16.double()) < 8e-3
 
 
 @pytest.mark.parametrize("g_dtype", DTYPES)
