@@ -30,6 +30,7 @@
 //             rows 8*(i/4) + 4*(l/32) + i%4 for i = 0..15
 // Which 8 of the k values a lane group multiplies is free as long as both operands agree.
 #include "common.h"
+#include "gemm_bf16_slices.h"
 #include "gemm_bf16_turns.h"
 #include <algorithm>
 #include <type_traits>
@@ -307,10 +308,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
 #define MAX_TURNS_PARTS 8   // what gemm_turns_parts cuts K into at most
 #define FINISH_COLUMNS 64
 typedef uint16_t u16x4_t __attribute__((ext_vector_type(4)));
+// blocks.c: a SwiGLU's bfloat16 output goes out in blocks of that many rows (bh_rows_index; 0: rows); blocks.behind: so do
+// the rows prepared for a norm behind (a thread's four columns lie in one 16-byte piece of a block).
 template <bool SWIGLU, typename TC>
 __global__ __launch_bounds__(256) void gemm_parts_finish_kernel(const float* __restrict__ sums, TC* __restrict__ c,
                                                                 int M, int N, int K, int parts, int accumulate,
-                                                                RidingNorm norm) {
+                                                                RidingNorm norm, RowBlocks blocks) {
   const int w_rows = SWIGLU ? 2 * N : N;
   const int col = threadIdx.x % 16, n = blockIdx.x * FINISH_COLUMNS + 4 * col, m = blockIdx.y * 16 + threadIdx.x / 16;
   const bool valid = m < M && n < N;
@@ -372,7 +375,7 @@ __global__ __launch_bounds__(256) void gemm_parts_finish_kernel(const float* __r
       u16x4_t packed;
 #pragma unroll
       for (int i = 0; i < 4; ++i) packed[i] = f32_to_bf16_bits(value[i]);
-      *reinterpret_cast<u16x4_t*>(reinterpret_cast<uint16_t*>(c) + at) = packed;
+      *reinterpret_cast<u16x4_t*>(reinterpret_cast<uint16_t*>(c) + (SWIGLU ? (size_t)bh_rows_index(blocks.c, m, n, N) : at)) = packed;
     }
   }
   if (!SWIGLU && norm.behind_weight) {   // float32 output
@@ -387,7 +390,7 @@ __global__ __launch_bounds__(256) void gemm_parts_finish_kernel(const float* __r
                                                : bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(norm.behind_weight)[n + i]);
         rows[i] = f32_to_bf16_bits(value[i] * g);
       }
-      *reinterpret_cast<u16x4_t*>(norm.behind_rows + at) = rows;
+      *reinterpret_cast<u16x4_t*>(norm.behind_rows + (size_t)bh_rows_index(blocks.behind, m, n, N)) = rows;
     }
     if (col == 0 && m < M) norm.behind_ss[(size_t)m * gridDim.x + blockIdx.x] = sq;
   }
@@ -1053,6 +1056,7 @@ static void launch_tiled(const void* a, const void* w, void* c, int M, int N, in
 extern "C" int bh_gemm_bf16_norm_blocks(int M, int N, int K, int layout, int activation) {
   if (activation || M <= 0 || M > NORM_RIDES_UP_TO_ROWS || N <= 0 || K % 8 != 0) return 0;
   int rows, columns, parts, each;
+  if (gemm_slices_takes(M, N, K, layout, 0)) return (N + FINISH_COLUMNS - 1) / FINISH_COLUMNS;   // always finished by that kernel
   tiled_config(M, N, false, &rows, &columns);
   if (!tiled_whole(M, N, K, layout, rows, columns)) return M <= 64 ? (N + 15) / 16 : 0;   // the skinny kernel's blocks
   tiled_parts(M, N, K, layout, false, &parts, &each);
@@ -1073,6 +1077,7 @@ extern "C" int bh_gemm_bf16_reads_blocked(int M, int N, int K, int layout, int a
   if (M <= 0 || N <= 0 || K <= 0 || K % 32 != 0) return 0;
   if (gemm_turns_blocks(M, N, K, layout, activation) || gemm_turns_parts(M, N, K, layout, activation) > 1) return 16;
   if (skinny_first(M, N, K, layout)) return M <= 8 ? 8 : 16;
+  if (gemm_slices_takes(M, N, K, layout, activation)) return 16;
   return 0;
 }
 
@@ -1082,6 +1087,7 @@ extern "C" int bh_gemm_bf16_reads_blocked(int M, int N, int K, int layout, int a
 extern "C" int bh_gemm_bf16_writes_blocked(int M, int N, int K, int layout, int activation) {
   if (M <= 0 || N <= 0 || K <= 0 || N % 32 != 0) return 0;
   if (gemm_turns_blocks(M, N, K, layout, activation)) return activation ? 1 : 0;
+  if (gemm_slices_takes(M, N, K, layout, activation)) return 2;    // the finishing kernel writes any blocks
   int rows, columns;
   tiled_config(M, N, activation != 0, &rows, &columns);
   return M <= 64 && !tiled_whole(M, N, K, layout, rows, columns) ? 2 : 0;
@@ -1089,14 +1095,22 @@ extern "C" int bh_gemm_bf16_writes_blocked(int M, int N, int K, int layout, int 
 
 // layout: 0 = rows, 1 = tiles.  activation: 0 = none; 1 = SwiGLU (W has 2 * N rows: gate rows then up rows).
 // Bytes of scratch memory that bh_gemm_bf16 wants for this product (0: none).
-extern "C" long bh_gemm_bf16_scratch(int M, int N, int K, int layout, int activation) {
-  if (M <= 0 || N <= 0 || K <= 0) return 0;
-  if (gemm_turns_blocks(M, N, K, layout, activation)) return 0;
-  if (const int turns_parts = gemm_turns_parts(M, N, K, layout, activation); turns_parts > 1)
-    return (long)turns_parts * M * N * (long)sizeof(float);
+// In how many parts of K the tiled kernels (whole tiles, or the kernel whose wave groups take turns) multiply a
+// product when they are given scratch memory (1: in one go).
+static int tiled_or_turns_parts(int M, int N, int K, int layout, int activation) {
+  if (gemm_turns_blocks(M, N, K, layout, activation)) return 1;
+  if (const int turns_parts = gemm_turns_parts(M, N, K, layout, activation); turns_parts > 1) return turns_parts;
   int parts, each;
   tiled_parts(M, N, K, layout, activation != 0, &parts, &each);
-  return parts == 1 ? 0 : (long)parts * M * (activation ? 2 * N : N) * (long)sizeof(float);
+  return parts;
+}
+extern "C" long bh_gemm_bf16_scratch(int M, int N, int K, int layout, int activation) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  int parts = tiled_or_turns_parts(M, N, K, layout, activation);
+  if (gemm_slices_takes(M, N, K, layout, activation))   // (a caller whose activations lie in rows gets the tiles: room for either)
+    parts = std::max(parts, gemm_slices_parts(M, N, K, activation, nullptr));
+  else if (parts == 1) return 0;
+  return (long)parts * M * (activation ? 2 * N : N) * (long)sizeof(float);
 }
 
 // The `ahead_*` and `behind_*` arguments (null when unused) let an RMSNorm ride on the products before and
@@ -1144,8 +1158,26 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
     tiled_config(M, N, activation != 0, &rows, &columns);
     return M <= 64 && !tiled_whole(M, N, K, layout, rows, columns);
   }();
-  BH_REQUIRE(skinny || (c_block_rows != 8 && behind_block_rows == 0 && (c_block_rows == 0 || gemm_turns_blocks(M, N, K, layout, activation))),
+  // 33 to 128 rows from blocks of 16: the kernel whose waves share the activations through LDS, then the finishing kernel
+  const bool slices = scratch != nullptr && a_block_rows == 16 && !skinny && gemm_slices_takes(M, N, K, layout, activation);
+  BH_REQUIRE(skinny || slices || (c_block_rows != 8 && behind_block_rows == 0 && (c_block_rows == 0 || gemm_turns_blocks(M, N, K, layout, activation))),
              "gemm_bf16: a product of M=%d N=%d K=%d does not write these blocks", M, N, K);
+  dim3 finish_grid((N + FINISH_COLUMNS - 1) / FINISH_COLUMNS, (M + 15) / 16);
+  const RowBlocks finish_blocks = {0, slices ? c_block_rows : 0, slices ? behind_block_rows : 0};
+#define BH_FINISH(SWIGLU, TC)                                                                                \
+  gemm_parts_finish_kernel<SWIGLU, TC><<<finish_grid, 256, 0, stream>>>((const float*)scratch, (TC*)c, M, N, K, \
+                                                                         parts, accumulate, norm, finish_blocks)
+  if (slices && !f32 && gemm_slices_gated(M, N, K, activation))   // the SwiGLU of many outputs: no parts, no finishing kernel
+    return gemm_slices_launch_gated(a, w, c, c_block_rows, M, N, K, ahead_ss, ahead_blocks, ahead_eps, stream);
+  if (slices) {
+    BH_REQUIRE(((uintptr_t)c | (uintptr_t)scratch | (uintptr_t)behind_rows) % 16 == 0,
+               "gemm_bf16: output, scratch memory and norm rows must be 16-byte aligned");
+    const int parts = gemm_slices_parts(M, N, K, activation, nullptr);
+    if (int status = gemm_slices_launch(a, w, (float*)scratch, M, N, K, activation, stream)) return status;
+    if (activation) { if (f32) BH_FINISH(true, float); else BH_FINISH(true, bf16_t); }
+    else { if (f32) BH_FINISH(false, float); else BH_FINISH(false, bf16_t); }
+    return bh_check_launch("gemm_parts_finish");
+  }
   const int a_blocked = a_block_rows == 16 && !skinny, c_blocked = c_block_rows == 16 && !skinny;
   if (!ahead_ss && !behind_weight && (f32 || !accumulate)) {   // many rows: the kernel whose wave groups take turns
     if (const int blocks = gemm_turns_blocks(M, N, K, layout, activation))
@@ -1156,10 +1188,10 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
     if (f32) FN<TILES, EXTRA, float>(__VA_ARGS__);                                  \
     else FN<TILES, EXTRA, bf16_t>(__VA_ARGS__);                                     \
   } while (0)
-  const bool in_parts = scratch != nullptr && bh_gemm_bf16_scratch(M, N, K, layout, activation) > 0;
+  const bool in_parts = scratch != nullptr && tiled_or_turns_parts(M, N, K, layout, activation) > 1;
   BH_REQUIRE(!a_blocked || (in_parts && gemm_turns_parts(M, N, K, layout, activation) > 1),
              "gemm_bf16: a product of M=%d N=%d K=%d that reads rows in blocks needs its scratch memory", M, N, K);
-  BH_REQUIRE(in_parts || !behind_weight || bh_gemm_bf16_scratch(M, N, K, layout, activation) == 0,
+  BH_REQUIRE(in_parts || !behind_weight || tiled_or_turns_parts(M, N, K, layout, activation) == 1,
              "gemm_bf16: a product of M=%d N=%d K=%d carries a norm through its finishing kernel and needs scratch memory", M, N, K);
   if (in_parts) {   // K in parts, then the finishing kernel
     BH_REQUIRE(((uintptr_t)c | (uintptr_t)scratch | (uintptr_t)behind_rows) % 16 == 0,
@@ -1175,10 +1207,6 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
       else launch_tiled<true, false, float>(a, w, nullptr, M, N, K, 0, none, (float*)scratch, stream);
       if (int status = bh_check_launch("gemm_tiled")) return status;
     }
-    dim3 finish_grid((N + FINISH_COLUMNS - 1) / FINISH_COLUMNS, (M + 15) / 16);
-#define BH_FINISH(SWIGLU, TC)                                                                                \
-  gemm_parts_finish_kernel<SWIGLU, TC><<<finish_grid, 256, 0, stream>>>((const float*)scratch, (TC*)c, M, N, K, \
-                                                                         parts, accumulate, norm)
     if (activation) { if (f32) BH_FINISH(true, float); else BH_FINISH(true, bf16_t); }
     else { if (f32) BH_FINISH(false, float); else BH_FINISH(false, bf16_t); }
 #undef BH_FINISH

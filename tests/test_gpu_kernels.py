@@ -112,7 +112,11 @@ def test_gemm(K, a_dtype, w_dtype, m, n, k):
                                    # many rows but few of the widest tiles: K in two or four parts of the kernel whose wave groups take turns
                                    (1800, 4096, 2048), (1000, 4096, 4096),
                                    # 65 to 127 rows: whole tiles of 64 rows
-                                   (100, 256, 1024), (127, 4096, 512), (65, 128, 64)])
+                                   (100, 256, 1024), (127, 4096, 512), (65, 128, 64),
+                                   # 33 to 64 rows, K from 512: the waves of a workgroup share the activations through LDS;
+                                   # a last slice of fewer than 512 k, weight blocks that do not fill the last workgroup
+                                   (33, 128, 512), (48, 144, 576), (64, 4096, 4096), (49, 1008, 1088), (40, 6144, 4096),
+                                   (64, 4096, 12288), (57, 5120, 5120), (80, 4096, 4096), (128, 6144, 4096), (97, 1008, 1280)])
 def test_gemm_with_packed_weights(K, m, n, k):
     """The same product from the regrouped (16 x 64 blocks) weight layout."""
     from beholdd.kernels import PackedWeight
@@ -143,12 +147,16 @@ def test_gemm_with_packed_weights(K, m, n, k):
 
 @pytest.mark.parametrize("g_dtype", DTYPES)
 @pytest.mark.parametrize("packed", [False, True])
-@pytest.mark.parametrize("m,n,k,n2", [(1, 192, 128, 48), (8, 4096, 256, 1000), (17, 200, 64, 64), (64, 320, 192, 130)])
+@pytest.mark.parametrize("m,n,k,n2", [(1, 192, 128, 48), (8, 4096, 256, 1000), (17, 200, 64, 64), (64, 320, 192, 130),
+                                      (48, 512, 1024, 256), (64, 4096, 4096, 2048), (33, 1024, 576, 640),
+                                      (96, 1024, 1024, 512), (128, 4096, 4096, 2048)])
 def test_norm_rides_on_the_products_around_it(K, g_dtype, packed, m, n, k, n2):
     """The product that completes the residual prepares the following RMSNorm (rows times the norm weight,
     partial sums of squares), and the product after it applies each row's factor to its result."""
     from beholdd.kernels import NormedRows
     from beholdd.parts.base import NormRequest
+    if m > 64 and not packed:
+        pytest.skip("beyond 64 rows a norm rides on products of packed weights only")
     gen = torch.Generator().manual_seed(m * 31 + n)
     a = torch.randn(m, k, generator=gen).to(torch.bfloat16)
     w = (torch.randn(n, k, generator=gen) * 0.1).to(torch.bfloat16)
@@ -367,8 +375,8 @@ def test_gemm_with_turns_reads_and_writes_rows_in_blocks(K, blocks, m, n, k):
 def test_products_of_few_rows_hand_each_other_blocks(K, m, g_dtype):
     """A layer's feed-forward and the norms around it as a decode step of m sequences runs them: the norm writes
     its rows for the gated product, that one its output for the down product, which adds into the residual and
-    prepares the next norm for the product after it.  Up to 32 rows every matrix on the way lies in blocks (of
-    8 rows up to 8, of 16 beyond), as `new_rows` hands them out for their readers; the numbers are those of float64
+    prepares the next norm for the product after it.  Every matrix on the way lies in blocks (of 8 rows up to 8,
+    of 16 beyond), as `new_rows` hands them out for their readers; the numbers are those of float64
     within bfloat16's rounding, and matrices handed over as plain rows give the same bits (they are regrouped)."""
     from beholdd.kernels.library import BlockedRows, NormedRows
     from beholdd.parts.base import NormRequest, ProductReader
@@ -399,7 +407,7 @@ def test_products_of_few_rows_hand_each_other_blocks(K, m, g_dtype):
     h_rows, again_rows, kinds_rows = chain(False)
     h_blocks, again_blocks, kinds_blocks = chain(True)
     assert not any(isinstance(t, BlockedRows) for t in kinds_rows)
-    want_blocks = 0 if m > 32 else 8 if m <= 8 else 16
+    want_blocks = 8 if m <= 8 else 16
     assert [t.block_rows if isinstance(t, BlockedRows) else 0 for t in kinds_blocks] == [want_blocks] * 3
     assert torch.equal(h_rows, h_blocks) and torch.equal(again_rows, again_blocks)
     on = lambda t: t.double().to("cuda:0")
@@ -525,7 +533,8 @@ def test_gemm_chooses_the_turns_kernel_where_it_fills_the_chip(K, m, n, k, swigl
 @pytest.mark.parametrize("m,width,k", [(1, 16, 64), (8, 160, 128), (40, 896, 320), (64, 48, 192), (65, 64, 64),
                                        (130, 208, 256), (300, 1000, 128), (7, 100, 64), (8, 12288, 4096), (5, 32, 72),
                                        (650, 33008, 128), (130, 208, 832), (256, 512, 1024), (100, 256, 512),
-                                       (127, 64, 64)])
+                                       (127, 64, 64), (48, 640, 512), (64, 12288, 4096), (33, 136, 1088), (96, 12288, 4096),
+                                       (80, 640, 768), (128, 10240, 512)])
 def test_gemm_swiglu(K, dtype, packed, m, width, k):
     """silu(a Wg^T) * (a Wu^T) in one pass (or in two where the sizes do not allow one), from both layouts."""
     g = torch.Generator().manual_seed(m + width)
