@@ -112,19 +112,23 @@ def decode_run(engine, batch, context, steps, warmup, torch):
     return elapsed / steps, mean_length
 
 
-def prefill_run(engine, n_tokens, torch, repeats=3):
+def prefill_run(engine, n_tokens, torch, repeats=3, prompts=1, host=False):
+    """Seconds of one step that brings `prompts` prompts of `n_tokens` tokens each (the best of `repeats`); with
+    `host` also the seconds until the step function returns, the device still busy."""
     from beholdd.engine import StepEntry
     tokens = [(31 * i + 5) % engine.model.vocab for i in range(n_tokens)]
-    times = []
+    times, returned = [], []
     for _ in range(repeats + 1):          # the first run warms up and is dropped
-        slot = engine.alloc_slot()
+        slots = [engine.alloc_slot() for _ in range(prompts)]
         torch.cuda.synchronize()
         begin = time.perf_counter()
-        engine.step([StepEntry(slot, tokens, [n_tokens - 1])])
+        engine.step([StepEntry(slot, tokens, [n_tokens - 1]) for slot in slots])
+        returned.append(time.perf_counter() - begin)
         torch.cuda.synchronize()
         times.append(time.perf_counter() - begin)
-        engine.free_slot(slot)
-    return min(times[1:])
+        for slot in slots:
+            engine.free_slot(slot)
+    return (min(times[1:]), min(returned[1:])) if host else min(times[1:])
 
 
 # Batches of the benchmark configurations: (prompts, shortest, longest, new tokens, temperature, context).
@@ -240,6 +244,24 @@ def main():
             s, length = decode_run(engine, batch, context, steps, 2, torch)
             points[name] = round(batch / s, 2)
             fractions[name] = round((weight_bytes + batch * length * kv_bytes_per_token) / s / 1e9 / PEAK_HBM_GBS, 4)
+    # Prompts of other lengths: tokens a second and the fraction of the matrix-core peak; for the short ones, which
+    # the host's launches bound, also the milliseconds until the step function returns.
+    prefill_points = {}
+    if not args.no_points:
+        def flops(tokens, prompts=1):
+            return prompts * (2.0 * cfg.n_layers * layer_params * tokens + cfg.n_layers * cfg.n_heads * 2.0 * tokens * tokens * cfg.head_dim
+                              + 2.0 * cfg.vocab * cfg.hidden)
+        for tokens in (16, 64, 128):
+            seconds_all, seconds_host = prefill_run(engine, tokens, torch, host=True)
+            prefill_points[f"tokens_{tokens}"] = {"ms": round(seconds_all * 1e3, 3), "host_ms": round(seconds_host * 1e3, 3),
+                                                  "tok_per_s": round(tokens / seconds_all, 1)}
+        for tokens, prompts in ((512, 1), (1024, 1), (4096, 1), (8192, 1), (2048, 4)):
+            if tokens > args.context:
+                continue
+            seconds_all = prefill_run(engine, tokens, torch, repeats=2, prompts=prompts)
+            name = f"tokens_{tokens}" if prompts == 1 else f"prompts_{prompts}x{tokens}"
+            prefill_points[name] = {"ms": round(seconds_all * 1e3, 3), "tok_per_s": round(prompts * tokens / seconds_all, 1),
+                                    "frac": round(flops(tokens, prompts) / seconds_all / PEAK_FLOPS[dtype_tag], 4)}
     generated = None
     if not args.no_points and args.shape == "8b":
         generated = workload_run(engine, args.shape, torch)     # the same batch through Engine.generate
@@ -273,10 +295,46 @@ def main():
         "points": points,
         "points_hbm_frac": fractions,
     }
+    if prefill_points:
+        line["prefill_points"] = prefill_points
     if generated is not None:
         line["generate"] = generated
+    if not args.no_points and args.shape == "8b" and args.layers is None and args.dtype == "bfloat16":
+        # the other two shapes of the family, full depth: decode at batch 8 and the prompt of 2,048 tokens
+        del engine, model, cache_tensor, span
+        line["shapes"] = {name: other_shape(name, args, torch) for name in ("14b", "32b")}
     print(json.dumps(line))
     return 0
+
+
+def other_shape(name, args, torch):
+    import gc
+
+    from beholdd.engine import Engine, random_model_on_device
+    gc.collect()
+    torch.cuda.empty_cache()
+    config = SHAPES[name][1]
+    model = random_model_on_device(dict(config), seed=0, dtype="bfloat16", device="cuda:0")
+    engine = Engine(model=model, dtype="bfloat16", max_tokens=8 * (-(-args.context // 64) * 64), max_slots=8, device="cuda:0")
+    randomise_cache(engine, torch)
+    cfg = engine.config
+    layer_params = (cfg.hidden * (cfg.q_width + 2 * cfg.kv_width) + cfg.q_width * cfg.hidden + 3 * cfg.hidden * cfg.intermediate)
+    weight_bytes = (cfg.n_layers * layer_params + cfg.vocab * cfg.hidden) * 2
+    kv_bytes_per_token = cfg.n_layers * 2 * cfg.kv_width * 2
+    steps = max(4, args.steps // 2)
+    seconds, mean_length = decode_run(engine, 8, args.context, steps, 2, torch)
+    t = args.prefill_tokens
+    prefill_seconds = prefill_run(engine, t, torch, repeats=2)
+    prefill_flops = (2.0 * cfg.n_layers * layer_params * t + cfg.n_layers * cfg.n_heads * 2.0 * t * t * cfg.head_dim
+                     + 2.0 * cfg.vocab * cfg.hidden)
+    out = {"layers": cfg.n_layers, "decode_b8_tok_per_s": round(8 / seconds, 2), "decode_b8_ms": round(seconds * 1e3, 4),
+           "decode_b8_hbm_frac": round((weight_bytes + 8 * mean_length * kv_bytes_per_token) / seconds / 1e9 / PEAK_HBM_GBS, 4),
+           "prefill_tok_per_s": round(t / prefill_seconds, 1), "prefill_ms": round(prefill_seconds * 1e3, 3),
+           "prefill_frac": round(prefill_flops / prefill_seconds / PEAK_FLOPS["bf16"], 4)}
+    del engine, model
+    gc.collect()
+    torch.cuda.empty_cache()
+    return out
 
 
 if __name__ == "__main__":
