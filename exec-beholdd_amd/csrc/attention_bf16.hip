@@ -453,9 +453,10 @@ extern "C" int bh_attention_bf16_splits(int n_seqs, int max_rows_per_seq, int H,
   const int G = H / KVH;
   const long tiles = (long)((max_rows_per_seq * G + 15) / 16) * KVH * n_seqs;
   const int pages = max_position / BH_PAGE + 1;
-  // about one workgroup per compute unit (256), every wave of a workgroup at least one page
-  if (tiles >= 256 || pages < 8) return 1;
-  long want = (256 + tiles - 1) / tiles;
+  // about one workgroup per compute unit (256 on an MI355X), every wave of a workgroup at least one page
+  const int units = bh_compute_units();
+  if (tiles >= units || pages < 8) return 1;
+  long want = (units + tiles - 1) / tiles;
   if (want > pages / 4) want = pages / 4;
   if (want < 1) want = 1;
   const int per = (int)((pages + want - 1) / want);
@@ -500,7 +501,7 @@ static int attention_bf16_run(const void* q, void* out, void* part_o, void* part
   BH_REQUIRE(out_blocked == 0 || ((out_blocked == 8 || out_blocked == 16) && (H * hd) % 32 == 0),
              "attention_bf16: the output's rows lie in blocks of 8 or 16, or one after the other (0), not %d", out_blocked);
   const int tile_groups = tiles, z_count = n_seqs * n_splits;
-  const bool lean = (long)tiles * KVH * z_count > 256;   // more workgroups than compute units: two of them per unit
+  const bool lean = (long)tiles * KVH * z_count > bh_compute_units();   // more workgroups than compute units: two of them per unit
   dim3 grid(tile_groups * KVH * z_count), block(256);
 #define BH_ATT_ONE(NS, STREAM, FUSED, ...)                                                                      \
   attention_mfma_kernel<NS, STREAM, FUSED, ##__VA_ARGS__><<<grid, block, 0, stream>>>(                          \

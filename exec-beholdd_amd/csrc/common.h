@@ -67,6 +67,9 @@ __device__ inline float block_max(float v, float* scratch) {
 // Every entry point returns 0 on success; otherwise bh_last_error() gives the reason.
 int bh_fail(const char* format, ...);
 int bh_check_launch(const char* what);
+// The compute units of the GPU that is current when it is first asked (256 on an MI355X): what launch plans count
+// workgroups against.  Where no GPU is visible (a byte plan made on another machine) it says 256.
+int bh_compute_units();
 
 #define BH_REQUIRE(cond, ...)                  \
   do {                                         \

@@ -960,10 +960,11 @@ static TiledConfig tiled_config(int M, int N, bool swiglu, int* rows, int* colum
   }
   const long tiles_128 = (long)((N + (swiglu ? 63 : 127)) / (swiglu ? 64 : 128)) * ((M + 127) / 128);
   const long tiles_256 = (long)((N + (swiglu ? 127 : 255)) / (swiglu ? 128 : 256)) * ((M + 255) / 256);
-  const bool big = tiles_256 >= 512;
+  const int units = bh_compute_units();   // measured with 256: two tiles each, and between two and four
+  const bool big = tiles_256 >= 2 * units;
   *rows = big ? 256 : 128;
   *columns = (big ? 256 : 128) / (swiglu ? 2 : 1);
-  return big ? TILED_256 : tiles_128 > 512 && tiles_128 <= 1024 ? TILED_128_ONE_BUFFER : TILED_128;
+  return big ? TILED_256 : tiles_128 > 2 * units && tiles_128 <= 4 * units ? TILED_128_ONE_BUFFER : TILED_128;
 }
 // Up to how many rows the skinny kernel takes a product of packed weights (it reads its activations in blocks,
 // see struct RowBlocks); without packed weights, or where the tiles do not fit, up to 64.
@@ -989,8 +990,8 @@ static bool tiled_whole(int M, int N, int K, int layout, int rows, int columns) 
 // one; one workgroup per compute unit is then enough (more parts only add scratch traffic) unless a part
 // would still be longer than 64 slices.
 #define TILED_FEW_ROWS 512
-#define TILED_FEW_ROWS_WORKGROUPS 384
-#define TILED_FEW_TILES 128
+#define TILED_FEW_ROWS_WORKGROUPS 384   // on 256 compute units; scaled to the chip's (bh_compute_units)
+#define TILED_FEW_TILES 128             // likewise
 static void tiled_parts(int M, int N, int K, int layout, bool swiglu, int* parts, int* slices_per_part) {
   int rows, columns;
   tiled_config(M, N, swiglu, &rows, &columns);
@@ -1000,11 +1001,13 @@ static void tiled_parts(int M, int N, int K, int layout, bool swiglu, int* parts
   const long tiles = (long)((N + columns - 1) / columns) * ((M + rows - 1) / rows);
   const int slices = K / TK;
   int p;
+  const int units = bh_compute_units();
+  const int few_rows_workgroups = TILED_FEW_ROWS_WORKGROUPS * units / 256, few_tiles = TILED_FEW_TILES * units / 256;
   if (M <= TILED_FEW_ROWS) {
-    p = (int)((TILED_FEW_ROWS_WORKGROUPS + tiles - 1) / tiles);
+    p = (int)((few_rows_workgroups + tiles - 1) / tiles);
   } else {
-    if (tiles > TILED_FEW_TILES) return;
-    p = (int)(2 * TILED_FEW_TILES / tiles);
+    if (tiles > few_tiles) return;
+    p = (int)(2 * few_tiles / tiles);
     if (slices / p > 64) p *= 2;
   }
   p = std::min(std::min(p, MAX_PARTS), slices / 4);    // at least four slices each

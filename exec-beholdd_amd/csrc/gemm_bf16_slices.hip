@@ -212,7 +212,8 @@ bool gemm_slices_takes(int M, int N, int K, int layout, int activation) {
 // 22.2 / 17.5 / 31.3; four waves (twice the activations' bytes from the L2, half the bytes of partial sums), stages of
 // four chunks, 384 workgroups 18.1 / 15.9 / 29.7; four waves, two chunks, 512 workgroups 18.6 / 15.6 / 28.2, and in the
 // whole model (decode step of 64 sequences, context 640) 5.50 against 5.56 and 5.67 ms for the other two, 5.98 before.
-constexpr int WAVES = 4, TARGET_WORKGROUPS = 512;
+constexpr int WAVES = 4;
+static int target_workgroups() { return 2 * bh_compute_units(); }      // 512 on the chip these were measured on
 // The SwiGLU that finishes itself has one workgroup of eight waves per 64 outputs (192 at Qwen3-8B's sizes, fewer than
 // compute units), so a wave may use twice the registers: stages of four chunks, 8 to 16 KB of W on their way per wave
 // (gate+up at 64 rows 46.4 us; with stages of two chunks 56.1; four waves per 32 outputs 49.7; K in two parts and the
@@ -221,7 +222,7 @@ constexpr int GATED_WAVES = 8, GATED_CHUNKS = 4;
 
 bool gemm_slices_gated(int M, int N, int K, int activation) {
   // with enough outputs that workgroups of 64 outputs each fill the chip, a SwiGLU needs no parts
-  return activation && gemm_slices_takes(M, N, K, 1, activation) && (N + 63) / 64 >= 160 && N % 32 == 0;
+  return activation && gemm_slices_takes(M, N, K, 1, activation) && (N + 63) / 64 >= bh_compute_units() * 5 / 8 && N % 32 == 0;
 }
 
 int gemm_slices_parts(int M, int N, int K, int activation, int* stages_per_part) {
@@ -231,7 +232,7 @@ int gemm_slices_parts(int M, int N, int K, int activation, int* stages_per_part)
     if (stages_per_part) *stages_per_part = stages;
     return 1;
   }
-  int parts = std::max(1, std::min({stages / 2, MOST_PARTS, (TARGET_WORKGROUPS + groups / 2) / groups}));   // 512 k each at least
+  int parts = std::max(1, std::min({stages / 2, MOST_PARTS, (target_workgroups() + groups / 2) / groups}));   // 512 k each at least
   const int each = (stages + parts - 1) / parts;
   parts = (stages + each - 1) / each;
   if (stages_per_part) *stages_per_part = each;       // in units of STAGE_K

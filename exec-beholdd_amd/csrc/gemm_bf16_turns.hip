@@ -311,13 +311,14 @@ TurnsPlan turns_plan(int M, int N, int K, int layout, int activation) {
   double best_rate = 600.0;    // TFLOP/s: what a tile of its own has to reach
   double direct_rate = 0.0;
   const double work = (double)M * (activation ? 2.0 * N : (double)N);   // rows x weight rows
+  const int units = bh_compute_units();   // a round is one tile per compute unit (the rates below were measured with 256)
   for (int blocks = 8; blocks >= 4; blocks -= 2) {
     if (!gemm_turns_can(M, N, K, layout, activation, blocks)) continue;
     const int outs = (activation ? 16 : 32) * blocks;
     const long tiles = (long)((N + outs - 1) / outs) * ((M + 255) / 256);
-    const long rounds = (tiles + 255) / 256;
+    const long rounds = (tiles + units - 1) / units;
     const double cost = blocks == 8 ? 1.0 : blocks == 6 ? 1.23 : 1.34;
-    const double rate = 1430.0 * work / ((double)rounds * 256 * 256 * (activation ? 2 : 1) * outs * cost);
+    const double rate = 1430.0 * (units / 256.0) * work / ((double)rounds * units * 256 * (activation ? 2 : 1) * outs * cost);
     if (rate >= best_rate) best_rate = direct_rate = rate, plan.blocks = blocks;
   }
   if (!activation && M >= 512 && gemm_turns_can(M, N, K, layout, 0, 8)) {
@@ -329,9 +330,9 @@ TurnsPlan turns_plan(int M, int N, int K, int layout, int activation) {
     // 2,048 rows: down 240 -> 199 in 2; 384 rows: slower for qkv and o, so not below 512.
     const long tiles = (long)((N + 255) / 256) * ((M + 255) / 256);
     int parts = 8;
-    while (parts > 1 && (tiles * parts > 256 || K / parts < 512 || K % (128 * parts) != 0)) parts /= 2;
-    if (parts > 1 && tiles * parts >= 160) {
-      const double rate = 0.85 * 1430.0 * work / (256.0 * 256 * 256 / parts);
+    while (parts > 1 && (tiles * parts > units || K / parts < 512 || K % (128 * parts) != 0)) parts /= 2;
+    if (parts > 1 && tiles * parts >= units * 5 / 8) {
+      const double rate = 0.85 * 1430.0 * (units / 256.0) * work / ((double)units * 256 * 256 / parts);
       if (rate > direct_rate) plan.blocks = 0, plan.parts = parts;
     }
   }

@@ -27,6 +27,20 @@ int bh_check_launch(const char* what) {
   return 0;
 }
 
+int bh_compute_units() {
+  static const int units = [] {
+    int device = 0;
+    hipDeviceProp_t properties;
+    if (hipGetDevice(&device) != hipSuccess || hipGetDeviceProperties(&properties, device) != hipSuccess ||
+        properties.multiProcessorCount <= 0) {
+      (void)hipGetLastError();   // no GPU here: the error is not a launch's
+      return 256;
+    }
+    return properties.multiProcessorCount;
+  }();
+  return units;
+}
+
 extern "C" const char* bh_last_error() { return g_error; }
 extern "C" int bh_page_size() { return BH_PAGE; }
 
@@ -508,6 +522,10 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_rows_kernel(
   *reinterpret_cast<uint4*>(block + bh_key_index(kv_order, token, 8 * c, HD)) = packed;   // 8 dims lie together in both orders
 }
 
+// Precondition: the rows of one sequence stand one after the other and in position order (row r + 1 of a
+// sequence is position p + 1), as a step lays them out.  The form for many rows relies on it: it takes eight
+// rows for one piece of values when the first and the last of them belong to one sequence, seven positions apart,
+// and does not look at the six between.
 extern "C" int bh_qk_norm_rope_cache(const void* qkv, int dtype, void* q_out, const void* q_weight,
                                      const void* k_weight, int w_dtype, float eps, const float* cos_table,
                                      const float* sin_table, int table_positions, int rot,

@@ -11,6 +11,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <vector>
 
 #include "layout.h"
@@ -205,6 +206,67 @@ int bhp_argmax(const float* logits, int32_t* tokens, int32_t* bad, int n_rows, i
   return 0;
 }
 
+// tokens[row] = a draw from softmax(logits / temperature) restricted to the top_k largest logits (0: all) and then to the
+// smallest set of most likely tokens whose mass reaches top_p of what is left (ties at a threshold are kept), by the
+// inverse CDF over the kept tokens in index order at uniform[row] in [0, 1); temperature <= 0: the argmax (sampling.hip:
+// bh_sample with temperatures).  Sums in double.  margin[row] (may be null): how far the draw's target lies from the
+// nearer end of the chosen token's interval, as a fraction of the kept mass: a kernel that sums in float32 may choose
+// a neighbour when that is within its rounding.
+int bhp_sample(const float* logits, const float* temperature, const int32_t* top_k, const float* top_p, const float* uniform,
+               int32_t* tokens, int32_t* bad, double* margin, int n_rows, int vocab) {
+  if (n_rows <= 0 || vocab <= 0 || !temperature || !uniform) return 1;
+  for (int r = 0; r < n_rows; ++r) {
+    const float* x = logits + (size_t)r * vocab;
+    if (margin) margin[r] = 1.0;
+    int best = 0;
+    bool finite = true;
+    for (int i = 0; i < vocab; ++i) {
+      if (!isfinite(x[i])) finite = false;
+      if (x[i] > x[best]) best = i;
+    }
+    bad[r] = finite ? 0 : 1;
+    tokens[r] = finite ? best : -1;
+    if (!finite || !(temperature[r] > 0.f)) continue;
+    std::vector<float> sorted(x, x + vocab);
+    std::sort(sorted.begin(), sorted.end(), [](float a, float b) { return a > b; });
+    const int k = top_k ? top_k[r] : 0;
+    float floor_value = (k > 0 && k < vocab) ? sorted[k - 1] : sorted[vocab - 1];   // ties at the k-th value are kept
+    auto weight = [&](float v) { return exp(((double)v - (double)x[best]) / (double)temperature[r]); };
+    const float p = top_p ? top_p[r] : 1.f;
+    if (p > 0.f && p < 1.f) {
+      double total = 0.0;
+      for (int i = 0; i < vocab; ++i)
+        if (x[i] >= floor_value) total += weight(x[i]);
+      double mass = 0.0;
+      for (int i = 0; i < vocab && sorted[i] >= floor_value; ++i) {   // most likely first; a value's ties all count
+        mass += weight(sorted[i]);
+        if ((i + 1 == vocab || sorted[i + 1] != sorted[i]) && mass >= (double)p * total) {
+          floor_value = sorted[i];
+          break;
+        }
+      }
+    }
+    double kept = 0.0;
+    for (int i = 0; i < vocab; ++i)
+      if (x[i] >= floor_value) kept += weight(x[i]);
+    const double target = (double)uniform[r] * kept;
+    double running = 0.0;
+    int pick = -1, last = -1;
+    for (int i = 0; i < vocab && pick < 0; ++i) {
+      if (x[i] < floor_value) continue;
+      last = i;
+      const double before = running;
+      running += weight(x[i]);
+      if (running > target) {
+        pick = i;
+        if (margin) margin[r] = fmin(target - before, running - target) / kept;
+      }
+    }
+    tokens[r] = pick >= 0 ? pick : last;
+  }
+  return 0;
+}
+
 int bhp_page_size() { return BH_PAGE; }
 int bhp_key_index(int order, int token, int dim, int hd) { return bh_key_index(order, token, dim, hd); }
 int bhp_value_index(int order, int token, int dim, int hd) { return bh_value_index(order, token, dim, hd); }
@@ -320,6 +382,23 @@ int main() {
     const float rows[8] = {-1, 3, 3, 2, 0, NAN, INFINITY, 0};
     int32_t tokens[2], bad[2];
     EXPECT(bhp_argmax(rows, tokens, bad, 2, 4) == 0 && tokens[0] == 1 && bad[0] == 0 && tokens[1] == -1 && bad[1] == 1);
+  }
+  // a draw: logits ln 1, ln 2, ln 5 at temperature 1 are the masses 1/8, 2/8, 5/8; top_k 2 leaves 2/7, 5/7; top_p 0.5 the last alone
+  {
+    const float row[3] = {0.f, logf(2.f), logf(5.f)};
+    const float one = 1.f, half = 0.5f;
+    const int32_t two = 2;
+    int32_t token, flag;
+    double margin;
+    const float draws[4] = {0.1f, 0.2f, 0.374f, 0.376f};
+    const int want_all[4] = {0, 1, 1, 2}, want_two[4] = {1, 1, 2, 2};
+    for (int i = 0; i < 4; ++i) {
+      EXPECT(bhp_sample(row, &one, nullptr, nullptr, &draws[i], &token, &flag, &margin, 1, 3) == 0 && token == want_all[i] && flag == 0);
+      EXPECT(bhp_sample(row, &one, &two, nullptr, &draws[i], &token, &flag, &margin, 1, 3) == 0 && token == want_two[i]);
+      EXPECT(bhp_sample(row, &one, nullptr, &half, &draws[i], &token, &flag, &margin, 1, 3) == 0 && token == 2);
+    }
+    const float zero = 0.f;
+    EXPECT(bhp_sample(row, &zero, nullptr, nullptr, &draws[0], &token, &flag, nullptr, 1, 3) == 0 && token == 2);
   }
   // swiglu: silu(0) = 0, silu(x) -> x for large x, no clamp
   {

@@ -158,3 +158,27 @@ def test_cache_write_and_attention_and_their_twins(K, twins, dtype, code, head_d
                 n_heads, kv_heads, head_dim, scale, window, layout=layout)
     want = twins.attention(host(q_dev), k_twin, v_twin, table, row_seq, positions, n_heads, kv_heads, head_dim, scale, window, order, code)
     assert rel(host(out), want) < (1e-5 if code == F32 else 1.2e-2)
+
+
+@pytest.mark.parametrize("vocab", [50, 1000, 4133])
+def test_the_draw_and_its_twin(K, twins, vocab):
+    """Temperature, top-k and top-p draws of the kernel against the plain twin's, row by row: the same token wherever the
+    draw's target lies further from the ends of its token's interval than float32 sums can move it."""
+    rng = np.random.default_rng(vocab)
+    rows = 96
+    logits = (rng.normal(size=(rows, vocab)) * 2.5).astype(np.float32)
+    logits[5, 7] = logits[5, 9]                    # ties at a threshold are kept
+    temperature = rng.choice([0.0, 0.5, 0.8, 1.0, 1.7], size=rows).astype(np.float32)
+    uniform = rng.random(rows).astype(np.float32)
+    for top_k, top_p in ((None, None), (rng.choice([0, 1, 5, 40, vocab], size=rows).astype(np.int32), None),
+                         (None, rng.choice([1.0, 0.9, 0.5, 0.05], size=rows).astype(np.float32)),
+                         (rng.choice([0, 3, 40], size=rows).astype(np.int32), rng.choice([1.0, 0.8, 0.3], size=rows).astype(np.float32))):
+        tokens, bad = torch.empty(rows, dtype=torch.int32, device=DEVICE), torch.empty(rows, dtype=torch.int32, device=DEVICE)
+        K.sample(dev(logits), tokens, bad, temperature=dev(temperature), top_k=None if top_k is None else dev(top_k),
+                 top_p=None if top_p is None else dev(top_p), uniform=dev(uniform))
+        want, want_bad, margin = twins.sample(logits, temperature, uniform, top_k, top_p)
+        got = tokens.cpu().numpy()
+        assert bad.cpu().tolist() == want_bad.tolist() == [0] * rows
+        sure = margin > 1e-5
+        assert sure.sum() > 0.9 * rows and np.array_equal(got[sure], want[sure])
+        assert len(set(want.tolist())) > rows // 4

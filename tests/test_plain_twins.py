@@ -116,3 +116,31 @@ def test_rows_in_blocks_are_a_permutation_in_operand_order(twins, block_rows):
             block = (r // block_rows) * (width // 32) + c // 32
             want = block * 32 * block_rows + (((c % 32) // 8) * block_rows + r % block_rows) * 8 + c % 8
             assert index[r, c] == want
+
+
+def test_the_draws_twin_is_an_inverse_cdf_over_the_kept_tokens(twins):
+    """The sampler's twin against NumPy and SciPy: the distribution it draws from is softmax(logits / temperature)
+    cut to the top k and to the smallest most likely set that reaches top_p, in index order."""
+    from scipy.special import softmax
+    rng = np.random.default_rng(3)
+    vocab = 200
+    logits = (rng.normal(size=(1, vocab)) * 2).astype(np.float32)
+    for temperature, k, p in ((1.0, 0, 1.0), (0.6, 0, 1.0), (1.3, 10, 1.0), (1.5, 0, 0.7), (1.6, 25, 0.9)):
+        masses = softmax(logits[0].astype(np.float64) / temperature)
+        keep = np.ones(vocab, bool)
+        if k:
+            keep &= logits[0] >= np.sort(logits[0])[-k]
+        if p < 1.0:
+            order = np.argsort(-masses * keep, kind="stable")
+            reached = np.cumsum((masses * keep)[order]) >= p * (masses * keep).sum()
+            keep &= masses >= masses[order[np.argmax(reached)]]
+        edges = np.concatenate([[0.0], np.cumsum(masses * keep)]) / (masses * keep).sum()
+        draws = rng.random(400).astype(np.float32)
+        got, bad, margin = twins.sample(np.repeat(logits, 400, axis=0), np.full(400, temperature), draws,
+                                        top_k=np.full(400, k, np.int32), top_p=np.full(400, p, np.float32))
+        want = np.searchsorted(edges, draws.astype(np.float64), side="right") - 1
+        sure = margin > 1e-9
+        assert bad.sum() == 0 and sure.sum() > 390 and np.array_equal(got[sure], want[sure])
+        assert keep[got].all() and len(set(got.tolist())) > 3
+    greedy, _, _ = twins.sample(logits, np.zeros(1), np.zeros(1, np.float32))
+    assert greedy[0] == int(np.argmax(logits[0]))

@@ -87,3 +87,61 @@ def test_sizes_beyond_the_static_array_are_refused_with_a_clear_error():
     assert "static array" in message and "45000" in message
     torch.cuda.synchronize()
     assert tokens.cpu().tolist() == [-7] * 4
+
+
+_CAPTURE = r"""
+import ctypes, sys
+import torch
+sys.path.insert(0, {root!r})
+from beholdd.kernels import build
+lib = ctypes.CDLL(build.ensure_built(verbose=False))
+p, i = ctypes.c_void_p, ctypes.c_int
+lib.bh_last_error.restype = ctypes.c_char_p
+lib.bh_sample_scratch.argtypes, lib.bh_sample_scratch.restype = [i, i], i
+lib.bh_sample.argtypes, lib.bh_sample.restype = [p, p, p, p, p, p, p, p, i, i, p], i
+lib.bh_sample_greedy_static.argtypes, lib.bh_sample_greedy_static.restype = [p, p, p, i, i, p], i
+rows, vocab = 6, 40_000
+logits = torch.randn(rows, vocab, device="cuda:0")
+tokens = torch.full((rows,), -7, dtype=torch.int32, device="cuda:0")
+bad = torch.full((rows,), -7, dtype=torch.int32, device="cuda:0")
+def static(stream):
+    status = lib.bh_sample_greedy_static(logits.data_ptr(), tokens.data_ptr(), bad.data_ptr(), rows, vocab, ctypes.c_void_p(stream))
+    assert status == 0, lib.bh_last_error()
+if {warm}:
+    static(torch.cuda.current_stream().cuda_stream)      # an eager call first: the array's address is known before the capture
+    torch.cuda.synchronize()
+graph = torch.cuda.CUDAGraph()
+with torch.cuda.graph(graph):
+    static(torch.cuda.current_stream().cuda_stream)
+words = lib.bh_sample_scratch(rows, vocab)
+scratch = torch.empty(max(words, 1), dtype=torch.float32, device="cuda:0")
+want, want_bad = torch.empty_like(tokens), torch.empty_like(bad)
+for replay in range(4):                # other work and synchronisations between the replays; every replay is checked
+    logits.normal_()
+    logits[replay % rows, 17] = 50.0
+    if replay == 2:
+        logits[1, 9] = float("nan")
+    tokens.fill_(-7)
+    torch.cuda.synchronize()
+    graph.replay()
+    status = lib.bh_sample(logits.data_ptr(), None, None, None, None, want.data_ptr(), want_bad.data_ptr(),
+                           scratch.data_ptr() if words else None, rows, vocab, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert status == 0, lib.bh_last_error()
+    torch.cuda.synchronize()
+    assert torch.equal(tokens, want) and torch.equal(bad, want_bad), (replay, tokens, want)
+    assert int(tokens[replay % rows]) in (17, -1)
+print("capture ok")
+"""
+
+
+@pytest.mark.parametrize("warm", [False, True])
+def test_the_call_inside_a_captured_graph(warm):
+    """What the entry point is for: the call recorded into a HIP graph, in a process of its own so that the capture
+    can be the very first call on the device (the array's address is asked for inside it), and after an eager call;
+    four replays with other work between them against the allocating entry point."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    run = subprocess.run([sys.executable, "-c", _CAPTURE.format(root=root, warm=warm)], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0 and "capture ok" in run.stdout, run.stderr[-2000:]

@@ -116,6 +116,19 @@ class Twins:
         assert self.lib.bhp_argmax(self._p(logits), self._p(tokens), self._p(bad), logits.shape[0], logits.shape[1]) == 0
         return tokens, bad
 
+    def sample(self, logits, temperature, uniform, top_k=None, top_p=None):
+        """(tokens, bad, margin): margin is how far each draw lies from the nearer end of its token's interval, as a
+        fraction of the kept mass."""
+        logits = np.ascontiguousarray(logits, dtype=np.float32)
+        n = logits.shape[0]
+        tokens, bad, margin = np.zeros(n, np.int32), np.zeros(n, np.int32), np.zeros(n, np.float64)
+        as_f32 = lambda v: None if v is None else np.ascontiguousarray(v, dtype=np.float32)
+        temperature, uniform, top_p = as_f32(temperature), as_f32(uniform), as_f32(top_p)
+        top_k = None if top_k is None else np.ascontiguousarray(top_k, dtype=np.int32)
+        assert self.lib.bhp_sample(self._p(logits), self._p(temperature), self._p(top_k), self._p(top_p), self._p(uniform),
+                                   self._p(tokens), self._p(bad), self._p(margin), n, logits.shape[1]) == 0
+        return tokens, bad, margin
+
     def rows_index(self, block_rows, rows, width):
         """Where each element of a [rows, width] matrix lies when its rows are in blocks of `block_rows`."""
         self.lib.bhp_rows_index.restype = ctypes.c_long
