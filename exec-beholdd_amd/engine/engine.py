@@ -140,14 +140,16 @@ class Engine:
         return self._last_selection
 
     # ---- the step function ----
-    def step(self, entries: list):
+    def step(self, entries: list, extras: dict | None = None):
         """Run the given tokens of each entry's sequence from the cache; return float32 logits
         [wanted, vocab] in the order of the entries and of their `want` lists (None if nothing is
-        wanted).  On an error no sequence's length changes.  The logits of a decode step stand in memory
+        wanted).  `extras`, a dictionary of the caller's, receives what parts left in the step's
+        `StepContext.extras` (one row per token of the step, in the order of the entries).
+        On an error no sequence's length changes.  The logits of a decode step stand in memory
         that a later decode step may write again: copy what has to outlive the next step."""
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
         if self.graphs is not None and entries and self.graphs.usable(entries):
-            return self._graph_step(entries)
+            return self._graph_step(entries, extras)
         if any(e.fed_row is not None for e in entries):
             # only the captured decode step reads tokens on the device; here the host waits for them
             if self._last_selection is None:
@@ -168,16 +170,18 @@ class Engine:
             self.cache.rollback(requests)
             raise
         self.cache.commit(requests)
+        if extras is not None:
+            extras.update(ctx.extras)
         return logits
 
-    def _graph_step(self, entries: list):
+    def _graph_step(self, entries: list, extras: dict | None = None):
         """A decode step (one token per sequence) replayed from a captured HIP graph."""
         check_entries(entries, self.cache, self.model.vocab)
         requests = [(e.slot, 1) for e in entries]
         self.cache.reserve(requests)
         try:
             pasts = [self.cache.length(e.slot) for e in entries]
-            logits = self.graphs.step(entries, pasts)
+            logits = self.graphs.step(entries, pasts, extras)
         except BaseException:
             self.cache.rollback(requests)
             raise

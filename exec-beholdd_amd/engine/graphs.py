@@ -133,7 +133,7 @@ class DecodeGraphs:
         return (getattr(model, "graph_safe", False) and self.engine.device.type == "cuda"
                 and all(len(e.tokens) == 1 for e in ctx_entries))
 
-    def step(self, entries, pasts):
+    def step(self, entries, pasts, extras=None):
         cache = self.engine.cache
         pages = max(-(-(past + 1) // cache.page_size) for past in pasts)
         width = -(-pages // PAGE_BUCKET) * PAGE_BUCKET
@@ -147,4 +147,7 @@ class DecodeGraphs:
             graph = DecodeGraph(self.engine, *key, pool=self.pool)
         self.graphs[key] = graph
         graph.fill(entries, pasts)
-        return graph.run()
+        logits = graph.run()
+        if extras is not None:
+            extras.update(graph.ctx.extras)      # what the parts left when the step was launched and captured: every replay writes it again
+        return logits

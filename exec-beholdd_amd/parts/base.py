@@ -95,6 +95,10 @@ class StepContext:
     sequence), seq_slot [B] (cache slot of each sequence), seq_past [B] (tokens the cache held
     before this step).  The `host_*` lists carry the same numbers for parts that decide on the
     host.  `is_decode` says that every sequence brings exactly one token.
+    `extras` is the step's second way out, beside the logits: a part may leave there what a caller wants to
+    inspect (a routed feed-forward its routing, a mixer its state's norm), under a key of its own; the step
+    function hands the dictionary to a caller who asks for it (`Engine.step(entries, extras={})`).  In a
+    captured step the tensors left there are written again by every replay.
     """
     kernels: object
     act_dtype: torch.dtype

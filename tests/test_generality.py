@@ -46,13 +46,17 @@ def test_toy_architectures_step_like_their_plain_forms(tmp_path, architecture):
         from beholdd.engine import StepEntry
         tokens = schedules.random_requests(90, [120], seed=4)[0]
         slot = engine.alloc_slot()
-        engine.step([StepEntry(slot, tokens, [])])
+        seen = {}
+        engine.step([StepEntry(slot, tokens, [])], extras=seen)
         engine.free_slot(slot)
         _, weights = toy_parts.load_plain_weights(folder)
         _, routing = toy_parts.plain_own_logits(toy_parts.OWN, weights, tokens)
         routed = [block.feed_forward for block in engine.model.blocks[::2]]
         for part, want in zip(routed, routing):
             assert part.last_routing.tolist() == want.tolist()
+        # what the parts leave in the step's extras comes out of the step function: one routing row per token and layer
+        assert sorted(seen["routing"]) == ["blocks.0.routed.router.weight", "blocks.2.routed.router.weight"][:len(routed)]
+        assert [seen["routing"][name].tolist() for name in sorted(seen["routing"])] == [want.tolist() for want in routing]
         assert sorted(set(routing[0].tolist())) == [0, 1, 2]
     else:
         assert sorted(needs) == [0, 2] and engine.model.run_writes == [True, False, True, False]
