@@ -1170,7 +1170,7 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
 #define BH_FINISH(SWIGLU, TC)                                                                                \
   gemm_parts_finish_kernel<SWIGLU, TC><<<finish_grid, 256, 0, stream>>>((const float*)scratch, (TC*)c, M, N, K, \
                                                                          parts, accumulate, norm, finish_blocks)
-  if (slices && !f32 && gemm_slices_gated(M, N, K, activation))   // the SwiGLU of many outputs: no parts, no finishing kernel
+  if (!f32 && a_block_rows == 16 && layout == 1 && gemm_slices_gated(M, N, K, activation))   // the SwiGLU of many outputs: no parts, no finishing kernel
     return gemm_slices_launch_gated(a, w, c, c_block_rows, M, N, K, ahead_ss, ahead_blocks, ahead_eps, stream);
   if (slices) {
     BH_REQUIRE(((uintptr_t)c | (uintptr_t)scratch | (uintptr_t)behind_rows) % 16 == 0,

@@ -9,7 +9,7 @@
 //   K in parts over workgroups of four waves, so that the chip is full (about 512 workgroups); the bare sums go to
 //   scratch memory as [part][row][weight row] and gemm_parts_finish_kernel (gemm_bf16.hip) adds them and applies
 //   norm factors, SwiGLU and accumulation;
-//   a SwiGLU of so many outputs that workgroups of eight waves per 64 outputs fill the chip walks over all of K
+//   a SwiGLU of so many outputs that workgroups of six waves per 48 outputs fill the chip walks over all of K
 //   and finishes itself (GATED below): no scratch memory, no second launch.
 //
 // Needs: W in the tiles layout (16 rows x 64 k blocks), the activations in blocks of 16 rows x 32 k in operand
@@ -105,15 +105,15 @@ __global__ __launch_bounds__(64 * WAVES, SC == 4 || MB > 4 ? 2 : 4) void gemm_sl
   // The norm ahead: eight threads per row add up its partial sums, each every eighth, in a fixed order.
   __shared__ float row_factor[GATED ? 16 * MB : 1];
   if (GATED && out.ahead_ss) {
-    const int part = threadIdx.x % WAVES;    // WAVES threads per row, 64 rows at a time
+    const int part = threadIdx.x % 4;    // four threads per row, 16 WAVES rows at a time
 #pragma unroll
-    for (int row0 = 0; row0 < 16 * MB; row0 += 64) {
-      const int row = row0 + threadIdx.x / WAVES;
+    for (int row0 = 0; row0 < 16 * MB; row0 += 16 * WAVES) {
+      const int row = row0 + threadIdx.x / 4;
       float ss = 0.f;
       if (row < M)
-        for (int block0 = part; block0 < out.ahead_blocks; block0 += WAVES) ss += out.ahead_ss[(size_t)row * out.ahead_blocks + block0];
-#pragma unroll
-      for (int step = WAVES / 2; step >= 1; step /= 2) ss += __shfl_xor(ss, step, 64);
+        for (int block0 = part; block0 < out.ahead_blocks; block0 += 4) ss += out.ahead_ss[(size_t)row * out.ahead_blocks + block0];
+      ss += __shfl_xor(ss, 2, 64);
+      ss += __shfl_xor(ss, 1, 64);
       if (part == 0 && row < 16 * MB) row_factor[row] = row < M ? 1.0f / sqrtf(ss / (float)K + out.ahead_eps) : 0.f;   // visible after the first meeting
     }
   }
@@ -214,15 +214,19 @@ bool gemm_slices_takes(int M, int N, int K, int layout, int activation) {
 // whole model (decode step of 64 sequences, context 640) 5.50 against 5.56 and 5.67 ms for the other two, 5.98 before.
 constexpr int WAVES = 4;
 static int target_workgroups() { return 2 * bh_compute_units(); }      // 512 on the chip these were measured on
-// The SwiGLU that finishes itself has one workgroup of eight waves per 64 outputs (192 at Qwen3-8B's sizes, fewer than
-// compute units), so a wave may use twice the registers: stages of four chunks, 8 to 16 KB of W on their way per wave
-// (gate+up at 64 rows 46.4 us; with stages of two chunks 56.1; four waves per 32 outputs 49.7; K in two parts and the
-// finishing kernel 52.1; the tiles 47.4).
-constexpr int GATED_WAVES = 8, GATED_CHUNKS = 4;
+// The SwiGLU that finishes itself has one workgroup per compute unit at most, so a wave may use twice the registers:
+// stages of four chunks, 8 to 16 KB of W on their way per wave (gate+up at 64 rows with eight waves per 64 outputs
+// 46.4 us; with stages of two chunks 56.1; four waves per 32 outputs 49.7; K in two parts and the finishing kernel
+// 52.1; the tiles 47.4).
+// Six waves (48 outputs a workgroup: 256 workgroups at these sizes) against eight (64 outputs, 192 workgroups), gate+up
+// alone: 40 rows 39.7 / 44.5 us, 64 rows 47.1 / 46.7, 96 rows 50.6 / 54.9.
+constexpr int GATED_WAVES = 6, GATED_CHUNKS = 4;
 
 bool gemm_slices_gated(int M, int N, int K, int activation) {
-  // with enough outputs that workgroups of 64 outputs each fill the chip, a SwiGLU needs no parts
-  return activation && gemm_slices_takes(M, N, K, 1, activation) && (N + 63) / 64 >= bh_compute_units() * 5 / 8 && N % 32 == 0;
+  // With enough outputs that its workgroups fill the chip, a SwiGLU needs no parts.  (Also tried for 9 to 32 rows, which
+  // the kernel with a workgroup per 16 weight rows takes: gate+up alone 38.4 against 40.1 us at 17 to 32 rows, 35.6 against
+  // 34.7 at 16, but the whole decode step slower, 16 sequences 4.53 against 4.30 ms, 32 sequences 5.53 against 5.48.)
+  return activation && gemm_slices_takes(M, N, K, 1, activation) && (N / 16 + GATED_WAVES / 2 - 1) / (GATED_WAVES / 2) >= bh_compute_units() * 5 / 8 && N % 32 == 0;
 }
 
 int gemm_slices_parts(int M, int N, int K, int activation, int* stages_per_part) {
