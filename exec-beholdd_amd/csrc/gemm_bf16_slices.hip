@@ -68,7 +68,7 @@ struct GatedOut {
 __device__ inline float silu_mul(float gate, float up) { return gate / (1.0f + expf(-gate)) * up; }
 
 template <int MB, int SC, int WAVES, bool GATED>
-__global__ __launch_bounds__(64 * WAVES, SC == 4 || MB > 4 ? 2 : 4) void gemm_slices_kernel(const uint16_t* __restrict__ a,
+__global__ __launch_bounds__(64 * WAVES, GATED ? (WAVES + 3) / 4 : MB > 4 ? 2 : 4) void gemm_slices_kernel(const uint16_t* __restrict__ a,
                                                                     const uint16_t* __restrict__ w,
                                                                     float* __restrict__ sums, int M, int w_rows, int K,
                                                                     int stages_per_part, GatedOut out) {
@@ -218,15 +218,32 @@ static int target_workgroups() { return 2 * bh_compute_units(); }      // 512 on
 // stages of four chunks, 8 to 16 KB of W on their way per wave (gate+up at 64 rows with eight waves per 64 outputs
 // 46.4 us; with stages of two chunks 56.1; four waves per 32 outputs 49.7; K in two parts and the finishing kernel
 // 52.1; the tiles 47.4).
-// Six waves (48 outputs a workgroup: 256 workgroups at these sizes) against eight (64 outputs, 192 workgroups), gate+up
-// alone: 40 rows 39.7 / 44.5 us, 64 rows 47.1 / 46.7, 96 rows 50.6 / 54.9.
-constexpr int GATED_WAVES = 6, GATED_CHUNKS = 4;
+// How many blocks of gate rows a workgroup takes (twice as many waves): a workgroup walks over all of K, so the
+// kernel lasts as long as the compute unit that carries the most bytes, and workgroups that share a compute unit share
+// its bandwidth: the fewest bytes per compute unit, ceil(workgroups / compute units) x blocks, decides, the smaller
+// workgroup at a tie.  Qwen3-8B (768 blocks of gate rows, 256 compute units): three blocks, 256 workgroups of six
+// waves; gate+up alone against four blocks (192 workgroups of eight waves): 40 rows 39.7 / 44.5 us, 64 rows 47.1 / 46.7,
+// 96 rows 50.6 / 54.9.  Qwen3-14B (1,088 blocks): five, gate+up at 64 rows 71.6 us (5.0 TB/s); three, with 363 workgroups,
+// 99.7.  Qwen3-32B (1,600 blocks): seven, 117.5 us (4.5 TB/s; 18 registers of a wave spilled); three 145.7.
+constexpr int GATED_CHUNKS = 4, GATED_MOST_BLOCKS = 8;
+// (Beyond 64 rows the registers of a wave hold six blocks of rows: more than eight waves a workgroup leave a wave too few
+// and it spills, 96 rows at Qwen3-14B's sizes 101.8 us with ten waves.)
+static int gated_blocks(int M, int N) {
+  const int gate_blocks = N / 16, units = bh_compute_units();
+  int best = 3, best_cost = 1 << 30;
+  for (int b = 3; b <= (M > 64 ? 4 : GATED_MOST_BLOCKS); ++b) {
+    const int workgroups = (gate_blocks + b - 1) / b, cost = ((workgroups + units - 1) / units) * b;
+    if (cost < best_cost) best = b, best_cost = cost;
+  }
+  return best;
+}
 
 bool gemm_slices_gated(int M, int N, int K, int activation) {
   // With enough outputs that its workgroups fill the chip, a SwiGLU needs no parts.  (Also tried for 9 to 32 rows, which
   // the kernel with a workgroup per 16 weight rows takes: gate+up alone 38.4 against 40.1 us at 17 to 32 rows, 35.6 against
   // 34.7 at 16, but the whole decode step slower, 16 sequences 4.53 against 4.30 ms, 32 sequences 5.53 against 5.48.)
-  return activation && gemm_slices_takes(M, N, K, 1, activation) && (N / 16 + GATED_WAVES / 2 - 1) / (GATED_WAVES / 2) >= bh_compute_units() * 5 / 8 && N % 32 == 0;
+  return activation && gemm_slices_takes(M, N, K, 1, activation) && N % 32 == 0 &&
+         (N / 16 + gated_blocks(M, N) - 1) / gated_blocks(M, N) >= bh_compute_units() * 5 / 8;
 }
 
 int gemm_slices_parts(int M, int N, int K, int activation, int* stages_per_part) {
@@ -268,15 +285,23 @@ int gemm_slices_launch_gated(const void* a, const void* w, void* gated, int gate
   BH_REQUIRE(gemm_slices_gated(M, N, K, 1), "gemm_slices: a SwiGLU of M=%d N=%d K=%d is not one this kernel finishes itself", M, N, K);
   BH_REQUIRE(((uintptr_t)a | (uintptr_t)w | (uintptr_t)gated) % 16 == 0, "gemm_slices: operands must be 16-byte aligned");
   BH_REQUIRE(!ahead_ss || (ahead_blocks > 0 && ahead_eps > 0.f), "gemm_slices: the norm ahead needs partial sums and an epsilon");
-  constexpr int SC = GATED_CHUNKS, WAVES = GATED_WAVES;
+  constexpr int SC = GATED_CHUNKS;
+  const int blocks_each = gated_blocks(M, N), WAVES = 2 * blocks_each;
   const GatedOut out = {(uint16_t*)gated, gated_block_rows, N, ahead_ss, ahead_blocks, ahead_eps};
   const dim3 grid((N / 16 + WAVES / 2 - 1) / (WAVES / 2)), block(64 * WAVES);
   const int stages = K / (64 * SC);
-#define BH_GATED(MB) gemm_slices_kernel<MB, SC, WAVES, true><<<grid, block, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, nullptr, M, 2 * N, K, stages, out)
-  if (M <= 48) BH_GATED(3);
-  else if (M <= 64) BH_GATED(4);
-  else if (M <= 96) BH_GATED(6);
-  else BH_GATED(8);
+#define BH_GATED(MB, NW) gemm_slices_kernel<MB, SC, NW, true><<<grid, block, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, nullptr, M, 2 * N, K, stages, out)
+#define BH_GATED_ROWS(NW) do { if (M <= 48) BH_GATED(3, NW); else if (M <= 64) BH_GATED(4, NW); else BH_GATED(6, NW); } while (0)
+  static_assert(MOST_ROWS_GATED <= 96 && GATED_MOST_BLOCKS == 8, "the forms below");
+  switch (blocks_each) {
+    case 3: BH_GATED_ROWS(6); break;
+    case 4: BH_GATED_ROWS(8); break;
+    case 5: BH_GATED_ROWS(10); break;
+    case 6: BH_GATED_ROWS(12); break;
+    case 7: BH_GATED_ROWS(14); break;
+    default: BH_GATED_ROWS(16); break;
+  }
+#undef BH_GATED_ROWS
 #undef BH_GATED
   return bh_check_launch("gemm_slices");
 }
