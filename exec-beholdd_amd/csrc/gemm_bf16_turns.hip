@@ -303,7 +303,8 @@ bool gemm_turns_can(int M, int N, int K, int layout, int activation, int blocks)
 namespace {
 struct TurnsPlan {
   int blocks;   // tile width for the product in one launch, or 0
-  int parts;    // parts of K with the widest tile, or 1
+  int parts;    // parts of K, or 1
+  int part_blocks = 8;   // the tile width of the parts
 };
 TurnsPlan turns_plan(int M, int N, int K, int layout, int activation) {
   TurnsPlan plan = {0, 1};
@@ -321,19 +322,32 @@ TurnsPlan turns_plan(int M, int N, int K, int layout, int activation) {
     const double rate = 1430.0 * (units / 256.0) * work / ((double)rounds * units * 256 * (activation ? 2 : 1) * outs * cost);
     if (rate >= best_rate) best_rate = direct_rate = rate, plan.blocks = blocks;
   }
-  if (!activation && M >= 512 && gemm_turns_can(M, N, K, layout, 0, 8)) {
+  if (!activation && M >= 320 && gemm_turns_can(M, N, K, layout, 0, 8)) {
     // As many parts (8, 4 or 2) as keep the workgroups within one round and every part at least 512 long; worth
     // it from about five eighths of the chip on.  Measured at the Qwen3-8B widths against the other kernels, us:
     // 512 rows: down in 8 parts 88 -> 72 (o in 4 parts, half the chip, 41 -> 45; in 8 parts of 512 the prefill step of
     // 512 tokens is 0.5 % faster than with the older tiles); 768 rows: o 71 -> 53,
     // down 195 -> 102 in 4; 1,024 rows: o 72 -> 57, down 196 -> 111 in 4; 1,536 rows: o 93 -> 77, down 219 -> 173 in 2;
-    // 2,048 rows: down 240 -> 199 in 2; 384 rows: slower for qkv and o, so not below 512.
-    const long tiles = (long)((N + 255) / 256) * ((M + 255) / 256);
-    int parts = 8;
-    while (parts > 1 && (tiles * parts > units || K / parts < 512 || K % (128 * parts) != 0)) parts /= 2;
-    if (parts > 1 && tiles * parts >= units * 5 / 8) {
-      const double rate = 0.85 * 1430.0 * (units / 256.0) * work / ((double)units * 256 * 256 / parts);
-      if (rate > direct_rate) plan.blocks = 0, plan.parts = parts;
+    // 2,048 rows: down 240 -> 199 in 2.  From 320 rows on (a whole prefill step of the Qwen3-8B shape with the parts from 257
+    // rows on instead of from 512 on: 272 tokens 9.15 -> 9.24 ms, 320 tokens 9.34 -> 9.25, 384 tokens 9.62 -> 9.48, 448 tokens
+    // 10.88 -> 9.77).
+    // With the widest tile first; where that needs eight parts (257 to 512 rows at these widths), four parts of the
+    // 128-wide tile instead: half the bare sums to write and to read again (512 rows at the Qwen3-8B widths, product +
+    // finishing kernel, o and down on average: 42.5 + 19.9 -> 40.9 + 14.1 us; where the widest tile needs four parts or
+    // two, the narrower one lost: 640 rows 51.8 + 16.0 -> 64.0 + 13.1, 1,024 rows 60.8 + 21.7 -> 73.8 + 17.4; the
+    // 192-wide tile lost everywhere).
+    auto parts_of = [&](int pb) {
+      const int outs = 32 * pb;
+      const long tiles = (long)((N + outs - 1) / outs) * ((M + 255) / 256);
+      int parts = 8;
+      while (parts > 1 && (tiles * parts > units || K / parts < 512 || K % (128 * parts) != 0)) parts /= 2;
+      return parts > 1 && tiles * parts >= units * 5 / 8 ? parts : 1;
+    };
+    int pb = 8, parts = parts_of(8);
+    if (parts == 8 && gemm_turns_can(M, N, K, layout, 0, 4) && parts_of(4) == 4) pb = 4, parts = 4;
+    if (parts > 1) {
+      const double rate = 0.85 * 1430.0 * (units / 256.0) * work / ((double)units * 256 * 32 * pb / parts * (pb == 8 ? 1.0 : 1.34));
+      if (rate > direct_rate) plan.blocks = 0, plan.parts = parts, plan.part_blocks = pb;
     }
   }
   return plan;
@@ -349,10 +363,11 @@ int gemm_turns_parts(int M, int N, int K, int layout, int activation) {
 
 int gemm_turns_launch_parts(const void* a, const void* w, float* sums, int M, int N, int K, int parts, int a_blocked,
                             hipStream_t stream) {
-  BH_REQUIRE(parts >= 1 && K % (128 * parts) == 0 && gemm_turns_can(M, N, K / parts, 1, 0, 8),
+  const int pb = turns_plan(M, N, K, 1, 0).part_blocks;
+  BH_REQUIRE(parts >= 1 && K % (128 * parts) == 0 && gemm_turns_can(M, N, K / parts, 1, 0, pb),
              "gemm_turns: M=%d N=%d K=%d cannot be multiplied in %d parts of K", M, N, K, parts);
   BH_REQUIRE(((uintptr_t)a | (uintptr_t)w | (uintptr_t)sums) % 16 == 0, "gemm_turns: operands must be 16-byte aligned");
-  launch<1>(a, w, sums, 8, M, N, K, 0, a_blocked, 0, stream, parts);
+  launch<1>(a, w, sums, pb, M, N, K, 0, a_blocked, 0, stream, parts);
   return bh_check_launch("gemm_turns");
 }
 

@@ -405,7 +405,7 @@ __device__ inline void load_eight(const bf16_t* p, float (&v)[8]) {
 }
 
 // The same for many bfloat16 rows: a lane takes 8 consecutive elements of a head (16 bytes), LPH = head_dim / 8
-// lanes a head, 64 / LPH heads a wave, four waves a block.  The rotation spans the whole head or is absent, so
+// lanes a head, 64 / LPH heads of RPW rows a wave, four waves a block.  The rotation spans the whole head or is absent, so
 // that an element's partner sits LPH / 2 lanes away.  Per q or k head: one 16-byte load, one 16-byte store.
 // The values have waves of their own, behind the `main_waves` that take the q and k heads (`n_heads` of them):
 // a value's neighbours in memory are the same dim of other tokens, eight tokens to a 16-byte piece in either
@@ -414,7 +414,28 @@ __device__ inline void load_eight(const bf16_t* p, float (&v)[8]) {
 // rows, turn the 8 x 8 elements and store whole pieces; rows whose piece is not whole in this step (a step's
 // first and last tokens) store their eight elements one by one.  (8,192 rows of 32 query and 8 kv heads of
 // 128: the stores of the values one by one were 35 of the kernel's 57 us.)
-template <typename TW, int LPH>
+// The value that the lane LPH / 2 further on (or back) in the same head holds, and a sum over a head's LPH lanes, in
+// all of them.  A head of 16 lanes is a row of the wave's data-parallel moves: rotations within the row, no trip through LDS.
+template <int LPH>
+__device__ inline float head_partner(float v) {
+  if constexpr (LPH == 16) return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x128, 0xf, 0xf, false));   // row_ror:8
+  else return __shfl_xor(v, LPH / 2, BH_WAVE);
+}
+template <int LPH>
+__device__ inline float head_sum(float v) {
+  if constexpr (LPH == 16) {
+    v += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x128, 0xf, 0xf, false));   // row_ror:8, 4, 2, 1
+    v += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x124, 0xf, 0xf, false));
+    v += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x122, 0xf, 0xf, false));
+    v += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x121, 0xf, 0xf, false));
+  } else {
+#pragma unroll
+    for (int off = LPH / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, BH_WAVE);
+  }
+  return v;
+}
+
+template <typename TW, int LPH, int RPW>   // RPW: rows that a wave of the q and k heads takes
 __global__ __launch_bounds__(256) void qk_norm_rope_cache_rows_kernel(
     const uint16_t* __restrict__ qkv, uint16_t* __restrict__ q_out, const TW* __restrict__ q_weight,
     const TW* __restrict__ k_weight, float eps, const float* __restrict__ cos_table,
@@ -427,24 +448,37 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_rows_kernel(
   if (wave >= main_waves) {   // the values of eight rows and HPW kv heads
     if (wave - main_waves >= value_waves) return;   // the last block's waves beyond the work (none at all without write_kv)
     const int chunks = (KVH + HPW - 1) / HPW, group = (wave - main_waves) / chunks;
-    const int kv_head = ((wave - main_waves) % chunks) * HPW + lane / LPH, c = lane % LPH;
-    if (kv_head >= KVH) return;
+    // lanes without a kv head of their own follow the last one and store nothing: every lane stays to the end,
+    // because the rows' positions below are read out of the first 24 lanes' registers
+    const int wanted_head = ((wave - main_waves) % chunks) * HPW + lane / LPH, c = lane % LPH;
+    const bool mine = wanted_head < KVH;
+    const int kv_head = mine ? wanted_head : KVH - 1;
     const size_t fused = (size_t)(H + 2 * KVH) * HD;
     const uint16_t* src = qkv + (size_t)(H + KVH + kv_head) * HD + 8 * c;   // + row * fused
+    // Positions and sequences of the rows 8 group - 8 .. 8 group + 15, one in each of the first 24 lanes, in one load
+    // each: everything that the eight rows' decisions below look at (asked for row by row inside the loop, eight
+    // waits for memory in a row were most of this kernel's time at a few hundred rows).
+    const int base = 8 * group - 8;
+    const int near = min(max(base + lane, 0), n_rows - 1);
+    const int near_pos = positions[near], near_seq = row_seq[near];
+    auto pos_of = [&](int row) { return __builtin_amdgcn_readlane(near_pos, __builtin_amdgcn_readfirstlane(row - base)); };
+    auto seq_of = [&](int row) { return __builtin_amdgcn_readlane(near_seq, __builtin_amdgcn_readfirstlane(row - base)); };
     for (int row = 8 * group; row < 8 * group + 8 && row < n_rows; ++row) {
-      const int pos = positions[row], seq = row_seq[row];
+      const int pos = pos_of(row), seq = seq_of(row);
       const int first = row - pos % 8;   // where the row of the piece's first token would lie
-      const bool whole = first >= 0 && first + 7 < n_rows && row_seq[first] == seq && row_seq[first + 7] == seq &&
-                         positions[first] == pos - pos % 8 && positions[first + 7] == pos - pos % 8 + 7;
+      const bool whole = first >= 0 && first + 7 < n_rows && seq_of(first) == seq && seq_of(first + 7) == seq &&
+                         pos_of(first) == pos - pos % 8 && pos_of(first + 7) == pos - pos % 8 + 7;
       if (whole && pos % 8 != 0) continue;   // the first row of the piece stores it
       const int page = page_table[(size_t)seq * table_stride + pos / BH_PAGE];
       uint16_t* block = v_pages + ((size_t)page * KVH + kv_head) * BH_PAGE * HD;
       if (!whole) {
         const uint4 raw = *reinterpret_cast<const uint4*>(src + (size_t)row * fused);
         const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+        if (mine) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          block[bh_value_index(kv_order, pos % BH_PAGE, 8 * c + e, HD)] = (uint16_t)(words[e / 2] >> (16 * (e % 2)));
+          for (int e = 0; e < 8; ++e)
+            block[bh_value_index(kv_order, pos % BH_PAGE, 8 * c + e, HD)] = (uint16_t)(words[e / 2] >> (16 * (e % 2)));
+        }
         continue;
       }
       uint4 raw[8];   // token t's dims 8 c .. 8 c + 7
@@ -461,65 +495,78 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_rows_kernel(
         piece.y = __builtin_amdgcn_perm(word[3], word[2], pick);
         piece.z = __builtin_amdgcn_perm(word[5], word[4], pick);
         piece.w = __builtin_amdgcn_perm(word[7], word[6], pick);
-        *reinterpret_cast<uint4*>(block + bh_value_index(kv_order, pos % BH_PAGE, 8 * c + e, HD)) = piece;
+        if (mine) *reinterpret_cast<uint4*>(block + bh_value_index(kv_order, pos % BH_PAGE, 8 * c + e, HD)) = piece;
       }
     }
     return;
   }
-  const int row = wave / waves_per_row;
-  if (row >= n_rows) return;   // whole waves leave; nothing below synchronises the block
+  const int first_row = (wave / waves_per_row) * RPW;
+  if (first_row >= n_rows) return;   // whole waves leave; nothing below synchronises the block
   const int wanted = (wave % waves_per_row) * HPW + lane / LPH, c = lane % LPH;
   const bool active = wanted < n_heads;
   const int head = active ? wanted : n_heads - 1;   // lanes without a head of their own follow the last one and store nothing
   const bool is_q = head < H;
-  const int pos = positions[row];
-  const uint16_t* src = qkv + ((size_t)row * (H + 2 * KVH) + head) * HD + 8 * c;
-  const uint4 raw = *reinterpret_cast<const uint4*>(src);
-  const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
-  float x[8];
+  // All of a wave's loads are asked for before anything is computed: RPW rows' 16 bytes, their positions and, behind
+  // those, their angles.  (With one row per wave the three waits in a row, for so little data each, were the kernel's time.)
+  int pos[RPW];
+  uint4 raw[RPW];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) x[e] = bf16_bits_to_f32((uint16_t)(words[e / 2] >> (16 * (e % 2))));
+  for (int r = 0; r < RPW; ++r) {
+    const int row = min(first_row + r, n_rows - 1);
+    pos[r] = positions[row];
+    raw[r] = *reinterpret_cast<const uint4*>(qkv + ((size_t)row * (H + 2 * KVH) + head) * HD + 8 * c);
+  }
   const TW* weight = is_q ? q_weight : k_weight;
-  {
+  float wv[8];
+  if (weight != nullptr) load_eight(weight + 8 * c, wv);
+  constexpr int HALF = HD / 2;
+  float cs[RPW][8], sn[RPW][8];
+  if (cos_table != nullptr) {
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) {
+      load_eight(cos_table + (size_t)pos[r] * HALF + 8 * (c % (LPH / 2)), cs[r]);
+      load_eight(sin_table + (size_t)pos[r] * HALF + 8 * (c % (LPH / 2)), sn[r]);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < RPW; ++r) {
+    const int row = first_row + r;
+    const uint32_t words[4] = {raw[r].x, raw[r].y, raw[r].z, raw[r].w};
+    float x[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = bf16_bits_to_f32((uint16_t)(words[e / 2] >> (16 * (e % 2))));
     if (weight != nullptr) {
       float ss = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
-#pragma unroll
-      for (int off = LPH / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, BH_WAVE);
+      ss = head_sum<LPH>(ss);
       const float inv = 1.0f / sqrtf(ss / (float)HD + eps);
-      float wv[8];
-      load_eight(weight + 8 * c, wv);
 #pragma unroll
       for (int e = 0; e < 8; ++e) x[e] = x[e] * inv * wv[e];
     }
     if (cos_table != nullptr) {
-      constexpr int HALF = HD / 2;
       const bool lower = c < LPH / 2;
-      float cs[8], sn[8];
-      load_eight(cos_table + (size_t)pos * HALF + 8 * (c % (LPH / 2)), cs);
-      load_eight(sin_table + (size_t)pos * HALF + 8 * (c % (LPH / 2)), sn);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float other = __shfl_xor(x[e], LPH / 2, BH_WAVE);
-        x[e] = lower ? x[e] * cs[e] - other * sn[e] : other * sn[e] + x[e] * cs[e];
+        const float other = head_partner<LPH>(x[e]);
+        x[e] = lower ? x[e] * cs[r][e] - other * sn[r][e] : other * sn[r][e] + x[e] * cs[r][e];
       }
+    }   // (all the lanes of a head take the same way through this: the exchanges stay within the head)
+    if (!active || row >= n_rows) continue;
+    uint4 packed;
+    packed.x = (uint32_t)f32_to_bf16_bits(x[0]) | ((uint32_t)f32_to_bf16_bits(x[1]) << 16);
+    packed.y = (uint32_t)f32_to_bf16_bits(x[2]) | ((uint32_t)f32_to_bf16_bits(x[3]) << 16);
+    packed.z = (uint32_t)f32_to_bf16_bits(x[4]) | ((uint32_t)f32_to_bf16_bits(x[5]) << 16);
+    packed.w = (uint32_t)f32_to_bf16_bits(x[6]) | ((uint32_t)f32_to_bf16_bits(x[7]) << 16);
+    if (is_q) {
+      *reinterpret_cast<uint4*>(q_out + ((size_t)row * H + head) * HD + 8 * c) = packed;
+      continue;
     }
-  }   // (all the lanes of a head take the same way through this: the exchanges stay within the head)
-  if (!active) return;
-  uint4 packed;
-  packed.x = (uint32_t)f32_to_bf16_bits(x[0]) | ((uint32_t)f32_to_bf16_bits(x[1]) << 16);
-  packed.y = (uint32_t)f32_to_bf16_bits(x[2]) | ((uint32_t)f32_to_bf16_bits(x[3]) << 16);
-  packed.z = (uint32_t)f32_to_bf16_bits(x[4]) | ((uint32_t)f32_to_bf16_bits(x[5]) << 16);
-  packed.w = (uint32_t)f32_to_bf16_bits(x[6]) | ((uint32_t)f32_to_bf16_bits(x[7]) << 16);
-  if (is_q) {
-    *reinterpret_cast<uint4*>(q_out + ((size_t)row * H + head) * HD + 8 * c) = packed;
-    return;
+    const int page = page_table[(size_t)row_seq[row] * table_stride + pos[r] / BH_PAGE];
+    const int token = pos[r] % BH_PAGE, kv_head = head - H;
+    uint16_t* block = k_pages + ((size_t)page * KVH + kv_head) * BH_PAGE * HD;
+    *reinterpret_cast<uint4*>(block + bh_key_index(kv_order, token, 8 * c, HD)) = packed;   // 8 dims lie together in both orders
   }
-  const int page = page_table[(size_t)row_seq[row] * table_stride + pos / BH_PAGE];
-  const int token = pos % BH_PAGE, kv_head = head - H;
-  uint16_t* block = k_pages + ((size_t)page * KVH + kv_head) * BH_PAGE * HD;
-  *reinterpret_cast<uint4*>(block + bh_key_index(kv_order, token, 8 * c, HD)) = packed;   // 8 dims lie together in both orders
 }
 
 // Precondition: the rows of one sequence stand one after the other and in position order (row r + 1 of a
@@ -546,12 +593,13 @@ extern "C" int bh_qk_norm_rope_cache(const void* qkv, int dtype, void* q_out, co
   if (dtype == BH_BF16 && n_rows >= 64 && (hd == 64 || hd == 128 || hd == 256) && (rot == 0 || rot == hd)) {
     // waves for the q and k heads of every row, then (write_kv) waves for the values of eight rows each
     const int lanes_per_head = hd / 8, heads_per_wave = 64 / lanes_per_head, main_heads = write_kv ? H + KVH : H;
-    const long main_waves = (long)n_rows * ((main_heads + heads_per_wave - 1) / heads_per_wave);
+    constexpr int RPW = 4;
+    const long main_waves = (long)((n_rows + RPW - 1) / RPW) * ((main_heads + heads_per_wave - 1) / heads_per_wave);
     const long value_waves = write_kv ? (long)((n_rows + 7) / 8) * ((KVH + heads_per_wave - 1) / heads_per_wave) : 0;
     BH_REQUIRE(main_waves + value_waves < (1L << 31), "qk_norm_rope: too many rows");
     dim3 wide_grid((unsigned)((main_waves + value_waves + 3) / 4)), wide_block(4 * BH_WAVE);
 #define BH_QK_ROWS(TW, LPH)                                                                                       \
-  qk_norm_rope_cache_rows_kernel<TW, LPH><<<wide_grid, wide_block, 0, stream>>>(                                   \
+  qk_norm_rope_cache_rows_kernel<TW, LPH, RPW><<<wide_grid, wide_block, 0, stream>>>(                                   \
       (const uint16_t*)qkv, (uint16_t*)q_out, (const TW*)q_weight, (const TW*)k_weight, eps,                        \
       rot ? cos_table : nullptr, rot ? sin_table : nullptr,                                                          \
       positions, row_seq, (uint16_t*)k_pages, (uint16_t*)v_pages, page_table, table_stride, H, KVH, kv_order,      \

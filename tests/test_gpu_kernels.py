@@ -241,7 +241,8 @@ def test_norm_rides_on_wide_products(K, m, n, k, n2, g_dtype):
 
 @pytest.mark.parametrize("g_dtype", DTYPES)
 @pytest.mark.parametrize("m,n,k", [(2048, 4096, 4096), (1000, 4096, 2048 * 4), (1800, 5120 - 1024, 2048),
-                                   (601, 4096, 12288), (2047, 4080, 4096)])   # eight parts; rows and pieces that fill no block
+                                   (601, 4096, 12288), (2047, 4080, 4096),    # rows and pieces that fill no block
+                                   (512, 4096, 4096), (333, 4080, 12288)])    # four parts of the 128-wide tile
 def test_product_in_parts_of_many_rows_finishes_the_norm(K, g_dtype, m, n, k):
     """Beyond 256 rows, where K goes through the turns kernel in parts, the finishing kernel owns whole rows and
     writes the norm's output itself: `gemm(..., then_norm=)` returns it as a plain bfloat16 matrix."""
