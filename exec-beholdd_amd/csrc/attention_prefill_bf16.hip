@@ -22,11 +22,17 @@
 // probabilities by one more row of the value product, a page's operands asked of LDS in two goes ahead of
 // the arithmetic that hides the wait, and the exponentials' reference moved (and the sums so far scaled) only
 // when the maximum has grown by more than 2^8.  Measured, one sequence at 32 query and 8 kv heads of 128:
-// 2,048 rows 72 -> 60 us, 4,096 rows 194 -> 166 us, 8,192 rows 604 -> 533 us.
+// 2,048 rows 72 -> 60 us, 4,096 rows 194 -> 166 us, 8,192 rows 604 -> 533 us.  With two column tiles a wave, one
+// tile's softmax stands between the matrix instructions of the other (and the score products start from a constant
+// instead of cleared registers): 56.5, 160 and 513 us.  Counters at 8,192 rows (SQ_VALU_MFMA_BUSY_CYCLES,
+// SQ_ACTIVE_INST_VALU, SQ_VALU_MFMA_COEXEC_CYCLES): the matrix cores are busy half of the time and so is the vector
+// issue port (three vector instructions per matrix instruction, the exponentials counting double), both at once
+// a tenth of it.
 // A wave skips pages none of whose keys any of its columns may see.  Values beyond the last position
 // of the workgroup's columns are zeroed in LDS before the last page is used (their probabilities are
 // zero, but what lies there may be anything).
 #include "attention_bf16.h"
+#include <type_traits>
 
 // The larger of two numbers, a NaN if either is one (v_maximum3_f32, which takes its operands as they are; fmaxf
 // has to make each of them a quiet number first, one more instruction per score).
@@ -58,7 +64,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
   // Workgroups go to the eight XCDs in turn, each with an L2 of its own: when the number of
   // (kv head, sequence) units allows it, all tile groups of a unit run on one XCD, one after the other,
   // so that the unit's keys and values stay in that L2; and the groups with the most keys (the last
-  // rows of a causal prefill) start first.
+  // rows of a causal prefill) start first.  (Handing them out so that the two workgroups of a compute unit carry
+  // the same number of pages together, the heaviest with the lightest, changed nothing at 2,048 or 4,096 rows: there
+  // the kernel takes as long as its heaviest workgroup alone, 1.8 us a page.)
   int tile_group, unit;
   const int units = KVH * n_seqs;
   if (units % 8 == 0) {
@@ -162,106 +170,138 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
   fetch(begin, 0);
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
-  auto attend = [&](int p, int buffer) {
+  // One column tile's scores of a page -> its probabilities (as bfloat16 operands of the value product) and the
+  // factor for what was summed so far.  Vector instructions only, so that it can run between the matrix
+  // instructions of another tile.
+  auto softmax_of = [&](auto masked, int ct, f32x4_t (&st)[4], int key0, u32x4_t (&p_vec)[2]) -> float {
+    if constexpr (decltype(masked)::value) {   // key k0 + d of the page is seen if lo <= k0 + d <= pos: two numbers per column, then constants
+      const int d_last = pos[ct] - key0, d_first = lo[ct] - key0;
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int d = 32 * (t / 2) + 4 * (t % 2) + r;
+          if (d > d_last || d < d_first) st[t][r] = -INFINITY;
+        }
+    }
+    // Online softmax with few instructions: the maximum is taken over the raw scores, the scale
+    // enters through one fused multiply-add per score, and the exponentials are bare v_exp_f32
+    // (arguments <= 0; results below the normal range may flush to zero).
+    float local_max = larger(larger(st[0][0], st[0][1]), st[0][2]);
+    local_max = larger(larger(local_max, st[0][3]), st[1][0]);
+#pragma unroll
+    for (int t = 1; t < 4; ++t) {
+      local_max = larger(larger(local_max, st[t][1]), st[t][2]);
+      local_max = larger(larger(local_max, st[t][3]), t < 3 ? st[t + 1][0] : run_max[ct]);
+    }
+    const float new_max = largest_of_column(local_max);               // raw (unscaled) scores, the earlier pages' too
+    // The exponentials' reference moves only when the maximum has grown by more than SLACK powers of two (or
+    // from nothing): until then probabilities may reach 2^SLACK, which float32 sums and bfloat16 operands
+    // hold as well as numbers up to one, and what was summed so far needs no factor.
+    const bool stays = (new_max - run_max[ct]) * scale_log2 <= SLACK;   // false from -inf, and while nothing was seen
+    const float reference = stays ? run_max[ct] : new_max;
+    const float shift = (reference == -INFINITY) ? 0.f : -reference * scale_log2;
+    // exactly 1 while the reference stands still, 0 when nothing was seen before
+    const float alpha =
+        (run_max[ct] == reference) ? 1.0f : __builtin_amdgcn_exp2f((run_max[ct] - reference) * scale_log2);
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const int t = 2 * u + half;
+        const float e0 = __builtin_amdgcn_exp2f(fmaf(st[t][0], scale_log2, shift));
+        const float e1 = __builtin_amdgcn_exp2f(fmaf(st[t][1], scale_log2, shift));
+        const float e2 = __builtin_amdgcn_exp2f(fmaf(st[t][2], scale_log2, shift));
+        const float e3 = __builtin_amdgcn_exp2f(fmaf(st[t][3], scale_log2, shift));
+        p_vec[u][2 * half] = pack_bf16(e0, e1);
+        p_vec[u][2 * half + 1] = pack_bf16(e2, e3);
+      }
+    run_max[ct] = reference;
+    return alpha;
+  };
+  auto scale_sums = [&](int ct, float alpha) {
+    if (__any(alpha != 1.0f)) {   // after the first pages the reference seldom moves
+      run_sum[ct] = run_sum[ct] * alpha;
+#pragma unroll
+      for (int dt = 0; dt < 2 * NS; ++dt) o[ct][dt] = o[ct][dt] * alpha;
+    }
+  };
+  // The matrix instructions of one tile and the vector instructions of another are independent of each other: side
+  // by side in one stretch of code they are issued in turn (a matrix instruction keeps the matrix core busy for 16
+  // clocks and the issue port for 4; this asks the compiler for five vector instructions after each), so that a
+  // wave's softmax runs under its own products and not only under another wave's.
+#define BH_TAKE_TURNS(n)                                            \
+  do {                                                              \
+    _Pragma("unroll") for (int turn = 0; turn < (n); ++turn) {      \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);            \
+      __builtin_amdgcn_sched_group_barrier(0x402, 5, 0);            \
+    }                                                               \
+  } while (0)
+  auto scores_of = [&](int ct, const u32x4_t (&kop)[4 * NS], f32x4_t (&st)[4]) {   // 4 NS matrix instructions
+    const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};   // (the first product of each chain adds to a constant: no registers to clear)
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+        st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kop[t * NS + s]), q_vec[ct][s], s == 0 ? zero : st[t], 0, 0, 0);
+  };
+  auto values_of = [&](int ct, const u32x4_t (&vop)[4 * NS], const u32x4_t (&p_vec)[2]) {   // 4 NS + 2 matrix instructions
+    run_sum[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(ones), as_bf16x8(p_vec[0]), run_sum[ct], 0, 0, 0);
+#pragma unroll
+    for (int dt = 0; dt < 2 * NS; ++dt)
+      o[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vop[dt * 2]), as_bf16x8(p_vec[0]), o[ct][dt], 0, 0, 0);
+    run_sum[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(ones), as_bf16x8(p_vec[1]), run_sum[ct], 0, 0, 0);
+#pragma unroll
+    for (int dt = 0; dt < 2 * NS; ++dt)
+      o[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vop[dt * 2 + 1]), as_bf16x8(p_vec[1]), o[ct][dt], 0, 0, 0);
+  };
+  auto attend_page = [&](auto masked, int p, int buffer) {
     const u32x4_t* kl = page_lds[buffer];
     const u32x4_t* vl = page_lds[buffer] + PIECES;
+    const int key0 = p * BH_PAGE + 8 * g;  // lane (j, g) holds keys key0 + 32 * (t / 2) + 4 * (t % 2) + r
+    // A page's operands are asked of LDS in two goes, each before the arithmetic that hides the wait: all the
+    // keys' before the first score product, all the values' behind it.
+    u32x4_t kop[4 * NS], vop[4 * NS];
+#pragma unroll
+    for (int i = 0; i < 4 * NS; ++i) kop[i] = kl[i * 64 + lane];
+    __builtin_amdgcn_sched_barrier(0);
+    f32x4_t st[CTW][4];
+    u32x4_t p_vec[CTW][2];
+    scores_of(0, kop, st[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (CTW == 1) {
+#pragma unroll
+      for (int i = 0; i < 4 * NS; ++i) vop[i] = vl[i * 64 + lane];
+      __builtin_amdgcn_sched_barrier(0);
+      const float alpha = softmax_of(masked, 0, st[0], key0, p_vec[0]);
+      scale_sums(0, alpha);
+      values_of(0, vop, p_vec[0]);
+    } else {
+      static_assert(CTW <= 2, "a wave takes one or two column tiles");
+      scores_of(1, kop, st[1]);                                              // the second tile's scores ...
+      const float alpha0 = softmax_of(masked, 0, st[0], key0, p_vec[0]);     // ... with the first tile's softmax between them
+#pragma unroll
+      for (int i = 0; i < 4 * NS; ++i) vop[i] = vl[i * 64 + lane];          // (into the registers that the keys leave)
+      BH_TAKE_TURNS(4 * NS);
+      __builtin_amdgcn_sched_barrier(0);
+      scale_sums(0, alpha0);
+      __builtin_amdgcn_sched_barrier(0);
+      values_of(0, vop, p_vec[0]);                                           // the first tile's values ...
+      const float alpha1 = softmax_of(masked, 1, st[1], key0, p_vec[1]);     // ... with the second tile's softmax
+      BH_TAKE_TURNS(4 * NS + 2);
+      __builtin_amdgcn_sched_barrier(0);
+      scale_sums(1, alpha1);
+      __builtin_amdgcn_sched_barrier(0);
+      values_of(1, vop, p_vec[1]);
+    }
+  };
+  auto attend = [&](int p, int buffer) {
     // a page none of whose keys this wave's columns may see changes nothing
     const bool visible = wave_active && p * BH_PAGE <= pos_max && p * BH_PAGE + BH_PAGE - 1 >= lo_min;
-    if (visible) {
-      // A page's operands are asked of LDS in two goes, each before the arithmetic that hides the wait: all the
-      // keys' before the first score product, all the values' before the softmax.
-      u32x4_t operand[4 * NS];
-#pragma unroll
-      for (int i = 0; i < 4 * NS; ++i) operand[i] = kl[i * 64 + lane];
-      __builtin_amdgcn_sched_barrier(0);
-      f32x4_t st[CTW][4];
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-#pragma unroll
-        for (int ct = 0; ct < CTW; ++ct) st[ct][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int s = 0; s < NS; ++s) {
-#pragma unroll
-          for (int ct = 0; ct < CTW; ++ct)
-            st[ct][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(operand[t * NS + s]), q_vec[ct][s], st[ct][t], 0, 0, 0);
-        }
-      }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int i = 0; i < 4 * NS; ++i) operand[i] = vl[i * 64 + lane];
-      __builtin_amdgcn_sched_barrier(0);
-      const int key0 = p * BH_PAGE + 8 * g;  // lane (j, g) holds keys key0 + 32 * (t / 2) + 4 * (t % 2) + r
-      const bool mask_needed = (p * BH_PAGE + BH_PAGE - 1 > pos_min) || (p * BH_PAGE < lo_max);
-      u32x4_t p_vec[CTW][2];
-#pragma unroll
-      for (int ct = 0; ct < CTW; ++ct) {
-        if (mask_needed) {   // key k0 + d of the page is seen if lo <= k0 + d <= pos: two numbers per column, then constants
-          const int d_last = pos[ct] - key0, d_first = lo[ct] - key0;
-#pragma unroll
-          for (int t = 0; t < 4; ++t)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const int d = 32 * (t / 2) + 4 * (t % 2) + r;
-              if (d > d_last || d < d_first) st[ct][t][r] = -INFINITY;
-            }
-        }
-        // Online softmax with few instructions: the maximum is taken over the raw scores, the scale
-        // enters through one fused multiply-add per score, and the exponentials are bare v_exp_f32
-        // (arguments <= 0; results below the normal range may flush to zero).
-        float local_max = larger(larger(st[ct][0][0], st[ct][0][1]), st[ct][0][2]);
-        local_max = larger(larger(local_max, st[ct][0][3]), st[ct][1][0]);
-#pragma unroll
-        for (int t = 1; t < 4; ++t) {
-          local_max = larger(larger(local_max, st[ct][t][1]), st[ct][t][2]);
-          local_max = larger(larger(local_max, st[ct][t][3]), t < 3 ? st[ct][t + 1][0] : run_max[ct]);
-        }
-        const float new_max = largest_of_column(local_max);               // raw (unscaled) scores, the earlier pages' too
-        // The exponentials' reference moves only when the maximum has grown by more than SLACK powers of two (or
-        // from nothing): until then probabilities may reach 2^SLACK, which float32 sums and bfloat16 operands
-        // hold as well as numbers up to one, and what was summed so far needs no factor.
-        const bool stays = (new_max - run_max[ct]) * scale_log2 <= SLACK;   // false from -inf, and while nothing was seen
-        const float reference = stays ? run_max[ct] : new_max;
-        const float shift = (reference == -INFINITY) ? 0.f : -reference * scale_log2;
-        // exactly 1 while the reference stands still, 0 when nothing was seen before
-        const float alpha =
-            (run_max[ct] == reference) ? 1.0f : __builtin_amdgcn_exp2f((run_max[ct] - reference) * scale_log2);
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-#pragma unroll
-          for (int half = 0; half < 2; ++half) {
-            const int t = 2 * u + half;
-            const float e0 = __builtin_amdgcn_exp2f(fmaf(st[ct][t][0], scale_log2, shift));
-            const float e1 = __builtin_amdgcn_exp2f(fmaf(st[ct][t][1], scale_log2, shift));
-            const float e2 = __builtin_amdgcn_exp2f(fmaf(st[ct][t][2], scale_log2, shift));
-            const float e3 = __builtin_amdgcn_exp2f(fmaf(st[ct][t][3], scale_log2, shift));
-            p_vec[ct][u][2 * half] = pack_bf16(e0, e1);
-            p_vec[ct][u][2 * half + 1] = pack_bf16(e2, e3);
-          }
-        run_max[ct] = reference;
-        if (__any(alpha != 1.0f)) {   // after the first pages the reference seldom moves
-          run_sum[ct] = run_sum[ct] * alpha;
-#pragma unroll
-          for (int dt = 0; dt < 2 * NS; ++dt) o[ct][dt] = o[ct][dt] * alpha;
-        }
-      }
-#pragma unroll
-      for (int ct = 0; ct < CTW; ++ct) {
-        run_sum[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(ones), as_bf16x8(p_vec[ct][0]), run_sum[ct], 0, 0, 0);
-        run_sum[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(ones), as_bf16x8(p_vec[ct][1]), run_sum[ct], 0, 0, 0);
-      }
-#pragma unroll
-      for (int dt = 0; dt < 2 * NS; ++dt) {
-        const bf16x8_t v0 = as_bf16x8(operand[dt * 2]);
-        const bf16x8_t v1 = as_bf16x8(operand[dt * 2 + 1]);
-#pragma unroll
-        for (int ct = 0; ct < CTW; ++ct) {
-          f32x4_t acc = o[ct][dt];
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v0, as_bf16x8(p_vec[ct][0]), acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v1, as_bf16x8(p_vec[ct][1]), acc, 0, 0, 0);
-          o[ct][dt] = acc;
-        }
-      }
-    }
+    if (!visible) return;
+    const bool mask_needed = (p * BH_PAGE + BH_PAGE - 1 > pos_min) || (p * BH_PAGE < lo_max);
+    if (mask_needed) attend_page(std::true_type(), p, buffer);
+    else attend_page(std::false_type(), p, buffer);
   };
   // all pages but the last in a loop whose body does not branch on the page count, so that the compiler may
   // interleave the next page's loads and staging writes with this page's arithmetic
@@ -294,6 +334,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
   }
 }
 
+#undef BH_TAKE_TURNS
+
 void bh_attention_prefill_launch(const void* q, void* out, const void* k_pages, const void* v_pages,
                                  const int32_t* page_table, int table_stride, const int32_t* positions,
                                  const int32_t* seq_start, int n_seqs, int tiles, int H, int KVH, int hd,
@@ -308,7 +350,8 @@ void bh_attention_prefill_launch(const void* q, void* out, const void* k_pages, 
   // Two column tiles per wave while the accumulators leave room for two workgroups per compute unit; one
   // where that gives fewer than two workgroups per compute unit (a page costs a workgroup nearly the same
   // time either way, so the steps are shorter with more and smaller workgroups: at 32 query and 8 kv heads
-  // of 128, 512 rows 24.5 -> 18.1 us, 1,024 rows 38.6 -> 30.2 us; from 4,096 rows on two tiles are faster).
+  // of 128, 512 rows 24.5 -> 18.1 us, 1,024 rows 38.6 -> 30.2 us; at 2,048 rows one tile is 3 % slower, at 4,096 rows
+  // 20 %).
   const bool few = (long)((tiles + 7) / 8) * KVH * n_seqs < 512;
   switch (hd / 32) {
     case 1: if (few) BH_PREFILL(1, 1); else BH_PREFILL(1, 2); break;
