@@ -1279,3 +1279,21 @@ extern "C" int bh_gemm_bf16_then_norm(const void* a, const void* w, float* resid
 #undef BH_FINISH_NORM
   return bh_check_launch("gemm_parts_finish_norm");
 }
+
+// A W^T of many rows left as the float32 sums of K's parts, [parts][M][N], for a consumer that adds them up itself
+// (the q/k norm, rotation and cache write: bh_qk_norm_rope_cache_sums): the product without its finishing kernel.
+// bh_gemm_bf16_bare_parts: how many parts such a product of these sizes has, 0 where the product is not one whose
+// K goes in parts through the kernel for many rows.  `sums`: parts * M * N floats.
+extern "C" int bh_gemm_bf16_bare_parts(int M, int N, int K, int layout) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  const int parts = gemm_turns_parts(M, N, K, layout, 0);
+  return parts > 1 && parts <= MAX_TURNS_PARTS ? parts : 0;
+}
+extern "C" int bh_gemm_bf16_bare(const void* a, const void* w, float* sums, int M, int N, int K, int layout, int a_blocked,
+                                 hipStream_t stream) {
+  const int parts = bh_gemm_bf16_bare_parts(M, N, K, layout);
+  BH_REQUIRE(parts > 0, "gemm_bf16_bare: a product of M=%d N=%d K=%d is not left in parts (bh_gemm_bf16_bare_parts)", M, N, K);
+  BH_REQUIRE(a && w && sums, "gemm_bf16_bare: every operand is needed");
+  BH_REQUIRE(((uintptr_t)a | (uintptr_t)w | (uintptr_t)sums) % 16 == 0, "gemm_bf16_bare: operands must be 16-byte aligned");
+  return gemm_turns_launch_parts(a, w, sums, M, N, K, parts, a_blocked, stream);
+}

@@ -435,9 +435,54 @@ __device__ inline float head_sum(float v) {
   return v;
 }
 
-template <typename TW, int LPH, int RPW>   // RPW: rows that a wave of the q and k heads takes
+// PARTS: `qkv` holds no bfloat16 rows but the float32 sums of a product whose K was cut into parts,
+// [parts][n_rows][(H + 2 KVH) * HD], as the kernel left them whose wave groups take turns: an element is the sum
+// of its parts in their order, rounded to bfloat16 (what that product's finishing kernel would have written, which
+// this takes the place of, and the bfloat16 rows' trip to memory and back with it).
+template <bool PARTS, int RN>
+__device__ inline void eight_of_each_row(const uint16_t* qkv, const size_t (&at)[RN], size_t part_stride, int parts,
+                                         uint4 (&raw)[RN]) {   // at[r]: element offset in a [rows][width] matrix
+  if constexpr (!PARTS) {
+#pragma unroll
+    for (int r = 0; r < RN; ++r) raw[r] = *reinterpret_cast<const uint4*>(qkv + at[r]);
+  } else {
+    const float* sums = reinterpret_cast<const float*>(qkv);
+    float4 lo[RN], hi[RN];
+#pragma unroll
+    for (int r = 0; r < RN; ++r) lo[r] = hi[r] = make_float4(0.f, 0.f, 0.f, 0.f);
+    constexpr int GROUP = RN >= 8 ? 2 : 4;   // parts whose loads, of all the rows, are on their way together
+    for (int p0 = 0; p0 < parts; p0 += GROUP) {
+      float4 a[GROUP][RN], b[GROUP][RN];
+#pragma unroll
+      for (int u = 0; u < GROUP; ++u)
+#pragma unroll
+        for (int r = 0; r < RN; ++r) {
+          const float* from = sums + (size_t)min(p0 + u, parts - 1) * part_stride + at[r];
+          const bool there = p0 + u < parts;
+          a[u][r] = there ? *reinterpret_cast<const float4*>(from) : make_float4(0.f, 0.f, 0.f, 0.f);
+          b[u][r] = there ? *reinterpret_cast<const float4*>(from + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+      for (int u = 0; u < GROUP; ++u)   // in the parts' order; a part that is not there adds zero
+#pragma unroll
+        for (int r = 0; r < RN; ++r) {
+          lo[r].x += a[u][r].x, lo[r].y += a[u][r].y, lo[r].z += a[u][r].z, lo[r].w += a[u][r].w;
+          hi[r].x += b[u][r].x, hi[r].y += b[u][r].y, hi[r].z += b[u][r].z, hi[r].w += b[u][r].w;
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < RN; ++r) {
+      raw[r].x = (uint32_t)f32_to_bf16_bits(lo[r].x) | ((uint32_t)f32_to_bf16_bits(lo[r].y) << 16);
+      raw[r].y = (uint32_t)f32_to_bf16_bits(lo[r].z) | ((uint32_t)f32_to_bf16_bits(lo[r].w) << 16);
+      raw[r].z = (uint32_t)f32_to_bf16_bits(hi[r].x) | ((uint32_t)f32_to_bf16_bits(hi[r].y) << 16);
+      raw[r].w = (uint32_t)f32_to_bf16_bits(hi[r].z) | ((uint32_t)f32_to_bf16_bits(hi[r].w) << 16);
+    }
+  }
+}
+
+template <typename TW, int LPH, int RPW, bool PARTS>   // RPW: rows that a wave of the q and k heads takes
 __global__ __launch_bounds__(256) void qk_norm_rope_cache_rows_kernel(
-    const uint16_t* __restrict__ qkv, uint16_t* __restrict__ q_out, const TW* __restrict__ q_weight,
+    const uint16_t* __restrict__ qkv, int parts, uint16_t* __restrict__ q_out, const TW* __restrict__ q_weight,
     const TW* __restrict__ k_weight, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
     uint16_t* __restrict__ k_pages, uint16_t* __restrict__ v_pages, const int32_t* __restrict__ page_table,
@@ -453,8 +498,8 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_rows_kernel(
     const int wanted_head = ((wave - main_waves) % chunks) * HPW + lane / LPH, c = lane % LPH;
     const bool mine = wanted_head < KVH;
     const int kv_head = mine ? wanted_head : KVH - 1;
-    const size_t fused = (size_t)(H + 2 * KVH) * HD;
-    const uint16_t* src = qkv + (size_t)(H + KVH + kv_head) * HD + 8 * c;   // + row * fused
+    const size_t fused = (size_t)(H + 2 * KVH) * HD, part_stride = (size_t)n_rows * fused;
+    const size_t src = (size_t)(H + KVH + kv_head) * HD + 8 * c;   // + row * fused
     // Positions and sequences of the rows 8 group - 8 .. 8 group + 15, one in each of the first 24 lanes, in one load
     // each: everything that the eight rows' decisions below look at (asked for row by row inside the loop, eight
     // waits for memory in a row were most of this kernel's time at a few hundred rows).
@@ -472,8 +517,10 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_rows_kernel(
       const int page = page_table[(size_t)seq * table_stride + pos / BH_PAGE];
       uint16_t* block = v_pages + ((size_t)page * KVH + kv_head) * BH_PAGE * HD;
       if (!whole) {
-        const uint4 raw = *reinterpret_cast<const uint4*>(src + (size_t)row * fused);
-        const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+        const size_t one_at[1] = {src + (size_t)row * fused};
+        uint4 one[1];
+        eight_of_each_row<PARTS, 1>(qkv, one_at, part_stride, parts, one);
+        const uint32_t words[4] = {one[0].x, one[0].y, one[0].z, one[0].w};
         if (mine) {
 #pragma unroll
           for (int e = 0; e < 8; ++e)
@@ -482,8 +529,10 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_rows_kernel(
         continue;
       }
       uint4 raw[8];   // token t's dims 8 c .. 8 c + 7
+      size_t raw_at[8];
 #pragma unroll
-      for (int t = 0; t < 8; ++t) raw[t] = *reinterpret_cast<const uint4*>(src + (size_t)(row + t) * fused);
+      for (int t = 0; t < 8; ++t) raw_at[t] = src + (size_t)(row + t) * fused;
+      eight_of_each_row<PARTS, 8>(qkv, raw_at, part_stride, parts, raw);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {   // dim 8 c + e of the eight tokens: the halves e % 2 of the words e / 2
         const uint32_t pick = e % 2 ? 0x07060302u : 0x05040100u;
@@ -510,12 +559,14 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_rows_kernel(
   // those, their angles.  (With one row per wave the three waits in a row, for so little data each, were the kernel's time.)
   int pos[RPW];
   uint4 raw[RPW];
+  size_t raw_at[RPW];
 #pragma unroll
   for (int r = 0; r < RPW; ++r) {
     const int row = min(first_row + r, n_rows - 1);
     pos[r] = positions[row];
-    raw[r] = *reinterpret_cast<const uint4*>(qkv + ((size_t)row * (H + 2 * KVH) + head) * HD + 8 * c);
+    raw_at[r] = ((size_t)row * (H + 2 * KVH) + head) * HD + 8 * c;
   }
+  eight_of_each_row<PARTS, RPW>(qkv, raw_at, (size_t)n_rows * (H + 2 * KVH) * HD, parts, raw);
   const TW* weight = is_q ? q_weight : k_weight;
   float wv[8];
   if (weight != nullptr) load_eight(weight + 8 * c, wv);
@@ -569,6 +620,44 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_rows_kernel(
   }
 }
 
+// The form for many bfloat16 rows (or, parts > 0, for a product's float32 sums in `parts` parts of K): whether it
+// takes these sizes, and its launch.
+static bool qk_rows_form_takes(int n_rows, int hd, int rot) {
+  return n_rows >= 64 && (hd == 64 || hd == 128 || hd == 256) && (rot == 0 || rot == hd);
+}
+static int qk_rows_form(const void* qkv, int parts, void* q_out, const void* q_weight, const void* k_weight, int w_dtype,
+                        float eps, const float* cos_table, const float* sin_table, int rot, const int32_t* positions,
+                        const int32_t* row_seq, void* k_pages, void* v_pages, const int32_t* page_table, int table_stride,
+                        int n_rows, int H, int KVH, int hd, int write_kv, int kv_order, hipStream_t stream) {
+  // waves for the q and k heads of every row, then (write_kv) waves for the values of eight rows each
+  const int lanes_per_head = hd / 8, heads_per_wave = 64 / lanes_per_head, main_heads = write_kv ? H + KVH : H;
+  constexpr int RPW = 4;
+  const long main_waves = (long)((n_rows + RPW - 1) / RPW) * ((main_heads + heads_per_wave - 1) / heads_per_wave);
+  const long value_waves = write_kv ? (long)((n_rows + 7) / 8) * ((KVH + heads_per_wave - 1) / heads_per_wave) : 0;
+  BH_REQUIRE(main_waves + value_waves < (1L << 31), "qk_norm_rope: too many rows");
+  BH_REQUIRE(w_dtype == BH_F32 || w_dtype == BH_BF16, "qk_norm_rope: unknown weight dtype %d", w_dtype);
+  dim3 wide_grid((unsigned)((main_waves + value_waves + 3) / 4)), wide_block(4 * BH_WAVE);
+#define BH_QK_ROWS(TW, LPH, PARTS)                                                                                  \
+  qk_norm_rope_cache_rows_kernel<TW, LPH, RPW, PARTS><<<wide_grid, wide_block, 0, stream>>>(                        \
+      (const uint16_t*)qkv, parts, (uint16_t*)q_out, (const TW*)q_weight, (const TW*)k_weight, eps,                 \
+      rot ? cos_table : nullptr, rot ? sin_table : nullptr,                                                          \
+      positions, row_seq, (uint16_t*)k_pages, (uint16_t*)v_pages, page_table, table_stride, H, KVH, kv_order,      \
+      n_rows, main_heads, (int)main_waves, (int)value_waves)
+#define BH_QK_ROWS_W(LPH)                                      \
+  do {                                                         \
+    if (parts > 0 && w_dtype == BH_F32) BH_QK_ROWS(float, LPH, true);   \
+    else if (parts > 0) BH_QK_ROWS(bf16_t, LPH, true);         \
+    else if (w_dtype == BH_F32) BH_QK_ROWS(float, LPH, false); \
+    else BH_QK_ROWS(bf16_t, LPH, false);                       \
+  } while (0)
+  if (hd == 64) BH_QK_ROWS_W(8);
+  else if (hd == 128) BH_QK_ROWS_W(16);
+  else BH_QK_ROWS_W(32);
+#undef BH_QK_ROWS_W
+#undef BH_QK_ROWS
+  return bh_check_launch("qk_norm_rope_cache_rows");
+}
+
 // Precondition: the rows of one sequence stand one after the other and in position order (row r + 1 of a
 // sequence is position p + 1), as a step lays them out.  The form for many rows relies on it: it takes eight
 // rows for one piece of values when the first and the last of them belong to one sequence, seven positions apart,
@@ -590,33 +679,9 @@ extern "C" int bh_qk_norm_rope_cache(const void* qkv, int dtype, void* q_out, co
              "qk_norm_rope: cache order %d does not exist for head size %d", kv_order, hd);
   if (cos_table == nullptr) rot = 0;
   const int n_heads = write_kv ? H + 2 * KVH : H;
-  if (dtype == BH_BF16 && n_rows >= 64 && (hd == 64 || hd == 128 || hd == 256) && (rot == 0 || rot == hd)) {
-    // waves for the q and k heads of every row, then (write_kv) waves for the values of eight rows each
-    const int lanes_per_head = hd / 8, heads_per_wave = 64 / lanes_per_head, main_heads = write_kv ? H + KVH : H;
-    constexpr int RPW = 4;
-    const long main_waves = (long)((n_rows + RPW - 1) / RPW) * ((main_heads + heads_per_wave - 1) / heads_per_wave);
-    const long value_waves = write_kv ? (long)((n_rows + 7) / 8) * ((KVH + heads_per_wave - 1) / heads_per_wave) : 0;
-    BH_REQUIRE(main_waves + value_waves < (1L << 31), "qk_norm_rope: too many rows");
-    dim3 wide_grid((unsigned)((main_waves + value_waves + 3) / 4)), wide_block(4 * BH_WAVE);
-#define BH_QK_ROWS(TW, LPH)                                                                                       \
-  qk_norm_rope_cache_rows_kernel<TW, LPH, RPW><<<wide_grid, wide_block, 0, stream>>>(                                   \
-      (const uint16_t*)qkv, (uint16_t*)q_out, (const TW*)q_weight, (const TW*)k_weight, eps,                        \
-      rot ? cos_table : nullptr, rot ? sin_table : nullptr,                                                          \
-      positions, row_seq, (uint16_t*)k_pages, (uint16_t*)v_pages, page_table, table_stride, H, KVH, kv_order,      \
-      n_rows, main_heads, (int)main_waves, (int)value_waves)
-#define BH_QK_ROWS_W(LPH)                              \
-  do {                                                 \
-    if (w_dtype == BH_F32) BH_QK_ROWS(float, LPH);     \
-    else BH_QK_ROWS(bf16_t, LPH);                      \
-  } while (0)
-    BH_REQUIRE(w_dtype == BH_F32 || w_dtype == BH_BF16, "qk_norm_rope: unknown weight dtype %d", w_dtype);
-    if (hd == 64) BH_QK_ROWS_W(8);
-    else if (hd == 128) BH_QK_ROWS_W(16);
-    else BH_QK_ROWS_W(32);
-#undef BH_QK_ROWS_W
-#undef BH_QK_ROWS
-    return bh_check_launch("qk_norm_rope_cache_rows");
-  }
+  if (dtype == BH_BF16 && qk_rows_form_takes(n_rows, hd, rot))
+    return qk_rows_form(qkv, 0, q_out, q_weight, k_weight, w_dtype, eps, cos_table, sin_table, rot, positions, row_seq,
+                        k_pages, v_pages, page_table, table_stride, n_rows, H, KVH, hd, write_kv, kv_order, stream);
   dim3 grid(n_rows, n_heads), block(BH_WAVE);
 #define BH_QK(T, TW)                                                                                         \
   qk_norm_rope_cache_kernel<T, TW><<<grid, block, 0, stream>>>(                                              \
@@ -629,6 +694,36 @@ extern "C" int bh_qk_norm_rope_cache(const void* qkv, int dtype, void* q_out, co
   else return bh_fail("qk_norm_rope: unknown dtypes %d/%d", dtype, w_dtype);
 #undef BH_QK
   return bh_check_launch("qk_norm_rope_cache");
+}
+
+// The same from the float32 sums that a product of many rows left in `parts` parts of K
+// ([parts][n_rows][(H + 2 KVH) * hd]; bh_gemm_bf16_bare_parts says which products do): every element is the sum of
+// its parts in their order, rounded to bfloat16, as that product's finishing kernel would have written it; q_out,
+// the cache and the weights as above, bfloat16 outputs.  bh_qk_norm_rope_cache_takes_sums: whether these sizes go.
+extern "C" int bh_qk_norm_rope_cache_takes_sums(int n_rows, int hd, int rot) {
+  return qk_rows_form_takes(n_rows, hd, rot) ? 1 : 0;
+}
+extern "C" int bh_qk_norm_rope_cache_sums(const float* sums, int parts, void* q_out, const void* q_weight,
+                                          const void* k_weight, int w_dtype, float eps, const float* cos_table,
+                                          const float* sin_table, int table_positions, int rot,
+                                          const int32_t* positions, const int32_t* row_seq, void* k_pages,
+                                          void* v_pages, const int32_t* page_table, int table_stride, int n_rows,
+                                          int H, int KVH, int hd, int write_kv, int kv_order, int max_position,
+                                          hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && H > 0 && KVH > 0 && hd > 0 && parts > 0, "qk_norm_rope: sizes must be positive");
+  BH_REQUIRE((q_weight == nullptr) == (k_weight == nullptr), "qk_norm_rope: give both norm weights or neither");
+  BH_REQUIRE(cos_table == nullptr || max_position < table_positions,
+             "qk_norm_rope: position %d is outside the rotation table of %d positions", max_position, table_positions);
+  BH_REQUIRE(H + 2 * KVH <= 65535, "qk_norm_rope: too many heads");
+  BH_REQUIRE(kv_order == BH_KV_ROWS || (kv_order == BH_KV_PIECES && hd % 32 == 0),
+             "qk_norm_rope: cache order %d does not exist for head size %d", kv_order, hd);
+  if (cos_table == nullptr) rot = 0;
+  BH_REQUIRE(qk_rows_form_takes(n_rows, hd, rot),
+             "qk_norm_rope: sums in parts are taken for at least 64 rows, heads of 64, 128 or 256 and a rotation over "
+             "the whole head or none (rows %d, head %d, rotation %d)", n_rows, hd, rot);
+  BH_REQUIRE(((uintptr_t)sums % 16) == 0 && ((long)(H + 2 * KVH) * hd) % 4 == 0, "qk_norm_rope: the sums must be 16-byte aligned");
+  return qk_rows_form(sums, parts, q_out, q_weight, k_weight, w_dtype, eps, cos_table, sin_table, rot, positions, row_seq,
+                      k_pages, v_pages, page_table, table_stride, n_rows, H, KVH, hd, write_kv, kv_order, stream);
 }
 
 // ---- attention over the paged cache, any size -------------------------------------------------

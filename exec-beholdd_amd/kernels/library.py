@@ -54,6 +54,21 @@ class NormedRows:
         return 2
 
 
+class PartSums:
+    """A bfloat16 matrix [rows, width] that was never written: `sums` [parts, rows, width] float32 holds a product's
+    sums over the parts its K was cut into, and an element of the matrix is the sum of its parts in their order,
+    rounded to bfloat16.  `HipKernels.gemm_bare` leaves it, `qk_norm_rope_cache` takes it in place of the rows
+    (and does what the product's finishing kernel would have done on the way).  `shape` and `dtype` are those of
+    the matrix it stands for."""
+
+    def __init__(self, sums: torch.Tensor):
+        self.sums, self.parts = sums, int(sums.shape[0])
+        self.shape, self.dtype, self.device = sums.shape[1:], torch.bfloat16, sums.device
+
+    def dim(self):
+        return 2
+
+
 class BlockedRows:
     """A bfloat16 activation matrix [rows, width] kept in blocks of `block_rows` (16 or 8) rows x 32 columns, each
     block in the order in which a matrix-core operand lies in a wave's lanes (`bh_rows_index` in csrc/layout.h):
@@ -124,6 +139,10 @@ class KernelSizes:
             "bh_rmsnorm": [p, p, p, i, p, i, i, i, f, i, p],
             "bh_gemm_generic": [p, i, p, i, p, i, i, i, i, i, p],
             "bh_qk_norm_rope_cache": [p, i, p, p, p, i, f, p, p, i, i, p, p, p, p, p, i, i, i, i, i, i, i, i, p],
+            "bh_qk_norm_rope_cache_sums": [p, i, p, p, p, i, f, p, p, i, i, p, p, p, p, p, i, i, i, i, i, i, i, i, p],
+            "bh_qk_norm_rope_cache_takes_sums": [i, i, i],
+            "bh_gemm_bf16_bare_parts": [i, i, i, i],
+            "bh_gemm_bf16_bare": [p, p, p, i, i, i, i, i, p],
             "bh_attention_generic": [p, p, i, p, p, p, i, p, p, i, i, i, i, f, i, i, p],
             "bh_swiglu": [p, p, i, i, i, p],
             "bh_sample": [p, p, p, p, p, p, p, p, i, i, p],
@@ -218,6 +237,7 @@ class HipKernels(KernelSizes):
         self.device = torch.device("cuda", self._device_index)
         self._raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
         self._plans: dict = {}      # (m, n, k, packed, activation) -> what the library says of such a product
+        self._bare: dict = {}       # (m, n, k) -> the parts that `gemm_bare` leaves such a product in, or 0
         self.page_size = int(self.lib.bh_page_size())
         if self.page_size != _build.source_page_size():
             raise KernelError(f"{self.library_path} was built for pages of {self.page_size} tokens, the sources say "
@@ -465,6 +485,32 @@ class HipKernels(KernelSizes):
             self._ptr(out, "gemm out"), _code(out, "gemm out"), int(bool(accumulate)), m, n, k, self._stream()))
         return None
 
+    def gemm_bare(self, a, w):
+        """a[M, K] @ w[N, K]^T left as `PartSums`, where the product of these operands is one of many rows whose K the
+        library cuts into parts (prompts of a few hundred to about 1,500 rows at the usual widths): the product
+        without its finishing kernel, for a consumer that adds the parts up itself.  None where it is not (then call
+        `gemm`)."""
+        if (not isinstance(w, PackedWeight) or isinstance(a, NormedRows) or a.dim() != 2 or a.dtype != torch.bfloat16
+                or a.shape[1] != w.shape[1]):
+            return None
+        m, k = a.shape
+        n = w.shape[0]
+        parts = self._bare.get((m, n, k))
+        if parts is None:
+            parts = self._bare[(m, n, k)] = int(self.lib.bh_gemm_bf16_bare_parts(m, n, k, 1))
+        if not parts:
+            return None
+        a_block_rows = self._product(m, n, k, 1, 0)[0]
+        a = self._in_blocks_of(a, a_block_rows)
+        sums = torch.empty((parts, m, n), dtype=torch.float32, device=self.device)
+        self._check(self.lib.bh_gemm_bf16_bare(self._ptr(a, "gemm a"), self._ptr(w.data, "gemm w"), self._ptr(sums, "gemm sums"),
+                                               m, n, k, 1, int(a_block_rows == 16), self._stream()))
+        return PartSums(sums)
+
+    def qk_norm_rope_takes_sums(self, n_rows, head_dim, rot) -> bool:
+        """Whether `qk_norm_rope_cache` takes `PartSums` for a step of these sizes (`rot`: the rotation's width, 0 for none)."""
+        return bool(self.lib.bh_qk_norm_rope_cache_takes_sums(int(n_rows), int(head_dim), int(rot)))
+
     def gemm_turns(self, a, w, out, blocks, accumulate=False, swiglu=False):
         """The product for many rows whose wave groups take turns, at a given tile width (`blocks` of 16
         weight rows per wave: 8, 6 or 4), whatever `gemm` would choose for these sizes: out[M, N] (+)= a @ w^T,
@@ -549,8 +595,15 @@ class HipKernels(KernelSizes):
                 raise KernelError("qk_norm_rope: norm weights must be [head_dim] and of one dtype")
             w_code = _code(q_weight, "qk_norm_rope weight")
         self._check_pages(k_pages, v_pages, page_table, n_kv_heads, head_dim, qkv.dtype, "qk_norm_rope")
-        self._check(self.lib.bh_qk_norm_rope_cache(
-            self._ptr(qkv, "qkv"), _code(qkv, "qkv"), self._ptr(q_out, "q_out"),
+        if isinstance(qkv, PartSums):
+            if not self.qk_norm_rope_takes_sums(n_rows, head_dim, rot):
+                raise KernelError(f"qk_norm_rope: sums in parts are not taken for {n_rows} rows, heads of {head_dim} "
+                                  f"and a rotation over {rot} (qk_norm_rope_takes_sums says so beforehand)")
+            first, second, entry = self._ptr(qkv.sums, "qkv sums", (torch.float32,)), qkv.parts, self.lib.bh_qk_norm_rope_cache_sums
+        else:
+            first, second, entry = self._ptr(qkv, "qkv"), _code(qkv, "qkv"), self.lib.bh_qk_norm_rope_cache
+        self._check(entry(
+            first, second, self._ptr(q_out, "q_out"),
             self._ptr(q_weight, "q_norm", None, True), self._ptr(k_weight, "k_norm", None, True), w_code,
             float(eps), self._ptr(cos, "cos", (torch.float32,), True), self._ptr(sin, "sin", (torch.float32,), True),
             table_positions, rot, self._ptr(positions, "positions", (torch.int32,)),

@@ -84,8 +84,14 @@ class GQAAttention:
 
     def forward(self, ctx, x, hidden, cache, then_norm=None):
         k = ctx.kernels
-        qkv = self.qkv.forward(ctx, x)
         cos, sin = self.position_encoding.tables() if self.position_encoding is not None else (None, None)
+        qkv = None
+        # a step of many rows: the projection may stay the sums of K's parts, which the norm/rotation kernel adds up
+        takes_sums = getattr(k, "qk_norm_rope_takes_sums", None)
+        if not ctx.is_decode and takes_sums is not None and takes_sums(ctx.n_rows, self.head_dim, 2 * cos.shape[1] if cos is not None else 0):
+            qkv = self.qkv.forward_bare(ctx, x)
+        if qkv is None:
+            qkv = self.qkv.forward(ctx, x)
         attended = ctx.new_activations(ctx.n_rows, self.n_heads * self.head_dim, reader=self.out.reader())
         # a decode step: norm, rotation, cache write and attention in one launch where the kernels offer it
         one_launch = getattr(k, "attention_decode_fused", None)

@@ -81,6 +81,13 @@ class Linear:
         ctx.kernels.gemm(x, self.weight, out, accumulate=accumulate)
         return out
 
+    def forward_bare(self, ctx, x):
+        """W x as the kernel library's unfinished form of it (the sums of the parts that K was cut into), for a
+        consumer that says it takes that form; None where the library has no such form for these operands or
+        does not cut this product (then call `forward`)."""
+        bare = getattr(ctx.kernels, "gemm_bare", None)
+        return bare(x, self.weight) if bare is not None else None
+
     def add_into(self, ctx, x, residual, then_norm=None):
         """residual += W x.  With `then_norm` (a NormRequest for the norm that reads the residual next)
         returns what the product prepared of that norm's output, or None."""

@@ -1045,6 +1045,72 @@ def test_qk_norm_rope_cache(K, dtype, w_dtype, n_heads, kv_heads, head_dim, rot,
     assert torch.equal(kp2.cpu(), kp) and torch.equal(vp2.cpu(), vp)
 
 
+@pytest.mark.parametrize("w_dtype", DTYPES)
+@pytest.mark.parametrize("parts", [2, 4, 8])
+@pytest.mark.parametrize("news,pasts", [([70, 5, 1], [0, 62, 130]), ([3, 70, 2], [5, 16, 7]), ([66, 5, 6], [0, 62, 130])])
+@pytest.mark.parametrize("n_heads,kv_heads,head_dim,rot", [(8, 2, 128, 128), (3, 3, 256, 256), (5, 1, 64, 64), (5, 1, 128, 0)])
+def test_qk_norm_rope_cache_from_the_sums_of_a_products_parts(K, w_dtype, parts, news, pasts, n_heads, kv_heads, head_dim, rot):
+    """The same kernel fed with the float32 sums of K's parts instead of finished bfloat16 rows writes, bit for bit,
+    what it writes from the rows that the parts add up to (in their order, rounded to bfloat16)."""
+    from beholdd.kernels import PartSums
+    g = torch.Generator().manual_seed(head_dim + parts)
+    n_rows = sum(news)
+    fused = (n_heads + 2 * kv_heads) * head_dim
+    sums = torch.randn(parts, n_rows, fused, generator=g) * torch.tensor([1.0, -0.7, 0.3, 2.0, 0.1, -1.3, 0.6, 0.9][:parts])[:, None, None]
+    total = torch.zeros(n_rows, fused)
+    for part in range(parts):
+        total = total + sums[part]
+    rows = total.to(torch.bfloat16)
+    qw = (1 + 0.2 * torch.randn(head_dim, generator=g)).to(w_dtype)
+    kw = (1 + 0.2 * torch.randn(head_dim, generator=g)).to(w_dtype)
+    max_pos = 256
+    cos = sin = None
+    if rot:
+        freqs = 1.0 / 10000.0 ** (torch.arange(0, rot, 2, dtype=torch.float64) / rot)
+        angles = torch.arange(max_pos, dtype=torch.float64)[:, None] * freqs
+        cos, sin = dev(angles.cos().float()), dev(angles.sin().float())
+    positions = torch.tensor([p + t for p, n in zip(pasts, news) for t in range(n)], dtype=torch.int32)
+    row_seq = torch.tensor([s for s, n in enumerate(news) for _ in range(n)], dtype=torch.int32)
+    table = torch.tensor([[4, 5, 0], [7, 2, 0], [1, 8, 3]], dtype=torch.int32)
+    assert K.qk_norm_rope_takes_sums(n_rows, head_dim, rot)
+    results = []
+    for source in (dev(rows), PartSums(dev(sums))):
+        kp = torch.full((9, kv_heads, PAGE, head_dim), 768.0).to(torch.bfloat16)
+        vp = torch.full((9, kv_heads, head_dim, PAGE), 768.0).to(torch.bfloat16)
+        kp_d, vp_d = stored(K, kp, vp)
+        q_out = torch.full((n_rows, n_heads * head_dim), 3.0, dtype=torch.bfloat16, device="cuda:0")
+        K.qk_norm_rope_cache(source, q_out, dev(qw), dev(kw), 1e-5, cos, sin, dev(positions), dev(row_seq), kp_d, vp_d,
+                             dev(table), n_heads, kv_heads, head_dim, True, int(positions.max()))
+        results.append((q_out.cpu(), kp_d.cpu(), vp_d.cpu()))
+    for from_rows, from_sums in zip(*results):
+        assert torch.equal(from_rows, from_sums)
+    assert not K.qk_norm_rope_takes_sums(63, head_dim, rot) and not K.qk_norm_rope_takes_sums(n_rows, 96, 96)
+    with pytest.raises(Exception, match="sums in parts"):
+        K.qk_norm_rope_cache(PartSums(dev(sums[:, :40].contiguous())), q_out[:40], dev(qw), dev(kw), 1e-5, cos, sin,
+                             dev(positions[:40]), dev(row_seq[:40]), kp_d, vp_d, dev(table), n_heads, kv_heads, head_dim, True, 255)
+
+
+@pytest.mark.parametrize("m,n,k", [(512, 6144, 4096), (1024, 6144, 4096), (333, 4080, 4096), (2048, 6144, 4096), (64, 6144, 4096)])
+def test_product_left_in_parts_adds_up_to_the_finished_product(K, m, n, k):
+    """`gemm_bare` leaves what `gemm` would have finished: the parts, added in their order and rounded, are its output bit
+    for bit; where the library does not cut such a product it says so by returning None."""
+    gen = torch.Generator().manual_seed(m + n)
+    a = dev((torch.randn(m, k, generator=gen) * 0.5).to(torch.bfloat16))
+    packed = K.pack_weight(dev((torch.randn(n, k, generator=gen) * 0.05).to(torch.bfloat16)))
+    finished = torch.empty(m, n, dtype=torch.bfloat16, device="cuda:0")
+    K.gemm(a, packed, finished)
+    bare = K.gemm_bare(a, packed)
+    if m in (2048, 64):           # a tile of its own, or few rows: not cut into parts for a finishing kernel of many rows
+        assert bare is None
+        return
+    assert bare is not None and bare.parts >= 2 and tuple(bare.shape) == (m, n) and bare.dtype == torch.bfloat16
+    total = torch.zeros(m, n, device="cuda:0")
+    for part in range(bare.parts):
+        total = total + bare.sums[part]
+    assert torch.equal(total.to(torch.bfloat16), finished)
+    assert K.gemm_bare(a.float(), packed) is None
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("rows,width", [(1, 10), (7, 200), (33, 12288), (2, 25600)])
 def test_swiglu(K, dtype, rows, width):
