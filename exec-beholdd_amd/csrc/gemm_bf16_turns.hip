@@ -1,5 +1,5 @@
 // bfloat16 matrix products of many rows, C[M, N] (+)= A[M, K] * W[N, K]^T with W in the tiles layout
-// (see gemm_bf16.hip), for the shapes where a 256-row tile fills the chip: prompts from about 512 tokens on.
+// (see gemm_bf16.hip), for the shapes where a 256-row tile fills the chip: prompts from 320 tokens on.
 //
 // A workgroup of eight waves owns 256 rows x 32 YB weight rows.  Its waves form two groups of four (one wave
 // of each group per SIMD) that take turns: while one group multiplies (32, 24 or 16 MFMAs on operands it holds
