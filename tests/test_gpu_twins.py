@@ -160,7 +160,40 @@ def test_cache_write_and_attention_and_their_twins(K, twins, dtype, code, head_d
     assert rel(host(out), want) < (1e-5 if code == F32 else 1.2e-2)
 
 
-@pytest.mark.parametrize("vocab", [50, 1000, 4133])
+def test_the_draws_thresholds_on_rows_made_to_trip_them(K, twins):
+    """Rows on which a search for the k-th largest logit or for top-p's threshold digit by digit could go wrong: all
+    logits equal (every token ties at every threshold), two values only, logits of both signs around zero and far
+    apart, a vocabulary that fills no trip of the draw, k one below the vocabulary, p so small that only the
+    largest logit stays, p just below one.  Against the plain twin, row by row."""
+    rng = np.random.default_rng(11)
+    vocab = 5003
+    shapes = [np.full(vocab, 1.25, np.float32),
+              np.where(rng.random(vocab) < 0.01, 3.0, -2.0).astype(np.float32),
+              (rng.normal(size=vocab) * 1e-3).astype(np.float32),
+              (rng.normal(size=vocab) * 40).astype(np.float32),
+              np.concatenate([np.full(vocab - 3, -1e30, np.float32), np.asarray([0.5, 0.5, 0.25], np.float32)]),
+              (-np.abs(rng.normal(size=vocab)) * 5 - 100).astype(np.float32)]
+    settings = [(0, 1.0), (5, 1.0), (vocab - 1, 1.0), (0, 1e-6), (0, 0.999999), (0, 0.5), (40, 0.7), (1, 0.3)]
+    logits = np.stack([shape for shape in shapes for _ in settings])
+    rows = logits.shape[0]
+    top_k = np.asarray([k for _ in shapes for k, _ in settings], np.int32)
+    top_p = np.asarray([p for _ in shapes for _, p in settings], np.float32)
+    temperature = rng.choice([0.6, 1.0, 1.5], size=rows).astype(np.float32)
+    for seed in range(3):
+        uniform = np.random.default_rng(seed).random(rows).astype(np.float32)
+        tokens, bad = torch.empty(rows, dtype=torch.int32, device=DEVICE), torch.empty(rows, dtype=torch.int32, device=DEVICE)
+        K.sample(dev(logits), tokens, bad, temperature=dev(temperature), top_k=dev(top_k), top_p=dev(top_p), uniform=dev(uniform))
+        want, want_bad, margin = twins.sample(logits, temperature, uniform, top_k, top_p)
+        got = tokens.cpu().numpy()
+        assert bad.cpu().tolist() == want_bad.tolist() == [0] * rows
+        sure = margin > 1e-5
+        assert sure.sum() > 0.8 * rows and np.array_equal(got[sure], want[sure]), (got[sure != (got == want)], want[sure != (got == want)])
+    # k = 1 and a tiny p keep the largest logit alone, whatever the uniform number
+    alone = [i for i in range(rows) if (top_k[i] == 1 or top_p[i] < 1e-5) and len(set(logits[i].tolist())) > 2]
+    assert alone and all(int(got[i]) == int(np.argmax(logits[i])) for i in alone)
+
+
+@pytest.mark.parametrize("vocab", [50, 1000, 4133, 151936])
 def test_the_draw_and_its_twin(K, twins, vocab):
     """Temperature, top-k and top-p draws of the kernel against the plain twin's, row by row: the same token wherever the
     draw's target lies further from the ends of its token's interval than float32 sums can move it."""
@@ -179,6 +212,6 @@ def test_the_draw_and_its_twin(K, twins, vocab):
         want, want_bad, margin = twins.sample(logits, temperature, uniform, top_k, top_p)
         got = tokens.cpu().numpy()
         assert bad.cpu().tolist() == want_bad.tolist() == [0] * rows
-        sure = margin > 1e-5
-        assert sure.sum() > 0.9 * rows and np.array_equal(got[sure], want[sure])
+        sure = margin > 1e-5      # (of 151,936 tokens most have intervals of that size: fewer rows are sure there)
+        assert sure.sum() > (0.9 if vocab < 10000 else 0.6) * rows and np.array_equal(got[sure], want[sure])
         assert len(set(want.tolist())) > rows // 4
