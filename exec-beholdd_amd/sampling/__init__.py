@@ -113,6 +113,15 @@ class Sampler:
         pin = self.device.type == "cuda"
         self._hosts = [torch.zeros((2, capacity), dtype=torch.int32, pin_memory=pin) for _ in range(self.RING)]
         self._turn = 0
+        # A draw's numbers (temperature, top-p, the uniform number; top-k) go to the device from pinned memory without
+        # a wait: a copy from ordinary memory would hold the host until the stream has run everything before it, and
+        # the loop that works a step ahead of the device would lose its lead at every step.
+        self._draw_hosts = [(torch.zeros((3, capacity), dtype=torch.float32, pin_memory=pin),
+                             torch.zeros(capacity, dtype=torch.int32, pin_memory=pin)) for _ in range(self.RING)]
+        self._draw_sent = [None] * self.RING      # the event behind each pair's last copy
+        self._draw_turn = 0
+        self._draw = (torch.zeros((3, capacity), dtype=torch.float32, device=self.device),
+                      torch.zeros(capacity, dtype=torch.int32, device=self.device))
 
     @property
     def device_tokens(self) -> torch.Tensor:
@@ -130,12 +139,26 @@ class Sampler:
         if all(p.greedy for p in params):
             self.kernels.sample(logits, tokens, bad)
         else:
-            host = torch.tensor([[p.temperature, p.top_p, uniform(p.seed, r, s)]
-                                 for p, r, s in zip(params, requests, steps)], dtype=torch.float32)
-            columns = host.t().contiguous().to(self.device)
-            top_k = torch.tensor([p.top_k for p in params], dtype=torch.int32).to(self.device)
-            self.kernels.sample(logits, tokens, bad, temperature=columns[0], top_k=top_k, top_p=columns[1],
-                                uniform=columns[2])
+            turn = self._draw_turn
+            self._draw_turn = (turn + 1) % self.RING
+            if self._draw_sent[turn] is not None:
+                self._draw_sent[turn].synchronize()      # (made RING selections ago: long done)
+            numbers, counts = self._draw_hosts[turn]
+            numbers[:, :n_rows] = torch.tensor([[p.temperature for p in params], [p.top_p for p in params],
+                                                [uniform(p.seed, r, s) for p, r, s in zip(params, requests, steps)]],
+                                               dtype=torch.float32)
+            counts[:n_rows] = torch.tensor([p.top_k for p in params], dtype=torch.int32)
+            on_device, counts_on_device = self._draw
+            if self.device.type == "cuda":
+                on_device.copy_(numbers, non_blocking=True)
+                counts_on_device.copy_(counts, non_blocking=True)
+                self._draw_sent[turn] = torch.cuda.Event()
+                self._draw_sent[turn].record()
+            else:
+                on_device.copy_(numbers)
+                counts_on_device.copy_(counts)
+            self.kernels.sample(logits, tokens, bad, temperature=on_device[0, :n_rows], top_k=counts_on_device[:n_rows],
+                                top_p=on_device[1, :n_rows], uniform=on_device[2, :n_rows])
         host = self._hosts[self._turn]
         self._turn = (self._turn + 1) % self.RING
         event = None
