@@ -20,7 +20,7 @@ from ..weights.random_init import random_tensor_on_device
 from . import generation
 from .graphs import DecodeGraphs
 from .memory import plan_memory
-from .step import StepEntry, StepError, build_step, cache_for_runs, check_entries
+from .step import StepEntry, StepError, StepStaging, build_step, cache_for_runs, check_entries
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
 
@@ -105,6 +105,7 @@ class Engine:
         self.cache_plan = self.cache.allocate()
         self.sampler = Sampler(kernels, self.device, capacity=self.cache.max_slots)
         self._last_selection = None
+        self._staging = StepStaging() if self.device.type == "cuda" else None
         self.graphs = DecodeGraphs(self, graph_limit) if with_graphs else None
 
     # ---- what the generation loop needs of a stepper ----
@@ -164,7 +165,7 @@ class Engine:
                             "(max_rows_per_step): feed the prompts in portions")
         self.cache.reserve(requests)
         try:
-            ctx, want_rows, tables = build_step(self.kernels, self.dtype, self.device, self.cache, entries)
+            ctx, want_rows, tables = build_step(self.kernels, self.dtype, self.device, self.cache, entries, self._staging)
             logits = self.model.forward(ctx, cache_for_runs(self.model, self.cache, tables), want_rows)
         except BaseException:
             self.cache.rollback(requests)

@@ -147,9 +147,39 @@ def cache_for_runs(model, cache, tables: dict):
     return cache_for_run
 
 
-def build_step(kernels, act_dtype, device, cache, entries: list):
+class StepStaging:
+    """Pinned host memory for the numbers of eager steps, a few buffers in turn: the copy to the device does not make
+    the host wait for what the stream still has to run (a copy from ordinary memory does), so that the host lays
+    out and launches a prompt's next portion while the device works on the one before."""
+
+    RING = 4
+
+    def __init__(self):
+        self._buffers = [None] * self.RING
+        self._sent = [None] * self.RING
+        self._turn = 0
+
+    def send(self, host_buffer: np.ndarray, device) -> torch.Tensor:
+        turn = self._turn
+        self._turn = (turn + 1) % self.RING
+        if self._sent[turn] is not None:
+            self._sent[turn].synchronize()      # its last copy, RING steps ago
+        pinned = self._buffers[turn]
+        if pinned is None or pinned.numel() < host_buffer.size:
+            pinned = self._buffers[turn] = torch.empty(max(4096, 2 * host_buffer.size), dtype=torch.int32, pin_memory=True)
+        staged = pinned[:host_buffer.size]
+        staged.copy_(torch.from_numpy(host_buffer))
+        on_device = torch.empty(host_buffer.size, dtype=torch.int32, device=device)
+        on_device.copy_(staged, non_blocking=True)
+        self._sent[turn] = torch.cuda.Event()
+        self._sent[turn].record()
+        return on_device
+
+
+def build_step(kernels, act_dtype, device, cache, entries: list, staging: StepStaging | None = None):
     """Lay out a step whose entries were checked and whose room was reserved: one buffer, one copy to the
-    device.  Returns (context, want_rows tensor, page tables by key/value group)."""
+    device (through `staging`, if given and the device is a GPU, without a wait).  Returns (context, want_rows
+    tensor, page tables by key/value group)."""
     pasts = [cache.length(entry.slot) for entry in entries]
     slots = [entry.slot for entry in entries]
     n_rows = sum(len(entry.tokens) for entry in entries)
@@ -161,7 +191,10 @@ def build_step(kernels, act_dtype, device, cache, entries: list):
     layout.fill(host, entries, pasts)
     for group in kv_groups:
         cache.write_page_table(group, slots, host["tables"][group])
-    views = layout.views(torch.from_numpy(host_buffer).to(device))
+    if staging is not None and torch.device(device).type == "cuda":
+        views = layout.views(staging.send(host_buffer, device))
+    else:
+        views = layout.views(torch.from_numpy(host_buffer).to(device))
     ctx = layout.context(views, kernels, act_dtype, device, host=host,
                          max_position=max(past + len(entry.tokens) for entry, past in zip(entries, pasts)) - 1,
                          max_rows_per_seq=max(len(entry.tokens) for entry in entries))
