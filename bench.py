@@ -53,6 +53,9 @@ def parse():
                              "128 tokens each at temperature 1) and print its tokens per second")
     parser.add_argument("--hbm-ceiling", action="store_true",
                         help="measure what a plain streaming read and a copy of 8 GB reach on this GPU, print it and exit")
+    parser.add_argument("--sampling", action="store_true",
+                        help="time the selection kernel on 1, 8 and 64 rows of 151,936 logits (greedy, at a temperature, with "
+                             "top-k, with top-p, with both), print the microseconds and exit")
     return parser.parse_args()
 
 
@@ -183,6 +186,41 @@ def hbm_ceiling(torch):
     return out
 
 
+def sampling_times(torch):
+    """Microseconds of one selection over rows of the benchmark's vocabulary, each mode replayed ten times from a
+    captured graph so that the launches' host cost stays out."""
+    from beholdd.kernels import HipKernels
+
+    kernels, vocab, out = HipKernels("cuda:0"), QWEN3_8B["vocab_size"], {}
+    for rows in (1, 8, 64):
+        logits = torch.randn(rows, vocab, device="cuda:0") * 3
+        tokens = torch.empty(rows, dtype=torch.int32, device="cuda:0")
+        bad = torch.empty_like(tokens)
+        temperature, uniform = torch.full((rows,), 0.8, device="cuda:0"), torch.rand(rows, device="cuda:0")
+        top_k = torch.full((rows,), 50, dtype=torch.int32, device="cuda:0")
+        top_p = torch.full((rows,), 0.9, device="cuda:0")
+        modes = {"greedy": {}, "temperature": dict(temperature=temperature, uniform=uniform),
+                 "top_k": dict(temperature=temperature, uniform=uniform, top_k=top_k),
+                 "top_p": dict(temperature=temperature, uniform=uniform, top_p=top_p),
+                 "top_k_top_p": dict(temperature=temperature, uniform=uniform, top_k=top_k, top_p=top_p)}
+        for name, arguments in modes.items():
+            kernels.sample(logits, tokens, bad, **arguments)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for _ in range(10):
+                    kernels.sample(logits, tokens, bad, **arguments)
+            graph.replay()
+            torch.cuda.synchronize()
+            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            begin.record()
+            graph.replay()
+            end.record()
+            torch.cuda.synchronize()
+            out[f"rows_{rows}_{name}_us"] = round(begin.elapsed_time(end) * 100, 1)
+    return out
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -191,6 +229,9 @@ def main():
     import torch
     if args.hbm_ceiling:
         print(json.dumps(hbm_ceiling(torch)))
+        return 0
+    if args.sampling:
+        print(json.dumps(sampling_times(torch)))
         return 0
 
     import beholdd
