@@ -296,6 +296,184 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
   }
 }
 
+// The skinny product of packed weights with workgroups that own 20 or 24 weight rows instead of 16 (parts of two
+// neighbouring blocks of the packed layout), for products whose blocks of 16 rows are
+// more than the compute units but fewer than twice as many: a quarter of the compute units would carry two blocks,
+// the others one, and the product takes as long as one with twice the compute units' blocks (Qwen3-14B's down
+// projection, 5120 x 17408 at 8 rows: 40.3 us, where 4096 x 17408 takes 25.4 and 8192 x 17408 47.2; with spans of
+// 20 rows 35.3 us, at 32 rows 59.6 -> 48.6; Qwen3-32B's, 5120 x 25600: 57.8 -> 49.9 and 86.8 -> 68.1; decode steps of 8,
+// 16 and 32 sequences at the 14B sizes 3 to 5 % faster, at the 32B sizes 6 to 8 %).  A lane asks
+// only for the rows its workgroup owns (the rows of a block lie side by side, 16 bytes each, so these are runs of 64
+// bytes and more), multiplies every block it touches and keeps what it owns.  Workgroups that run on one XCD own
+// neighbouring rows, so that a line of the weights that two of them share is fetched into that L2 once.  RT = 1 only.
+#define SPAN_TILES 2
+template <int MB, int WAVES, typename TC, int XB>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_span_kernel(const uint16_t* __restrict__ a,
+                                                                      const uint16_t* __restrict__ w,
+                                                                      TC* __restrict__ c, int M, int N, int K,
+                                                                      int accumulate, int span, RidingNorm norm,
+                                                                      RowBlocks blocks) {
+  __shared__ float partial[WAVES][SPAN_TILES][MB][256];
+  __shared__ float row_factor[MB * 16];
+  constexpr int ROWS_PER_PASS = WAVES * 2, PASSES = (MB * 16 + ROWS_PER_PASS - 1) / ROWS_PER_PASS;
+  const int part = threadIdx.x % 32;
+  float early[PASSES][8];
+  if (norm.ahead_ss) {
+#pragma unroll
+    for (int pass = 0; pass < PASSES; ++pass) {
+      const int r = pass * ROWS_PER_PASS + threadIdx.x / 32;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int block = part + 32 * u;
+        early[pass][u] = (r < M && block < norm.ahead_blocks) ? norm.ahead_ss[(size_t)r * norm.ahead_blocks + block] : 0.f;
+      }
+    }
+  }
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int i = lane % 16, g = lane / 16;
+  const int full = K / 64;
+  // workgroups go to the XCDs in turn: the ones of an XCD own a run of neighbouring spans
+  const int owner = gridDim.x % 8 == 0 ? (int)(blockIdx.x % 8) * (int)(gridDim.x / 8) + (int)(blockIdx.x / 8) : (int)blockIdx.x;
+  const int first_row = owner * span, first_tile = first_row / 16;
+  int lo[SPAN_TILES], hi[SPAN_TILES];   // the rows of each block that this workgroup owns: lo <= row < hi (none: hi <= lo)
+  const uint16_t* wp[SPAN_TILES];
+#pragma unroll
+  for (int t = 0; t < SPAN_TILES; ++t) {
+    const int tile_row = (first_tile + t) * 16;
+    lo[t] = max(first_row, tile_row) - tile_row;
+    hi[t] = min(min(first_row + span, N), tile_row + 16) - tile_row;
+    const int tile = min(first_tile + t, N / 16 - 1);   // (a block beyond the matrix is never loaded; its address stays inside)
+    wp[t] = w + (size_t)tile * full * 1024 + lane * 8;
+  }
+  const uint16_t* xp[MB];
+  constexpr int x_half = XB ? XB * 8 : 8, x_chunk = XB ? 64 * XB : 64;
+#pragma unroll
+  for (int b = 0; b < MB; ++b) {
+    if (XB) {
+      constexpr int step = 32 * (XB ? XB : 1);
+      xp[b] = a + (size_t)(b * 16 / (XB ? XB : 1)) * (K / 32) * step + (g / 2) * step + ((2 * g) % 4 * XB + (XB == 8 ? i : i % (XB ? XB : 1))) * 8;
+    } else {
+      const int row = (b * 16 + i < M) ? b * 16 + i : M - 1;
+      xp[b] = a + (size_t)row * K + g * 16;
+    }
+  }
+  f32x4_t acc[SPAN_TILES][MB];
+#pragma unroll
+  for (int t = 0; t < SPAN_TILES; ++t)
+#pragma unroll
+    for (int b = 0; b < MB; ++b) acc[t][b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const u32x4_t zero = {0u, 0u, 0u, 0u};
+  bool mine[SPAN_TILES];
+#pragma unroll
+  for (int t = 0; t < SPAN_TILES; ++t) mine[t] = i >= lo[t] && i < hi[t];
+
+  constexpr int U = MB == 1 ? 4 : 2;   // chunks per trip, all their loads issued before the first multiply
+  int chunk = wave;
+  for (; chunk + (U - 1) * WAVES < full; chunk += U * WAVES) {
+    u32x4_t wv[U][SPAN_TILES][2], xv[U][MB][2];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int at = chunk + u * WAVES;
+#pragma unroll
+      for (int t = 0; t < SPAN_TILES; ++t) {
+        const uint16_t* p = wp[t] + (size_t)at * 1024;
+        wv[u][t][0] = mine[t] ? load16_stream(p) : zero;
+        wv[u][t][1] = mine[t] ? load16_stream(p + 512) : zero;
+      }
+#pragma unroll
+      for (int b = 0; b < MB; ++b) {
+        xv[u][b][0] = load16(xp[b] + at * x_chunk);
+        if (XB != 8) xv[u][b][1] = load16(xp[b] + at * x_chunk + x_half);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int b = 0; b < MB; ++b) {
+        if (XB == 8) xv[u][b][1] = from_lane_plus_8(xv[u][b][0]);
+#pragma unroll
+        for (int t = 0; t < SPAN_TILES; ++t) {
+          if (hi[t] <= lo[t]) continue;   // the same for the whole workgroup
+          acc[t][b] = MFMA16(wv[u][t][0], xv[u][b][0], acc[t][b]);
+          acc[t][b] = MFMA16(wv[u][t][1], xv[u][b][1], acc[t][b]);
+        }
+      }
+  }
+  for (; chunk < full; chunk += WAVES) {
+    u32x4_t x0[MB], x1[MB];
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+      x0[b] = load16(xp[b] + chunk * x_chunk);
+      x1[b] = XB == 8 ? from_lane_plus_8(x0[b]) : load16(xp[b] + chunk * x_chunk + x_half);
+    }
+#pragma unroll
+    for (int t = 0; t < SPAN_TILES; ++t) {
+      if (hi[t] <= lo[t]) continue;
+      const uint16_t* p = wp[t] + (size_t)chunk * 1024;
+      const u32x4_t w0 = mine[t] ? load16(p) : zero, w1 = mine[t] ? load16(p + 512) : zero;
+#pragma unroll
+      for (int b = 0; b < MB; ++b) {
+        acc[t][b] = MFMA16(w0, x0[b], acc[t][b]);
+        acc[t][b] = MFMA16(w1, x1[b], acc[t][b]);
+      }
+    }
+  }
+  if (norm.ahead_ss) {
+#pragma unroll
+    for (int pass = 0; pass < PASSES; ++pass) {
+      const int r = pass * ROWS_PER_PASS + threadIdx.x / 32;
+      float ss = 0.f;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) ss += early[pass][u];
+      if (r < M)
+        for (int block = part + 256; block < norm.ahead_blocks; block += 32) ss += norm.ahead_ss[(size_t)r * norm.ahead_blocks + block];
+#pragma unroll
+      for (int off = 16; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+      if (part == 0 && r < MB * 16) row_factor[r] = (r < M) ? 1.0f / sqrtf(ss / (float)K + norm.ahead_eps) : 0.f;
+    }
+  }
+  // D: lane holds column (activation row) i and rows (W rows) 4g..4g+3 of each block; lay it out as [m][n]
+#pragma unroll
+  for (int t = 0; t < SPAN_TILES; ++t)
+#pragma unroll
+    for (int b = 0; b < MB; ++b)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) partial[wave][t][b][i * 16 + 4 * g + r] = acc[t][b][r];
+  __syncthreads();
+  for (int e = threadIdx.x; e < MB * 256; e += WAVES * 64) {   // whole waves enter or stay out
+    const int b = e / 256, m = b * 16 + (e % 256) / 16, column = e % 16;
+    float sq = 0.f;   // of what this workgroup adds to row m of the residual (norm.behind_weight)
+#pragma unroll
+    for (int t = 0; t < SPAN_TILES; ++t) {
+      const int n = (first_tile + t) * 16 + column;
+      const bool valid = m < M && column >= lo[t] && column < hi[t];
+      float sum = 0.f;
+#pragma unroll
+      for (int v = 0; v < WAVES; ++v) sum += partial[v][t][b][e % 256];
+      if (norm.ahead_ss) sum *= row_factor[m];
+      if (!valid) continue;
+      if (norm.behind_weight) {   // float32 output
+        float* cf = reinterpret_cast<float*>(c);
+        const float value = accumulate ? cf[(size_t)m * N + n] + sum : sum;
+        cf[(size_t)m * N + n] = value;
+        sq += value * value;
+        const float gw = norm.behind_weight_f32 ? reinterpret_cast<const float*>(norm.behind_weight)[n]
+                                                : bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(norm.behind_weight)[n]);
+        norm.behind_rows[bh_rows_index(blocks.behind, m, n, N)] = f32_to_bf16_bits(value * gw);
+      } else {
+        store_out<TC>(c, (size_t)m * N + n, sum, accumulate != 0);
+      }
+    }
+    if (norm.behind_weight) {
+      sq += __shfl_xor(sq, 8, 64);   // the 16 columns of a row sit in 16 neighbouring lanes
+      sq += __shfl_xor(sq, 4, 64);
+      sq += __shfl_xor(sq, 2, 64);
+      sq += __shfl_xor(sq, 1, 64);
+      if (column == 0 && m < M) norm.behind_ss[(size_t)m * gridDim.x + blockIdx.x] = sq;
+    }
+  }
+}
+
 // ---- K in parts: the finishing kernel ---------------------------------------------------------
 // Whole tiles that are too few to fill the chip cut K into parts over workgroups (gemm_tiled_whole_kernel
 // with `parts_out`); the bare sums go to scratch memory as [K part][row][weight row].  This kernel adds the
@@ -907,10 +1085,37 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_whole_kernel(const ui
 
 // ---- entry -------------------------------------------------------------------------------------
 
+// The weight rows per workgroup (20 or 24) with which the skinny product of packed weights runs as
+// gemm_skinny_span_kernel, or 0: where its blocks of 16 rows are more than the compute units and fewer than twice as
+// many, and some such span divides the rows into no more workgroups than there are compute units.
+static int skinny_span_rows(int M, int N, int K) {
+  if (M > 32 || N % 16 != 0 || K % 64 != 0) return 0;
+  const int tiles = N / 16, units = bh_compute_units();
+  if (tiles <= units || tiles >= 2 * units) return 0;
+  for (int rows = 20; rows <= 24; rows += 4)   // (28 rows can lie in three blocks: 7168 x 5120 at 8 rows 14.6 -> 17.1 us)
+    if (N % rows == 0 && N / rows <= units) return rows;
+  return 0;
+}
+
 template <bool TILES, int RT, typename TC>
 static void launch_skinny(const void* a, const void* w, void* c, int M, int N, int K, int accumulate,
                           int pair_blocks, const RidingNorm& norm, const RowBlocks& blocks, hipStream_t stream) {
   constexpr int WAVES = 8;
+  if constexpr (TILES && RT == 1) {
+    if (const int span = skinny_span_rows(M, N, K)) {
+      dim3 span_grid(N / span), span_block(WAVES * 64);
+#define BH_SPAN(MB, XB)                                                                                  \
+  gemm_skinny_span_kernel<MB, WAVES, TC, XB><<<span_grid, span_block, 0, stream>>>(                      \
+      (const uint16_t*)a, (const uint16_t*)w, (TC*)c, M, N, K, accumulate, span, norm, blocks)
+      if (blocks.a == 8) BH_SPAN(1, 8);
+      else if (blocks.a == 16 && M <= 16) BH_SPAN(1, 16);
+      else if (blocks.a == 16) BH_SPAN(2, 16);
+      else if (M <= 16) BH_SPAN(1, 0);
+      else BH_SPAN(2, 0);
+#undef BH_SPAN
+      return;
+    }
+  }
   dim3 grid((N + 15) / 16), block(WAVES * 64);
 #define BH_SKINNY(MB, XB)                                                                                 \
   gemm_skinny_kernel<MB, WAVES, TILES, RT, TC, XB><<<grid, block, 0, stream>>>(                           \
@@ -1061,7 +1266,11 @@ extern "C" int bh_gemm_bf16_norm_blocks(int M, int N, int K, int layout, int act
   int rows, columns, parts, each;
   if (gemm_slices_takes(M, N, K, layout, 0)) return (N + FINISH_COLUMNS - 1) / FINISH_COLUMNS;   // always finished by that kernel
   tiled_config(M, N, false, &rows, &columns);
-  if (!tiled_whole(M, N, K, layout, rows, columns)) return M <= 64 ? (N + 15) / 16 : 0;   // the skinny kernel's blocks
+  if (!tiled_whole(M, N, K, layout, rows, columns)) {   // the skinny kernel's blocks, or its workgroups of wider spans
+    if (layout == 1 && skinny_first(M, N, K, layout))
+      if (const int span = skinny_span_rows(M, N, K)) return N / span;
+    return M <= 64 ? (N + 15) / 16 : 0;
+  }
   tiled_parts(M, N, K, layout, false, &parts, &each);
   return parts > 1 ? (N + FINISH_COLUMNS - 1) / FINISH_COLUMNS : (N + columns - 1) / columns;   // the finishing kernel's blocks, or the tiles'
 }

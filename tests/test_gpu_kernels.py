@@ -116,7 +116,10 @@ def test_gemm(K, a_dtype, w_dtype, m, n, k):
                                    # 33 to 64 rows, K from 512: the waves of a workgroup share the activations through LDS;
                                    # a last slice of fewer than 512 k, weight blocks that do not fill the last workgroup
                                    (33, 128, 512), (48, 144, 576), (64, 4096, 4096), (49, 1008, 1088), (40, 6144, 4096),
-                                   (64, 4096, 12288), (57, 5120, 5120), (80, 4096, 4096), (128, 6144, 4096), (97, 1008, 1280)])
+                                   (64, 4096, 12288), (57, 5120, 5120), (80, 4096, 4096), (128, 6144, 4096), (97, 1008, 1280),
+                                   # up to 32 rows, blocks of 16 weight rows between one and two per compute unit: workgroups
+                                   # that own 20, 24 or 28 rows (parts of two or three blocks); a last chunk trip that is not whole
+                                   (8, 5120, 1024), (1, 5120, 5120), (32, 7168, 512), (17, 6144, 192), (9, 7168, 5120), (3, 5120, 17408)])
 def test_gemm_with_packed_weights(K, m, n, k):
     """The same product from the regrouped (16 x 64 blocks) weight layout."""
     from beholdd.kernels import PackedWeight
@@ -149,7 +152,9 @@ def test_gemm_with_packed_weights(K, m, n, k):
 @pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("m,n,k,n2", [(1, 192, 128, 48), (8, 4096, 256, 1000), (17, 200, 64, 64), (64, 320, 192, 130),
                                       (48, 512, 1024, 256), (64, 4096, 4096, 2048), (33, 1024, 576, 640),
-                                      (96, 1024, 1024, 512), (128, 4096, 4096, 2048)])
+                                      (96, 1024, 1024, 512), (128, 4096, 4096, 2048),
+                                      # workgroups that own 20, 24 or 28 weight rows, on both sides of the norm
+                                      (8, 5120, 512, 7168), (20, 6144, 256, 5120), (1, 5120, 128, 6144)])
 def test_norm_rides_on_the_products_around_it(K, g_dtype, packed, m, n, k, n2):
     """The product that completes the residual prepares the following RMSNorm (rows times the norm weight,
     partial sums of squares), and the product after it applies each row's factor to its result."""
