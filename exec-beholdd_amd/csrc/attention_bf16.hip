@@ -453,12 +453,20 @@ extern "C" int bh_attention_bf16_splits(int n_seqs, int max_rows_per_seq, int H,
   const int G = H / KVH;
   const long tiles = (long)((max_rows_per_seq * G + 15) / 16) * KVH * n_seqs;
   const int pages = max_position / BH_PAGE + 1;
-  // about one workgroup per compute unit (256 on an MI355X), every wave of a workgroup at least one page
+  // Every wave of a workgroup at least one page.  The workgroups run in rounds of one per compute unit (256 on an
+  // MI355X), so what a launch costs is its rounds times a workgroup's pages (and about four pages' worth of start and
+  // merge): the split count with the least of that, the smaller one among equals.  One workgroup per compute unit or
+  // just beyond, as it was before, made 288 to 384 workgroups of 9 to 14 and of 17 to 24 sequences: two rounds of
+  // nearly whole-sized workgroups (decode steps of the Qwen3-8B shape at context 8,192, 8 layers: 6 sequences 1.18 ->
+  // 1.11 ms, 10 1.48 -> 1.40, 12 1.63 -> 1.48, 20 2.18 -> 2.02, 24 2.23 -> 2.19; 8, 16 and 32 sequences as before).
   const int units = bh_compute_units();
   if (tiles >= units || pages < 8) return 1;
-  long want = (units + tiles - 1) / tiles;
-  if (want > pages / 4) want = pages / 4;
-  if (want < 1) want = 1;
+  long want = 1, least = -1;
+  for (long splits = 1; splits <= pages / 4 && splits <= 64; ++splits) {
+    const long rounds = (tiles * splits + units - 1) / units, each = (pages + splits - 1) / splits;
+    const long cost = rounds * (each + 4);
+    if (least < 0 || cost < least) least = cost, want = splits;
+  }
   const int per = (int)((pages + want - 1) / want);
   return (pages + per - 1) / per;
 }
