@@ -460,12 +460,24 @@ extern "C" int bh_attention_bf16_splits(int n_seqs, int max_rows_per_seq, int H,
   // nearly whole-sized workgroups (decode steps of the Qwen3-8B shape at context 8,192, 8 layers: 6 sequences 1.18 ->
   // 1.11 ms, 10 1.48 -> 1.40, 12 1.63 -> 1.48, 20 2.18 -> 2.02, 24 2.23 -> 2.19; 8, 16 and 32 sequences as before).
   const int units = bh_compute_units();
-  if (tiles >= units || pages < 8) return 1;
+  if (pages < 8) return 1;
   long want = 1, least = -1;
-  for (long splits = 1; splits <= pages / 4 && splits <= 64; ++splits) {
-    const long rounds = (tiles * splits + units - 1) / units, each = (pages + splits - 1) / splits;
-    const long cost = rounds * (each + 4);
-    if (least < 0 || cost < least) least = cost, want = splits;
+  if (tiles > units) {
+    // More workgroups than compute units: two of the lean kernel's share a compute unit.  Just above one per compute
+    // unit (and just above two) the few compute units that carry one more hold the launch up, and three (two) splits
+    // spread the pages evenly; from about 1.4 per compute unit on the whole workgroups are as fast or faster
+    // (Qwen3-8B shape, context 8,192, 8 layers, ms per step with 1 / 2 / 3 / 4 / 6 splits: 33 sequences 3.04 / 2.80 / 2.72 /
+    // 2.69 / 2.66, 40: 3.20 / 2.92 / 2.89 / 2.90 / 2.91, 48: 3.27 / 3.35 / 3.25 / 3.25 / 3.25, 56: 3.66 / 3.75 / 3.75 / 3.69 /
+    // 3.73, 72: 4.55 / 4.43 / 4.43 / 4.52 / 4.54).
+    const double each_unit = (double)tiles / units;
+    want = each_unit < 1.4 ? 3 : (each_unit > 2.0 && each_unit < 2.4) ? 2 : 1;
+    if (want > pages / 4) want = pages / 4;
+  } else {
+    for (long splits = 1; splits <= pages / 4 && splits <= 64; ++splits) {
+      const long rounds = (tiles * splits + units - 1) / units, each = (pages + splits - 1) / splits;
+      const long cost = rounds * (each + 4);
+      if (least < 0 || cost < least) least = cost, want = splits;
+    }
   }
   const int per = (int)((pages + want - 1) / want);
   return (pages + per - 1) / per;
