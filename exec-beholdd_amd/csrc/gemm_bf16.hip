@@ -1385,6 +1385,10 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
     BH_REQUIRE(((uintptr_t)c | (uintptr_t)scratch | (uintptr_t)behind_rows) % 16 == 0,
                "gemm_bf16: output, scratch memory and norm rows must be 16-byte aligned");
     const int parts = gemm_slices_parts(M, N, K, activation, nullptr);
+    // One part, float32 rows out, nothing to add, to scale or to prepare: the sums are the output, in its own order
+    // (the head product of 33 to 128 rows: 151,936 x 4,096 at 64 rows 279 us with the finishing kernel's copy).
+    if (parts == 1 && f32 && !activation && !accumulate && !ahead_ss && !behind_weight)
+      return gemm_slices_launch(a, w, (float*)c, M, N, K, activation, stream);
     if (int status = gemm_slices_launch(a, w, (float*)scratch, M, N, K, activation, stream)) return status;
     if (activation) { if (f32) BH_FINISH(true, float); else BH_FINISH(true, bf16_t); }
     else { if (f32) BH_FINISH(false, float); else BH_FINISH(false, bf16_t); }
