@@ -270,8 +270,8 @@ def main():
     achieved = step_bytes / seconds / 1e9
     value = args.batch / seconds
 
-    prefill_seconds = prefill_run(engine, args.prefill_tokens, torch)
-    t = args.prefill_tokens
+    t = min(args.prefill_tokens, args.context)      # (a context shorter than the prompt: a prompt of the context's length)
+    prefill_seconds = prefill_run(engine, t, torch)
     prefill_flops = (2.0 * cfg.n_layers * layer_params * t + cfg.n_layers * cfg.n_heads * 2.0 * t * t * cfg.head_dim
                      + 2.0 * cfg.vocab * cfg.hidden)
     # Other batch sizes and contexts: tokens a second, and beside each the fraction of the HBM peak that the
@@ -364,7 +364,7 @@ def other_shape(name, args, torch):
     kv_bytes_per_token = cfg.n_layers * 2 * cfg.kv_width * 2
     steps = max(4, args.steps // 2)
     seconds, mean_length = decode_run(engine, 8, args.context, steps, 2, torch)
-    t = args.prefill_tokens
+    t = min(args.prefill_tokens, args.context)
     prefill_seconds = prefill_run(engine, t, torch, repeats=2)
     prefill_flops = (2.0 * cfg.n_layers * layer_params * t + cfg.n_layers * cfg.n_heads * 2.0 * t * t * cfg.head_dim
                      + 2.0 * cfg.vocab * cfg.hidden)
