@@ -310,12 +310,14 @@ def main():
     # what a kernel that does nothing but read reaches on this GPU (the library's yardstick kernel over 4 GB of the cache)
     cache_tensor = engine.cache.groups[0].k
     span = cache_tensor.view(-1)[: min(cache_tensor.numel(), 2 << 30)]
-    engine.kernels.stream_read(span)
-    torch.cuda.synchronize()
-    begin = time.perf_counter()
-    read = sum(engine.kernels.stream_read(span) for _ in range(4))
-    torch.cuda.synchronize()
-    yardstick = read / (time.perf_counter() - begin) / 1e9
+    yardstick = None
+    if span.numel() * span.element_size() >= 256 << 20:      # (a cache of a few MB says nothing about streaming)
+        engine.kernels.stream_read(span)
+        torch.cuda.synchronize()
+        begin = time.perf_counter()
+        read = sum(engine.kernels.stream_read(span) for _ in range(4))
+        torch.cuda.synchronize()
+        yardstick = read / (time.perf_counter() - begin) / 1e9
 
     line = {
         "metric": f"decode tok/s @ batch {args.batch} ({shape_name}, context {args.context})", "value": round(value, 2), "unit": "tok/s",
@@ -332,7 +334,7 @@ def main():
         "prefill": {"value": round(t / prefill_seconds, 1), "tokens": t, "ms": round(prefill_seconds * 1e3, 3),
                     "frac": round(prefill_flops / prefill_seconds / PEAK_FLOPS[dtype_tag], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(achieved / PEAK_HBM_GBS, 4), "plain_read_GBs": round(yardstick, 1)},
+                     "frac": round(achieved / PEAK_HBM_GBS, 4), "plain_read_GBs": round(yardstick, 1) if yardstick is not None else None},
         "points": points,
         "points_hbm_frac": fractions,
     }
