@@ -102,7 +102,10 @@ def test_batches_of_many_sequences(model_dirs, dtype):
 
 # (layers, hidden, query heads, kv heads, feed-forward width, prompt lengths)
 LARGE_SHAPES = {"8b": (2, 4096, 32, 8, 12288, [70, 9, 131, 300]), "14b": (1, 5120, 40, 8, 17408, [70, 9, 131]),
-                "32b": (1, 5120, 64, 8, 25600, [70, 9, 131])}
+                "32b": (1, 5120, 64, 8, 25600, [70, 9, 131]),
+                # narrower layers of the same make: other counts of weight blocks per compute unit, other tile plans
+                "w1024": (2, 1024, 16, 8, 3072, [70, 9, 131]), "w2048": (2, 2048, 16, 8, 6144, [70, 9, 131]),
+                "w2560": (1, 2560, 32, 8, 9728, [70, 9, 131, 300])}
 
 
 @pytest.fixture(scope="module")
@@ -131,7 +134,7 @@ def large_expected(tmp_path_factory):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("shape", ["8b", "14b", "32b"])
+@pytest.mark.parametrize("shape", ["8b", "14b", "32b", "w1024", "w2048", "w2560"])
 def test_layers_of_the_large_models_sizes(large_expected, shape, dtype):
     """The layer sizes of Qwen3-8B, 14B and 32B (five and eight query heads per kv head, heads that do not
     add up to the width) in one or two layers with a small vocabulary: the kernels at the shapes they are
