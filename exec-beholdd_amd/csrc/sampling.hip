@@ -14,10 +14,10 @@
 // the order-preserving integer key of a logit): a pass over the row adds each token's count (top-k) or weight
 // (top-p) to the bin of its digit, among the tokens whose higher digits are the ones found so far; the bins are
 // walked from the top until the count reaches k, or the weight top_p of the total.  Three passes each, where a
-// search bit by bit took 32 (a row of 151,936 logits, one row or eight: temperature alone 121 -> 55 us, with
-// top-k of 50 711 -> 93, with top-p of 0.9 2,224 -> 115, with both 2,634 -> 134; 64 rows: 216 -> 59, 1,707 -> 102,
-// 5,146 -> 125, 5,835 -> 151).  What is left is arithmetic on the one compute unit that a row has: a pass costs
-// 10 to 13 us, the draw's pass with its sums per trip about 30 (holding twice the loads in flight changed nothing).
+// search bit by bit took 32 (a row of 151,936 logits, one row or eight: temperature alone 121 -> 48 us, with
+// top-k of 50 711 -> 86, with top-p of 0.9 2,224 -> 110, with both 2,634 -> 128; 64 rows: 216 -> 52, 1,707 -> 94,
+// 5,146 -> 117, 5,835 -> 142).  What is left is arithmetic on the one compute unit that a row has: a pass costs
+// 10 to 13 us, the draw's about 25 (holding twice the loads in flight changed nothing).
 #include "sampling.h"
 
 #include <mutex>
@@ -230,12 +230,13 @@ __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ lo
 
   // The draw.  A wave owns a contiguous span of the vocabulary and walks it in trips of 256 tokens, lane l taking
   // tokens 64 u + l of a trip (u = 0..3): in index order a trip is its four quarters one after the other, a quarter its
-  // lanes.  First every trip's kept weight (into `bins`), then the wave whose span holds the target finds the trip,
-  // the quarter and the lane.
+  // lanes.  First every span's kept weight (a lane adds up its own tokens, one sum over the lanes at the end), which
+  // says whose span holds the target; then all waves share that span's trips and leave each trip's weight in `bins`;
+  // then one wave finds the trip, the quarter and the lane.  (A sum over the lanes for every trip of every span made
+  // this pass 30 us of arithmetic on the one compute unit that a row has.)
   constexpr int WAVES = SB / BH_WAVE, TRIP = 4 * BH_WAVE;
   const int wave = tid / BH_WAVE, lane = tid % BH_WAVE;
-  const int trips = ((vocab + WAVES - 1) / WAVES + TRIP - 1) / TRIP;   // per wave; at most SAMPLE_BINS / WAVES (the entry point checks)
-  const int begin = wave * trips * TRIP;
+  const int trips = ((vocab + WAVES - 1) / WAVES + TRIP - 1) / TRIP;   // per span; at most SAMPLE_BINS (the entry point checks)
   auto kept_weight = [&](int i) -> sample_u64 {
     if (i >= vocab) return 0;
     const float v = x[i];
@@ -246,44 +247,51 @@ __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ lo
     for (int off = BH_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, BH_WAVE);
     return v;
   };
-  sample_u64 of_wave = 0;
-  constexpr int AHEAD = 8;   // trips whose loads are on their way together
-  for (int trip0 = 0; trip0 < trips; trip0 += AHEAD) {
-    float v[AHEAD][4];
+  {
+    const int begin = wave * trips * TRIP;
+    sample_u64 mine = 0;
+    constexpr int AHEAD = 8;   // trips whose loads are on their way together
+    for (int trip0 = 0; trip0 < trips; trip0 += AHEAD) {
+      float v[AHEAD][4];
 #pragma unroll
-    for (int a = 0; a < AHEAD; ++a)
+      for (int a = 0; a < AHEAD; ++a)
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int i = begin + (trip0 + a) * TRIP + BH_WAVE * u + lane;
-        v[a][u] = (trip0 + a < trips && i < vocab) ? x[i] : -INFINITY;   // what is not there weighs nothing
-      }
+        for (int u = 0; u < 4; ++u) {
+          const int i = begin + (trip0 + a) * TRIP + BH_WAVE * u + lane;
+          v[a][u] = (trip0 + a < trips && i < vocab) ? x[i] : -INFINITY;   // what is not there weighs nothing
+        }
 #pragma unroll
-    for (int a = 0; a < AHEAD; ++a) {
-      if (trip0 + a >= trips) break;
-      sample_u64 w = 0;
+      for (int a = 0; a < AHEAD; ++a)
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
-        if (v[a][u] != -INFINITY && order_key(v[a][u]) >= floor_key) w += weight_of(v[a][u]);
-      w = wave_total(w);
-      if (lane == 0) bins[wave * trips + trip0 + a] = w;
-      of_wave += w;
+        for (int u = 0; u < 4; ++u)
+          if (v[a][u] != -INFINITY && order_key(v[a][u]) >= floor_key) mine += weight_of(v[a][u]);
     }
+    mine = wave_total(mine);
+    __syncthreads();
+    if (lane == 0) scratch[wave] = mine;
+    if (tid == 0) chosen = arg_max;
+    __syncthreads();
   }
-  __syncthreads();
-  if (lane == 0) scratch[wave] = of_wave;
-  if (tid == 0) chosen = arg_max;
-  __syncthreads();
-  sample_u64 before = 0, kept = 0;
-  for (int w = 0; w < WAVES; ++w) {
-    if (w < wave) before += scratch[w];
-    kept += scratch[w];
-  }
+  sample_u64 kept = 0;
+  for (int w = 0; w < WAVES; ++w) kept += scratch[w];
   sample_u64 target = (sample_u64)__double2ull_rd((double)uniform[row] * (double)kept);
   if (target >= kept) target = kept - 1;   // (uniform is below 1; the largest token alone weighs 2^32 - 1)
-  if (target >= before && target < before + of_wave) {   // one wave, all of its lanes
+  int span = 0;
+  sample_u64 before = 0;   // the kept weight of the spans before the target's
+  for (; span < WAVES - 1 && before + scratch[span] <= target; ++span) before += scratch[span];
+  const int span_begin = span * trips * TRIP;
+  for (int trip = wave; trip < trips; trip += WAVES) {   // the waves share the span's trips
+    sample_u64 w = 0;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) w += kept_weight(span_begin + trip * TRIP + BH_WAVE * u + lane);
+    w = wave_total(w);
+    if (lane == 0) bins[trip] = w;
+  }
+  __syncthreads();
+  if (wave == 0) {
     int trip = 0;
-    for (; trip < trips - 1 && before + bins[wave * trips + trip] <= target; ++trip) before += bins[wave * trips + trip];
-    const int base = begin + trip * TRIP;
+    for (; trip < trips - 1 && before + bins[trip] <= target; ++trip) before += bins[trip];
+    const int base = span_begin + trip * TRIP;
     sample_u64 w[4], quarter[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
@@ -409,8 +417,8 @@ extern "C" int bh_sample(const float* logits, const float* temperature, const in
     argmax_rows_kernel<<<dim3(n_rows), dim3(BH_WAVE), 0, stream>>>(part_val, part_idx, tokens, bad, chunks);
     return bh_check_launch("argmax_rows");
   }
-  BH_REQUIRE(temperature == nullptr || vocab <= SAMPLE_BINS * 256,
-             "sample: a draw takes vocabularies of up to %d tokens, not %d", SAMPLE_BINS * 256, vocab);
+  BH_REQUIRE(temperature == nullptr || vocab <= SAMPLE_BINS * 256 * (SB / BH_WAVE),
+             "sample: a draw takes vocabularies of up to %d tokens, not %d", SAMPLE_BINS * 256 * (SB / BH_WAVE), vocab);
   sample_kernel<<<dim3(n_rows), dim3(SB), 0, stream>>>(logits, temperature, top_k, top_p, uniform, tokens, bad,
                                                        vocab);
   return bh_check_launch("sample");
