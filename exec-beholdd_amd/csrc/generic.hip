@@ -410,7 +410,7 @@ __device__ inline void load_eight(const bf16_t* p, float (&v)[8]) {
 // The values have waves of their own, behind the `main_waves` that take the q and k heads (`n_heads` of them):
 // a value's neighbours in memory are the same dim of other tokens, eight tokens to a 16-byte piece in either
 // cache order, so a wave takes eight rows and (up to) 64 / LPH kv heads, and where the eight tokens of a piece
-// are rows of this step (the same sequence, positions 8 x .. 8 x + 7) the lanes of its first row load all eight
+// are consecutive rows of this step (the same sequence, positions 8 x .. 8 x + 7) the lanes of its first row load all eight
 // rows, turn the 8 x 8 elements and store whole pieces; rows whose piece is not whole in this step (a step's
 // first and last tokens) store their eight elements one by one.  (8,192 rows of 32 query and 8 kv heads of
 // 128: the stores of the values one by one were 35 of the kernel's 57 us.)
@@ -511,8 +511,11 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_rows_kernel(
     for (int row = 8 * group; row < 8 * group + 8 && row < n_rows; ++row) {
       const int pos = pos_of(row), seq = seq_of(row);
       const int first = row - pos % 8;   // where the row of the piece's first token would lie
-      const bool whole = first >= 0 && first + 7 < n_rows && seq_of(first) == seq && seq_of(first + 7) == seq &&
-                         pos_of(first) == pos - pos % 8 && pos_of(first + 7) == pos - pos % 8 + 7;
+      bool whole = first >= 0 && first + 7 < n_rows;   // the piece's eight tokens are the rows first .. first + 7, in order
+      if (whole) {
+#pragma unroll
+        for (int t = 0; t < 8; ++t) whole = whole && seq_of(first + t) == seq && pos_of(first + t) == pos - pos % 8 + t;
+      }
       if (whole && pos % 8 != 0) continue;   // the first row of the piece stores it
       const int page = page_table[(size_t)seq * table_stride + pos / BH_PAGE];
       uint16_t* block = v_pages + ((size_t)page * KVH + kv_head) * BH_PAGE * HD;
@@ -658,10 +661,9 @@ static int qk_rows_form(const void* qkv, int parts, void* q_out, const void* q_w
   return bh_check_launch("qk_norm_rope_cache_rows");
 }
 
-// Precondition: the rows of one sequence stand one after the other and in position order (row r + 1 of a
-// sequence is position p + 1), as a step lays them out.  The form for many rows relies on it: it takes eight
-// rows for one piece of values when the first and the last of them belong to one sequence, seven positions apart,
-// and does not look at the six between.
+// Rows may come in any order (every (sequence, position) once).  The form for many rows stores the values of eight
+// consecutive positions as one piece where the step holds all eight as consecutive rows of one sequence, which it
+// checks row by row (a step lays a sequence's rows out that way); any other row stores its own elements.
 extern "C" int bh_qk_norm_rope_cache(const void* qkv, int dtype, void* q_out, const void* q_weight,
                                      const void* k_weight, int w_dtype, float eps, const float* cos_table,
                                      const float* sin_table, int table_positions, int rot,

@@ -572,9 +572,9 @@ class HipKernels(KernelSizes):
                            k_pages, v_pages, page_table, n_heads, n_kv_heads, head_dim, write_kv, max_position):
         """Per head of the fused [q | k | v] projection rows: RMSNorm (when weights are given),
         split-half rotation at the row's position (when tables are given), then q to `q_out`
-        and k, v into the cache pages of (sequence, position).  The rows of one sequence must stand one after
-        the other and in position order, as a step lays them out (the kernel for many rows writes the values of
-        eight consecutive positions as one piece and checks only the first and the last of the eight)."""
+        and k, v into the cache pages of (sequence, position).  Rows may come in any order, each
+        (sequence, position) once; where eight consecutive positions of a sequence are consecutive rows, as a step
+        lays them out, the kernel for many rows writes their values as one piece."""
         n_rows = qkv.shape[0]
         fused = (n_heads + 2 * n_kv_heads) * head_dim
         if qkv.shape != (n_rows, fused) or q_out.shape != (n_rows, n_heads * head_dim) or q_out.dtype != qkv.dtype:

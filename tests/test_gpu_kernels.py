@@ -1050,6 +1050,45 @@ def test_qk_norm_rope_cache(K, dtype, w_dtype, n_heads, kv_heads, head_dim, rot,
     assert torch.equal(kp2.cpu(), kp) and torch.equal(vp2.cpu(), vp)
 
 
+def test_qk_norm_rope_cache_takes_rows_in_any_order(K):
+    """The kernel for many rows writes whole pieces of eight values only where the eight positions are consecutive rows;
+    rows of two sequences interleaved, a sequence's rows backwards and a gap in the positions land where they belong."""
+    n_heads, kv_heads, head_dim = 8, 2, 128
+    g = torch.Generator().manual_seed(5)
+    # sequence 0: positions 0..39 interleaved with sequence 1's 64..103 backwards; sequence 2: 8..23 then 32..39
+    order = []
+    for t in range(40):
+        order += [(0, t), (1, 103 - t)]
+    order += [(2, p) for p in list(range(8, 24)) + list(range(32, 40))]
+    n_rows = len(order)
+    row_seq = torch.tensor([s for s, _ in order], dtype=torch.int32)
+    positions = torch.tensor([p for _, p in order], dtype=torch.int32)
+    fused = (n_heads + 2 * kv_heads) * head_dim
+    qkv = torch.randn(n_rows, fused, generator=g).to(torch.bfloat16)
+    table = torch.tensor([[4, 5], [7, 2], [1, 8]], dtype=torch.int32)
+    results = []
+    for permuted in (False, True):      # the same rows sorted by (sequence, position): the kernel's pieces of eight
+        index = sorted(range(n_rows), key=lambda r: order[r]) if permuted else list(range(n_rows))
+        kp = torch.full((9, kv_heads, PAGE, head_dim), 768.0).to(torch.bfloat16)
+        vp = torch.full((9, kv_heads, head_dim, PAGE), 768.0).to(torch.bfloat16)
+        kp_d, vp_d = stored(K, kp, vp)
+        q_out = torch.empty(n_rows, n_heads * head_dim, dtype=torch.bfloat16, device="cuda:0")
+        K.qk_norm_rope_cache(dev(qkv[index]), q_out, None, None, 0.0, None, None, dev(positions[index]), dev(row_seq[index]),
+                             kp_d, vp_d, dev(table), n_heads, kv_heads, head_dim, True, 103)
+        back = torch.empty_like(q_out)
+        back[torch.tensor(index, device="cuda:0")] = q_out
+        kp_r, vp_r = as_rows(K, kp_d, vp_d)
+        results.append((back.cpu(), kp_r.cpu(), vp_r.cpu()))
+    for any_order, sorted_rows in zip(*results):
+        assert torch.equal(any_order, sorted_rows)
+    kp_r, vp_r = results[0][1], results[0][2]
+    for row, (seq, pos) in enumerate(order):
+        page = int(table[seq, pos // PAGE])
+        want_v = qkv[row, (n_heads + kv_heads) * head_dim:].reshape(kv_heads, head_dim)
+        assert torch.equal(vp_r[page, :, :, pos % PAGE], want_v)
+        assert torch.equal(kp_r[page, :, pos % PAGE], qkv[row, n_heads * head_dim:(n_heads + kv_heads) * head_dim].reshape(kv_heads, head_dim))
+
+
 @pytest.mark.parametrize("w_dtype", DTYPES)
 @pytest.mark.parametrize("parts", [2, 4, 8])
 @pytest.mark.parametrize("news,pasts", [([70, 5, 1], [0, 62, 130]), ([3, 70, 2], [5, 16, 7]), ([66, 5, 6], [0, 62, 130])])
