@@ -7,8 +7,12 @@ extern "C" {
 // Float-sized words of scratch that bh_sample wants for these rows when every row is greedy (0: none).
 int bh_sample_scratch(int n_rows, int vocab);
 
+// Words of scratch for a draw at a temperature without top-k and top-p (0: none is used).
+int bh_sample_draw_scratch(int n_rows, int vocab);
+
 // One token per row of float32 logits [n_rows, vocab]: argmax where `temperature` is null or <= 0, else
-// a draw (see sampling.hip).  `scratch` (bh_sample_scratch words, or null) is the caller's.
+// a draw (see sampling.hip).  `scratch` (bh_sample_scratch words for greedy rows, bh_sample_draw_scratch words
+// for a draw at a temperature alone, or null) is the caller's.
 int bh_sample(const float* logits, const float* temperature, const int32_t* top_k, const float* top_p,
               const float* uniform, int32_t* tokens, int32_t* bad, void* scratch, int n_rows, int vocab,
               hipStream_t stream);

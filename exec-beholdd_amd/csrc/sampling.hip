@@ -396,6 +396,201 @@ __global__ __launch_bounds__(BH_WAVE) void argmax_rows_kernel(const float* __res
   }
 }
 
+// ---- a draw at a temperature alone, over chunks of the row ---------------------------------------
+// Without top-k and top-p nothing has to be known of the whole row before its weights can be added up, so the row
+// need not stay with one block: a block per (row, chunk of DC tokens) leaves the chunk's largest logit (with its
+// lowest index, or -1 beside a logit that is not finite) and the chunk's weights relative to that logit, summed as
+// integers; a block per row then scales the chunks' sums to the row's largest logit (one float32 factor each, a fixed
+// computation), finds the chunk that holds the target, weighs that chunk's tokens against the row's largest logit
+// and walks them in index order.  The target's place inside the chunk is taken in proportion, the chunk's scaled sum
+// and the sum of its tokens' weights differing by their rounding.  (151,936 logits at a temperature: 48 us with a
+// block per row, which is one compute unit; this way 1 to 64 rows take 12 to 16.)
+
+#define DC 2048   // tokens per chunk
+#define DT 256    // threads per block: eight tokens of a chunk each, token 256 u + thread in turn u
+
+__device__ inline sample_u64 fixed_weight(float logit, float reference, float per_logit) {
+  return (sample_u64)__float2uint_rn(__builtin_amdgcn_exp2f((logit - reference) * per_logit) * 4294967296.f);
+}
+
+// Sum over a block of DT threads, the same in every thread; `scratch` holds DT / 64 words.
+__device__ inline sample_u64 draw_total(sample_u64 v, sample_u64* scratch) {
+#pragma unroll
+  for (int off = BH_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, BH_WAVE);
+  __syncthreads();
+  if (threadIdx.x % BH_WAVE == 0) scratch[threadIdx.x / BH_WAVE] = v;
+  __syncthreads();
+  sample_u64 total = 0;
+  for (int w = 0; w < DT / BH_WAVE; ++w) total += scratch[w];
+  return total;
+}
+
+__global__ __launch_bounds__(DT) void draw_chunk_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
+                                                        uint32_t* __restrict__ records, int vocab, int chunks) {
+  __shared__ float wave_val[DT / BH_WAVE];
+  __shared__ int wave_idx[DT / BH_WAVE];
+  __shared__ sample_u64 scratch[DT / BH_WAVE];
+  const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
+  const float* x = logits + (size_t)row * vocab;
+  float v[DC / DT];
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  bool not_finite = false;
+#pragma unroll
+  for (int u = 0; u < DC / DT; ++u) {
+    const int i = chunk * DC + u * DT + tid;
+    v[u] = i < vocab ? x[i] : -INFINITY;
+    if (i < vocab && !isfinite(v[u])) not_finite = true;
+    if (i < vocab && (v[u] > bv || bi == 0x7fffffff)) bv = v[u], bi = i;   // (a thread's indices rise with u)
+  }
+#pragma unroll
+  for (int off = BH_WAVE / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, BH_WAVE);
+    const int oi = __shfl_xor(bi, off, BH_WAVE);
+    if (ov > bv || (ov == bv && oi < bi)) bv = ov, bi = oi;
+  }
+  const bool any_bad = __syncthreads_or(not_finite);
+  if (tid % BH_WAVE == 0) wave_val[tid / BH_WAVE] = bv, wave_idx[tid / BH_WAVE] = bi;
+  __syncthreads();
+  for (int w = 0; w < DT / BH_WAVE; ++w)
+    if (wave_val[w] > bv || (wave_val[w] == bv && wave_idx[w] < bi)) bv = wave_val[w], bi = wave_idx[w];
+  const float temp = temperature[row];
+  sample_u64 mass = 0;
+  if (!any_bad && temp > 0.f) {
+    const float per_logit = 1.4426950408889634f / temp;
+#pragma unroll
+    for (int u = 0; u < DC / DT; ++u)
+      if (chunk * DC + u * DT + tid < vocab) mass += fixed_weight(v[u], bv, per_logit);
+  }
+  mass = draw_total(mass, scratch);
+  if (tid == 0) {
+    uint32_t* record = records + ((size_t)row * chunks + chunk) * 4;
+    record[0] = __float_as_uint(bv);
+    record[1] = (uint32_t)(any_bad ? -1 : bi);
+    record[2] = (uint32_t)mass;
+    record[3] = (uint32_t)(mass >> 32);
+  }
+}
+
+#define DRAW_MOST_CHUNKS 1024
+__global__ __launch_bounds__(DT) void draw_rows_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
+                                                       const float* __restrict__ uniform, const uint32_t* __restrict__ records,
+                                                       int32_t* __restrict__ tokens, int32_t* __restrict__ bad, int vocab,
+                                                       int chunks) {
+  __shared__ sample_u64 scaled[DRAW_MOST_CHUNKS];
+  __shared__ sample_u64 scratch[DT / BH_WAVE];
+  __shared__ float wave_val[DT / BH_WAVE];
+  __shared__ int wave_idx[DT / BH_WAVE];
+  __shared__ int found_chunk;
+  __shared__ sample_u64 found_before;
+  __shared__ int chosen;
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const uint32_t* mine = records + (size_t)row * chunks * 4;
+  // the row's largest logit with its lowest index; chunks come in index order, so among equals the first chunk's
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  bool any_bad = false;
+  for (int c = tid; c < chunks; c += DT) {
+    const float value = __uint_as_float(mine[4 * c]);
+    const int index = (int)mine[4 * c + 1];
+    if (index < 0) any_bad = true;
+    if (value > bv || bi == 0x7fffffff) bv = value, bi = index;   // (a thread's chunks rise)
+  }
+#pragma unroll
+  for (int off = BH_WAVE / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, BH_WAVE);
+    const int oi = __shfl_xor(bi, off, BH_WAVE);
+    if (ov > bv || (ov == bv && oi < bi)) bv = ov, bi = oi;
+  }
+  any_bad = __syncthreads_or(any_bad);
+  if (tid % BH_WAVE == 0) wave_val[tid / BH_WAVE] = bv, wave_idx[tid / BH_WAVE] = bi;
+  __syncthreads();
+  for (int w = 0; w < DT / BH_WAVE; ++w)
+    if (wave_val[w] > bv || (wave_val[w] == bv && wave_idx[w] < bi)) bv = wave_val[w], bi = wave_idx[w];
+  const float temp = temperature[row];
+  if (any_bad || !(temp > 0.f)) {
+    if (tid == 0) {
+      tokens[row] = any_bad ? -1 : bi;
+      bad[row] = any_bad ? 1 : 0;
+    }
+    return;
+  }
+  const float per_logit = 1.4426950408889634f / temp;
+  sample_u64 sum = 0;
+  for (int c = tid; c < chunks; c += DT) {
+    const sample_u64 mass = (sample_u64)mine[4 * c + 2] | ((sample_u64)mine[4 * c + 3] << 32);
+    const float factor = __builtin_amdgcn_exp2f((__uint_as_float(mine[4 * c]) - bv) * per_logit);   // 1 for the chunk of the largest logit
+    const sample_u64 part = (sample_u64)__double2ull_rd((double)mass * (double)factor);
+    scaled[c] = part;
+    sum += part;
+  }
+  const sample_u64 kept = draw_total(sum, scratch);   // (its barriers also put `scaled` in place)
+  sample_u64 target = (sample_u64)__double2ull_rd((double)uniform[row] * (double)kept);
+  if (target >= kept) target = kept - 1;
+  if (tid == 0) {
+    int c = 0;
+    sample_u64 before = 0;
+    for (; c < chunks - 1 && before + scaled[c] <= target; ++c) before += scaled[c];
+    found_chunk = c;
+    found_before = before;
+    chosen = bi;
+  }
+  __syncthreads();
+  const int chunk = found_chunk;
+  const float* x = logits + (size_t)row * vocab;
+  sample_u64 w[DC / DT], of_chunk = 0;
+#pragma unroll
+  for (int u = 0; u < DC / DT; ++u) {
+    const int i = chunk * DC + u * DT + tid;
+    w[u] = i < vocab ? fixed_weight(x[i], bv, per_logit) : 0;
+    of_chunk += w[u];
+  }
+  of_chunk = draw_total(of_chunk, scratch);
+  if (of_chunk == 0) {   // every token of the chunk rounds to nothing against the row's largest: the chunk's own largest
+    if (tid == 0) tokens[row] = (int)mine[4 * chunk + 1], bad[row] = 0;
+    return;
+  }
+  // the target's place inside the chunk, in the units of its tokens' weights
+  const sample_u64 inside = target - found_before, of_scaled = scaled[chunk];
+  sample_u64 local = (sample_u64)__double2ull_rd((double)inside * ((double)of_chunk / (double)of_scaled));
+  if (local >= of_chunk) local = of_chunk - 1;
+  sample_u64 before = 0;
+  int turn = 0;
+  sample_u64 of_turn[DC / DT];
+#pragma unroll
+  for (int u = 0; u < DC / DT; ++u) of_turn[u] = draw_total(w[u], scratch);
+  for (; turn < DC / DT - 1 && before + of_turn[turn] <= local; ++turn) before += of_turn[turn];
+  sample_u64 own = 0;
+#pragma unroll
+  for (int u = 0; u < DC / DT; ++u)
+    if (u == turn) own = w[u];
+  // the weights of the turn's tokens before this thread's
+  const int lane = tid % BH_WAVE, wave = tid / BH_WAVE;
+  sample_u64 through = own;
+#pragma unroll
+  for (int off = 1; off < BH_WAVE; off <<= 1) {
+    const sample_u64 other = __shfl_up(through, off, BH_WAVE);
+    if (lane >= off) through += other;
+  }
+  __syncthreads();
+  if (lane == BH_WAVE - 1) scratch[wave] = through;
+  __syncthreads();
+  for (int v = 0; v < wave; ++v) before += scratch[v];
+  if (own > 0 && before + through - own <= local && local < before + through) chosen = chunk * DC + turn * DT + tid;
+  __syncthreads();
+  if (tid == 0) {
+    tokens[row] = chosen;
+    bad[row] = 0;
+  }
+}
+
+// Words of scratch for a draw at a temperature alone over these rows (0: the rows are drawn by a block each).
+extern "C" int bh_sample_draw_scratch(int n_rows, int vocab) {
+  const int chunks = (vocab + DC - 1) / DC;
+  if (n_rows <= 0 || n_rows > 65535 || vocab < 4 * DC || chunks > DRAW_MOST_CHUNKS) return 0;
+  return 4 * n_rows * chunks;
+}
+
 // Float-sized words of scratch that bh_sample wants for these rows when every row is greedy (0: none).
 extern "C" int bh_sample_scratch(int n_rows, int vocab) {
   if (n_rows <= 0 || vocab < 4 * AC || n_rows >= 128) return 0;   // enough rows fill the compute units by themselves
@@ -419,6 +614,14 @@ extern "C" int bh_sample(const float* logits, const float* temperature, const in
   }
   BH_REQUIRE(temperature == nullptr || vocab <= SAMPLE_BINS * 256 * (SB / BH_WAVE),
              "sample: a draw takes vocabularies of up to %d tokens, not %d", SAMPLE_BINS * 256 * (SB / BH_WAVE), vocab);
+  if (temperature != nullptr && top_k == nullptr && top_p == nullptr && scratch != nullptr && bh_sample_draw_scratch(n_rows, vocab) > 0) {
+    const int chunks = (vocab + DC - 1) / DC;
+    draw_chunk_kernel<<<dim3(chunks, n_rows), dim3(DT), 0, stream>>>(logits, temperature, (uint32_t*)scratch, vocab, chunks);
+    if (int status = bh_check_launch("draw_chunk")) return status;
+    draw_rows_kernel<<<dim3(n_rows), dim3(DT), 0, stream>>>(logits, temperature, uniform, (const uint32_t*)scratch, tokens, bad,
+                                                            vocab, chunks);
+    return bh_check_launch("draw_rows");
+  }
   sample_kernel<<<dim3(n_rows), dim3(SB), 0, stream>>>(logits, temperature, top_k, top_p, uniform, tokens, bad,
                                                        vocab);
   return bh_check_launch("sample");

@@ -147,6 +147,7 @@ class KernelSizes:
             "bh_swiglu": [p, p, i, i, i, p],
             "bh_sample": [p, p, p, p, p, p, p, p, i, i, p],
             "bh_sample_scratch": [i, i],
+            "bh_sample_draw_scratch": [i, i],
             "bh_gemm_bf16": [p, p, p, i, i, i, i, i, i, i, p, i, f, p, i, p, p, p, i, i, i, p],
             "bh_gemm_bf16_turns": [p, p, p, i, i, i, i, i, i, i, i, i, p],
             "bh_gemm_bf16_then_norm": [p, p, p, i, i, i, i, p, i, f, p, p, i, i, p],
@@ -210,7 +211,9 @@ class KernelSizes:
         return _rounded(n_rows * n_heads * n_splits * head_dim * 4) + _rounded(n_rows * n_heads * n_splits * 2 * 4)
 
     def sample_working_bytes(self, n_rows, vocab) -> int:
-        return _rounded(int(self.lib.bh_sample_scratch(int(n_rows), int(vocab))) * 4) + 4 * _rounded(n_rows * 4)
+        words = max(int(self.lib.bh_sample_scratch(int(n_rows), int(vocab))),
+                    int(self.lib.bh_sample_draw_scratch(int(n_rows), int(vocab))))
+        return _rounded(words * 4) + 4 * _rounded(n_rows * 4)
 
     def packs(self, rows, cols, act_size) -> bool:
         """Whether `pack_weight` regroups a matrix of this shape and element size."""
@@ -764,6 +767,10 @@ class HipKernels(KernelSizes):
         scratch = None
         if temperature is None:      # greedy rows of a long vocabulary are searched chunk by chunk
             words = int(self.lib.bh_sample_scratch(n_rows, vocab))
+            if words:
+                scratch = torch.empty(words, dtype=torch.float32, device=self.device)
+        elif top_k is None and top_p is None:      # a draw from the whole distribution likewise
+            words = int(self.lib.bh_sample_draw_scratch(n_rows, vocab))
             if words:
                 scratch = torch.empty(words, dtype=torch.float32, device=self.device)
         self._check(self.lib.bh_sample(

@@ -193,6 +193,53 @@ def test_the_draws_thresholds_on_rows_made_to_trip_them(K, twins):
     assert alone and all(int(got[i]) == int(np.argmax(logits[i])) for i in alone)
 
 
+def test_a_draw_from_the_whole_distribution_goes_chunk_by_chunk_and_keeps_index_order(K, twins):
+    """A draw at a temperature without top-k and top-p is spread over chunks of the row.  Rows made so that a fault of
+    that shows: three tokens in three different chunks (one in the ragged last chunk) hold all of the weight, 0.5, 0.3
+    and 0.2 of it, and uniform numbers step through [0, 1): the token follows the cumulative weights in index order.
+    Then shapes against the plain twin: all logits equal, one chunk far above the others, a very low temperature, a
+    greedy row among drawn ones, and a logit that is not finite in a chunk that is not the first."""
+    vocab = 4 * 2048 + 808
+    assert K.lib.bh_sample_draw_scratch(4, vocab) > 0
+    places, shares = [700, 2048 + 1999, 4 * 2048 + 807], [0.5, 0.3, 0.2]
+    steps = 200
+    logits = np.full((steps, vocab), -1e4, np.float32)
+    for place, share in zip(places, shares):
+        logits[:, place] = np.log(share)
+    uniform = ((np.arange(steps) + 0.5) / steps).astype(np.float32)
+    temperature = np.ones(steps, np.float32)
+    tokens, bad = torch.empty(steps, dtype=torch.int32, device=DEVICE), torch.empty(steps, dtype=torch.int32, device=DEVICE)
+    K.sample(dev(logits), tokens, bad, temperature=dev(temperature), uniform=dev(uniform))
+    want = [places[0] if u < 0.5 else places[1] if u < 0.8 else places[2] for u in uniform]
+    assert tokens.cpu().tolist() == want and bad.cpu().tolist() == [0] * steps
+
+    rng = np.random.default_rng(23)
+    lifted = (rng.normal(size=vocab) * 2).astype(np.float32)
+    lifted[3 * 2048:4 * 2048] += 30.0
+    shapes = [np.full(vocab, -3.5, np.float32), lifted, (rng.normal(size=vocab) * 3).astype(np.float32),
+              (rng.normal(size=vocab) * 1e-3).astype(np.float32), (rng.normal(size=vocab) * 40).astype(np.float32)]
+    logits = np.stack([shape for shape in shapes for _ in range(12)])
+    rows = logits.shape[0]
+    temperature = rng.choice([0.01, 0.3, 1.0, 2.5], size=rows).astype(np.float32)
+    temperature[7] = 0.0
+    for seed in range(3):
+        uniform = np.random.default_rng(seed).random(rows).astype(np.float32)
+        tokens, bad = torch.empty(rows, dtype=torch.int32, device=DEVICE), torch.empty(rows, dtype=torch.int32, device=DEVICE)
+        K.sample(dev(logits), tokens, bad, temperature=dev(temperature), uniform=dev(uniform))
+        want, want_bad, margin = twins.sample(logits, temperature, uniform)
+        got = tokens.cpu().numpy()
+        assert bad.cpu().tolist() == want_bad.tolist() == [0] * rows
+        sure = margin > 1e-5
+        assert sure.sum() > 0.8 * rows and np.array_equal(got[sure], want[sure]), (got[sure & (got != want)], want[sure & (got != want)])
+        assert int(got[7]) == int(np.argmax(logits[7]))
+    spoiled = logits.copy()
+    spoiled[3, 2 * 2048 + 5] = np.nan
+    spoiled[4, vocab - 1] = np.inf
+    K.sample(dev(spoiled), tokens, bad, temperature=dev(temperature), uniform=dev(uniform))
+    assert bad.cpu().tolist() == [int(i in (3, 4)) for i in range(rows)]
+    assert tokens.cpu().tolist()[3:5] == [-1, -1] and np.array_equal(tokens.cpu().numpy()[5:], got[5:])
+
+
 @pytest.mark.parametrize("vocab", [50, 1000, 4133, 151936])
 def test_the_draw_and_its_twin(K, twins, vocab):
     """Temperature, top-k and top-p draws of the kernel against the plain twin's, row by row: the same token wherever the
