@@ -10,9 +10,12 @@ int bh_sample_scratch(int n_rows, int vocab);
 // Words of scratch for a draw at a temperature without top-k and top-p (0: none is used).
 int bh_sample_draw_scratch(int n_rows, int vocab);
 
+// Words of scratch for draws with a top-k (0: none is used).
+int bh_sample_top_k_scratch(int n_rows, int vocab);
+
 // One token per row of float32 logits [n_rows, vocab]: argmax where `temperature` is null or <= 0, else
 // a draw (see sampling.hip).  `scratch` (bh_sample_scratch words for greedy rows, bh_sample_draw_scratch words
-// for a draw at a temperature alone, or null) is the caller's.
+// for a draw at a temperature alone, bh_sample_top_k_scratch words for draws with a top-k, or null) is the caller's.
 int bh_sample(const float* logits, const float* temperature, const int32_t* top_k, const float* top_p,
               const float* uniform, int32_t* tokens, int32_t* bad, void* scratch, int n_rows, int vocab,
               hipStream_t stream);

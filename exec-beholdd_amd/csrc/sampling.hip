@@ -143,62 +143,27 @@ __device__ inline uint32_t threshold_key(const float* __restrict__ x, int vocab,
   return prefix;
 }
 
-__global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ logits,
-                                                    const float* __restrict__ temperature,
-                                                    const int32_t* __restrict__ top_k,
-                                                    const float* __restrict__ top_p,
-                                                    const float* __restrict__ uniform,
-                                                    int32_t* __restrict__ tokens, int32_t* __restrict__ bad,
-                                                    int vocab) {
-  __shared__ sample_u64 bins[SAMPLE_BINS];
-  __shared__ sample_u64 scratch[SB / BH_WAVE];
-  __shared__ float wave_val[SB / BH_WAVE];
-  __shared__ int wave_idx[SB / BH_WAVE];
-  __shared__ int wave_bad[SB / BH_WAVE];
-  __shared__ uint32_t found_bin;
-  __shared__ sample_u64 found_above;
-  __shared__ int chosen;
+// What a block that selects for a row keeps in LDS.
+struct SampleShared {
+  sample_u64 bins[SAMPLE_BINS];
+  sample_u64 scratch[SB / BH_WAVE];
+  float wave_val[SB / BH_WAVE];
+  int wave_idx[SB / BH_WAVE];
+  int wave_bad[SB / BH_WAVE];
+  uint32_t found_bin;
+  sample_u64 found_above;
+  int chosen;
+};
 
-  const int row = blockIdx.x, tid = threadIdx.x;
-  const float* x = logits + (size_t)row * vocab;
-
-  // the maximum with lowest-index ties, and the finiteness check
-  float bv = -INFINITY;
-  int bi = 0x7fffffff, not_finite = 0;
-  over_the_row(x, vocab, [&](int i, float v) {
-    if (!isfinite(v)) not_finite = 1;
-    if (v > bv || (v == bv && i < bi) || bi == 0x7fffffff) bv = v, bi = i;
-  });
-#pragma unroll
-  for (int off = BH_WAVE / 2; off > 0; off >>= 1) {
-    const float ov = __shfl_xor(bv, off, BH_WAVE);
-    const int oi = __shfl_xor(bi, off, BH_WAVE);
-    not_finite |= __shfl_xor(not_finite, off, BH_WAVE);
-    if (ov > bv || (ov == bv && oi < bi)) bv = ov, bi = oi;
-  }
-  if (tid % BH_WAVE == 0) wave_val[tid / BH_WAVE] = bv, wave_idx[tid / BH_WAVE] = bi, wave_bad[tid / BH_WAVE] = not_finite;
-  __syncthreads();
-  for (int w = 0; w < SB / BH_WAVE; ++w) {
-    not_finite |= wave_bad[w];
-    if (wave_val[w] > bv || (wave_val[w] == bv && wave_idx[w] < bi)) bv = wave_val[w], bi = wave_idx[w];
-  }
-  if (not_finite) {
-    if (tid == 0) {
-      tokens[row] = -1;
-      bad[row] = 1;
-    }
-    return;
-  }
-  const float max_logit = bv;
-  const int arg_max = bi;
-  const float temp = temperature ? temperature[row] : 0.f;
-  if (!(temp > 0.f)) {
-    if (tid == 0) {
-      tokens[row] = arg_max;
-      bad[row] = 0;
-    }
-    return;
-  }
+// The draw from x[0..vocab) at a temperature above zero, the largest logit and its place known: the filters, then
+// the inverse-CDF draw over the kept tokens in index order; thread 0 leaves the token.  `ids` (or null): the token
+// that each element of x stands for, when x is a row's candidates and not the row itself.
+__device__ inline void draw_from(const float* __restrict__ x, int vocab, const int32_t* __restrict__ ids, float max_logit,
+                                 int arg_max, float temp, int k, float p_keep, float uniform_number, int32_t* token,
+                                 SampleShared& sh) {
+  sample_u64* bins = sh.bins;
+  sample_u64* scratch = sh.scratch;
+  const int tid = threadIdx.x;
   // exp((v - max) / temperature) as 2^((v - max) * log2(e) / temperature): one multiplication and the hardware's
   // exponential; times 2^32 and rounded (the conversion stops at 2^32 - 1, which the largest token gets)
   const float per_logit = 1.4426950408889634f / temp;
@@ -208,13 +173,11 @@ __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ lo
 
   // top-k: the k-th largest logit's key; tokens with key >= floor_key are kept (ties at the k-th are)
   uint32_t floor_key = 0;
-  const int k = top_k ? top_k[row] : 0;
   if (k > 0 && k < vocab)
-    floor_key = threshold_key(x, vocab, 0u, (sample_u64)k, bins, scratch, &found_bin, &found_above,
+    floor_key = threshold_key(x, vocab, 0u, (sample_u64)k, bins, scratch, &sh.found_bin, &sh.found_above,
                               [](float) -> sample_u64 { return 1; });
 
   // top-p: the largest key whose tokens, with all above them, weigh top_p of what top-k has left
-  const float p_keep = top_p ? top_p[row] : 1.f;
   if (p_keep > 0.f && p_keep < 1.f) {
     sample_u64 total = 0;
     over_the_row(x, vocab, [&](int, float v) {
@@ -224,7 +187,7 @@ __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ lo
     sample_u64 need = (sample_u64)__double2ull_rn((double)p_keep * (double)total);
     if (need < 1) need = 1;
     if (need > total) need = total;
-    const uint32_t key = threshold_key(x, vocab, floor_key, need, bins, scratch, &found_bin, &found_above, weight_of);
+    const uint32_t key = threshold_key(x, vocab, floor_key, need, bins, scratch, &sh.found_bin, &sh.found_above, weight_of);
     if (key > floor_key) floor_key = key;
   }
 
@@ -269,12 +232,12 @@ __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ lo
     mine = wave_total(mine);
     __syncthreads();
     if (lane == 0) scratch[wave] = mine;
-    if (tid == 0) chosen = arg_max;
+    if (tid == 0) sh.chosen = arg_max;
     __syncthreads();
   }
   sample_u64 kept = 0;
   for (int w = 0; w < WAVES; ++w) kept += scratch[w];
-  sample_u64 target = (sample_u64)__double2ull_rd((double)uniform[row] * (double)kept);
+  sample_u64 target = (sample_u64)__double2ull_rd((double)uniform_number * (double)kept);
   if (target >= kept) target = kept - 1;   // (uniform is below 1; the largest token alone weighs 2^32 - 1)
   int span = 0;
   sample_u64 before = 0;   // the kept weight of the spans before the target's
@@ -309,13 +272,56 @@ __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ lo
     }
     // the first lane whose token carries the sum beyond the target
     const unsigned long long beyond = __ballot(own > 0 && before + through > target);
-    if (beyond != 0 && lane == __ffsll((long long)beyond) - 1) chosen = base + BH_WAVE * u + lane;
+    if (beyond != 0 && lane == __ffsll((long long)beyond) - 1) {
+      const int place = base + BH_WAVE * u + lane;
+      sh.chosen = ids ? ids[place] : place;
+    }
   }
   __syncthreads();
-  if (tid == 0) {
-    tokens[row] = chosen;
-    bad[row] = 0;
+  if (tid == 0) *token = sh.chosen;
+}
+
+__global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ logits,
+                                                    const float* __restrict__ temperature,
+                                                    const int32_t* __restrict__ top_k,
+                                                    const float* __restrict__ top_p,
+                                                    const float* __restrict__ uniform,
+                                                    int32_t* __restrict__ tokens, int32_t* __restrict__ bad,
+                                                    int vocab) {
+  __shared__ SampleShared sh;
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const float* x = logits + (size_t)row * vocab;
+
+  // the maximum with lowest-index ties, and the finiteness check
+  float bv = -INFINITY;
+  int bi = 0x7fffffff, not_finite = 0;
+  over_the_row(x, vocab, [&](int i, float v) {
+    if (!isfinite(v)) not_finite = 1;
+    if (v > bv || (v == bv && i < bi) || bi == 0x7fffffff) bv = v, bi = i;
+  });
+#pragma unroll
+  for (int off = BH_WAVE / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, BH_WAVE);
+    const int oi = __shfl_xor(bi, off, BH_WAVE);
+    not_finite |= __shfl_xor(not_finite, off, BH_WAVE);
+    if (ov > bv || (ov == bv && oi < bi)) bv = ov, bi = oi;
   }
+  if (tid % BH_WAVE == 0) sh.wave_val[tid / BH_WAVE] = bv, sh.wave_idx[tid / BH_WAVE] = bi, sh.wave_bad[tid / BH_WAVE] = not_finite;
+  __syncthreads();
+  for (int w = 0; w < SB / BH_WAVE; ++w) {
+    not_finite |= sh.wave_bad[w];
+    if (sh.wave_val[w] > bv || (sh.wave_val[w] == bv && sh.wave_idx[w] < bi)) bv = sh.wave_val[w], bi = sh.wave_idx[w];
+  }
+  const float temp = temperature ? temperature[row] : 0.f;
+  if (not_finite || !(temp > 0.f)) {
+    if (tid == 0) {
+      tokens[row] = not_finite ? -1 : bi;
+      bad[row] = not_finite ? 1 : 0;
+    }
+    return;
+  }
+  if (tid == 0) bad[row] = 0;
+  draw_from(x, vocab, nullptr, bv, bi, temp, top_k ? top_k[row] : 0, top_p ? top_p[row] : 1.f, uniform[row], tokens + row, sh);
 }
 
 // ---- argmax of long rows in two steps ---------------------------------------------------------
@@ -591,6 +597,203 @@ extern "C" int bh_sample_draw_scratch(int n_rows, int vocab) {
   return 4 * n_rows * chunks;
 }
 
+// ---- a draw among the top k, from the candidates of the row's chunks ------------------------------
+// Each of the k largest logits of a row is among the k largest of its chunk.  So a block per (row, chunk of DC tokens)
+// leaves the chunk's largest logit and, in index order, every token of the chunk that is not below the chunk's k-th
+// largest (ties kept; `used` places per chunk, filled up with minus infinity, which weighs nothing and lies below
+// every threshold); the block of the row then does on these few thousand candidates exactly what it would do on the
+// row: the k-th largest's key, top-p's threshold among what top-k leaves, the draw in index order.  The tokens kept
+// are the same as over the whole row, and so are their integer weights, the target and the token drawn.  A row
+// whose k is off or above CANDIDATES_UP_TO_K, or one of whose chunks has more ties at its threshold than fit, is
+// drawn from the whole row as before, by the same block (only the search for the largest logit is saved).
+// 151,936 logits, top-k of 50: 86 -> 29 us for one row, 33 for eight, 94 -> 61 for 64; with top-p of 0.9 as well 128 -> 39, 42, 143 -> 70.
+
+#define CANDIDATES_UP_TO_K 128
+#define CANDIDATE_PLACES 144   // per chunk at most; used(k) = k + 8 rounded up to 16
+
+__host__ __device__ inline int candidate_places(int k) { return (k + 8 + 15) / 16 * 16; }
+
+__global__ __launch_bounds__(DT) void candidates_chunk_kernel(const float* __restrict__ logits, const int32_t* __restrict__ top_k,
+                                                              uint32_t* __restrict__ headers, float* __restrict__ values,
+                                                              int32_t* __restrict__ ids, int vocab, int chunks) {
+  __shared__ float wave_val[DT / BH_WAVE];
+  __shared__ int wave_idx[DT / BH_WAVE];
+  __shared__ uint32_t counts[256];
+  __shared__ uint32_t found_digit, found_above;
+  __shared__ int wave_kept[DT / BH_WAVE];
+  constexpr int PER = DC / DT;   // a thread's tokens: PER neighbours, so that the threads' order is the index order
+  const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x, lane = tid % BH_WAVE, wave = tid / BH_WAVE;
+  const float* x = logits + (size_t)row * vocab;
+  const int first = chunk * DC + PER * tid;
+  float v[PER];
+  uint32_t key[PER];
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  bool not_finite = false;
+#pragma unroll
+  for (int u = 0; u < PER; ++u) v[u] = first + u < vocab ? x[first + u] : -INFINITY;
+#pragma unroll
+  for (int u = 0; u < PER; ++u) {
+    const bool there = first + u < vocab;
+    if (there && !isfinite(v[u])) not_finite = true;
+    if (there && (v[u] > bv || bi == 0x7fffffff)) bv = v[u], bi = first + u;
+    key[u] = there ? order_key(v[u]) : 0u;   // (no float has the key 0)
+  }
+#pragma unroll
+  for (int off = BH_WAVE / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, BH_WAVE);
+    const int oi = __shfl_xor(bi, off, BH_WAVE);
+    if (ov > bv || (ov == bv && oi < bi)) bv = ov, bi = oi;
+  }
+  const bool any_bad = __syncthreads_or(not_finite);
+  if (lane == 0) wave_val[wave] = bv, wave_idx[wave] = bi;
+  __syncthreads();
+  for (int w = 0; w < DT / BH_WAVE; ++w)
+    if (wave_val[w] > bv || (wave_val[w] == bv && wave_idx[w] < bi)) bv = wave_val[w], bi = wave_idx[w];
+  uint32_t* header = headers + ((size_t)row * chunks + chunk) * 4;
+  const int k = top_k[row];
+  if (any_bad || k <= 0 || k > CANDIDATES_UP_TO_K || k >= vocab) {   // (the same for all of the row's chunks)
+    if (tid == 0) {
+      header[0] = __float_as_uint(bv);
+      header[1] = (uint32_t)(any_bad ? -1 : bi);
+      header[2] = (uint32_t)-1;   // no candidates
+    }
+    return;
+  }
+  // the key of the chunk's k-th largest logit, digit by digit from the top (all of a chunk that has no more than k)
+  const int here = min(DC, vocab - chunk * DC);
+  uint32_t floor_key = 0;
+  if (here > k) {
+    uint32_t need = (uint32_t)k;
+#pragma unroll 1
+    for (int shift = 24; shift >= 0; shift -= 8) {
+      counts[tid] = 0;   // (DT == 256 bins)
+      __syncthreads();
+#pragma unroll
+      for (int u = 0; u < PER; ++u)
+        if (key[u] != 0u && (shift == 24 || (key[u] >> (shift + 8)) == (floor_key >> (shift + 8))))
+          atomicAdd(&counts[(key[u] >> shift) & 255u], 1u);
+      __syncthreads();
+      if (wave == 0) {   // lane l has the bins 255 - 4 l .. 252 - 4 l, the highest first
+        uint32_t mine[4], sum = 0;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) mine[u] = counts[255 - (4 * lane + u)], sum += mine[u];
+        uint32_t through = sum;
+#pragma unroll
+        for (int off = 1; off < BH_WAVE; off <<= 1) {
+          const uint32_t other = __shfl_up(through, off, BH_WAVE);
+          if (lane >= off) through += other;
+        }
+        uint32_t above = through - sum;
+        if (above < need && above + sum >= need) {
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            if (above < need && above + mine[u] >= need) found_digit = 255u - (4 * lane + u), found_above = above;
+            above += mine[u];
+          }
+        }
+      }
+      __syncthreads();
+      floor_key |= found_digit << shift;
+      need -= found_above;
+      __syncthreads();
+    }
+  }
+  // the kept tokens' places among the chunk's candidates, in index order
+  int mine = 0;
+#pragma unroll
+  for (int u = 0; u < PER; ++u) mine += key[u] != 0u && key[u] >= floor_key;
+  int through = mine;
+#pragma unroll
+  for (int off = 1; off < BH_WAVE; off <<= 1) {
+    const int other = __shfl_up(through, off, BH_WAVE);
+    if (lane >= off) through += other;
+  }
+  if (lane == BH_WAVE - 1) wave_kept[wave] = through;
+  __syncthreads();
+  int before = through - mine, kept = 0;
+  for (int w = 0; w < DT / BH_WAVE; ++w) {
+    if (w < wave) before += wave_kept[w];
+    kept += wave_kept[w];
+  }
+  const int places = candidate_places(k);
+  if (tid == 0) {
+    header[0] = __float_as_uint(bv);
+    header[1] = (uint32_t)bi;
+    header[2] = (uint32_t)(kept <= places ? kept : -1);   // more ties than places: the row is drawn whole
+  }
+  if (kept > places) return;
+  const size_t base = (size_t)row * chunks * CANDIDATE_PLACES + (size_t)chunk * places;
+#pragma unroll
+  for (int u = 0; u < PER; ++u)
+    if (key[u] != 0u && key[u] >= floor_key) {
+      values[base + before] = v[u];
+      ids[base + before] = first + u;
+      ++before;
+    }
+  for (int j = kept + tid; j < places; j += DT) values[base + j] = -INFINITY, ids[base + j] = 0;
+}
+
+__global__ __launch_bounds__(SB) void sample_candidates_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
+                                                               const int32_t* __restrict__ top_k, const float* __restrict__ top_p,
+                                                               const float* __restrict__ uniform, const uint32_t* __restrict__ headers,
+                                                               const float* __restrict__ values, const int32_t* __restrict__ ids,
+                                                               int32_t* __restrict__ tokens, int32_t* __restrict__ bad, int vocab,
+                                                               int chunks) {
+  __shared__ SampleShared sh;
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const uint32_t* mine = headers + (size_t)row * chunks * 4;
+  // the row's largest logit with its lowest index (chunks are in index order), from the chunks' own
+  float bv = -INFINITY;
+  int bi = 0x7fffffff, not_finite = 0, whole = 0;
+  for (int c = tid; c < chunks; c += SB) {
+    const float value = __uint_as_float(mine[4 * c]);
+    const int index = (int)mine[4 * c + 1];
+    if (index < 0) not_finite = 1;
+    if ((int)mine[4 * c + 2] < 0) whole = 1;
+    if (value > bv || bi == 0x7fffffff) bv = value, bi = index;
+  }
+#pragma unroll
+  for (int off = BH_WAVE / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, BH_WAVE);
+    const int oi = __shfl_xor(bi, off, BH_WAVE);
+    not_finite |= __shfl_xor(not_finite, off, BH_WAVE);
+    whole |= __shfl_xor(whole, off, BH_WAVE);
+    if (ov > bv || (ov == bv && oi < bi)) bv = ov, bi = oi;
+  }
+  if (tid % BH_WAVE == 0) sh.wave_val[tid / BH_WAVE] = bv, sh.wave_idx[tid / BH_WAVE] = bi, sh.wave_bad[tid / BH_WAVE] = not_finite | (whole << 1);
+  __syncthreads();
+  for (int w = 0; w < SB / BH_WAVE; ++w) {
+    not_finite |= sh.wave_bad[w] & 1;
+    whole |= sh.wave_bad[w] >> 1;
+    if (sh.wave_val[w] > bv || (sh.wave_val[w] == bv && sh.wave_idx[w] < bi)) bv = sh.wave_val[w], bi = sh.wave_idx[w];
+  }
+  const float temp = temperature[row];
+  if (not_finite || !(temp > 0.f)) {
+    if (tid == 0) {
+      tokens[row] = not_finite ? -1 : bi;
+      bad[row] = not_finite ? 1 : 0;
+    }
+    return;
+  }
+  if (tid == 0) bad[row] = 0;
+  const int k = top_k[row];
+  const float p_keep = top_p ? top_p[row] : 1.f;
+  if (whole)
+    draw_from(logits + (size_t)row * vocab, vocab, nullptr, bv, bi, temp, k, p_keep, uniform[row], tokens + row, sh);
+  else
+    draw_from(values + (size_t)row * chunks * CANDIDATE_PLACES, chunks * candidate_places(k),
+              ids + (size_t)row * chunks * CANDIDATE_PLACES, bv, bi, temp, k, p_keep, uniform[row], tokens + row, sh);
+}
+
+// Words of scratch for draws with a top-k over these rows (0: the rows are drawn by a block each from the whole row).
+extern "C" int bh_sample_top_k_scratch(int n_rows, int vocab) {
+  const long chunks = (vocab + DC - 1) / DC;
+  const long words = (long)n_rows * chunks * (4 + 2 * CANDIDATE_PLACES);
+  if (n_rows <= 0 || n_rows > 65535 || vocab < 4 * DC || chunks > SB || words >= (1L << 31)) return 0;
+  return (int)words;
+}
+
 // Float-sized words of scratch that bh_sample wants for these rows when every row is greedy (0: none).
 extern "C" int bh_sample_scratch(int n_rows, int vocab) {
   if (n_rows <= 0 || vocab < 4 * AC || n_rows >= 128) return 0;   // enough rows fill the compute units by themselves
@@ -621,6 +824,17 @@ extern "C" int bh_sample(const float* logits, const float* temperature, const in
     draw_rows_kernel<<<dim3(n_rows), dim3(DT), 0, stream>>>(logits, temperature, uniform, (const uint32_t*)scratch, tokens, bad,
                                                             vocab, chunks);
     return bh_check_launch("draw_rows");
+  }
+  if (temperature != nullptr && top_k != nullptr && scratch != nullptr && bh_sample_top_k_scratch(n_rows, vocab) > 0) {
+    const int chunks = (vocab + DC - 1) / DC;
+    uint32_t* headers = (uint32_t*)scratch;
+    float* values = (float*)scratch + (size_t)n_rows * chunks * 4;
+    int32_t* ids = (int32_t*)values + (size_t)n_rows * chunks * CANDIDATE_PLACES;
+    candidates_chunk_kernel<<<dim3(chunks, n_rows), dim3(DT), 0, stream>>>(logits, top_k, headers, values, ids, vocab, chunks);
+    if (int status = bh_check_launch("candidates_chunk")) return status;
+    sample_candidates_kernel<<<dim3(n_rows), dim3(SB), 0, stream>>>(logits, temperature, top_k, top_p, uniform, headers, values,
+                                                                    ids, tokens, bad, vocab, chunks);
+    return bh_check_launch("sample_candidates");
   }
   sample_kernel<<<dim3(n_rows), dim3(SB), 0, stream>>>(logits, temperature, top_k, top_p, uniform, tokens, bad,
                                                        vocab);

@@ -148,6 +148,7 @@ class KernelSizes:
             "bh_sample": [p, p, p, p, p, p, p, p, i, i, p],
             "bh_sample_scratch": [i, i],
             "bh_sample_draw_scratch": [i, i],
+            "bh_sample_top_k_scratch": [i, i],
             "bh_gemm_bf16": [p, p, p, i, i, i, i, i, i, i, p, i, f, p, i, p, p, p, i, i, i, p],
             "bh_gemm_bf16_turns": [p, p, p, i, i, i, i, i, i, i, i, i, p],
             "bh_gemm_bf16_then_norm": [p, p, p, i, i, i, i, p, i, f, p, p, i, i, p],
@@ -212,7 +213,8 @@ class KernelSizes:
 
     def sample_working_bytes(self, n_rows, vocab) -> int:
         words = max(int(self.lib.bh_sample_scratch(int(n_rows), int(vocab))),
-                    int(self.lib.bh_sample_draw_scratch(int(n_rows), int(vocab))))
+                    int(self.lib.bh_sample_draw_scratch(int(n_rows), int(vocab))),
+                    int(self.lib.bh_sample_top_k_scratch(int(n_rows), int(vocab))))
         return _rounded(words * 4) + 4 * _rounded(n_rows * 4)
 
     def packs(self, rows, cols, act_size) -> bool:
@@ -771,6 +773,10 @@ class HipKernels(KernelSizes):
                 scratch = torch.empty(words, dtype=torch.float32, device=self.device)
         elif top_k is None and top_p is None:      # a draw from the whole distribution likewise
             words = int(self.lib.bh_sample_draw_scratch(n_rows, vocab))
+            if words:
+                scratch = torch.empty(words, dtype=torch.float32, device=self.device)
+        elif top_k is not None:                    # and the chunks' candidates for the top k
+            words = int(self.lib.bh_sample_top_k_scratch(n_rows, vocab))
             if words:
                 scratch = torch.empty(words, dtype=torch.float32, device=self.device)
         self._check(self.lib.bh_sample(

@@ -157,11 +157,13 @@ class Sampler:
             else:
                 on_device.copy_(numbers)
                 counts_on_device.copy_(counts)
-            # rows that all draw from the whole distribution say so: their draw is spread over the chip
-            unfiltered = all(p.top_k == 0 and p.top_p == 1.0 for p in params)
+            # a filter that no row uses is left out: the kernels then spread the rows' work over the chip where they can
+            # (a draw from the whole distribution over chunks of the row, a top-k through the chunks' candidates)
+            any_k = any(p.top_k > 0 for p in params)
+            any_p = any(p.top_p < 1.0 for p in params)
             self.kernels.sample(logits, tokens, bad, temperature=on_device[0, :n_rows],
-                                top_k=None if unfiltered else counts_on_device[:n_rows],
-                                top_p=None if unfiltered else on_device[1, :n_rows], uniform=on_device[2, :n_rows])
+                                top_k=counts_on_device[:n_rows] if any_k else None,
+                                top_p=on_device[1, :n_rows] if any_p else None, uniform=on_device[2, :n_rows])
         host = self._hosts[self._turn]
         self._turn = (self._turn + 1) % self.RING
         event = None

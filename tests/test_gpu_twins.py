@@ -240,6 +240,53 @@ def test_a_draw_from_the_whole_distribution_goes_chunk_by_chunk_and_keeps_index_
     assert tokens.cpu().tolist()[3:5] == [-1, -1] and np.array_equal(tokens.cpu().numpy()[5:], got[5:])
 
 
+def test_a_top_k_draw_goes_through_the_candidates_of_the_rows_chunks(K, twins):
+    """With a top-k the row's chunks hand in their own k largest and the draw is made among those.  Rows made for what
+    could go wrong there: the k largest all in one chunk (the first, or the ragged last one, which has fewer tokens
+    than k), ties at the threshold within a chunk and across chunks (more of them than a chunk has places for sends
+    the row down the other path), all logits equal, k of 1, the largest k that goes this way and the first that does
+    not, k off in some rows.  The token must be the one that the one-block kernel draws from the whole row, for every
+    row, and the plain twin's wherever the target is not at an interval's very end."""
+    rng = np.random.default_rng(31)
+    vocab = 4 * 2048 + 30
+    assert K.lib.bh_sample_top_k_scratch(4, vocab) > 0
+    ramp = np.linspace(8.0, -8.0, vocab).astype(np.float32)
+    coarse = (np.round(rng.normal(size=vocab) * 4) / 4).astype(np.float32)
+    few_ties = (rng.normal(size=vocab) * 3).astype(np.float32)
+    few_ties[[5, 2048 + 17, 3 * 2048 + 1, vocab - 2]] = np.sort(few_ties)[-20]      # the 20th largest, in four chunks
+    shapes = [(rng.normal(size=vocab) * 3).astype(np.float32), ramp, ramp[::-1].copy(), coarse, few_ties,
+              np.full(vocab, 0.75, np.float32), np.where(rng.random(vocab) < 0.01, 3.0, -2.0).astype(np.float32)]
+    settings = [(1, 1.0), (5, 0.9), (20, 1.0), (40, 0.3), (50, 0.9), (128, 1.0), (129, 0.9), (0, 0.5), (vocab - 1, 1.0)]
+    logits = np.stack([shape for shape in shapes for _ in settings])
+    rows = logits.shape[0]
+    top_k = np.asarray([k for _ in shapes for k, _ in settings], np.int32)
+    top_p = np.asarray([p for _ in shapes for _, p in settings], np.float32)
+    temperature = rng.choice([0.6, 1.0, 1.5], size=rows).astype(np.float32)
+    temperature[3] = 0.0
+    on_device = dict(logits=dev(logits), temperature=dev(temperature), top_k=dev(top_k), top_p=dev(top_p))
+    for seed in range(4):
+        uniform = np.random.default_rng(seed).random(rows).astype(np.float32)
+        tokens, bad = torch.empty(rows, dtype=torch.int32, device=DEVICE), torch.empty(rows, dtype=torch.int32, device=DEVICE)
+        K.sample(on_device["logits"], tokens, bad, temperature=on_device["temperature"], top_k=on_device["top_k"],
+                 top_p=on_device["top_p"] if seed % 2 else None, uniform=dev(uniform))
+        whole, whole_bad = torch.empty_like(tokens), torch.empty_like(bad)
+        K._check(K.lib.bh_sample(K._ptr(on_device["logits"], "logits"), K._ptr(on_device["temperature"], "temperature"),
+                                 K._ptr(on_device["top_k"], "top_k"), K._ptr(on_device["top_p"] if seed % 2 else None, "top_p", None, True),
+                                 K._ptr(dev(uniform), "uniform"), K._ptr(whole, "tokens"), K._ptr(whole_bad, "bad"),
+                                 K._ptr(None, "scratch", None, True), rows, vocab, K._stream()))
+        got = tokens.cpu().numpy()
+        assert np.array_equal(got, whole.cpu().numpy())
+        want, want_bad, margin = twins.sample(logits, temperature, uniform, top_k, top_p if seed % 2 else None)
+        assert bad.cpu().tolist() == want_bad.tolist() == [0] * rows
+        sure = margin > 1e-5
+        assert sure.sum() > 0.8 * rows and np.array_equal(got[sure], want[sure]), (got[sure & (got != want)], want[sure & (got != want)])
+        assert int(got[3]) == int(np.argmax(logits[3]))
+    spoiled = logits.copy()
+    spoiled[2, 3 * 2048 + 5] = np.nan
+    K.sample(dev(spoiled), tokens, bad, temperature=on_device["temperature"], top_k=on_device["top_k"], uniform=dev(uniform))
+    assert bad.cpu().tolist() == [int(i == 2) for i in range(rows)] and int(tokens[2]) == -1
+
+
 @pytest.mark.parametrize("vocab", [50, 1000, 4133, 151936])
 def test_the_draw_and_its_twin(K, twins, vocab):
     """Temperature, top-k and top-p draws of the kernel against the plain twin's, row by row: the same token wherever the
