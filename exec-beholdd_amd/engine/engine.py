@@ -57,7 +57,7 @@ class Engine:
     def __init__(self, model_dir: str | None = None, dtype="bfloat16", max_tokens: int = 4096,
                  max_slots: int | None = None, device="cuda:0", kernels=None, model=None,
                  memory_limit_bytes: int | None = None, use_graphs: bool = True,
-                 max_rows_per_step: int | None = None, graph_limit: int = GRAPH_LIMIT):
+                 max_rows_per_step: int | None = None, graph_limit: int = GRAPH_LIMIT, graph_rows_per_sequence: int = 1):
         self.dtype = parse_dtype(dtype)
         self.device = torch.device(device)
         if kernels is None:
@@ -78,7 +78,8 @@ class Engine:
             self.max_rows_per_step = min(max(int(max_rows_per_step), cache.max_slots), capacity) if max_rows_per_step else capacity
             self.plan = plan_memory(model, weight_bytes, cache.plan(), 2 if self.dtype == torch.bfloat16 else 4,
                                     kernels if hasattr(kernels, "gemm_working_bytes") else None, self.max_rows_per_step,
-                                    cache.max_slots, cache.max_position, cache.page_size, graph_limit, with_graphs)
+                                    cache.max_slots, cache.max_position, cache.page_size, graph_limit, with_graphs,
+                                    max(int(graph_rows_per_sequence), 1))
             if memory_limit_bytes is not None and self.plan.total_bytes > memory_limit_bytes:
                 raise MemoryBudgetError(f"the engine needs {self.plan.total_bytes} bytes, the limit is "
                                         f"{memory_limit_bytes}:\n{self.plan.describe()}")
@@ -106,7 +107,7 @@ class Engine:
         self.sampler = Sampler(kernels, self.device, capacity=self.cache.max_slots)
         self._last_selection = None
         self._staging = StepStaging() if self.device.type == "cuda" else None
-        self.graphs = DecodeGraphs(self, graph_limit) if with_graphs else None
+        self.graphs = DecodeGraphs(self, graph_limit, graph_rows_per_sequence) if with_graphs else None
 
     # ---- what the generation loop needs of a stepper ----
     @property
@@ -176,9 +177,10 @@ class Engine:
         return logits
 
     def _graph_step(self, entries: list, extras: dict | None = None):
-        """A decode step (one token per sequence) replayed from a captured HIP graph."""
+        """A decode step (every sequence bringing the same few tokens, as a rule one) replayed from a captured HIP graph."""
         check_entries(entries, self.cache, self.model.vocab)
-        requests = [(e.slot, 1) for e in entries]
+        rows = len(entries[0].tokens)
+        requests = [(e.slot, rows) for e in entries]
         self.cache.reserve(requests)
         try:
             pasts = [self.cache.length(e.slot) for e in entries]
@@ -187,10 +189,10 @@ class Engine:
             self.cache.rollback(requests)
             raise
         self.cache.commit(requests)
-        wanted = [row for row, e in enumerate(entries) if e.want]
+        wanted = [index * rows + place for index, e in enumerate(entries) for place in e.want]
         if not wanted:
             return None
-        if len(wanted) == len(entries):
+        if wanted == list(range(len(entries) * rows)):
             return logits
         return logits[torch.tensor(wanted, device=self.device)]
 

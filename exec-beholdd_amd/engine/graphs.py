@@ -1,10 +1,11 @@
 """Decode steps as HIP graphs.
 
 A decode step launches a few hundred small kernels; replaying them as one captured graph takes
-the host out of the loop.  A graph is captured for a given number of sequences and a given
-page-table width (the longest sequence's pages, rounded up to a bucket) and replayed for every
-later step of that shape: the step's numbers (tokens, positions, slots, page tables) live in one
-static device buffer that is refreshed with a single copy before each replay.
+the host out of the loop.  A graph is captured for a given number of sequences, a given number of
+tokens that each of them brings (one, unless `DecodeGraphs.rows_per_sequence` allows short steps
+of several) and a given page-table width (the longest sequence's pages, rounded up to a bucket)
+and replayed for every later step of that shape: the step's numbers (tokens, positions, slots,
+page tables) live in one static device buffer that is refreshed with a single copy before each replay.
 
 Only kernels go into a graph: no memset nodes, no library calls (torch only hands out the
 temporaries, from the graph's private pool).  Parts whose `forward` reads the step's host-side
@@ -30,20 +31,20 @@ PAGE_BUCKET = 16      # page-table widths are rounded up to a multiple of this m
 
 
 class DecodeGraph:
-    def __init__(self, engine, n_seqs: int, table_width: int, pool=None):
-        self.pool = pool
+    def __init__(self, engine, n_seqs: int, table_width: int, rows: int = 1, pool=None):
+        self.pool, self.rows = pool, rows
         # the engine owns its graphs; they point back weakly, so that an engine nobody holds any more is
         # freed at once and not by a later garbage collection
         self.engine, self.n_seqs, self.table_width = _weakly(engine), n_seqs, table_width
         cache = engine.cache
-        self.layout = StepLayout(n_seqs, n_seqs, n_seqs, cache.kv_group_indices(), table_width)
+        self.layout = StepLayout(n_seqs * rows, n_seqs, n_seqs * rows, cache.kv_group_indices(), table_width)
         self.host = torch.zeros(self.layout.total, dtype=torch.int32).pin_memory()
         self.device = torch.zeros(self.layout.total, dtype=torch.int32, device=engine.device)
         self.host_views = self.layout.views(self.host.numpy())
         views = self.layout.views(self.device)
         self.tables = views["tables"]
         self.ctx = self.layout.context(
-            views, engine.kernels, engine.dtype, engine.device, max_rows_per_seq=1,
+            views, engine.kernels, engine.dtype, engine.device, max_rows_per_seq=rows,
             max_position=min(table_width * cache.page_size, cache.max_position) - 1,
             fed_tokens=engine.sampler.device_tokens)
         self.want_rows = views["want_rows"]
@@ -114,14 +115,17 @@ class _every_row_wanted:
     engine picks the wanted ones afterwards."""
 
     def __init__(self, entry):
-        self.slot, self.tokens, self.fed_row, self.want = entry.slot, entry.tokens, entry.fed_row, (0,)
+        self.slot, self.tokens, self.fed_row, self.want = entry.slot, entry.tokens, entry.fed_row, tuple(range(len(entry.tokens)))
 
 
 class DecodeGraphs:
-    """The graphs of one engine, by (sequences, page-table width)."""
+    """The graphs of one engine, by (sequences, page-table width, tokens per sequence)."""
 
-    def __init__(self, engine, limit: int = 48):
+    def __init__(self, engine, limit: int = 48, rows_per_sequence: int = 1):
         self.engine, self.limit = _weakly(engine), max(int(limit), 1)
+        # The most tokens per sequence of a step that is captured (every sequence of the step bringing as many).  The
+        # generation loop decodes one token per sequence; a caller whose steps bring a few each may raise this.
+        self.rows_per_sequence = max(int(rows_per_sequence), 1)
         self.graphs: dict = {}
         # One pool of device memory for all captures of the engine: only one of them runs at a time, on one
         # stream, so the temporaries of one step may stand where another's stood; what a capture returns (its
@@ -130,14 +134,17 @@ class DecodeGraphs:
 
     def usable(self, ctx_entries) -> bool:
         model = self.engine.model
+        rows = len(ctx_entries[0].tokens)
         return (getattr(model, "graph_safe", False) and self.engine.device.type == "cuda"
-                and all(len(e.tokens) == 1 for e in ctx_entries))
+                and 1 <= rows <= self.rows_per_sequence and all(len(e.tokens) == rows for e in ctx_entries)
+                and (rows == 1 or all(e.fed_row is None for e in ctx_entries)))
 
     def step(self, entries, pasts, extras=None):
         cache = self.engine.cache
-        pages = max(-(-(past + 1) // cache.page_size) for past in pasts)
+        rows = len(entries[0].tokens)
+        pages = max(-(-(past + rows) // cache.page_size) for past in pasts)
         width = -(-pages // PAGE_BUCKET) * PAGE_BUCKET
-        key = (len(entries), width)
+        key = (len(entries), width, rows)
         graph = self.graphs.pop(key, None)
         if graph is not None and graph.fed_buffer is not self.engine.sampler.out:
             graph = None                 # the sampler has a new buffer: what was captured reads the old one

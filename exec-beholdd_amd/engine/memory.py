@@ -108,7 +108,7 @@ def tables_bytes(model) -> int:
 
 
 def plan_memory(model, weight_bytes: int, cache_plan, act_size: int, sizes, max_rows_per_step: int, max_slots: int,
-                max_position: int, page_size: int, graph_limit: int, graphs: bool = True) -> MemoryPlan:
+                max_position: int, page_size: int, graph_limit: int, graphs: bool = True, graph_rows: int = 1) -> MemoryPlan:
     plan = MemoryPlan()
     kept, transient = weights_as_kept(model, act_size, sizes)
     plan.add("weights", int(weight_bytes))
@@ -127,9 +127,10 @@ def plan_memory(model, weight_bytes: int, cache_plan, act_size: int, sizes, max_
                  + step_numbers_bytes(rows, big.seqs, kv_groups, width))
         plan.unaccounted = model.unaccounted_parts() if hasattr(model, "unaccounted_parts") else []
         if graphs and getattr(model, "graph_safe", False):
-            small = step_size(model, max_slots, max_slots, act_size, max_position, sizes, max_rows_per_seq=1)
+            most = max_slots * graph_rows       # every sequence of a captured step brings the same one to graph_rows tokens
+            small = step_size(model, most, max_slots, act_size, max_position, sizes, max_rows_per_seq=graph_rows)
             pool = model.working_bytes(small)
-            each = _rounded(max_slots * model.vocab * 4) + step_numbers_bytes(max_slots, max_slots, kv_groups, width + 16)
+            each = _rounded(most * model.vocab * 4) + step_numbers_bytes(most, max_slots, kv_groups, width + 16)
             plan.add(f"captured decode steps (one pool; up to {graph_limit} captures' logits and numbers)",
                      pool + graph_limit * each)
     else:

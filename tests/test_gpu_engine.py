@@ -364,6 +364,51 @@ def test_graph_replays_equal_eager_steps(model_dirs, dtype):
     assert schedules.relative_error(outs[0][0], final) < TOLERANCE[dtype]
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_steps_of_a_few_tokens_per_sequence(model_dirs, dtype):
+    """An engine that is told to capture steps of up to four tokens per sequence: steps in which every sequence brings
+    three tokens are captured and replayed (across a page boundary and a change of the batch), steps of one token go on
+    as before, a step of unequal counts is launched kernel by kernel; logits asked for at some of a step's places only.
+    Every step against an engine without captures, the end against the plain implementation."""
+    from beholdd.engine import Engine, StepEntry
+    folder = model_dirs("D", "bfloat16")
+    graphed = Engine(folder, dtype=dtype, max_tokens=4096, graph_rows_per_sequence=4)
+    eager = Engine(folder, dtype=dtype, max_tokens=4096, use_graphs=False)
+    requests = schedules.random_requests(1500, [400, 300, 200], seed=23)
+    done = [50, 30, 1]
+    for engine in (graphed, eager):
+        engine.slots = [engine.alloc_slot() for _ in requests]
+        engine.step([StepEntry(s, r[:p], []) for s, r, p in zip(engine.slots, requests, done)])
+    live = [0, 1, 2]
+    worst = 0.0
+    counts = []
+    for step in range(30):
+        if step == 14:
+            live = [0, 2]
+        each = [1, 1, 1] if step % 7 == 3 else [3, 2, 3] if step == 9 else [3, 3, 3]
+        want = [[0, 2], [1], [0, 1, 2]] if each == [3, 3, 3] else [[n - 1] for n in each]
+        outs = []
+        for engine in (graphed, eager):
+            logits = engine.step([StepEntry(engine.slots[i], requests[i][done[i]:done[i] + each[i]], want[i]) for i in live])
+            outs.append(logits.float().cpu().numpy())
+        counts.append(outs[0].shape[0])
+        for i in live:
+            done[i] += each[i]
+        if dtype == "float32":
+            assert np.array_equal(outs[0], outs[1]), step
+        else:
+            worst = max(worst, schedules.relative_error(outs[0], outs[1]))
+    assert worst < 5e-3, worst
+    assert counts[0] == 6 and counts[3] == 3 and counts[20] == 5
+    keys = set(graphed.graphs.graphs)
+    assert {(3, 16, 3), (2, 16, 3), (3, 16, 1), (2, 16, 1)} <= keys and not any(key[2] == 2 for key in keys), keys
+    assert max(done) > 64           # the steps of three crossed a page's end
+    cfg, weights = plain.load_plain(folder)
+    final = plain.forward_logits(cfg, weights, requests[0][:done[0]])[-1]
+    assert schedules.relative_error(outs[0][1], final) < TOLERANCE[dtype]
+    graphed.cache.check_invariants()
+
+
 def _varied(model_dirs):
     """Tiny configuration B (separate head) with weights of a larger scale: greedy continuations that change
     from token to token, so that a wrong position, a stale page or a wrong length after the prompt changes
