@@ -1,4 +1,6 @@
-// Token selection from float32 logits, one block per row.
+// Token selection from float32 logits.  One block per row does all of it (sample_kernel); long rows get help from
+// blocks per chunk of the row where the work can be cut: the argmax in two steps, a draw from the whole distribution
+// through the chunks' weight sums, a draw with a top-k through the chunks' own k largest (further down).
 //   temperature <= 0: argmax, ties to the lowest id.
 //   temperature  > 0: softmax(logits / temperature) with the maximum subtracted,
 //                     optionally restricted to the top_k largest logits and then to the
@@ -16,8 +18,8 @@
 // walked from the top until the count reaches k, or the weight top_p of the total.  Three passes each, where a
 // search bit by bit took 32 (a row of 151,936 logits, one row or eight: temperature alone 121 -> 48 us, with
 // top-k of 50 711 -> 86, with top-p of 0.9 2,224 -> 110, with both 2,634 -> 128; 64 rows: 216 -> 52, 1,707 -> 94,
-// 5,146 -> 117, 5,835 -> 142).  What is left is arithmetic on the one compute unit that a row has: a pass costs
-// 10 to 13 us, the draw's about 25 (holding twice the loads in flight changed nothing).
+// 5,146 -> 117, 5,835 -> 142).  What is left there is arithmetic on the one compute unit that a row has: a pass costs
+// 10 to 13 us, the draw's about 25 (holding twice the loads in flight changed nothing); hence the chunks.
 #include "sampling.h"
 
 #include <mutex>
