@@ -55,7 +55,7 @@ def parse():
                         help="measure what a plain streaming read and a copy of 8 GB reach on this GPU, print it and exit")
     parser.add_argument("--sampling", action="store_true",
                         help="time the selection kernel on 1, 8 and 64 rows of 151,936 logits (greedy, at a temperature, with "
-                             "top-k, with top-p, with both), print the microseconds and exit")
+                             "top-k, with top-p on rows of three spreads, with both), print the microseconds and exit")
     return parser.parse_args()
 
 
@@ -199,11 +199,17 @@ def sampling_times(torch):
         temperature, uniform = torch.full((rows,), 0.8, device="cuda:0"), torch.rand(rows, device="cuda:0")
         top_k = torch.full((rows,), 50, dtype=torch.int32, device="cuda:0")
         top_p = torch.full((rows,), 0.9, device="cuda:0")
+        # (top-p's share of these rows is a thousand tokens or so; of the "peaked" rows, three times the spread, under a
+        # hundred, as of a trained model's mostly; of the "wide" rows, a sixth of the spread, most of the vocabulary)
+        usual, peaked, wide = logits, logits * 3, logits / 6
         modes = {"greedy": {}, "temperature": dict(temperature=temperature, uniform=uniform),
                  "top_k": dict(temperature=temperature, uniform=uniform, top_k=top_k),
                  "top_p": dict(temperature=temperature, uniform=uniform, top_p=top_p),
+                 "top_p_peaked": dict(temperature=temperature, uniform=uniform, top_p=top_p),
+                 "top_p_wide": dict(temperature=temperature, uniform=uniform, top_p=top_p),
                  "top_k_top_p": dict(temperature=temperature, uniform=uniform, top_k=top_k, top_p=top_p)}
         for name, arguments in modes.items():
+            logits = peaked if name.endswith("peaked") else wide if name.endswith("wide") else usual
             kernels.sample(logits, tokens, bad, **arguments)
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()

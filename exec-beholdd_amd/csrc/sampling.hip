@@ -159,10 +159,13 @@ struct SampleShared {
 
 // The draw from x[0..vocab) at a temperature above zero, the largest logit and its place known: the filters, then
 // the inverse-CDF draw over the kept tokens in index order; thread 0 leaves the token.  `ids` (or null): the token
-// that each element of x stands for, when x is a row's candidates and not the row itself.
-__device__ inline void draw_from(const float* __restrict__ x, int vocab, const int32_t* __restrict__ ids, float max_logit,
+// that each element of x stands for, when x is a row's candidates and not the row itself.  `whole_total` (or 0):
+// the weight of the whole row where top-p is to keep its share of that and not of what top-k leaves of x (
+// x's elements from the key `complete_from` on are then all of the row's with such keys); false, and no token, if
+// top-p's share reaches beyond them.
+__device__ inline bool draw_from(const float* __restrict__ x, int vocab, const int32_t* __restrict__ ids, float max_logit,
                                  int arg_max, float temp, int k, float p_keep, float uniform_number, int32_t* token,
-                                 SampleShared& sh) {
+                                 SampleShared& sh, sample_u64 whole_total = 0, uint32_t complete_from = 0) {
   sample_u64* bins = sh.bins;
   sample_u64* scratch = sh.scratch;
   const int tid = threadIdx.x;
@@ -174,7 +177,7 @@ __device__ inline void draw_from(const float* __restrict__ x, int vocab, const i
   };
 
   // top-k: the k-th largest logit's key; tokens with key >= floor_key are kept (ties at the k-th are)
-  uint32_t floor_key = 0;
+  uint32_t floor_key = complete_from;
   if (k > 0 && k < vocab)
     floor_key = threshold_key(x, vocab, 0u, (sample_u64)k, bins, scratch, &sh.found_bin, &sh.found_above,
                               [](float) -> sample_u64 { return 1; });
@@ -182,13 +185,19 @@ __device__ inline void draw_from(const float* __restrict__ x, int vocab, const i
   // top-p: the largest key whose tokens, with all above them, weigh top_p of what top-k has left
   if (p_keep > 0.f && p_keep < 1.f) {
     sample_u64 total = 0;
-    over_the_row(x, vocab, [&](int, float v) {
-      if (order_key(v) >= floor_key) total += weight_of(v);
-    });
-    total = block_total(total, scratch);
-    sample_u64 need = (sample_u64)__double2ull_rn((double)p_keep * (double)total);
+    if (whole_total != 0 && floor_key == 0u) {
+      total = whole_total;   // x is the whole row, and its weight is known
+    } else {
+      over_the_row(x, vocab, [&](int, float v) {
+        if (order_key(v) >= floor_key) total += weight_of(v);
+      });
+      total = block_total(total, scratch);
+    }
+    const sample_u64 of = whole_total != 0 ? whole_total : total;
+    sample_u64 need = (sample_u64)__double2ull_rn((double)p_keep * (double)of);
     if (need < 1) need = 1;
-    if (need > total) need = total;
+    if (need > of) need = of;
+    if (need > total) return false;   // (the same in every thread)
     const uint32_t key = threshold_key(x, vocab, floor_key, need, bins, scratch, &sh.found_bin, &sh.found_above, weight_of);
     if (key > floor_key) floor_key = key;
   }
@@ -281,6 +290,7 @@ __device__ inline void draw_from(const float* __restrict__ x, int vocab, const i
   }
   __syncthreads();
   if (tid == 0) *token = sh.chosen;
+  return true;
 }
 
 __global__ __launch_bounds__(SB) void sample_kernel(const float* __restrict__ logits,
@@ -606,16 +616,37 @@ extern "C" int bh_sample_draw_scratch(int n_rows, int vocab) {
 // every threshold); the block of the row then does on these few thousand candidates exactly what it would do on the
 // row: the k-th largest's key, top-p's threshold among what top-k leaves, the draw in index order.  The tokens kept
 // are the same as over the whole row, and so are their integer weights, the target and the token drawn.  A row
-// whose k is off or above CANDIDATES_UP_TO_K, or one of whose chunks has more ties at its threshold than fit, is
+// whose k is above CANDIDATES_UP_TO_K, or one of whose chunks has more ties at its threshold than fit, is
 // drawn from the whole row as before, by the same block (only the search for the largest logit is saved).
+// Up to 32 rows with a top-p and no top-k go the same way with the chunks' CANDIDATES_UP_TO_K largest: the chunks'
+// blocks, which then know the row's largest logit from a launch before them (the argmax's first step), also leave
+// their tokens' weight, so that the row's block knows the whole row's, and the key of their last candidate: from the
+// largest of those keys on, the candidates are all of the row's tokens.  If top-p's share of the row's weight lies
+// within these, threshold and draw among the candidates are those of the whole row; if not (a flat distribution),
+// the row is drawn whole, its largest logit and its weight already known.  (One row of 151,936 random logits, top-p
+// of 0.9: at a spread that keeps a thousand tokens or so 107 -> 42 us, at three times the spread 40, at a sixth of it,
+// where most of the vocabulary is kept and the row is drawn whole, 106; the candidates are about the largest 6 % of the
+// row.  With 64 rows the launches before the row's block cost what they save.)
 // 151,936 logits, top-k of 50: 86 -> 29 us for one row, 33 for eight, 94 -> 61 for 64; with top-p of 0.9 as well 128 -> 39, 42, 143 -> 70.
 
 #define CANDIDATES_UP_TO_K 128
 #define CANDIDATE_PLACES 144   // per chunk at most; used(k) = k + 8 rounded up to 16
+#define CANDIDATES_FOR_TOP_P_UP_TO_ROWS 32
 
 __host__ __device__ inline int candidate_places(int k) { return (k + 8 + 15) / 16 * 16; }
 
-__global__ __launch_bounds__(DT) void candidates_chunk_kernel(const float* __restrict__ logits, const int32_t* __restrict__ top_k,
+#define CANDIDATE_HEADER 8   // words a chunk leaves beside its candidates: largest logit, its place (-1: not finite), count (-1: none), last candidate's key, weight (2)
+
+// The k whose candidates a row's chunks hand in: its top-k, or for a top-p alone the most there is room for.
+__device__ inline int candidates_k(const int32_t* top_k, const float* top_p, int row) {
+  if (top_k != nullptr) return top_k[row];
+  const float p = top_p[row];
+  return p > 0.f && p < 1.f ? CANDIDATES_UP_TO_K : 0;
+}
+
+__global__ __launch_bounds__(DT) void candidates_chunk_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
+                                                              const int32_t* __restrict__ top_k, const float* __restrict__ top_p,
+                                                              const float* __restrict__ chunk_max,
                                                               uint32_t* __restrict__ headers, float* __restrict__ values,
                                                               int32_t* __restrict__ ids, int vocab, int chunks) {
   __shared__ float wave_val[DT / BH_WAVE];
@@ -652,8 +683,29 @@ __global__ __launch_bounds__(DT) void candidates_chunk_kernel(const float* __res
   __syncthreads();
   for (int w = 0; w < DT / BH_WAVE; ++w)
     if (wave_val[w] > bv || (wave_val[w] == bv && wave_idx[w] < bi)) bv = wave_val[w], bi = wave_idx[w];
-  uint32_t* header = headers + ((size_t)row * chunks + chunk) * 4;
-  const int k = top_k[row];
+  uint32_t* header = headers + ((size_t)row * chunks + chunk) * CANDIDATE_HEADER;
+  const int k = candidates_k(top_k, top_p, row);
+  if (chunk_max != nullptr) {   // the chunk's weight against the row's largest logit, which the launch before left chunk by chunk
+    __shared__ sample_u64 sums[DT / BH_WAVE];
+    float top = -INFINITY;
+    for (int c = tid; c < chunks; c += DT) top = fmaxf(top, chunk_max[(size_t)row * chunks + c]);
+#pragma unroll
+    for (int off = BH_WAVE / 2; off > 0; off >>= 1) top = fmaxf(top, __shfl_xor(top, off, BH_WAVE));
+    __syncthreads();
+    if (lane == 0) wave_val[wave] = top;
+    __syncthreads();
+    for (int w = 0; w < DT / BH_WAVE; ++w) top = fmaxf(top, wave_val[w]);
+    const float temp = temperature[row];
+    sample_u64 weight = 0;
+    if (!any_bad && temp > 0.f) {
+      const float per_logit = 1.4426950408889634f / temp;
+#pragma unroll
+      for (int u = 0; u < PER; ++u)
+        if (first + u < vocab) weight += fixed_weight(v[u], top, per_logit);
+    }
+    weight = draw_total(weight, sums);
+    if (tid == 0) header[4] = (uint32_t)weight, header[5] = (uint32_t)(weight >> 32);
+  }
   if (any_bad || k <= 0 || k > CANDIDATES_UP_TO_K || k >= vocab) {   // (the same for all of the row's chunks)
     if (tid == 0) {
       header[0] = __float_as_uint(bv);
@@ -723,6 +775,7 @@ __global__ __launch_bounds__(DT) void candidates_chunk_kernel(const float* __res
     header[0] = __float_as_uint(bv);
     header[1] = (uint32_t)bi;
     header[2] = (uint32_t)(kept <= places ? kept : -1);   // more ties than places: the row is drawn whole
+    header[3] = floor_key;
   }
   if (kept > places) return;
   const size_t base = (size_t)row * chunks * CANDIDATE_PLACES + (size_t)chunk * places;
@@ -742,18 +795,26 @@ __global__ __launch_bounds__(SB) void sample_candidates_kernel(const float* __re
                                                                const float* __restrict__ values, const int32_t* __restrict__ ids,
                                                                int32_t* __restrict__ tokens, int32_t* __restrict__ bad, int vocab,
                                                                int chunks) {
+  constexpr int HW = CANDIDATE_HEADER;
   __shared__ SampleShared sh;
   const int row = blockIdx.x, tid = threadIdx.x;
-  const uint32_t* mine = headers + (size_t)row * chunks * 4;
+  const uint32_t* mine = headers + (size_t)row * chunks * HW;
   // the row's largest logit with its lowest index (chunks are in index order), from the chunks' own
   float bv = -INFINITY;
   int bi = 0x7fffffff, not_finite = 0, whole = 0;
+  const bool share_of_the_row = top_k == nullptr;   // a top-p alone: the chunks have left their weights and last keys
+  sample_u64 weight = 0;
+  uint32_t complete_from = 0;
   for (int c = tid; c < chunks; c += SB) {
-    const float value = __uint_as_float(mine[4 * c]);
-    const int index = (int)mine[4 * c + 1];
+    const float value = __uint_as_float(mine[HW * c]);
+    const int index = (int)mine[HW * c + 1];
     if (index < 0) not_finite = 1;
-    if ((int)mine[4 * c + 2] < 0) whole = 1;
+    if ((int)mine[HW * c + 2] < 0) whole = 1;
     if (value > bv || bi == 0x7fffffff) bv = value, bi = index;
+    if (share_of_the_row) {
+      weight += (sample_u64)mine[HW * c + 4] | ((sample_u64)mine[HW * c + 5] << 32);
+      if ((int)mine[HW * c + 2] >= 0) complete_from = max(complete_from, mine[HW * c + 3]);
+    }
   }
 #pragma unroll
   for (int off = BH_WAVE / 2; off > 0; off >>= 1) {
@@ -779,19 +840,32 @@ __global__ __launch_bounds__(SB) void sample_candidates_kernel(const float* __re
     return;
   }
   if (tid == 0) bad[row] = 0;
-  const int k = top_k[row];
+  const int k = top_k ? top_k[row] : 0;
   const float p_keep = top_p ? top_p[row] : 1.f;
-  if (whole)
-    draw_from(logits + (size_t)row * vocab, vocab, nullptr, bv, bi, temp, k, p_keep, uniform[row], tokens + row, sh);
-  else
-    draw_from(values + (size_t)row * chunks * CANDIDATE_PLACES, chunks * candidate_places(k),
-              ids + (size_t)row * chunks * CANDIDATE_PLACES, bv, bi, temp, k, p_keep, uniform[row], tokens + row, sh);
+  if (share_of_the_row) {
+    weight = block_total(weight, sh.scratch);
+#pragma unroll
+    for (int off = BH_WAVE / 2; off > 0; off >>= 1) complete_from = max(complete_from, (uint32_t)__shfl_xor((int)complete_from, off, BH_WAVE));
+    __syncthreads();
+    if (tid % BH_WAVE == 0) sh.wave_idx[tid / BH_WAVE] = (int)complete_from;
+    __syncthreads();
+    for (int w = 0; w < SB / BH_WAVE; ++w) complete_from = max(complete_from, (uint32_t)sh.wave_idx[w]);
+  }
+  const int places = candidate_places(candidates_k(top_k, top_p, row));
+  // with a top-k, top-p keeps its share of what top-k leaves; alone, its share of the whole row
+  if (!whole && draw_from(values + (size_t)row * chunks * CANDIDATE_PLACES, chunks * places,
+                          ids + (size_t)row * chunks * CANDIDATE_PLACES, bv, bi, temp, k, p_keep, uniform[row],
+                          tokens + row, sh, weight, complete_from))
+    return;
+  __syncthreads();
+  draw_from(logits + (size_t)row * vocab, vocab, nullptr, bv, bi, temp, k, p_keep, uniform[row], tokens + row, sh, weight);
 }
 
-// Words of scratch for draws with a top-k over these rows (0: the rows are drawn by a block each from the whole row).
+// Words of scratch for draws with a top-k or a top-p over these rows (0: the rows are drawn by a block each from the whole row).
 extern "C" int bh_sample_top_k_scratch(int n_rows, int vocab) {
+  static_assert(AC == DC, "the argmax's chunks are the candidates' chunks");
   const long chunks = (vocab + DC - 1) / DC;
-  const long words = (long)n_rows * chunks * (4 + 2 * CANDIDATE_PLACES);
+  const long words = (long)n_rows * chunks * (CANDIDATE_HEADER + 2 * CANDIDATE_PLACES + 2);
   if (n_rows <= 0 || n_rows > 65535 || vocab < 4 * DC || chunks > SB || words >= (1L << 31)) return 0;
   return (int)words;
 }
@@ -827,12 +901,21 @@ extern "C" int bh_sample(const float* logits, const float* temperature, const in
                                                             vocab, chunks);
     return bh_check_launch("draw_rows");
   }
-  if (temperature != nullptr && top_k != nullptr && scratch != nullptr && bh_sample_top_k_scratch(n_rows, vocab) > 0) {
+  if (temperature != nullptr && (top_k != nullptr || (top_p != nullptr && n_rows <= CANDIDATES_FOR_TOP_P_UP_TO_ROWS)) && scratch != nullptr &&
+      bh_sample_top_k_scratch(n_rows, vocab) > 0) {
     const int chunks = (vocab + DC - 1) / DC;
     uint32_t* headers = (uint32_t*)scratch;
-    float* values = (float*)scratch + (size_t)n_rows * chunks * 4;
+    float* values = (float*)scratch + (size_t)n_rows * chunks * CANDIDATE_HEADER;
     int32_t* ids = (int32_t*)values + (size_t)n_rows * chunks * CANDIDATE_PLACES;
-    candidates_chunk_kernel<<<dim3(chunks, n_rows), dim3(DT), 0, stream>>>(logits, top_k, headers, values, ids, vocab, chunks);
+    float* chunk_max = nullptr;
+    if (top_k == nullptr) {   // a top-p alone: the chunks' weights need the row's largest logit first
+      chunk_max = (float*)(ids + (size_t)n_rows * chunks * CANDIDATE_PLACES);
+      argmax_chunk_kernel<<<dim3(chunks, n_rows), dim3(AT), 0, stream>>>(logits, chunk_max, (int32_t*)chunk_max + (size_t)n_rows * chunks,
+                                                                         vocab, chunks);
+      if (int status = bh_check_launch("argmax_chunk")) return status;
+    }
+    candidates_chunk_kernel<<<dim3(chunks, n_rows), dim3(DT), 0, stream>>>(logits, temperature, top_k, top_p, chunk_max, headers, values,
+                                                                           ids, vocab, chunks);
     if (int status = bh_check_launch("candidates_chunk")) return status;
     sample_candidates_kernel<<<dim3(n_rows), dim3(SB), 0, stream>>>(logits, temperature, top_k, top_p, uniform, headers, values,
                                                                     ids, tokens, bad, vocab, chunks);

@@ -775,7 +775,7 @@ class HipKernels(KernelSizes):
             words = int(self.lib.bh_sample_draw_scratch(n_rows, vocab))
             if words:
                 scratch = torch.empty(words, dtype=torch.float32, device=self.device)
-        elif top_k is not None:                    # and the chunks' candidates for the top k
+        else:                                      # and the chunks' candidates for a top-k or a top-p
             words = int(self.lib.bh_sample_top_k_scratch(n_rows, vocab))
             if words:
                 scratch = torch.empty(words, dtype=torch.float32, device=self.device)

@@ -287,6 +287,56 @@ def test_a_top_k_draw_goes_through_the_candidates_of_the_rows_chunks(K, twins):
     assert bad.cpu().tolist() == [int(i == 2) for i in range(rows)] and int(tokens[2]) == -1
 
 
+def test_a_top_p_draw_goes_through_the_candidates_where_its_share_lies_within_them(K, twins):
+    """A top-p without a top-k: the chunks hand in their 128 largest and their tokens' weight, and the row's block stays
+    among the candidates if top-p's share of the whole row's weight lies within the row's 128 largest, else it goes
+    through the whole row.  Rows on both sides of that (peaked ones, flat ones, one whose share ends exactly around the
+    128th largest token, all logits equal, two values), rows with a top-k as well and rows with no filter in the same call.
+    The token must be the one-block kernel's for every row, and the plain twin's wherever the target is not at an
+    interval's very end."""
+    rng = np.random.default_rng(37)
+    vocab = 5 * 2048 + 100
+    base = rng.normal(size=vocab).astype(np.float32)
+    edge = np.full(vocab, -30.0, np.float32)             # 256 equal tokens carry all the weight: p = 0.5 ends at the 128th
+    edge[rng.choice(vocab, size=256, replace=False)] = 2.0
+    shapes = [base * 12, base * 6, base * 3, base, base * 0.05, edge, np.full(vocab, -1.5, np.float32),
+              np.where(rng.random(vocab) < 0.002, 4.0, -4.0).astype(np.float32)]
+    settings = [(0, 0.9), (0, 0.5), (0, 0.1), (0, 0.999), (0, 1.0), (20, 0.9), (50, 1.0), (200, 0.7)]
+    logits = np.stack([shape for shape in shapes for _ in settings])
+    rows = logits.shape[0]
+    top_k = np.asarray([k for _ in shapes for k, _ in settings], np.int32)
+    top_p = np.asarray([p for _ in shapes for _, p in settings], np.float32)
+    temperature = rng.choice([0.6, 1.0, 1.5], size=rows).astype(np.float32)
+    temperature[9] = 0.0
+    device = dict(logits=dev(logits), temperature=dev(temperature), top_k=dev(top_k), top_p=dev(top_p))
+    for seed in range(4):
+        with_k = seed % 2 == 1
+        uniform = np.random.default_rng(seed).random(rows).astype(np.float32)
+        tokens, bad = torch.empty(rows, dtype=torch.int32, device=DEVICE), torch.empty(rows, dtype=torch.int32, device=DEVICE)
+        uniform_device = dev(uniform)
+        for some in (slice(0, 32), slice(32, rows)):      # (a top-p alone goes this way for up to 32 rows a call)
+            K.sample(device["logits"][some], tokens[some], bad[some], temperature=device["temperature"][some],
+                     top_k=device["top_k"][some] if with_k else None, top_p=device["top_p"][some], uniform=uniform_device[some])
+        whole, whole_bad = torch.empty_like(tokens), torch.empty_like(bad)
+        K._check(K.lib.bh_sample(K._ptr(device["logits"], "logits"), K._ptr(device["temperature"], "temperature"),
+                                 K._ptr(device["top_k"] if with_k else None, "top_k", None, True), K._ptr(device["top_p"], "top_p"),
+                                 K._ptr(dev(uniform), "uniform"), K._ptr(whole, "tokens"), K._ptr(whole_bad, "bad"),
+                                 K._ptr(None, "scratch", None, True), rows, vocab, K._stream()))
+        got = tokens.cpu().numpy()
+        assert np.array_equal(got, whole.cpu().numpy()), np.nonzero(got != whole.cpu().numpy())
+        want, want_bad, margin = twins.sample(logits, temperature, uniform, top_k if with_k else None, top_p)
+        assert bad.cpu().tolist() == want_bad.tolist() == [0] * rows
+        sure = margin > 1e-5
+        assert sure.sum() > 0.7 * rows and np.array_equal(got[sure], want[sure]), (got[sure & (got != want)], want[sure & (got != want)])
+        assert int(got[9]) == int(np.argmax(logits[9]))
+    spoiled = logits.copy()
+    spoiled[2, 3 * 2048 + 5] = np.inf
+    K.sample(dev(spoiled[:32]), tokens[:32], bad[:32], temperature=device["temperature"][:32], top_p=device["top_p"][:32],
+             uniform=uniform_device[:32])
+    assert bad[:32].cpu().tolist() == [int(i == 2) for i in range(32)] and int(tokens[2]) == -1
+    assert K.lib.bh_sample_top_k_scratch(32, vocab) > 0
+
+
 @pytest.mark.parametrize("vocab", [50, 1000, 4133, 151936])
 def test_the_draw_and_its_twin(K, twins, vocab):
     """Temperature, top-k and top-p draws of the kernel against the plain twin's, row by row: the same token wherever the
