@@ -174,6 +174,32 @@ def test_the_real_vocabulary(tmp_path_factory, dtype):
             tokens.append(token)
             seen.add(token)
     assert len(seen) >= 6 and max(seen) >= 2048          # tokens from several chunks of the vocabulary
+    # Draws at this vocabulary go through chunks of the row (weight sums, the chunks' candidates): every token drawn
+    # with a top-k must be among the k largest of the plain logits, with a top-p within the smallest set that holds
+    # that share (one token of slack at its end, and the tolerance's worth of logit), and the same seed must give the
+    # same tokens again.
+    slack = TOLERANCE[dtype]
+    for filters in (dict(top_k=5), dict(top_p=0.3), dict(top_k=40, top_p=0.5), dict()):
+        drawn = engine.generate(prompts, max_new_tokens=5, temperature=0.7, seed=11, **filters)
+        again = engine.generate(prompts, max_new_tokens=5, temperature=0.7, seed=11, **filters)
+        assert [r.token_ids for r in drawn] == [r.token_ids for r in again]
+        for prompt, result in zip(prompts, drawn):
+            tokens = list(prompt)
+            for token in result.token_ids:
+                row = plain.forward_logits(cfg, weights, tokens)[-1].astype(np.float64)
+                order = np.argsort(-row, kind="stable")
+                allowed = len(order)
+                if filters.get("top_k"):
+                    allowed = min(allowed, filters["top_k"])
+                floor = row[order[allowed - 1]]
+                assert row[token] >= floor - slack * np.abs(row).max(), (filters, tokens, token)
+                if filters.get("top_p"):
+                    kept = order[:allowed]
+                    weights_kept = np.exp((row[kept] - row[kept[0]]) / 0.7)
+                    share = np.cumsum(weights_kept) / weights_kept.sum()
+                    last = min(int(np.searchsorted(share, filters["top_p"])) + 1, allowed - 1)
+                    assert row[token] >= row[kept[last]] - slack * np.abs(row).max(), (filters, tokens, token)
+                tokens.append(token)
 
 
 def test_more_decode_shapes_than_the_engine_keeps(model_dirs):
