@@ -52,6 +52,11 @@ constexpr int STAGE_K = 256;             // K is cut into parts at multiples of 
 // MB: blocks of 16 activation rows (3 or 4).  A stage is SC chunks of 64 k: each wave holds its SC x 2 KB of W for it
 // in registers and the workgroup the activations' MB x SC x 2 KB in LDS; while a stage is multiplied the next one's
 // loads are on their way (registers and LDS hold two stages), one meeting of the waves per stage.
+// DEEP: W is asked for two stages ahead (three sets of registers; the activations, which come from the L2, stay one
+// stage ahead).  Qwen3-8B sizes, each product alone, us without / with: K in parts, 64 rows qkv 18.6 / 18.1, down 28.3 /
+// 27.5, 96 rows qkv 21.2 / 20.5, down 33.4 / 32.1, o the same; the SwiGLU that finishes itself 48 rows 39.4 / 41.3, 64 rows
+// 47.3 / 44.5, 96 rows 50.7 / 55.4, so that one takes it at 49 to 64 rows only; a decode step of 64 sequences at context
+// 640 5.50 -> 5.40 ms.
 // GATED: SwiGLU with all of K in one workgroup (one part): waves 0 to 3 own four blocks of gate rows, waves 4 to 7 the
 // blocks of up rows of the same outputs (N / 16 blocks further on); at the end the up waves hand their sums over
 // through LDS and the gate waves write bfloat16(silu(gate) * up), times the row factors of a norm ahead, into `gated`
@@ -67,7 +72,7 @@ struct GatedOut {
 
 __device__ inline float silu_mul(float gate, float up) { return gate / (1.0f + expf(-gate)) * up; }
 
-template <int MB, int SC, int WAVES, bool GATED>
+template <int MB, int SC, int WAVES, bool GATED, bool DEEP = false>
 __global__ __launch_bounds__(64 * WAVES, GATED ? (WAVES + 3) / 4 : MB > 4 ? 2 : 4) void gemm_slices_kernel(const uint16_t* __restrict__ a,
                                                                     const uint16_t* __restrict__ w,
                                                                     float* __restrict__ sums, int M, int w_rows, int K,
@@ -118,13 +123,19 @@ __global__ __launch_bounds__(64 * WAVES, GATED ? (WAVES + 3) / 4 : MB > 4 ? 2 : 
     }
   }
 
-  auto ask = [&](int t, u32x4_t (&wv)[SC][2], u32x4_t (&xv)[MINE]) {
+  auto ask_x = [&](int t, u32x4_t (&xv)[MINE]) {
 #pragma unroll
     for (int j = 0; j < MINE; ++j) xv[j] = *reinterpret_cast<const u32x4_t*>(a + (size_t)(x_from[j] + t * (STEPS * 512)));
+  };
+  auto ask_w = [&](int t, u32x4_t (&wv)[SC][2]) {
 #pragma unroll
     for (int c = 0; c < SC; ++c)
 #pragma unroll
       for (int u = 0; u < 2; ++u) wv[c][u] = load16_stream(wp + ((size_t)t * SC + c) * 1024 + u * 512);
+  };
+  auto ask = [&](int t, u32x4_t (&wv)[SC][2], u32x4_t (&xv)[MINE]) {
+    ask_x(t, xv);
+    ask_w(t, wv);
   };
   auto stash = [&](int turn, const u32x4_t (&xv)[MINE]) {
 #pragma unroll
@@ -145,17 +156,42 @@ __global__ __launch_bounds__(64 * WAVES, GATED ? (WAVES + 3) / 4 : MB > 4 ? 2 : 
   // Stage t lies in turn (t - first) % 2.  Before a wave writes a turn's LDS again, every wave has passed the
   // meeting that follows the other turn's writes, which it reaches only after it has multiplied this turn's.
   u32x4_t w0[SC][2], w1[SC][2], x0[MINE], x1[MINE];
-  ask(first, w0, x0);
-  for (int t = first; t < end; t += 2) {
-    stash(0, x0);
-    MEET();
-    if (t + 1 < end) ask(t + 1, w1, x1);
-    multiply(0, w0);
-    if (t + 1 >= end) break;
-    stash(1, x1);
-    MEET();
-    if (t + 2 < end) ask(t + 2, w0, x0);
-    multiply(1, w1);
+  if (DEEP) {
+    // W two stages ahead (three sets of registers), the activations one (they come from the L2): a stage's
+    // activations are asked for before the W of the stage after it, so that waiting for them leaves that W on its way.
+    u32x4_t w2[SC][2];
+    ask_x(first, x0);
+    ask_w(first, w0);
+    if (first + 1 < end) ask_w(first + 1, w1);
+#define BH_STAGE(at, turn, w_now, w_then, x_now, x_then)  \
+    stash(turn, x_now);                                   \
+    MEET();                                               \
+    if (t + (at) + 1 < end) ask_x(t + (at) + 1, x_then);  \
+    if (t + (at) + 2 < end) ask_w(t + (at) + 2, w_then);  \
+    multiply(turn, w_now);                                \
+    if (t + (at) + 1 >= end) break;
+    for (int t = first; t < end; t += 6) {
+      BH_STAGE(0, 0, w0, w2, x0, x1)
+      BH_STAGE(1, 1, w1, w0, x1, x0)
+      BH_STAGE(2, 0, w2, w1, x0, x1)
+      BH_STAGE(3, 1, w0, w2, x1, x0)
+      BH_STAGE(4, 0, w1, w0, x0, x1)
+      BH_STAGE(5, 1, w2, w1, x1, x0)
+    }
+#undef BH_STAGE
+  } else {
+    ask(first, w0, x0);
+    for (int t = first; t < end; t += 2) {
+      stash(0, x0);
+      MEET();
+      if (t + 1 < end) ask(t + 1, w1, x1);
+      multiply(0, w0);
+      if (t + 1 >= end) break;
+      stash(1, x1);
+      MEET();
+      if (t + 2 < end) ask(t + 2, w0, x0);
+      multiply(1, w1);
+    }
   }
   // acc[b][i]: activation row 16 b + r, weight row 16 block + 4 q + i
   if (GATED) {
@@ -271,7 +307,7 @@ int gemm_slices_launch(const void* a, const void* w, float* sums, int M, int N, 
   const dim3 grid((w_rows / 16 + WAVES - 1) / WAVES, parts), block(64 * WAVES);
   const GatedOut none = {};
   constexpr int SC = 2;
-#define BH_SLICES(MB) gemm_slices_kernel<MB, SC, WAVES, false><<<grid, block, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, sums, M, w_rows, K, each * (STAGE_K / 64 / SC), none)
+#define BH_SLICES(MB) gemm_slices_kernel<MB, SC, WAVES, false, true><<<grid, block, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, sums, M, w_rows, K, each * (STAGE_K / 64 / SC), none)
   if (M <= 48) BH_SLICES(3);
   else if (M <= 64) BH_SLICES(4);
   else if (M <= 96) BH_SLICES(6);
@@ -290,7 +326,7 @@ int gemm_slices_launch_gated(const void* a, const void* w, void* gated, int gate
   const GatedOut out = {(uint16_t*)gated, gated_block_rows, N, ahead_ss, ahead_blocks, ahead_eps};
   const dim3 grid((N / 16 + WAVES / 2 - 1) / (WAVES / 2)), block(64 * WAVES);
   const int stages = K / (64 * SC);
-#define BH_GATED(MB, NW) gemm_slices_kernel<MB, SC, NW, true><<<grid, block, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, nullptr, M, 2 * N, K, stages, out)
+#define BH_GATED(MB, NW) gemm_slices_kernel<MB, SC, NW, true, MB == 4><<<grid, block, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, nullptr, M, 2 * N, K, stages, out)
 #define BH_GATED_ROWS(NW) do { if (M <= 48) BH_GATED(3, NW); else if (M <= 64) BH_GATED(4, NW); else BH_GATED(6, NW); } while (0)
   static_assert(MOST_ROWS_GATED <= 96 && GATED_MOST_BLOCKS == 8, "the forms below");
   switch (blocks_each) {
