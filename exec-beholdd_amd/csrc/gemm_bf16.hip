@@ -1176,8 +1176,9 @@ static TiledConfig tiled_config(int M, int N, bool swiglu, int* rows, int* colum
 // Decode steps of the Qwen3-8B sizes at context 8,192, against tiles with K in parts from 17 rows on: 16
 // sequences 6.88 -> 6.64 ms, 32 sequences 10.38 -> 9.93 ms, 48 sequences 14.24 -> 14.43 ms (so not those).
 #define SKINNY_UP_TO_ROWS 32
-static bool skinny_first(int M, int N, int K, int layout) {
-  return layout == 1 && K % TK == 0 && N % 16 == 0 && M <= SKINNY_UP_TO_ROWS;
+static bool skinny_first(int M, int N, int K, int layout, int activation) {
+  // (but for the products of 17 to 32 rows and very many outputs that the kernel for 33 to 128 rows takes)
+  return layout == 1 && K % TK == 0 && N % 16 == 0 && M <= SKINNY_UP_TO_ROWS && !gemm_slices_takes(M, N, K, layout, activation);
 }
 // Whether the product runs as whole tiles (gemm_tiled_whole_kernel): the way that cuts K into parts and
 // the only tiled way a norm rides on.
@@ -1267,7 +1268,7 @@ extern "C" int bh_gemm_bf16_norm_blocks(int M, int N, int K, int layout, int act
   if (gemm_slices_takes(M, N, K, layout, 0)) return (N + FINISH_COLUMNS - 1) / FINISH_COLUMNS;   // always finished by that kernel
   tiled_config(M, N, false, &rows, &columns);
   if (!tiled_whole(M, N, K, layout, rows, columns)) {   // the skinny kernel's blocks, or its workgroups of wider spans
-    if (layout == 1 && skinny_first(M, N, K, layout))
+    if (layout == 1 && skinny_first(M, N, K, layout, 0))
       if (const int span = skinny_span_rows(M, N, K)) return N / span;
     return M <= 64 ? (N + 15) / 16 : 0;
   }
@@ -1288,7 +1289,7 @@ extern "C" int bh_gemm_bf16_takes_norm(int M, int N, int K, int layout, int acti
 extern "C" int bh_gemm_bf16_reads_blocked(int M, int N, int K, int layout, int activation) {
   if (M <= 0 || N <= 0 || K <= 0 || K % 32 != 0) return 0;
   if (gemm_turns_blocks(M, N, K, layout, activation) || gemm_turns_parts(M, N, K, layout, activation) > 1) return 16;
-  if (skinny_first(M, N, K, layout)) return M <= 8 ? 8 : 16;
+  if (skinny_first(M, N, K, layout, activation)) return M <= 8 ? 8 : 16;
   if (gemm_slices_takes(M, N, K, layout, activation)) return 16;
   return 0;
 }
@@ -1368,7 +1369,7 @@ extern "C" int bh_gemm_bf16(const void* a, const void* w, void* c, int c_dtype, 
   const bool skinny = [&] {
     int rows, columns;
     tiled_config(M, N, activation != 0, &rows, &columns);
-    return M <= 64 && !tiled_whole(M, N, K, layout, rows, columns);
+    return M <= 64 && !tiled_whole(M, N, K, layout, rows, columns) && !(M <= SKINNY_UP_TO_ROWS && gemm_slices_takes(M, N, K, layout, activation));
   }();
   // 33 to 128 rows from blocks of 16: the kernel whose waves share the activations through LDS, then the finishing kernel
   const bool slices = scratch != nullptr && a_block_rows == 16 && !skinny && gemm_slices_takes(M, N, K, layout, activation);

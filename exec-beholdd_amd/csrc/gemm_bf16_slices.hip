@@ -49,7 +49,7 @@ __device__ inline u32x4_t load16_stream(const uint16_t* p) {
 
 constexpr int STAGE_K = 256;             // K is cut into parts at multiples of this
 
-// MB: blocks of 16 activation rows (3 or 4).  A stage is SC chunks of 64 k: each wave holds its SC x 2 KB of W for it
+// MB: blocks of 16 activation rows (2 to 8).  A stage is SC chunks of 64 k: each wave holds its SC x 2 KB of W for it
 // in registers and the workgroup the activations' MB x SC x 2 KB in LDS; while a stage is multiplied the next one's
 // loads are on their way (registers and LDS hold two stages), one meeting of the waves per stage.
 // DEEP: W is asked for two stages ahead (three sets of registers; the activations, which come from the L2, stay one
@@ -238,8 +238,13 @@ constexpr int MOST_ROWS = 128, MOST_ROWS_GATED = 96;
 
 }  // namespace
 
+// From 33 rows on; a product of very many outputs (the head over a long vocabulary, whose workgroups fill the chip many
+// times over without a cut of K) from 17 rows on: 151,936 x 4,096, us with the kernel for up to 32 rows / here: 17 rows
+// 275 / 221, 32 rows 286 / 234 (16 rows there 225).
+constexpr int FEW_ROWS_FROM = 17, FEW_ROWS_OUTPUTS = 32768;
 bool gemm_slices_takes(int M, int N, int K, int layout, int activation) {
-  return layout == 1 && M > 32 && M <= (activation ? MOST_ROWS_GATED : MOST_ROWS) && K >= 512 && K % STAGE_K == 0 && N % 16 == 0 && N >= 128 &&
+  const bool rows_fit = M > 32 || (M >= FEW_ROWS_FROM && !activation && N >= FEW_ROWS_OUTPUTS);
+  return layout == 1 && rows_fit && M <= (activation ? MOST_ROWS_GATED : MOST_ROWS) && K >= 512 && K % STAGE_K == 0 && N % 16 == 0 && N >= 128 &&
          (long)64 * K < (1L << 31);
 }
 
@@ -308,7 +313,8 @@ int gemm_slices_launch(const void* a, const void* w, float* sums, int M, int N, 
   const GatedOut none = {};
   constexpr int SC = 2;
 #define BH_SLICES(MB) gemm_slices_kernel<MB, SC, WAVES, false, true><<<grid, block, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, sums, M, w_rows, K, each * (STAGE_K / 64 / SC), none)
-  if (M <= 48) BH_SLICES(3);
+  if (M <= 32) BH_SLICES(2);
+  else if (M <= 48) BH_SLICES(3);
   else if (M <= 64) BH_SLICES(4);
   else if (M <= 96) BH_SLICES(6);
   else BH_SLICES(8);
