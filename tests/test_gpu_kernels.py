@@ -121,7 +121,9 @@ def test_gemm(K, a_dtype, w_dtype, m, n, k):
                                    # that own 20, 24 or 28 rows (parts of two or three blocks); a last chunk trip that is not whole
                                    (8, 5120, 1024), (1, 5120, 5120), (32, 7168, 512), (17, 6144, 192), (9, 7168, 5120), (3, 5120, 17408),
                                    # 17 to 32 rows and very many outputs (a head over a long vocabulary): the kernel for 33 to 128 rows
-                                   (17, 32768, 512), (32, 40016, 768), (24, 32784, 1024), (16, 32768, 512)])
+                                   (17, 32768, 512), (32, 40016, 768), (24, 32784, 1024), (16, 32768, 512),
+                                   # 49 to 96 rows and many times the chip's workgroups in one part: eight waves a workgroup
+                                   (64, 65568, 512), (90, 65536, 768), (49, 66000, 512)])
 def test_gemm_with_packed_weights(K, m, n, k):
     """The same product from the regrouped (16 x 64 blocks) weight layout."""
     from beholdd.kernels import PackedWeight
