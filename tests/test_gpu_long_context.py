@@ -136,7 +136,7 @@ def test_the_32b_layer_sizes_at_a_context_of_16384(tmp_path):
             engine.free_slot(slot)
         engine.cache.check_invariants()
         if dtype == "bfloat16":
-            assert engine.graphs.graphs and all(key == (4, 256) for key in engine.graphs.graphs)
+            assert engine.graphs.graphs and all(key == (4, 256, 1) for key in engine.graphs.graphs)
         got[dtype] = np.stack(rows, axis=1)
         del engine
     for index, n in enumerate(lengths):
