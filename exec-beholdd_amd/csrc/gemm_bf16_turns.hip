@@ -345,8 +345,14 @@ TurnsPlan turns_plan(int M, int N, int K, int layout, int activation) {
     };
     int pb = 8, parts = parts_of(8);
     if (parts == 8 && gemm_turns_can(M, N, K, layout, 0, 4) && parts_of(4) == 4) pb = 4, parts = 4;
+    // Where the widest tile finds no cut that fills five eighths of the chip within one round (the q/k/v projection of the
+    // Qwen3-8B shape at 513 to 768 rows: 72 tiles, 144 workgroups in two parts, 288 in four) and no tile of its own is worth it
+    // either, the 192-wide tile may (96 tiles, 192 workgroups in two parts), then the 128-wide one.
+    if (parts == 1 && plan.blocks == 0)
+      for (int narrower = 6; narrower >= 4 && parts == 1; narrower -= 2)
+        if (gemm_turns_can(M, N, K, layout, 0, narrower) && parts_of(narrower) > 1) pb = narrower, parts = parts_of(narrower);
     if (parts > 1) {
-      const double rate = 0.85 * 1430.0 * (units / 256.0) * work / ((double)units * 256 * 32 * pb / parts * (pb == 8 ? 1.0 : 1.34));
+      const double rate = 0.85 * 1430.0 * (units / 256.0) * work / ((double)units * 256 * 32 * pb / parts * (pb == 8 ? 1.0 : pb == 6 ? 1.23 : 1.34));
       if (rate > direct_rate) plan.blocks = 0, plan.parts = parts, plan.part_blocks = pb;
     }
   }

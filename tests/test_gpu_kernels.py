@@ -110,7 +110,7 @@ def test_gemm(K, a_dtype, w_dtype, m, n, k):
                                    # few whole tiles: K in parts (equal and unequal ones) and a finishing kernel
                                    (200, 320, 832), (512, 4096, 4096), (128, 128, 4096),
                                    # many rows but few of the widest tiles: K in two or four parts of the kernel whose wave groups take turns
-                                   (1800, 4096, 2048), (1000, 4096, 4096),
+                                   (1800, 4096, 2048), (1000, 4096, 4096), (600, 6144, 4096), (760, 6032, 1024),
                                    # 65 to 127 rows: whole tiles of 64 rows
                                    (100, 256, 1024), (127, 4096, 512), (65, 128, 64),
                                    # 33 to 64 rows, K from 512: the waves of a workgroup share the activations through LDS;
@@ -1138,7 +1138,8 @@ def test_qk_norm_rope_cache_from_the_sums_of_a_products_parts(K, w_dtype, parts,
                              dev(positions[:40]), dev(row_seq[:40]), kp_d, vp_d, dev(table), n_heads, kv_heads, head_dim, True, 255)
 
 
-@pytest.mark.parametrize("m,n,k", [(512, 6144, 4096), (1024, 6144, 4096), (333, 4080, 4096), (2048, 6144, 4096), (64, 6144, 4096)])
+@pytest.mark.parametrize("m,n,k", [(512, 6144, 4096), (1024, 6144, 4096), (333, 4080, 4096), (2048, 6144, 4096), (64, 6144, 4096),
+                                   (640, 6144, 4096), (700, 6160, 2048)])        # two parts of the 192-wide tile
 def test_product_left_in_parts_adds_up_to_the_finished_product(K, m, n, k):
     """`gemm_bare` leaves what `gemm` would have finished: the parts, added in their order and rounded, are its output bit
     for bit; where the library does not cut such a product it says so by returning None."""
