@@ -136,7 +136,8 @@ class DecodeGraphs:
         model = self.engine.model
         rows = len(ctx_entries[0].tokens)
         return (getattr(model, "graph_safe", False) and self.engine.device.type == "cuda"
-                and 1 <= rows <= self.rows_per_sequence and all(len(e.tokens) == rows for e in ctx_entries)
+                and 1 <= rows <= self.rows_per_sequence and (rows == 1 or rows <= getattr(model, "graph_safe_rows", 1))
+                and all(len(e.tokens) == rows for e in ctx_entries)
                 and (rows == 1 or all(e.fed_row is None for e in ctx_entries)))
 
     def step(self, entries, pasts, extras=None):

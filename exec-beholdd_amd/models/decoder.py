@@ -10,7 +10,7 @@ the rows that are asked for (crates/beholdd-model/src/qwen3moe/forward.rs:811-91
 
 from __future__ import annotations
 
-from ..parts.base import BLOCKS, NORMS, POSITION_ENCODINGS
+from ..parts.base import BLOCKS, NORMS, POSITION_ENCODINGS, graph_rows_allowed
 from ..parts.embedding import Embedding, LMHead
 
 
@@ -58,6 +58,11 @@ class DecoderModel:
         forward depends on the step's device tensors only."""
         return all(getattr(part, "graph_safe", False)
                    for part in (self.embedding, *self.blocks, self.final_norm, self.head))
+
+    @property
+    def graph_safe_rows(self) -> int:
+        """Up to how many tokens per sequence a captured step may bring (every sequence the same number)."""
+        return graph_rows_allowed((self.embedding, *self.blocks, self.final_norm, self.head))
 
     def tensor_specs(self):
         return [spec for part in self.parts() for spec in part.tensor_specs()]

@@ -25,6 +25,7 @@ from .linear import Linear
 
 class GQAAttention:
     graph_safe = True      # forward reads only the step's device tensors
+    graph_safe_rows = None # ... whatever the number of tokens a sequence brings
     prepares_next_norm = True      # the output projection can carry the norm that follows
     takes_prepared_input = True    # x goes to the q/k/v product untouched
     def __init__(self, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int, prefix: str, *,

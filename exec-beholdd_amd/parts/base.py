@@ -46,7 +46,10 @@ Every part may say what its forward allocates: working_bytes(step: StepSize) -> 
 engine's byte plan adds them up before anything is allocated and names the parts that do not say.
 A part may declare `graph_safe = True`: its forward uses only the device tensors of the step
 context (never the host_* lists, never a host-side decision that changes from step to step).
-Decode steps of a model whose parts all say so are captured and replayed as HIP graphs.
+Decode steps of a model whose parts all say so are captured and replayed as HIP graphs.  That speaks of steps
+of one token per sequence; a part whose forward keeps to the device tensors for steps of several tokens per sequence too
+says `graph_safe_rows = n` (up to n tokens) or `None` (any number), and an engine that is told to capture such steps
+captures them only for models whose parts all allow it (`graph_rows_allowed`).
 """
 
 from __future__ import annotations
@@ -54,6 +57,18 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 
 import torch
+
+
+def graph_rows_allowed(parts) -> int:
+    """Up to how many tokens per sequence a captured step of these parts may bring (0: none may be captured)."""
+    most = 1 << 30
+    for part in parts:
+        if not getattr(part, "graph_safe", False):
+            return 0
+        rows = getattr(part, "graph_safe_rows", 1)
+        if rows is not None:
+            most = min(most, int(rows))
+    return most
 
 
 # ---- what a mixer keeps between steps ------------------------------------------------------

@@ -7,7 +7,7 @@ and is updated in place; the mixer and the feed-forward add into it.
 
 from __future__ import annotations
 
-from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS
+from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, graph_rows_allowed
 
 
 class PreNormBlock:
@@ -21,6 +21,10 @@ class PreNormBlock:
     @property
     def graph_safe(self):
         return all(getattr(part, "graph_safe", False) for part in self.parts())
+
+    @property
+    def graph_safe_rows(self):
+        return graph_rows_allowed(self.parts())
 
     def tensor_specs(self):
         return [spec for part in self.parts() for spec in part.tensor_specs()]

@@ -16,6 +16,7 @@ from .linear import Linear
 
 class Embedding:
     graph_safe = True      # forward reads only the step's device tensors
+    graph_safe_rows = None # ... whatever the number of tokens a sequence brings
     def __init__(self, vocab: int, width: int, name: str):
         self.vocab, self.width, self.name = vocab, width, name
         self.weight: torch.Tensor | None = None
@@ -40,6 +41,7 @@ class Embedding:
 
 class LMHead:
     graph_safe = True      # forward reads only the step's device tensors
+    graph_safe_rows = None # ... whatever the number of tokens a sequence brings
     def __init__(self, vocab: int, width: int, name: str | None, tied_to: Embedding | None = None):
         if (name is None) == (tied_to is None):
             raise ValueError("a head has either its own tensor or an embedding it is tied to")

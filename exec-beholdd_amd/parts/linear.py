@@ -16,6 +16,7 @@ from .base import ProductReader
 
 class Linear:
     graph_safe = True      # forward reads only the step's device tensors
+    graph_safe_rows = None # ... whatever the number of tokens a sequence brings
     def __init__(self, in_features: int, out_features, names):
         """`names` and `out_features` are one name and size, or equal-length lists to stack."""
         self.in_features = int(in_features)

@@ -13,6 +13,7 @@ from .linear import Linear
 
 class SwiGLU:
     graph_safe = True      # forward reads only the step's device tensors
+    graph_safe_rows = None # ... whatever the number of tokens a sequence brings
     prepares_next_norm = True      # the down projection can carry the norm that follows
     takes_prepared_input = True    # x goes to the gate/up product untouched
     def __init__(self, hidden: int, intermediate: int, prefix: str):

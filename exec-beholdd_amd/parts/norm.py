@@ -15,6 +15,7 @@ from .base import NORMS, NormRequest
 
 class RMSNorm:
     graph_safe = True      # forward reads only the step's device tensors
+    graph_safe_rows = None # ... whatever the number of tokens a sequence brings
     def __init__(self, width: int, eps: float, name: str):
         if not (eps > 0.0):
             raise ValueError(f"RMSNorm epsilon must be positive, got {eps}")

@@ -23,7 +23,7 @@ def cpu_engine(folder):
 
 
 @pytest.mark.parametrize("architecture", ["ToyHybridForCausalLM", "ToyTwiceForCausalLM", "ToySharedCacheForCausalLM",
-                                          "ToyOwnForCausalLM"])
+                                          "ToyParallelForCausalLM", "ToyOwnForCausalLM"])
 def test_toy_architectures_step_like_their_plain_forms(tmp_path, architecture):
     folder = beholdd.write_random_model(str(tmp_path), toy_parts.config_dict(architecture), seed=3, dtype="float32")
     engine = toy_parts.check_architecture(architecture, folder, cpu_engine, 1e-4)
@@ -33,8 +33,18 @@ def test_toy_architectures_step_like_their_plain_forms(tmp_path, architecture):
         assert kinds == ["kv", "state"] and len(engine.cache.groups) == 2
         state = [g for g in engine.cache.groups if g.need.kind == "state"][0].state
         assert state.shape == (2, engine.cache.max_slots, 48)
+        # the toy mixer scans a step of several tokens on the host: its decode steps may be captured, longer ones not
+        assert engine.model.graph_safe and engine.model.graph_safe_rows == 1
     elif architecture == "ToyTwiceForCausalLM":
         assert sorted(needs) == [0, 1, 2, 3, 4] and engine.model.run_writes == [True] * 5
+    elif architecture == "ToyParallelForCausalLM":
+        # a norm and a block of another make in the odd layers: their own tensors are in the model folder, and the model
+        # may still be captured, for steps of any number of tokens per sequence
+        kinds = [type(block).__name__ for block in engine.model.blocks]
+        assert kinds == ["PreNormBlock", "ToyParallelBlock"] * 2
+        names = {spec.name for spec in engine.model.tensor_specs()}
+        assert "model.layers.1.input_layernorm.bias" in names and "model.layers.1.post_attention_layernorm.weight" not in names
+        assert engine.model.graph_safe and engine.model.graph_safe_rows > 1000
     elif architecture == "ToyOwnForCausalLM":
         # a configuration class of its own, tensors under names of its own, a routed feed-forward whose
         # experts are all in use, a rotation of part of each head

@@ -14,7 +14,7 @@ from dataclasses import dataclass
 
 from beholdd.config import ConfigReader, LayerKinds, Qwen3Config
 from beholdd.models import build_decoder
-from beholdd.parts import (FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, CacheNeed, GQAAttention, Linear, RMSNorm,
+from beholdd.parts import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, CacheNeed, GQAAttention, Linear, RMSNorm,
                            RotaryEncoding, SwiGLU)
 from beholdd.weights import TensorSpec
 
@@ -86,6 +86,95 @@ class ToySharedCacheConfig(Qwen3Config):
 
     def schedule(self):
         return [(i, i - (i % 2)) for i in range(self.n_layers)]
+
+
+# ---- a norm and an arrangement of a layer's parts of another make ----------------------------------------
+
+class ToyCentredNorm:
+    """y = (x - mean) / sqrt(mean((x - mean)^2) + eps) * weight + bias, the statistics in float32 on the float32
+    residual: two tensors and a mean where the package's norm has one tensor and none.  Device tensors only, for
+    steps of any shape."""
+
+    graph_safe = True
+    graph_safe_rows = None
+
+    def __init__(self, width: int, eps: float, name: str):
+        self.width, self.eps, self.name, self.bias_name = width, eps, name, name.replace(".weight", ".bias")
+        self.weight = self.bias = None
+
+    def tensor_specs(self):
+        return [TensorSpec(self.name, (self.width,), "norm"), TensorSpec(self.bias_name, (self.width,), "linear")]
+
+    def load(self, get):
+        self.weight, self.bias = get(self.name), get(self.bias_name)
+
+    def forward(self, ctx, hidden, rows=None):
+        x = hidden if rows is None else hidden.index_select(0, rows.long())
+        centred = x - x.mean(dim=-1, keepdim=True)
+        y = centred * torch.rsqrt(centred.pow(2).mean(dim=-1, keepdim=True) + self.eps) * self.weight.float() + self.bias.float()
+        return y.to(ctx.act_dtype)
+
+
+def plain_centred_norm(x, weight, bias, eps):
+    x = x.astype(np.float32)
+    centred = x - x.mean(axis=-1, keepdims=True, dtype=np.float32)
+    inv = np.float32(1) / np.sqrt((centred * centred).mean(axis=-1, keepdims=True, dtype=np.float32) + np.float32(eps))
+    return (centred * inv * weight.astype(np.float32) + bias.astype(np.float32)).astype(np.float32)
+
+
+class ToyParallelBlock:
+    """h = h + Mixer(Norm(h)) + FeedForward(Norm(h)): one norm, and the mixer and the feed-forward both read what it
+    wrote of the layer's input (the package's block norms twice and feeds the second norm what the mixer added)."""
+
+    def __init__(self, norm, mixer, feed_forward):
+        self.norm, self.mixer, self.feed_forward = norm, mixer, feed_forward
+
+    def parts(self):
+        return [self.norm, self.mixer, self.feed_forward]
+
+    @property
+    def graph_safe(self):
+        return all(getattr(part, "graph_safe", False) for part in self.parts())
+
+    @property
+    def graph_safe_rows(self):
+        from beholdd.parts.base import graph_rows_allowed
+        return graph_rows_allowed(self.parts())
+
+    def tensor_specs(self):
+        return [spec for part in self.parts() for spec in part.tensor_specs()]
+
+    def load(self, get):
+        for part in self.parts():
+            part.load(get)
+
+    def prepare(self, kernels):
+        for part in self.parts():
+            if hasattr(part, "prepare"):
+                part.prepare(kernels)
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def forward(self, ctx, hidden, cache, prepared=None, next_block=None):
+        x = self.norm.forward(ctx, hidden)
+        self.mixer.forward(ctx, x, hidden, cache)
+        self.feed_forward.forward(ctx, x, hidden)
+        return None
+
+
+class ToyParallelConfig(Qwen3Config):
+    """Odd layers in the parallel arrangement with the centred norm, even ones as the package has them."""
+
+    def layer_kinds(self):
+        return [LayerKinds(mixer="gqa_attention", feed_forward="swiglu", norm="toy_centred_norm" if i % 2 else "rmsnorm",
+                           block="toy_parallel" if i % 2 else "pre_norm") for i in range(self.n_layers)]
+
+
+def _build_toy_parallel(config, layer_index, prefix, kinds, shared):
+    return ToyParallelBlock(NORMS.get(kinds.norm)(config, config.hidden, prefix + "input_layernorm.weight", shared),
+                            MIXERS.get(kinds.mixer)(config, layer_index, prefix, shared),
+                            FEED_FORWARDS.get(kinds.feed_forward)(config, layer_index, prefix, shared))
 
 
 # ---- an architecture with a configuration of its own ----------------------------------------------------
@@ -199,6 +288,8 @@ OWN_PARTS = (
     (FEED_FORWARDS, "toy_own_swiglu", lambda c, index, prefix, shared: SwiGLU(c.width, c.inner, prefix + "dense.")),
     (NORMS, "toy_own_rmsnorm", lambda c, width, name, shared: RMSNorm(width, c.floor, name)),
     (POSITION_ENCODINGS, "toy_stretched_rotary", lambda c, shared: ToyStretchedRotary(c.turned, c.base, c.longest, c.stretch)),
+    (NORMS, "toy_centred_norm", lambda c, width, name, shared: ToyCentredNorm(width, c.rms_eps, name)),
+    (BLOCKS, "toy_parallel", _build_toy_parallel),
 )
 
 OWN = {
@@ -217,6 +308,7 @@ def register():
     for name, cls, build in (("ToyHybridForCausalLM", ToyHybridConfig, build_decoder),
                              ("ToyTwiceForCausalLM", ToyTwiceConfig, build_decoder),
                              ("ToySharedCacheForCausalLM", ToySharedCacheConfig, build_decoder),
+                             ("ToyParallelForCausalLM", ToyParallelConfig, build_decoder),
                              ("ToyOwnForCausalLM", ToyOwnConfig, build_toy_own)):
         if name not in beholdd.registered_architectures():
             beholdd.register_architecture(name, cls, build)
@@ -226,7 +318,8 @@ def unregister():
     MIXERS.unregister("toy_running_mean")
     for registry, name, _ in OWN_PARTS:
         registry.unregister(name)
-    for name in ("ToyHybridForCausalLM", "ToyTwiceForCausalLM", "ToySharedCacheForCausalLM", "ToyOwnForCausalLM"):
+    for name in ("ToyHybridForCausalLM", "ToyTwiceForCausalLM", "ToySharedCacheForCausalLM", "ToyParallelForCausalLM",
+                 "ToyOwnForCausalLM"):
         beholdd.registry.unregister_architecture(name)
 
 
@@ -340,6 +433,28 @@ def plain_logits(architecture, cfg, w, tokens):
             attended = plain.causal_attention(q, shared[0], shared[1], cfg.n_heads, cfg.n_kv_heads, cfg.head_dim, scale)
             hidden = (hidden + plain.linear(attended, w[prefix + "self_attn.o_proj.weight"])).astype(np.float32)
             hidden = plain.mlp_block(cfg, w, prefix, hidden)
+    elif architecture == "ToyParallelForCausalLM":
+        freqs = plain.rope_frequencies(cfg.theta, cfg.head_dim)
+        for i in range(cfg.n_layers):
+            prefix = f"model.layers.{i}."
+            if i % 2 == 0:
+                hidden = plain.layer(cfg, w, i, hidden)
+                continue
+            t_len, hd = hidden.shape[0], cfg.head_dim
+            xn = plain_centred_norm(hidden, w[prefix + "input_layernorm.weight"], w[prefix + "input_layernorm.bias"], cfg.eps)
+            q = plain.rmsnorm(plain.linear(xn, w[prefix + "self_attn.q_proj.weight"]).reshape(t_len, cfg.n_heads, hd),
+                              w[prefix + "self_attn.q_norm.weight"], cfg.eps)
+            k = plain.rmsnorm(plain.linear(xn, w[prefix + "self_attn.k_proj.weight"]).reshape(t_len, cfg.n_kv_heads, hd),
+                              w[prefix + "self_attn.k_norm.weight"], cfg.eps)
+            v = plain.linear(xn, w[prefix + "self_attn.v_proj.weight"])
+            for t in range(t_len):
+                cs = plain.rope_cos_sin(freqs, t)
+                q[t], k[t] = plain.rope_split_half(q[t], *cs), plain.rope_split_half(k[t], *cs)
+            attended = plain.causal_attention(q.reshape(t_len, -1), k.reshape(t_len, -1), v, cfg.n_heads, cfg.n_kv_heads, hd, scale)
+            mixed = plain.linear(attended, w[prefix + "self_attn.o_proj.weight"])
+            fed = plain.linear(plain.swiglu(plain.linear(xn, w[prefix + "mlp.gate_proj.weight"]), plain.linear(xn, w[prefix + "mlp.up_proj.weight"])),
+                               w[prefix + "mlp.down_proj.weight"])
+            hidden = ((hidden + mixed).astype(np.float32) + fed).astype(np.float32)      # the engine adds the two in this order
     else:
         raise ValueError(architecture)
     return plain.head(cfg, w, hidden)
