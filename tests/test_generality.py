@@ -23,7 +23,7 @@ def cpu_engine(folder):
 
 
 @pytest.mark.parametrize("architecture", ["ToyHybridForCausalLM", "ToyTwiceForCausalLM", "ToySharedCacheForCausalLM",
-                                          "ToyParallelForCausalLM", "ToyOwnForCausalLM"])
+                                          "ToyParallelForCausalLM", "ToyWindowedForCausalLM", "ToyOwnForCausalLM"])
 def test_toy_architectures_step_like_their_plain_forms(tmp_path, architecture):
     folder = beholdd.write_random_model(str(tmp_path), toy_parts.config_dict(architecture), seed=3, dtype="float32")
     engine = toy_parts.check_architecture(architecture, folder, cpu_engine, 1e-4)
@@ -37,6 +37,19 @@ def test_toy_architectures_step_like_their_plain_forms(tmp_path, architecture):
         assert engine.model.graph_safe and engine.model.graph_safe_rows == 1
     elif architecture == "ToyTwiceForCausalLM":
         assert sorted(needs) == [0, 1, 2, 3, 4] and engine.model.run_writes == [True] * 5
+    elif architecture == "ToyWindowedForCausalLM":
+        # two groups of storage, one per need; a sequence of 150 tokens keeps only the pages that its window touches there
+        windows = sorted(group.need.window for group in engine.cache.groups)
+        assert windows == [0, toy_parts.WINDOW] and [len(group.entries) for group in engine.cache.groups] == [2, 2]
+        import schedules
+        from beholdd.engine import StepEntry
+        slot = engine.alloc_slot()
+        engine.step([StepEntry(slot, schedules.random_requests(101, [150], seed=1)[0], [])])
+        windowed = [group for group in engine.cache.groups if group.need.window][0]
+        full = [group for group in engine.cache.groups if not group.need.window][0]
+        assert [page >= 0 for page in windowed.pages_of[slot]] == [False, True, True] and all(page >= 0 for page in full.pages_of[slot])
+        engine.free_slot(slot)
+        engine.cache.check_invariants()
     elif architecture == "ToyParallelForCausalLM":
         # a norm and a block of another make in the odd layers: their own tensors are in the model folder, and the model
         # may still be captured, for steps of any number of tokens per sequence

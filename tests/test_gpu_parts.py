@@ -239,12 +239,14 @@ def toys():
 # (the architecture with routing runs in float32 only: top-1 routing on rounded inputs may choose another expert
 # than the plain form does)
 @pytest.mark.parametrize("architecture,dtype", [(a, d) for a in ("ToyHybridForCausalLM", "ToyTwiceForCausalLM",
-                                                                 "ToySharedCacheForCausalLM", "ToyParallelForCausalLM")
+                                                                 "ToySharedCacheForCausalLM", "ToyParallelForCausalLM",
+                                                                 "ToyWindowedForCausalLM")
                                                 for d in ("float32", "bfloat16")]
                          + [("ToyOwnForCausalLM", "float32")])
 def test_toy_architectures_on_the_gpu(toys, tmp_path, architecture, dtype):
     """A mixer with state of its own (whose decode steps are captured and replayed), a layer that runs twice, a
-    layer that reads another layer's cache, a norm and an arrangement of a layer's parts of another make, and an
+    layer that reads another layer's cache, a norm and an arrangement of a layer's parts of another make, layers
+    whose attention sees a window of the keys beside layers that see all of them, and an
     architecture with a configuration class, tensor names, a routed feed-forward and a position encoding of its own: registered from the test, built, loaded and
     stepped by the unchanged engine."""
     folder = beholdd.write_random_model(str(tmp_path), toy_parts.config_dict(architecture), seed=3, dtype="bfloat16")

@@ -177,6 +177,34 @@ def _build_toy_parallel(config, layer_index, prefix, kinds, shared):
                             FEED_FORWARDS.get(kinds.feed_forward)(config, layer_index, prefix, shared))
 
 
+# ---- attention over a window of the keys in some layers, over all of them in the others ---------------------
+
+WINDOW = 24
+
+
+class ToyWindowedConfig(Qwen3Config):
+    """Odd layers see the last WINDOW keys only: their keys and values get storage of their own, which gives
+    pages back as a sequence moves on; even layers see all keys."""
+
+    def layer_kinds(self):
+        return [LayerKinds(mixer="toy_windowed_attention" if i % 2 else "gqa_attention", feed_forward="swiglu",
+                           norm="rmsnorm", block="pre_norm") for i in range(self.n_layers)]
+
+
+def plain_windowed_attention(q, k, v, n_heads, n_kv_heads, head_dim, scale, window):
+    """Query t sees keys max(0, t - window + 1) .. t: scores in float32 from float64 dot products, softmax in float32."""
+    t_len = q.shape[0]
+    qh, kh, vh = (a.astype(np.float64).reshape(t_len, -1, head_dim) for a in (q, k, v))
+    out = np.zeros((t_len, n_heads, head_dim), np.float32)
+    for h in range(n_heads):
+        g = h // (n_heads // n_kv_heads)
+        for t in range(t_len):
+            lo = max(0, t - window + 1)
+            scores = ((kh[lo:t + 1, g] @ qh[t, h]) * np.float64(np.float32(scale))).astype(np.float32)
+            out[t, h] = (plain.softmax(scores).astype(np.float64) @ vh[lo:t + 1, g]).astype(np.float32)
+    return out.reshape(t_len, -1)
+
+
 # ---- an architecture with a configuration of its own ----------------------------------------------------
 # Its config.json has other keys, its configuration class inherits nothing from Qwen3's, its tensors have
 # other names, and it brings a feed-forward with routing and a position encoding of its own; the builders
@@ -289,6 +317,9 @@ OWN_PARTS = (
     (NORMS, "toy_own_rmsnorm", lambda c, width, name, shared: RMSNorm(width, c.floor, name)),
     (POSITION_ENCODINGS, "toy_stretched_rotary", lambda c, shared: ToyStretchedRotary(c.turned, c.base, c.longest, c.stretch)),
     (NORMS, "toy_centred_norm", lambda c, width, name, shared: ToyCentredNorm(width, c.rms_eps, name)),
+    (MIXERS, "toy_windowed_attention", lambda c, index, prefix, shared: GQAAttention(
+        c.hidden, c.n_heads, c.n_kv_heads, c.head_dim, prefix + "self_attn.", position_encoding=shared["position_encoding"],
+        qk_norm_eps=c.rms_eps, window=WINDOW)),
     (BLOCKS, "toy_parallel", _build_toy_parallel),
 )
 
@@ -309,6 +340,7 @@ def register():
                              ("ToyTwiceForCausalLM", ToyTwiceConfig, build_decoder),
                              ("ToySharedCacheForCausalLM", ToySharedCacheConfig, build_decoder),
                              ("ToyParallelForCausalLM", ToyParallelConfig, build_decoder),
+                             ("ToyWindowedForCausalLM", ToyWindowedConfig, build_decoder),
                              ("ToyOwnForCausalLM", ToyOwnConfig, build_toy_own)):
         if name not in beholdd.registered_architectures():
             beholdd.register_architecture(name, cls, build)
@@ -319,7 +351,7 @@ def unregister():
     for registry, name, _ in OWN_PARTS:
         registry.unregister(name)
     for name in ("ToyHybridForCausalLM", "ToyTwiceForCausalLM", "ToySharedCacheForCausalLM", "ToyParallelForCausalLM",
-                 "ToyOwnForCausalLM"):
+                 "ToyWindowedForCausalLM", "ToyOwnForCausalLM"):
         beholdd.registry.unregister_architecture(name)
 
 
@@ -433,6 +465,16 @@ def plain_logits(architecture, cfg, w, tokens):
             attended = plain.causal_attention(q, shared[0], shared[1], cfg.n_heads, cfg.n_kv_heads, cfg.head_dim, scale)
             hidden = (hidden + plain.linear(attended, w[prefix + "self_attn.o_proj.weight"])).astype(np.float32)
             hidden = plain.mlp_block(cfg, w, prefix, hidden)
+    elif architecture == "ToyWindowedForCausalLM":
+        for i in range(cfg.n_layers):
+            prefix = f"model.layers.{i}."
+            if i % 2:
+                q, k, v = _attention_parts(cfg, w, prefix, hidden)
+                attended = plain_windowed_attention(q, k, v, cfg.n_heads, cfg.n_kv_heads, cfg.head_dim, scale, WINDOW)
+                hidden = (hidden + plain.linear(attended, w[prefix + "self_attn.o_proj.weight"])).astype(np.float32)
+            else:
+                hidden = plain.attention_block(cfg, w, prefix, hidden)
+            hidden = plain.mlp_block(cfg, w, prefix, hidden)
     elif architecture == "ToyParallelForCausalLM":
         freqs = plain.rope_frequencies(cfg.theta, cfg.head_dim)
         for i in range(cfg.n_layers):
@@ -470,7 +512,8 @@ def check_architecture(architecture, folder, make_engine, tolerance):
     else:
         cfg, weights = plain.load_plain(folder)
         vocab = cfg.vocab
-    requests = schedules.random_requests(vocab, [3, 70, 21, 40], seed=13)
+    # (with a window, one request long enough for the windowed layers to give pages back while it is decoded)
+    requests = schedules.random_requests(vocab, [3, 70, 21, 40] + ([150] if architecture == "ToyWindowedForCausalLM" else []), seed=13)
     want = [plain_logits(architecture, cfg, weights, r) for r in requests]
     engine = make_engine(folder)
     for label, got in (("whole", schedules.whole(engine, requests)),
