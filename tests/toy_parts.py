@@ -16,6 +16,7 @@ from beholdd.config import ConfigReader, LayerKinds, Qwen3Config
 from beholdd.models import build_decoder
 from beholdd.parts import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, CacheNeed, GQAAttention, Linear, RMSNorm,
                            RotaryEncoding, SwiGLU)
+from beholdd.parts.embedding import Embedding, LMHead
 from beholdd.weights import TensorSpec
 
 DECAY = 0.75
@@ -161,6 +162,29 @@ class ToyParallelBlock:
         self.mixer.forward(ctx, x, hidden, cache)
         self.feed_forward.forward(ctx, x, hidden)
         return None
+
+
+class ToyScaledEmbedding(Embedding):
+    """The embedding's rows times sqrt(width), in float32."""
+
+    def forward(self, ctx):
+        return super().forward(ctx).mul_(float(np.sqrt(np.float32(self.width))))
+
+
+LOGIT_CAP = 0.5
+
+
+class ToyCappedHead(LMHead):
+    """Logits held within (-LOGIT_CAP, LOGIT_CAP): cap * tanh(logits / cap), in float32."""
+
+    def forward(self, ctx, x):
+        logits = super().forward(ctx, x)
+        return torch.tanh(logits / LOGIT_CAP) * LOGIT_CAP
+
+
+def build_toy_parallel_model(config):
+    return build_decoder(config, make_embedding=lambda c: ToyScaledEmbedding(c.vocab, c.hidden, "model.embed_tokens.weight"),
+                         make_head=lambda c, embedding: ToyCappedHead(c.vocab, c.hidden, "lm_head.weight"))
 
 
 class ToyParallelConfig(Qwen3Config):
@@ -339,7 +363,7 @@ def register():
     for name, cls, build in (("ToyHybridForCausalLM", ToyHybridConfig, build_decoder),
                              ("ToyTwiceForCausalLM", ToyTwiceConfig, build_decoder),
                              ("ToySharedCacheForCausalLM", ToySharedCacheConfig, build_decoder),
-                             ("ToyParallelForCausalLM", ToyParallelConfig, build_decoder),
+                             ("ToyParallelForCausalLM", ToyParallelConfig, build_toy_parallel_model),
                              ("ToyWindowedForCausalLM", ToyWindowedConfig, build_decoder),
                              ("ToyOwnForCausalLM", ToyOwnConfig, build_toy_own)):
         if name not in beholdd.registered_architectures():
@@ -476,6 +500,7 @@ def plain_logits(architecture, cfg, w, tokens):
                 hidden = plain.attention_block(cfg, w, prefix, hidden)
             hidden = plain.mlp_block(cfg, w, prefix, hidden)
     elif architecture == "ToyParallelForCausalLM":
+        hidden = (hidden * np.sqrt(np.float32(cfg.hidden))).astype(np.float32)      # the scaled embedding
         freqs = plain.rope_frequencies(cfg.theta, cfg.head_dim)
         for i in range(cfg.n_layers):
             prefix = f"model.layers.{i}."
@@ -497,6 +522,8 @@ def plain_logits(architecture, cfg, w, tokens):
             fed = plain.linear(plain.swiglu(plain.linear(xn, w[prefix + "mlp.gate_proj.weight"]), plain.linear(xn, w[prefix + "mlp.up_proj.weight"])),
                                w[prefix + "mlp.down_proj.weight"])
             hidden = ((hidden + mixed).astype(np.float32) + fed).astype(np.float32)      # the engine adds the two in this order
+        logits = plain.head(cfg, w, hidden).astype(np.float32)
+        return (np.tanh(logits / np.float32(LOGIT_CAP)) * np.float32(LOGIT_CAP)).astype(np.float32)      # the capped head
     else:
         raise ValueError(architecture)
     return plain.head(cfg, w, hidden)
