@@ -29,8 +29,11 @@
 
 typedef unsigned long long sample_u64;
 
+// An integer that orders as the floats do; minus zero and zero, which compare equal, get one key (ties at a threshold
+// are kept, and a tie must not depend on a sign bit).
 __device__ inline uint32_t order_key(float x) {
   uint32_t u = __float_as_uint(x);
+  if (u == 0x80000000u) u = 0u;
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 

@@ -172,7 +172,8 @@ def test_the_draws_thresholds_on_rows_made_to_trip_them(K, twins):
               (rng.normal(size=vocab) * 1e-3).astype(np.float32),
               (rng.normal(size=vocab) * 40).astype(np.float32),
               np.concatenate([np.full(vocab - 3, -1e30, np.float32), np.asarray([0.5, 0.5, 0.25], np.float32)]),
-              (-np.abs(rng.normal(size=vocab)) * 5 - 100).astype(np.float32)]
+              (-np.abs(rng.normal(size=vocab)) * 5 - 100).astype(np.float32),
+              np.where(rng.random(vocab) < 0.5, np.float32(0.0), np.float32(-0.0)).astype(np.float32)]     # zero and minus zero tie
     settings = [(0, 1.0), (5, 1.0), (vocab - 1, 1.0), (0, 1e-6), (0, 0.999999), (0, 0.5), (40, 0.7), (1, 0.3)]
     logits = np.stack([shape for shape in shapes for _ in settings])
     rows = logits.shape[0]
@@ -254,8 +255,10 @@ def test_a_top_k_draw_goes_through_the_candidates_of_the_rows_chunks(K, twins):
     coarse = (np.round(rng.normal(size=vocab) * 4) / 4).astype(np.float32)
     few_ties = (rng.normal(size=vocab) * 3).astype(np.float32)
     few_ties[[5, 2048 + 17, 3 * 2048 + 1, vocab - 2]] = np.sort(few_ties)[-20]      # the 20th largest, in four chunks
+    signed_zeros = np.where(rng.random(vocab) < 0.5, np.float32(0.0), np.float32(-0.0)).astype(np.float32)
+    signed_zeros[[9, 5000]] = 1.0          # two tokens above a sea of zeros of both signs, which all tie
     shapes = [(rng.normal(size=vocab) * 3).astype(np.float32), ramp, ramp[::-1].copy(), coarse, few_ties,
-              np.full(vocab, 0.75, np.float32), np.where(rng.random(vocab) < 0.01, 3.0, -2.0).astype(np.float32)]
+              np.full(vocab, 0.75, np.float32), np.where(rng.random(vocab) < 0.01, 3.0, -2.0).astype(np.float32), signed_zeros]
     settings = [(1, 1.0), (5, 0.9), (20, 1.0), (40, 0.3), (50, 0.9), (128, 1.0), (129, 0.9), (0, 0.5), (vocab - 1, 1.0)]
     logits = np.stack([shape for shape in shapes for _ in settings])
     rows = logits.shape[0]
