@@ -621,7 +621,7 @@ extern "C" int bh_sample_draw_scratch(int n_rows, int vocab) {
 // are the same as over the whole row, and so are their integer weights, the target and the token drawn.  A row
 // whose k is above CANDIDATES_UP_TO_K, or one of whose chunks has more ties at its threshold than fit, is
 // drawn from the whole row as before, by the same block (only the search for the largest logit is saved).
-// Up to 32 rows with a top-p and no top-k go the same way with the chunks' CANDIDATES_UP_TO_K largest: the chunks'
+// Up to 64 rows with a top-p and no top-k go the same way with the chunks' CANDIDATES_UP_TO_K largest: the chunks'
 // blocks, which then know the row's largest logit from a launch before them (the argmax's first step), also leave
 // their tokens' weight, so that the row's block knows the whole row's, and the key of their last candidate: from the
 // largest of those keys on, the candidates are all of the row's tokens.  If top-p's share of the row's weight lies
@@ -629,12 +629,12 @@ extern "C" int bh_sample_draw_scratch(int n_rows, int vocab) {
 // the row is drawn whole, its largest logit and its weight already known.  (One row of 151,936 random logits, top-p
 // of 0.9: at a spread that keeps a thousand tokens or so 107 -> 42 us, at three times the spread 40, at a sixth of it,
 // where most of the vocabulary is kept and the row is drawn whole, 106; the candidates are about the largest 6 % of the
-// row.  With 64 rows the launches before the row's block cost what they save.)
+// row.  64 rows: 125 -> 91, 120 -> 86 and, drawn whole, 135 -> 160.)
 // 151,936 logits, top-k of 50: 86 -> 29 us for one row, 33 for eight, 94 -> 61 for 64; with top-p of 0.9 as well 128 -> 39, 42, 143 -> 70.
 
 #define CANDIDATES_UP_TO_K 128
 #define CANDIDATE_PLACES 144   // per chunk at most; used(k) = k + 8 rounded up to 16
-#define CANDIDATES_FOR_TOP_P_UP_TO_ROWS 32
+#define CANDIDATES_FOR_TOP_P_UP_TO_ROWS 64
 
 __host__ __device__ inline int candidate_places(int k) { return (k + 8 + 15) / 16 * 16; }
 

@@ -317,7 +317,7 @@ def test_a_top_p_draw_goes_through_the_candidates_where_its_share_lies_within_th
         uniform = np.random.default_rng(seed).random(rows).astype(np.float32)
         tokens, bad = torch.empty(rows, dtype=torch.int32, device=DEVICE), torch.empty(rows, dtype=torch.int32, device=DEVICE)
         uniform_device = dev(uniform)
-        for some in (slice(0, 32), slice(32, rows)):      # (a top-p alone goes this way for up to 32 rows a call)
+        for some in (slice(0, 32), slice(32, rows)):      # (a top-p alone goes this way for up to 64 rows a call; here in two calls)
             K.sample(device["logits"][some], tokens[some], bad[some], temperature=device["temperature"][some],
                      top_k=device["top_k"][some] if with_k else None, top_p=device["top_p"][some], uniform=uniform_device[some])
         whole, whole_bad = torch.empty_like(tokens), torch.empty_like(bad)
