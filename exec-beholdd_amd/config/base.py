@@ -56,7 +56,10 @@ class ConfigReader:
             return default
         return self.data[key]
 
-    def integer(self, key: str, default=_MISSING, minimum: int | None = None) -> int:
+    # The kernels take their sizes as 32-bit integers: no size in a configuration may be larger.
+    MOST = 2 ** 31 - 1
+
+    def integer(self, key: str, default=_MISSING, minimum: int | None = None, maximum: int | None = MOST) -> int:
         value = self.raw(key, default)
         if isinstance(value, bool) or not isinstance(value, int):
             if isinstance(value, float) and value.is_integer():
@@ -65,6 +68,8 @@ class ConfigReader:
                 raise ConfigError(f"{self.origin}: {key!r} must be an integer, got {value!r}")
         if minimum is not None and value < minimum:
             raise ConfigError(f"{self.origin}: {key!r} must be at least {minimum}, got {value}")
+        if maximum is not None and value > maximum:
+            raise ConfigError(f"{self.origin}: {key!r} must be at most {maximum}, got {value}")
         return value
 
     def number(self, key: str, default=_MISSING) -> float:

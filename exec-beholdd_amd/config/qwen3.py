@@ -58,7 +58,7 @@ class Qwen3Config:
         names = data.get("architectures")
         architecture = names[0] if isinstance(names, list) and names else "Qwen3ForCausalLM"
 
-        n_layers = r.integer("num_hidden_layers", minimum=1)
+        n_layers = r.integer("num_hidden_layers", minimum=1, maximum=1 << 20)      # (a part object and a cache entry each)
         hidden = r.integer("hidden_size", minimum=1)
         n_heads = r.integer("num_attention_heads", minimum=1)
         n_kv_heads = r.integer("num_key_value_heads", minimum=1)

@@ -50,6 +50,8 @@ def test_head_dim_defaults_only_when_it_divides(tiny_configs):
     ({"rms_norm_eps": -1e-6}, "epsilon"),
     ({"rope_theta": 0}, "RoPE base"),
     ({"num_hidden_layers": 0}, "at least 1"),
+    ({"num_hidden_layers": 2 ** 40}, "at most"),         # (a list of that many layers would never be finished)
+    ({"hidden_size": 2 ** 31}, "at most"),               # the kernels take 32-bit sizes
     ({"vocab_size": "many"}, "integer"),
     ({"hidden_size": 64.5}, "integer"),
     ({"attention_bias": True}, "attention_bias"),
