@@ -116,6 +116,15 @@ class Replayer:
             if item["id"] in seen:
                 raise TraceError(f"step {step}: request {item['id']!r} occurs twice")
             seen.add(item["id"])
+        ended = set()
+        for name in record.get("end", []):      # and an end that cannot be, before anything has run
+            if not isinstance(name, (str, int)) or isinstance(name, bool):
+                raise TraceError(f"step {step}: 'end' lists request ids (strings or integers), got {name!r}")
+            if name in ended:
+                raise TraceError(f"step {step}: request {name!r} ends twice")
+            if name not in self.slot_of and name not in seen:
+                raise TraceError(f"step {step}: request {name!r} ends but was never started")
+            ended.add(name)
         entries, fresh, places = [], [], []
         for item in record["entries"]:
             name = item["id"]
@@ -141,8 +150,6 @@ class Replayer:
             os.replace(path + ".tmp", path)
             self.capture.add(step, places, data)
         for name in record.get("end", []):
-            if name not in self.slot_of:
-                raise TraceError(f"step {step}: request {name!r} ends but was never started")
             self.engine.free_slot(self.slot_of.pop(name))
             self.generation[name] = self.generation.get(name, 0) + 1
 

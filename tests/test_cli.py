@@ -148,6 +148,11 @@ def test_trace_replay_on_the_kernel_double(model_dirs, tmp_path):
         with pytest.raises(replay.TraceError, match=message):
             player.run_step({"step": 6, "entries": entries, "end": []})
         assert engine.cache.live_slots() == [] and player.slot_of == {}
+    # an end that cannot be is refused before anything runs: the step's own requests are not started either
+    for end, message in ((["nobody"], "never started"), (["f", "f"], "ends twice"), ([["f"]], "strings or integers"), ([True], "strings or integers")):
+        with pytest.raises(replay.TraceError, match=message):
+            player.run_step({"step": 7, "entries": [{"id": "f", "tokens": [1, 2], "want": [1]}], "end": end})
+        assert engine.cache.live_slots() == [] and player.slot_of == {} and not os.path.exists(tmp_path / "out" / "7.f32")
     # an id that is used again after its request ended is another request in the capture
     player.run_step({"step": 5, "entries": [{"id": "a", "tokens": b, "want": [1]}], "end": ["a"]})
     player.close()
