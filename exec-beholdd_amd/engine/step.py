@@ -37,6 +37,10 @@ def check_entries(entries: list, cache, vocab: int) -> None:
     if not entries:
         raise StepError("a step needs at least one entry")
     for index, entry in enumerate(entries):
+        if not isinstance(entry.slot, (int, np.integer)) or isinstance(entry.slot, bool):
+            raise StepError(f"entry {index}: the slot is an integer, got {entry.slot!r}")
+        if not isinstance(entry.tokens, (list, tuple)) or not isinstance(entry.want, (list, tuple)):
+            raise StepError(f"entry {index} (slot {entry.slot}): tokens and wanted places are lists")
         n_new = len(entry.tokens)
         if n_new == 0:
             raise StepError(f"entry {index} (slot {entry.slot}) brings no tokens")

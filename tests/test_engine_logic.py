@@ -61,7 +61,10 @@ def test_step_refuses_bad_entries_without_changing_lengths(model_dirs):
     engine.step([StepEntry(slot, [1, 2, 3], [2])])
     for bad in ([StepEntry(slot, [], [])], [StepEntry(slot, [256], [0])], [StepEntry(slot, [-1], [0])],
                 [StepEntry(slot, [1], [1])], [StepEntry(slot, [1], [0]), StepEntry(slot, [2], [0])],
-                [StepEntry(slot + 1, [1], [0])], []):
+                [StepEntry(slot + 1, [1], [0])], [],
+                # wrong types are refused with a reason too, not with a traceback from the middle of the step
+                [StepEntry(slot, 7, [0])], [StepEntry(slot, [1], 0)], [StepEntry([slot], [1], [0])], [StepEntry(True, [1], [0])],
+                [StepEntry(slot, [1.5], [0])], [StepEntry(slot, None, [])]):
         with pytest.raises((StepError, beholdd.cache.CacheError)):
             engine.step(bad)
         assert engine.cache.length(slot) == 3
