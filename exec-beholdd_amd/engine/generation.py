@@ -31,6 +31,7 @@ reasons are those of the plain loop.
 
 from __future__ import annotations
 
+import numbers
 from dataclasses import dataclass, field
 
 from ..sampling import SamplingParams
@@ -83,6 +84,10 @@ def plan_batches(prompt_lens: list, max_new: list, page_size: int, capacity_page
     return batches
 
 
+def _whole_number(value) -> bool:
+    return isinstance(value, numbers.Integral) and not isinstance(value, bool)
+
+
 def generate(stepper, prompts: list, max_new_tokens, sampling=None, stop_token_ids=(), on_token=None,
              batch_size: int | None = None, control=None, on_logits=None) -> list:
     """Generate for every prompt (a list of token ids each).
@@ -92,6 +97,8 @@ def generate(stepper, prompts: list, max_new_tokens, sampling=None, stop_token_i
     `control()` is polled before every step and may raise to cancel;
     `on_logits(request_index, step, logits_row)` sees the device row each token is chosen from.
     """
+    if not isinstance(prompts, (list, tuple)):
+        raise GenerationError(f"prompts are a list of lists of token ids, got {prompts!r}")
     n = len(prompts)
     max_new = list(max_new_tokens) if isinstance(max_new_tokens, (list, tuple)) else [max_new_tokens] * n
     if sampling is None:
@@ -99,10 +106,18 @@ def generate(stepper, prompts: list, max_new_tokens, sampling=None, stop_token_i
     params = list(sampling) if isinstance(sampling, (list, tuple)) else [sampling] * n
     if len(max_new) != n or len(params) != n:
         raise GenerationError("one max_new_tokens and one sampling parameter set per prompt")
+    if not isinstance(stop_token_ids, (list, tuple, set, frozenset)) or not all(_whole_number(t) for t in stop_token_ids):
+        raise GenerationError(f"stop_token_ids are a list of token ids, got {stop_token_ids!r}")
     stops = frozenset(int(t) for t in stop_token_ids)
+    if batch_size is not None and not _whole_number(batch_size):
+        raise GenerationError(f"batch_size is an integer or None, got {batch_size!r}")
     for index, (prompt, n_new) in enumerate(zip(prompts, max_new)):
+        if not isinstance(prompt, (list, tuple)):
+            raise GenerationError(f"request {index}: a prompt is a list of token ids, got {prompt!r}")
         if len(prompt) == 0:
             raise GenerationError(f"request {index}: generation requires at least one prompt token")
+        if not _whole_number(n_new):
+            raise GenerationError(f"request {index}: max_new_tokens is an integer, got {n_new!r}")
         if n_new < 0:
             raise GenerationError(f"request {index}: max_new_tokens must not be negative")
         needed = positions_needed(len(prompt), n_new)

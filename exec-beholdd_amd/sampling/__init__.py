@@ -10,11 +10,13 @@ batch a request happens to be in.
 
 from __future__ import annotations
 
+import numbers
 from dataclasses import dataclass
 
 import torch
 
 _MASK = (1 << 64) - 1
+_MOST_TOP_K = (1 << 31) - 1     # the kernel takes it as a 32-bit integer; beyond the vocabulary it filters nothing
 
 
 @dataclass(frozen=True)
@@ -25,10 +27,18 @@ class SamplingParams:
     seed: int = 0
 
     def __post_init__(self):
-        if not (self.temperature >= 0.0):
-            raise ValueError(f"temperature must not be negative, got {self.temperature}")
-        if self.top_k < 0:
-            raise ValueError(f"top_k must not be negative, got {self.top_k}")
+        for name in ("temperature", "top_p"):
+            value = getattr(self, name)
+            if isinstance(value, bool) or not isinstance(value, numbers.Real):
+                raise ValueError(f"{name} is a number, got {value!r}")
+        for name in ("top_k", "seed"):
+            value = getattr(self, name)
+            if isinstance(value, bool) or not isinstance(value, numbers.Integral):
+                raise ValueError(f"{name} is an integer, got {value!r}")
+        if not (0.0 <= self.temperature < float("inf")):
+            raise ValueError(f"temperature must be finite and not negative, got {self.temperature}")
+        if not (0 <= self.top_k <= _MOST_TOP_K):
+            raise ValueError(f"top_k must be in 0 .. {_MOST_TOP_K} (0 = off), got {self.top_k}")
         if not (0.0 < self.top_p <= 1.0):
             raise ValueError(f"top_p must be in (0, 1], got {self.top_p}")
 

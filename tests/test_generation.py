@@ -182,9 +182,32 @@ def test_uniform_numbers_are_a_pure_function_of_seed_request_step():
     assert uniform(1, 2, 3) == uniform(1, 2, 3)
     mean = sum(uniform(0, 0, t) for t in range(4000)) / 4000
     assert abs(mean - 0.5) < 0.03
-    for bad in (dict(temperature=-1.0), dict(top_k=-1), dict(top_p=0.0), dict(top_p=1.5)):
+    for bad in (dict(temperature=-1.0), dict(top_k=-1), dict(top_p=0.0), dict(top_p=1.5),
+                dict(temperature=float("nan")), dict(temperature=float("inf")), dict(temperature="0.8"),
+                dict(temperature=[0.8]), dict(top_k=1.5), dict(top_k=None), dict(top_k=1 << 40), dict(top_k=True),
+                dict(top_p=None), dict(top_p=[0.5]), dict(top_p=float("nan")), dict(seed=None), dict(seed=0.5)):
         with pytest.raises(ValueError):
             SamplingParams(**bad)
+    import numpy as np
+    assert SamplingParams(temperature=np.float32(0.5), top_k=np.int64(3), seed=np.int32(2)).top_k == 3
+
+
+def test_arguments_of_the_wrong_type_are_refused_with_a_reason():
+    s = ScriptedStepper()
+    for prompts, wrong in ((7, "prompts are a list"), ([[1], 5], "request 1: a prompt is a list"),
+                           ([[1], "ab"], "request 1: a prompt is a list")):
+        with pytest.raises(GenerationError, match=wrong):
+            generate(s, prompts, 1)
+    for n_new in ("3", 1.5, None, True):
+        with pytest.raises(GenerationError, match="max_new_tokens is an integer"):
+            generate(s, [[1]], n_new)
+    for stops in (3, None, [0.5], ["a"], 2.0):
+        with pytest.raises(GenerationError, match="stop_token_ids are a list"):
+            generate(s, [[1]], 1, stop_token_ids=stops)
+    for size in ("2", 1.5, (1, 2)):
+        with pytest.raises(GenerationError, match="batch_size is an integer"):
+            generate(s, [[1]], 1, batch_size=size)
+    assert s.state == {} and s.steps == []
 
 
 # ---- the loop that runs one step ahead of the host ------------------------------------------------
