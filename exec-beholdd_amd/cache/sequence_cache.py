@@ -23,6 +23,7 @@ before anything is allocated (recorded_attention.rs:244-299).
 from __future__ import annotations
 
 import heapq
+import numbers
 from dataclasses import dataclass, field
 
 import torch
@@ -85,11 +86,22 @@ class _Group:
         self.pages_of: dict = {}     # slot -> list of page ids (or -1 once released), position order
 
 
+_MOST_SLOTS = 1 << 20     # every slot has a place in the free list and a row in each table
+
+
 class SequenceCache:
     def __init__(self, entry_needs: dict, max_tokens: int, dtype: torch.dtype, device, page_size: int,
                  max_slots: int | None = None, max_position: int | None = None):
+        for name, value, optional in (("max_tokens", max_tokens, False), ("max_slots", max_slots, True),
+                                      ("max_position", max_position, True)):
+            if value is None and optional:
+                continue
+            if isinstance(value, bool) or not isinstance(value, numbers.Integral) or not 0 <= value < 1 << 40:
+                raise ValueError(f"{name} is a count of tokens or sequences (an integer below 2^40), got {value!r}")
         if max_tokens <= 0:
             raise ValueError("the cache must hold at least one token")
+        if max_slots is not None and max_slots > _MOST_SLOTS:
+            raise ValueError(f"max_slots is at most {_MOST_SLOTS}, got {max_slots}")
         self.page_size = int(page_size)
         self.n_pages = -(-int(max_tokens) // self.page_size)
         self.max_slots = int(max_slots) if max_slots else min(self.n_pages, 1024)

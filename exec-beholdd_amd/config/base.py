@@ -96,7 +96,10 @@ class ConfigReader:
 
 def read_config_json(model_dir_or_file: str) -> tuple[dict, str]:
     """Return (dictionary, path) of a model folder's config.json or of a JSON file itself."""
-    path = model_dir_or_file
+    if not isinstance(model_dir_or_file, (str, os.PathLike)):
+        # an integer would be taken for an open file's number by the calls below
+        raise ConfigError(f"a model folder is named by a path, got {model_dir_or_file!r}")
+    path = os.fspath(model_dir_or_file)
     if os.path.isdir(path):
         path = os.path.join(path, "config.json")
     try:

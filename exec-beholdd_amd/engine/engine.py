@@ -9,6 +9,8 @@ reference's embedded API (crates/beholdd-embed/src/lib.rs:51-105): construct onc
 
 from __future__ import annotations
 
+import numbers
+
 import torch
 
 from ..cache import SequenceCache
@@ -64,8 +66,13 @@ class Engine:
             from ..kernels import HipKernels   # fails loudly without a GPU or the library
             kernels = HipKernels(self.device)
         self.kernels = kernels
-        if max_rows_per_step is not None and max_rows_per_step <= 0:
-            raise ValueError("max_rows_per_step must be positive")
+        for name, value, least, optional in (("max_rows_per_step", max_rows_per_step, 1, True), ("graph_limit", graph_limit, 0, False),
+                                             ("graph_rows_per_sequence", graph_rows_per_sequence, 1, False),
+                                             ("memory_limit_bytes", memory_limit_bytes, 0, True)):
+            if value is None and optional:
+                continue
+            if isinstance(value, bool) or not isinstance(value, numbers.Integral) or value < least:
+                raise ValueError(f"{name} is an integer of at least {least}{' or None' if optional else ''}, got {value!r}")
         with_graphs = bool(use_graphs and self.device.type == "cuda")
 
         def make_cache(built):

@@ -161,3 +161,17 @@ def test_no_gpu_means_no_engine(model_dirs):
         pytest.skip("a GPU is present")
     with pytest.raises(beholdd.kernels.KernelError, match="no CPU fallback"):
         Engine(model_dirs("A", "float32"), dtype="float32", max_tokens=64)
+
+
+def test_an_engine_refuses_arguments_that_cannot_be_meant(model_dirs):
+    folder = model_dirs("A", "float32")
+    for number in (0, 1, 64):       # an integer would name an open file of the process, not a folder
+        with pytest.raises(beholdd.ConfigError, match="named by a path"):
+            make_engine(number)
+    for bad in (dict(max_tokens="64"), dict(max_tokens=1 << 70), dict(max_tokens=1.5), dict(max_tokens=0),
+                dict(max_slots=-1), dict(max_slots=[1]), dict(max_slots=1 << 39), dict(max_rows_per_step="7"),
+                dict(max_rows_per_step=float("inf")), dict(max_rows_per_step=0), dict(graph_rows_per_sequence={}),
+                dict(graph_rows_per_sequence=0), dict(graph_limit=None), dict(memory_limit_bytes="1000"),
+                dict(memory_limit_bytes=1.5), dict(dtype="float16")):
+        with pytest.raises(ValueError):
+            make_engine(folder, **bad)
