@@ -154,9 +154,15 @@ __global__ __launch_bounds__(256, (LEAN ? 2 : 1)) void attention_mfma_kernel(
   const int kvh = unit % KVH, z = unit / KVH;
   const int seq = z / n_splits, split = z % n_splits;
   const int G = H / KVH;
-  const int row0 = seq_start[seq];
-  const int n_cols = (seq_start[seq + 1] - row0) * G;
+  // FUSED is a decode step: sequence s has the one row s, and nobody waits for `seq_start` to say so
+  const int row0 = FUSED ? seq : seq_start[seq];
+  const int n_cols = FUSED ? G : (seq_start[seq + 1] - row0) * G;
   if (tile * 16 >= n_cols) return;
+  // The number of this wave's first page, if no window cuts the front off, is asked for beside the row's position
+  // instead of after it: one trip to memory less before the first key is on its way.
+  const int32_t* table = page_table + (size_t)seq * table_stride;
+  const int first_guess = split * pages_per_split + (int)(threadIdx.x / 64);
+  const int page_guess = first_guess < table_stride ? table[first_guess] : 0;
 
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int j = lane % 16, g = lane / 16;
@@ -212,7 +218,6 @@ __global__ __launch_bounds__(256, (LEAN ? 2 : 1)) void attention_mfma_kernel(
   const int begin = lo_min / BH_PAGE + split * pages_per_split;
   const int last = pos_max >= 0 ? pos_max / BH_PAGE : -1;
   const int end = (begin + pages_per_split < last + 1) ? begin + pages_per_split : last + 1;
-  const int32_t* table = page_table + (size_t)seq * table_stride;
 
   f32x4_t o[2 * NS];
   float run_max = -INFINITY, run_sum = 0.f;  // run_sum: this lane's share of the column's sum
@@ -295,7 +300,8 @@ __global__ __launch_bounds__(256, (LEAN ? 2 : 1)) void attention_mfma_kernel(
     }
   };
 
-  int page_ahead = (begin + wave < end) ? table[begin + wave] : 0;   // a page's number is asked for one page early
+  // a page's number is asked for one page early
+  int page_ahead = (begin + wave < end) ? (begin + wave == first_guess ? page_guess : table[begin + wave]) : 0;
   for (int p = begin + wave; p < end; p += 4) {
     const int page = page_ahead;
     if (p + 4 < end) page_ahead = table[p + 4];
@@ -415,6 +421,12 @@ __global__ void attention_combine_kernel(const float* __restrict__ part_o, const
   const size_t column = blockIdx.x;
   const float* ml = part_ml + column * n_splits * 2;
   const int lane = threadIdx.x % BH_WAVE;
+  // the first eight splits' outputs are asked for beside the maxima and sums, not after them
+  float first_part[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (threadIdx.x < HD) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) first_part[u] = part_o[(column * n_splits + (u < n_splits ? u : n_splits - 1)) * HD + threadIdx.x];
+  }
   float top = -INFINITY;
   for (int s = lane; s < n_splits; s += BH_WAVE) top = fmaxf(top, ml[2 * s]);
 #pragma unroll
@@ -432,7 +444,7 @@ __global__ void attention_combine_kernel(const float* __restrict__ part_o, const
       for (int u = 0; u < 8; ++u) {
         const int s = s0 + u < n_splits ? s0 + u : n_splits - 1;
         weight[u] = s0 + u < n_splits ? ml[2 * s] : -INFINITY;
-        part[u] = part_o[(column * n_splits + s) * HD + d];
+        part[u] = (s0 == 0 && d == threadIdx.x) ? first_part[u] : part_o[(column * n_splits + s) * HD + d];
       }
 #pragma unroll
       for (int u = 0; u < 8; ++u) value += part[u] * exp2f(weight[u] - top);
@@ -570,7 +582,8 @@ extern "C" int bh_attention_bf16(const void* q, void* out, void* part_o, void* p
 // A decode step (one row per sequence) straight from the fused projection rows [q heads | k heads | v heads]:
 // per-head RMSNorm of q and k (weights may be null), rotation over the whole head at the row's position
 // (tables may be null), the new key and value into the cache (unless write_kv is 0: the entry is another
-// layer's), and attention over the cache and the new key.  See struct FusedQkv.
+// layer's), and attention over the cache and the new key.  See struct FusedQkv.  Row s is sequence s's: `seq_start`
+// can only say so (0, 1, ..., n_seqs) and is not read.
 extern "C" int bh_attention_decode_fused(const void* qkv, void* out, void* part_o, void* part_ml, void* k_pages,
                                          void* v_pages, const int32_t* page_table, int table_stride,
                                          const int32_t* positions, const int32_t* seq_start, int n_seqs, int H,

@@ -140,6 +140,25 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
   const int i = lane % 16, g = lane / 16;
   const int n0 = blockIdx.x * 16;
   const int full = K / 64;
+  // What a float32 output holds before this product adds to it, and the weight of the norm behind: each thread knows
+  // the elements it will write, and asks for them here, so that nobody waits for them behind the main loop (the
+  // residual was written by another kernel, on other XCDs: it comes from beyond this XCD's L2).
+  constexpr int OUT_PASSES = (MB * 256 + WAVES * 64 - 1) / (WAVES * 64);
+  constexpr bool OUT_EARLY = RT == 1 && sizeof(TC) == 4;
+  float before[OUT_PASSES], behind_gain[OUT_PASSES];
+  if (OUT_EARLY) {
+#pragma unroll
+    for (int pass = 0; pass < OUT_PASSES; ++pass) {
+      const int e = threadIdx.x + pass * WAVES * 64;
+      const int m = e / 256 * 16 + (e % 256) / 16, n = n0 + e % 16;
+      const bool valid = e < MB * 256 && m < M && n < N;
+      before[pass] = (valid && accumulate) ? reinterpret_cast<const float*>(c)[(size_t)m * N + n] : 0.f;
+      behind_gain[pass] = 0.f;
+      if (valid && norm.behind_weight)
+        behind_gain[pass] = norm.behind_weight_f32 ? reinterpret_cast<const float*>(norm.behind_weight)[n]
+                                                   : bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(norm.behind_weight)[n]);
+    }
+  }
   // per row block: base pointer, distance between consecutive 64-wide chunks, distance to the second half
   const uint16_t* wp[RT];
   const size_t chunk_stride = TILES ? 1024 : 64;
@@ -257,7 +276,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
 #pragma unroll
       for (int r = 0; r < 4; ++r) partial[wave][t][b][i * 16 + 4 * g + r] = acc[t][b][r];
   __syncthreads();
-  for (int e = threadIdx.x; e < MB * 256; e += WAVES * 64) {   // whole waves enter or stay out
+#pragma unroll
+  for (int pass = 0; pass < OUT_PASSES; ++pass) {
+    const int e = threadIdx.x + pass * WAVES * 64;
+    if (e >= MB * 256) break;   // whole waves enter or stay out
     const int b = e / 256, m = b * 16 + (e % 256) / 16, n = n0 + e % 16;
     const bool valid = m < M && n < N;
     float sum[RT];
@@ -272,24 +294,21 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const uint16_t*
     if (valid) {
       if (RT == 2) {
         store_out<TC>(c, (size_t)bh_rows_index(blocks.c, m, n, N), silu_mul(sum[0], sum[RT - 1]), false);
-      } else if (norm.behind_weight) {
-        float* cf = reinterpret_cast<float*>(c);
-        value = accumulate ? cf[(size_t)m * N + n] + sum[0] : sum[0];
-        cf[(size_t)m * N + n] = value;
+      } else if (OUT_EARLY) {
+        value = accumulate ? before[pass] + sum[0] : sum[0];
+        reinterpret_cast<float*>(c)[(size_t)m * N + n] = value;
       } else {
         store_out<TC>(c, (size_t)m * N + n, sum[0], accumulate != 0);
       }
     }
-    if (RT == 1 && norm.behind_weight) {
+    if (RT == 1 && norm.behind_weight) {   // (float32 output)
       float sq = value * value;   // 0 where there is no element
       sq += __shfl_xor(sq, 8, 64);   // the 16 columns of a row sit in 16 neighbouring lanes
       sq += __shfl_xor(sq, 4, 64);
       sq += __shfl_xor(sq, 2, 64);
       sq += __shfl_xor(sq, 1, 64);
       if (valid) {
-        const float g = norm.behind_weight_f32 ? reinterpret_cast<const float*>(norm.behind_weight)[n]
-                                               : bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(norm.behind_weight)[n]);
-        norm.behind_rows[bh_rows_index(blocks.behind, m, n, N)] = f32_to_bf16_bits(value * g);
+        norm.behind_rows[bh_rows_index(blocks.behind, m, n, N)] = f32_to_bf16_bits(value * behind_gain[pass]);
         if (e % 16 == 0) norm.behind_ss[(size_t)m * gridDim.x + blockIdx.x] = sq;
       }
     }
@@ -344,6 +363,26 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_span_kernel(const uint
     hi[t] = min(min(first_row + span, N), tile_row + 16) - tile_row;
     const int tile = min(first_tile + t, N / 16 - 1);   // (a block beyond the matrix is never loaded; its address stays inside)
     wp[t] = w + (size_t)tile * full * 1024 + lane * 8;
+  }
+  // what a float32 output holds before this product adds to it, and the weight of the norm behind, asked for here as
+  // in the kernel above
+  constexpr int OUT_PASSES = (MB * 256 + WAVES * 64 - 1) / (WAVES * 64);
+  constexpr bool OUT_EARLY = sizeof(TC) == 4;
+  float before[OUT_PASSES][SPAN_TILES], behind_gain[OUT_PASSES][SPAN_TILES];
+  if (OUT_EARLY) {
+#pragma unroll
+    for (int pass = 0; pass < OUT_PASSES; ++pass)
+#pragma unroll
+      for (int t = 0; t < SPAN_TILES; ++t) {
+        const int e = threadIdx.x + pass * WAVES * 64;
+        const int m = e / 256 * 16 + (e % 256) / 16, column = e % 16, n = (first_tile + t) * 16 + column;
+        const bool valid = e < MB * 256 && m < M && column >= lo[t] && column < hi[t];
+        before[pass][t] = (valid && accumulate) ? reinterpret_cast<const float*>(c)[(size_t)m * N + n] : 0.f;
+        behind_gain[pass][t] = 0.f;
+        if (valid && norm.behind_weight)
+          behind_gain[pass][t] = norm.behind_weight_f32 ? reinterpret_cast<const float*>(norm.behind_weight)[n]
+                                                        : bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(norm.behind_weight)[n]);
+      }
   }
   const uint16_t* xp[MB];
   constexpr int x_half = XB ? XB * 8 : 8, x_chunk = XB ? 64 * XB : 64;
@@ -440,7 +479,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_span_kernel(const uint
 #pragma unroll
       for (int r = 0; r < 4; ++r) partial[wave][t][b][i * 16 + 4 * g + r] = acc[t][b][r];
   __syncthreads();
-  for (int e = threadIdx.x; e < MB * 256; e += WAVES * 64) {   // whole waves enter or stay out
+#pragma unroll
+  for (int pass = 0; pass < OUT_PASSES; ++pass) {
+    const int e = threadIdx.x + pass * WAVES * 64;
+    if (e >= MB * 256) break;   // whole waves enter or stay out
     const int b = e / 256, m = b * 16 + (e % 256) / 16, column = e % 16;
     float sq = 0.f;   // of what this workgroup adds to row m of the residual (norm.behind_weight)
 #pragma unroll
@@ -452,14 +494,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_span_kernel(const uint
       for (int v = 0; v < WAVES; ++v) sum += partial[v][t][b][e % 256];
       if (norm.ahead_ss) sum *= row_factor[m];
       if (!valid) continue;
-      if (norm.behind_weight) {   // float32 output
-        float* cf = reinterpret_cast<float*>(c);
-        const float value = accumulate ? cf[(size_t)m * N + n] + sum : sum;
-        cf[(size_t)m * N + n] = value;
-        sq += value * value;
-        const float gw = norm.behind_weight_f32 ? reinterpret_cast<const float*>(norm.behind_weight)[n]
-                                                : bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(norm.behind_weight)[n]);
-        norm.behind_rows[bh_rows_index(blocks.behind, m, n, N)] = f32_to_bf16_bits(value * gw);
+      if (OUT_EARLY) {
+        const float value = accumulate ? before[pass][t] + sum : sum;
+        reinterpret_cast<float*>(c)[(size_t)m * N + n] = value;
+        if (norm.behind_weight) {
+          sq += value * value;
+          norm.behind_rows[bh_rows_index(blocks.behind, m, n, N)] = f32_to_bf16_bits(value * behind_gain[pass][t]);
+        }
       } else {
         store_out<TC>(c, (size_t)m * N + n, sum, accumulate != 0);
       }
