@@ -240,7 +240,6 @@ def main():
         print(json.dumps(sampling_times(torch)))
         return 0
 
-    import beholdd
     from beholdd.engine import Engine, random_model_on_device
 
     shape_name, shape = SHAPES[args.shape]

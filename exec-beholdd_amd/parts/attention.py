@@ -16,8 +16,6 @@ from __future__ import annotations
 
 import math
 
-import torch
-
 from ..weights.binder import TensorSpec
 from .base import MIXERS, CacheNeed
 from .linear import Linear

@@ -9,7 +9,7 @@ import pytest
 import torch
 
 import beholdd
-from beholdd.weights import (SafetensorsError, SafetensorsReader, TensorSpec, WeightError, bind, check_manifest,
+from beholdd.weights import (SafetensorsError, SafetensorsReader, TensorSpec, WeightError, check_manifest,
                              random_tensor, stored_dtype, write_safetensors)
 
 
