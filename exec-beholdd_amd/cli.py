@@ -280,3 +280,16 @@ def main(argv=None, out=None) -> int:
     except UsageError as error:
         print(f"error: {error}\n{USAGE}", file=sys.stderr)
         return 2
+    except (ValueError, OSError, *_library_errors()) as error:
+        # a value that some part refuses, a file that is not there, a model that does not fit: one line, not a traceback
+        print(f"error: {error}", file=sys.stderr)
+        return 1
+
+
+def _library_errors() -> tuple:
+    from .cache import CacheError
+    from .engine.engine import MemoryBudgetError
+    from .kernels import KernelError
+    from .kernels.build import BuildError
+    from .sampling import SamplingError
+    return (CacheError, MemoryBudgetError, BuildError, KernelError, SamplingError)

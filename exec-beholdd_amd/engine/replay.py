@@ -16,7 +16,7 @@ import sys
 
 import numpy as np
 
-from .engine import Engine
+from .engine import Engine, MemoryBudgetError
 from ..cache.sequence_cache import CacheError
 from .step import StepEntry, StepError
 
@@ -170,9 +170,15 @@ def main(argv=None, stdin=None, stdout=None) -> int:
         print(f"trace_run: {error}\nusage: trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N "
               "[--capture FILE]", file=sys.stderr)
         return 2
-    engine = Engine(args["--model"], dtype=args["--dtype"], max_tokens=args["--max-tokens"])
-    replayer = Replayer(engine, args["--out"], args["--capture"],
-                        notes={"dtype": args["--dtype"], "max_tokens": args["--max-tokens"], "tool": "trace_run"})
+    from ..kernels import KernelError
+    from ..kernels.build import BuildError
+    try:
+        engine = Engine(args["--model"], dtype=args["--dtype"], max_tokens=args["--max-tokens"])
+        replayer = Replayer(engine, args["--out"], args["--capture"],
+                            notes={"dtype": args["--dtype"], "max_tokens": args["--max-tokens"], "tool": "trace_run"})
+    except (ValueError, OSError, CacheError, MemoryBudgetError, KernelError, BuildError) as error:
+        print(f"trace_run: {error}", file=sys.stderr)      # no such model, a tensor that does not fit, no GPU: its reason
+        return 1
     try:
         for line in stdin:
             line = line.strip()

@@ -249,3 +249,20 @@ def test_compare_command(tmp_path, capsys):
     assert run(["compare", str(tmp_path / "g1"), whole])[0] == 1
     assert run(["compare", whole])[0] == 2
 
+
+
+def test_refused_values_and_missing_files_are_one_line_not_a_traceback(tmp_path, capsys, model_dirs):
+    base = ["generate", "--model", model_dirs("A"), "--plan-only"]
+    for extra, message in ((["--prompt-ids-file", str(tmp_path / "absent")], "No such file"),
+                           (["--prompt-ids", "1,2", "--dtype", "float16"], "engine dtype must be bfloat16 or float32"),
+                           (["--prompt-ids", "1,2", "--max-tokens", "-1"], "max_tokens")):
+        code, _ = run(base + extra)
+        error = capsys.readouterr().err
+        assert code == 1 and error.startswith("error: ") and message in error and "Traceback" not in error, error
+    code, _ = run(["generate", "--model", str(tmp_path / "no_model"), "--prompt-ids", "1", "--plan-only"])
+    assert code == 1 and "no such file" in capsys.readouterr().err
+    import torch
+    if not torch.cuda.is_available():
+        argv = ["--model", model_dirs("A"), "--dtype", "float32", "--out", str(tmp_path / "out"), "--max-tokens", "64"]
+        assert replay.main(argv, stdin=io.StringIO("")) == 1
+        assert capsys.readouterr().err.startswith("trace_run: no GPU is visible")
