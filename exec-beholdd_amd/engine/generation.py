@@ -88,6 +88,11 @@ def _whole_number(value) -> bool:
     return isinstance(value, numbers.Integral) and not isinstance(value, bool)
 
 
+def _token_sequence(value) -> bool:
+    """A list, a tuple, an array: something with a length that can be gone through, and no text."""
+    return hasattr(value, "__len__") and hasattr(value, "__iter__") and not isinstance(value, (str, bytes, dict))
+
+
 def generate(stepper, prompts: list, max_new_tokens, sampling=None, stop_token_ids=(), on_token=None,
              batch_size: int | None = None, control=None, on_logits=None) -> list:
     """Generate for every prompt (a list of token ids each).
@@ -97,7 +102,7 @@ def generate(stepper, prompts: list, max_new_tokens, sampling=None, stop_token_i
     `control()` is polled before every step and may raise to cancel;
     `on_logits(request_index, step, logits_row)` sees the device row each token is chosen from.
     """
-    if not isinstance(prompts, (list, tuple)):
+    if not _token_sequence(prompts):
         raise GenerationError(f"prompts are a list of lists of token ids, got {prompts!r}")
     n = len(prompts)
     max_new = list(max_new_tokens) if isinstance(max_new_tokens, (list, tuple)) else [max_new_tokens] * n
@@ -112,7 +117,7 @@ def generate(stepper, prompts: list, max_new_tokens, sampling=None, stop_token_i
     if batch_size is not None and not _whole_number(batch_size):
         raise GenerationError(f"batch_size is an integer or None, got {batch_size!r}")
     for index, (prompt, n_new) in enumerate(zip(prompts, max_new)):
-        if not isinstance(prompt, (list, tuple)):
+        if not _token_sequence(prompt):
             raise GenerationError(f"request {index}: a prompt is a list of token ids, got {prompt!r}")
         if len(prompt) == 0:
             raise GenerationError(f"request {index}: generation requires at least one prompt token")

@@ -32,6 +32,12 @@ class StepEntry:
                                                # at this row of the sampler's device buffer, not yet seen by the host
 
 
+def _sequence(value) -> bool:
+    """A list, a tuple or a one-dimensional array: something with a length that can be gone through, and no text."""
+    return (hasattr(value, "__len__") and hasattr(value, "__iter__") and not isinstance(value, (str, bytes, dict))
+            and getattr(value, "ndim", 1) == 1)
+
+
 def check_entries(entries: list, cache, vocab: int) -> None:
     """Refuse malformed entries before anything is changed or computed."""
     if not entries:
@@ -39,7 +45,7 @@ def check_entries(entries: list, cache, vocab: int) -> None:
     for index, entry in enumerate(entries):
         if not isinstance(entry.slot, (int, np.integer)) or isinstance(entry.slot, bool):
             raise StepError(f"entry {index}: the slot is an integer, got {entry.slot!r}")
-        if not isinstance(entry.tokens, (list, tuple)) or not isinstance(entry.want, (list, tuple)):
+        if not _sequence(entry.tokens) or not _sequence(entry.want):
             raise StepError(f"entry {index} (slot {entry.slot}): tokens and wanted places are lists")
         n_new = len(entry.tokens)
         if n_new == 0:

@@ -208,6 +208,10 @@ def test_arguments_of_the_wrong_type_are_refused_with_a_reason():
         with pytest.raises(GenerationError, match="batch_size is an integer"):
             generate(s, [[1]], 1, batch_size=size)
     assert s.state == {} and s.steps == []
+    import numpy as np
+    listed = generate(ScriptedStepper(), [[1, 2, 3], [4]], 3)
+    arrays = generate(ScriptedStepper(), [np.array([1, 2, 3]), np.array([4], dtype=np.int32)], np.int64(3))
+    assert [r.token_ids for r in arrays] == [r.token_ids for r in listed]      # arrays of token ids are as good as lists
 
 
 # ---- the loop that runs one step ahead of the host ------------------------------------------------
