@@ -111,7 +111,7 @@ def generate(stepper, prompts: list, max_new_tokens, sampling=None, stop_token_i
     params = list(sampling) if isinstance(sampling, (list, tuple)) else [sampling] * n
     if len(max_new) != n or len(params) != n:
         raise GenerationError("one max_new_tokens and one sampling parameter set per prompt")
-    if not isinstance(stop_token_ids, (list, tuple, set, frozenset)) or not all(_whole_number(t) for t in stop_token_ids):
+    if not _token_sequence(stop_token_ids) or not all(_whole_number(t) for t in stop_token_ids):
         raise GenerationError(f"stop_token_ids are a list of token ids, got {stop_token_ids!r}")
     stops = frozenset(int(t) for t in stop_token_ids)
     if batch_size is not None and not _whole_number(batch_size):
