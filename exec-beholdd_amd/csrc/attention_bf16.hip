@@ -415,18 +415,19 @@ __global__ __launch_bounds__(256, (LEAN ? 2 : 1)) void attention_mfma_kernel(
 
 // One block per column.  Nothing here may wait for one split's numbers before asking for the next
 // one's: with 32 splits that is 32 trips to the L2 in a row.  So the lanes of a wave fetch the splits'
-// (maximum, sum) pairs side by side, and the partial outputs are fetched eight splits at a time.
+// (maximum, sum) pairs side by side, and the partial outputs are fetched WIDTH splits at a time (8, or 4 where there are
+// no more); the sums run over the splits in their order either way.
+template <int WIDTH>
 __global__ void attention_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                          uint16_t* __restrict__ out, int n_splits, int HD, int H, int out_block_rows) {
   const size_t column = blockIdx.x;
   const float* ml = part_ml + column * n_splits * 2;
   const int lane = threadIdx.x % BH_WAVE;
-  // the first eight splits' outputs are asked for beside the maxima and sums, not after them
-  float first_part[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  if (threadIdx.x < HD) {
+  // the first splits' outputs are asked for beside the maxima and sums, not after them
+  float first_part[WIDTH];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) first_part[u] = part_o[(column * n_splits + (u < n_splits ? u : n_splits - 1)) * HD + threadIdx.x];
-  }
+  for (int u = 0; u < WIDTH; ++u)
+    first_part[u] = threadIdx.x < HD ? part_o[(column * n_splits + (u < n_splits ? u : n_splits - 1)) * HD + threadIdx.x] : 0.f;
   float top = -INFINITY;
   for (int s = lane; s < n_splits; s += BH_WAVE) top = fmaxf(top, ml[2 * s]);
 #pragma unroll
@@ -438,16 +439,16 @@ __global__ void attention_combine_kernel(const float* __restrict__ part_o, const
   const float inv = 1.0f / sum;
   for (int d = threadIdx.x; d < HD; d += blockDim.x) {
     float value = 0.f;
-    for (int s0 = 0; s0 < n_splits; s0 += 8) {
-      float weight[8], part[8];
+    for (int s0 = 0; s0 < n_splits; s0 += WIDTH) {
+      float weight[WIDTH], part[WIDTH];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
+      for (int u = 0; u < WIDTH; ++u) {
         const int s = s0 + u < n_splits ? s0 + u : n_splits - 1;
         weight[u] = s0 + u < n_splits ? ml[2 * s] : -INFINITY;
         part[u] = (s0 == 0 && d == threadIdx.x) ? first_part[u] : part_o[(column * n_splits + s) * HD + d];
       }
 #pragma unroll
-      for (int u = 0; u < 8; ++u) value += part[u] * exp2f(weight[u] - top);
+      for (int u = 0; u < WIDTH; ++u) value += part[u] * exp2f(weight[u] - top);
     }
     out[bh_rows_index(out_block_rows, (int)(column / H), (int)(column % H) * HD + d, H * HD)] = f32_to_bf16_bits(value * inv);
   }
@@ -561,8 +562,13 @@ static int attention_bf16_run(const void* q, void* out, void* part_o, void* part
 #undef BH_ATT_ONE
   if (int status = bh_check_launch("attention_mfma")) return status;
   if (n_splits > 1) {
-    attention_combine_kernel<<<dim3(n_rows * H), dim3(hd >= 128 ? 128 : 64), 0, stream>>>(
-        (const float*)part_o, (const float*)part_ml, (uint16_t*)out, n_splits, hd, H, out_blocked);
+    const dim3 columns(n_rows * H), threads(hd >= 128 ? 128 : 64);
+    if (n_splits <= 4)
+      attention_combine_kernel<4><<<columns, threads, 0, stream>>>((const float*)part_o, (const float*)part_ml, (uint16_t*)out,
+                                                                   n_splits, hd, H, out_blocked);
+    else
+      attention_combine_kernel<8><<<columns, threads, 0, stream>>>((const float*)part_o, (const float*)part_ml, (uint16_t*)out,
+                                                                   n_splits, hd, H, out_blocked);
     return bh_check_launch("attention_combine");
   }
   return 0;
